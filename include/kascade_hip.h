@@ -1,0 +1,192 @@
+/*
+ * kascade_hip.h -- C ABI of libkascade_hip.so (gfx950 / MI355X).
+ *
+ * One shared library replaces the per-kernel shared objects the reference
+ * builds with tilelang's LibraryGenerator and loads through
+ * JITKernel.from_database (reference src/kernels/kernel_utils.py:15-81).  Each
+ * of those objects exports `int init()`, `int call(<device pointers>, <dims>,
+ * stream)` and `const char* get_last_error()`; this header keeps that
+ * convention: every entry point takes raw device pointers owned by the
+ * caller, plain integer sizes and a stream handle, allocates nothing, returns
+ * 0 on success and -1 on failure, and leaves a message retrievable through
+ * kascade_get_last_error().
+ *
+ * Conventions
+ *   H = 32 query heads, G = 8 KV heads, D = 128, fp16 data, fp32 accumulate,
+ *   prefill tile = 32 queries (the shapes the reference kernels are specialised
+ *   to: EfficientKascadeStrategy.py:19-21).  `stream` is a hipStream_t passed
+ *   as void* (NULL = the default stream).  Index tensors hold logical token ids.
+ *   All softmax arithmetic is in the exp2 domain with
+ *   scale = D^-0.5 * log2(e); log-sum values are log2(sum) + max*scale.
+ *
+ * Paged KV cache (extension of the reference's padded [B, maxL, G, D] cache)
+ *   K/V pages are [num_pages, page_size, G, D] fp16; logical token i of
+ *   sequence b lives in page block_table[b*max_pages + i/page_size], slot
+ *   i % page_size.  page_size must be a power of two.  Passing
+ *   block_table == NULL selects the reference's contiguous layout: K/V are
+ *   [B, kv_stride_tokens, G, D] and token i of sequence b is row
+ *   b*kv_stride_tokens + i.
+ */
+#ifndef KASCADE_HIP_H
+#define KASCADE_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef uint16_t kascade_half; /* IEEE binary16 bit pattern */
+
+/* Replaces `init()` of every reference kernel object (e.g. decode reuse .cu:253-258):
+ * one-time device query and kernel attribute set-up for the current device. */
+int kascade_init(void);
+
+/* Replaces `get_last_error()` (e.g. decode reuse .cu:249-251).  Thread-local buffer. */
+const char* kascade_get_last_error(void);
+
+/* ABI version of this header (bumped on any signature change). */
+int kascade_abi_version(void);
+
+/* Number of compute units of the current device (0 before kascade_init). */
+int kascade_device_cu_count(void);
+
+/* ------------------------------------------------------------------ decode */
+
+/* Reuse-layer decode, contiguous cache.  Same argument list as the reference's
+ * `call` of dynamic_alllen_reuse_cp_async_dim128_gsize4_heads32_groups8.cu:260
+ * (DSL: reuse_kascade_gqa_decode.py:180-191) plus the split count that the
+ * reference fixes at 8 through the shape of its scratch tensors.
+ *   Q [B,H,D]  K,V [B,kv_seqlen,G,D]  topk_indices [B,G,topk] i32
+ *   head_mapping [G] i32  glse [B,H,num_split] f32
+ *   Output_partial [B,H,num_split,D] f32  Output [B,H,D] f16 */
+int kascade_decode_reuse_call(const kascade_half* Q, const kascade_half* K, const kascade_half* V,
+                              const int32_t* topk_indices, const int32_t* head_mapping,
+                              float* glse, float* Output_partial, kascade_half* Output,
+                              int batch, int kv_seqlen, int topk, int num_split, void* stream);
+
+/* Reuse-layer decode over a padded or paged cache with per-sequence lengths.
+ * Argument order follows the reference's kvcache `call`
+ * (dynamic_alllen_reuse_cp_async_dim128_gsize4_heads32_groups8_with_kvcache.cu:249;
+ * DSL reuse_kascade_gqa_decode_with_kvcache.py:160-173) with the block table
+ * added.  Sequence b consumes the first n(b) entries of its index rows,
+ *   n(b) = 128*ceil(floor(topk_percent*cache_seqlens[b]/100)/128)  if topk_percent > 0
+ *   n(b) = topk                                                   otherwise,
+ * clamped to `topk` (the row width of topk_indices).
+ *   block_table [B,max_pages] i32 or NULL (then K,V are [B,kv_stride_tokens,G,D]). */
+int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K,
+                                    const kascade_half* V, const int32_t* cache_seqlens,
+                                    const int32_t* topk_indices, const int32_t* head_mapping,
+                                    float topk_percent, float* glse, float* Output_partial,
+                                    kascade_half* Output, int batch, int kv_stride_tokens,
+                                    int topk, int num_split, const int32_t* block_table,
+                                    int max_pages, int page_size, void* stream);
+
+/* Dense split-K decode (the reference's TileLang dense baseline, gqa_decode.py:117-254 and
+ * gqa_decode_with_kvcache.py:118-257), same cache conventions as above.
+ * cache_seqlens may be NULL (all sequences have kv_stride_tokens tokens). */
+int kascade_decode_dense_paged_call(const kascade_half* Q, const kascade_half* K,
+                                    const kascade_half* V, const int32_t* cache_seqlens,
+                                    float* glse, float* Output_partial, kascade_half* Output,
+                                    int batch, int kv_stride_tokens, int num_split,
+                                    const int32_t* block_table, int max_pages, int page_size,
+                                    void* stream);
+
+/* Anchor-layer decode: split QK^T (+PV when with_output != 0), log-sum merge and
+ * pooled post-softmax scores.  Replaces the three launches of the reference's
+ * flashattn_gqa_decode_split_{0,1} (recompute_kascade_gqa_decode.py:318-348;
+ * kvcache form recompute_kascade_gqa_decode_with_kvcache.py:302-333).
+ *   scores            [B,H,scores_stride] f32 scratch (raw q.k; the reference
+ *                     stores fp16 here, fp32 avoids that extra rounding)
+ *   row_sums          [B,H] f32: global log2-domain log-sum per head
+ *   aggregated_scores [B,G,scores_stride] f16: sum over the 4 heads of a KV head
+ *                     of softmax probabilities; 0 at positions >= cache_seqlens[b]
+ *   Output            [B,H,D] f16, written only when with_output != 0. */
+int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_half* K,
+                                        const kascade_half* V, const int32_t* cache_seqlens,
+                                        float* glse, float* Output_partial, float* row_sums,
+                                        float* scores, kascade_half* Output,
+                                        kascade_half* aggregated_scores, int batch,
+                                        int kv_stride_tokens, int scores_stride, int num_split,
+                                        int with_output, const int32_t* block_table,
+                                        int max_pages, int page_size, void* stream);
+
+/* ------------------------------------------------------------------- top-k */
+
+/* Exact per-row top-n selection over non-negative-or--inf fp16 scores; replaces
+ * the ATen torch.topk call sites (EfficientKascadeStrategy.py:82, 90, 111).
+ *   scores  [rows, row_stride] f16
+ *   out_idx [rows, k] i32
+ * Row r looks at its first valid_len[r % period] entries (valid_len == NULL:
+ * uniform_len) and must select n_sel[r % period] of them (n_sel == NULL: k).
+ * Slots [0, n) receive exactly the n largest entries (ties broken towards the
+ * lower index), ordered by ascending index; when fewer than n entries are valid
+ * all valid ones are emitted followed by the first invalid positions, as
+ * torch.topk does for -inf padding.  Slots [n, k) are set to fill_value.
+ *   workspace: device scratch of at least kascade_topk_workspace_bytes(rows) bytes. */
+int64_t kascade_topk_workspace_bytes(int rows);
+int kascade_topk_call(const kascade_half* scores, int32_t* out_idx, int rows, int64_t row_stride,
+                      int uniform_len, const int32_t* valid_len, const int32_t* n_sel, int period,
+                      int k, int fill_value, void* workspace, void* stream);
+
+/* ----------------------------------------------------------------- prefill */
+
+/* Strides are in elements; the innermost (D) dimension is contiguous.  A tensor
+ * laid out [B,L,H,D] has (s_b, s_l, s_h) = (L*H*D, H*D, D); HF's [B,H,L,D]
+ * seen as [B,L,H,D] has (H*L*D, D, L*D). */
+typedef struct {
+    int64_t b, l, h;
+} kascade_strides;
+
+/* Anchor layer 0: dense causal GQA flash attention that also emits the log2
+ * log-sum per (token, head).  Replaces `prefill`
+ * (recompute_kascade_gqa_prefill.py:225-274).  with_output == 0 gives
+ * `compute_scores` (same file :277-312): log_sum only, V and Output unused.
+ *   Q [B,L,H,D]  K,V [B,L,G,D]  log_sum [B,L,H] f32  Output [B,L,H,D] f16 (contiguous) */
+int kascade_prefill_dense_call(const kascade_half* Q, const kascade_half* K, const kascade_half* V,
+                               float* log_sum, kascade_half* Output, int batch, int seq_len,
+                               kascade_strides q_strides, kascade_strides kv_strides,
+                               int with_output, void* stream);
+
+/* Pooled tile scores.  Same argument list as the reference's aggregate `call`
+ * (dynamic_alllen_aggregate_cp_async_ts32_dim128_gsize4_heads32_groups8.cu:138;
+ * DSL recompute_kascade_gqa_prefill.py:192-222) plus strides and fill_invalid:
+ *   aggregate_scores [B,G,ceil(L/32),L] f16; entry (t, j) for j < 32 t is
+ *   sum over the 32 queries of tile t and the 4 heads of the KV head of
+ *   exp2(q.k*scale - log_sum).  With fill_invalid != 0 the entries j >= 32 t are
+ *   written as -inf (the reference pre-fills the tensor on the host instead). */
+int kascade_prefill_aggregate_call(const kascade_half* Q, const kascade_half* K,
+                                   const float* log_sum, kascade_half* aggregate_scores, int batch,
+                                   int seq_len, kascade_strides q_strides,
+                                   kascade_strides kv_strides, int fill_invalid, void* stream);
+
+/* Reuse-layer prefill.  Same argument list as the reference's reuse `call`s
+ * (…reuse_cp_async_ts32…groups8_rolling.cu:268 and …groups8.cu:260; DSL
+ * reuse_kascade_gqa_prefill.py:147-198) plus strides and the rolling switch that
+ * the reference bakes into two separate objects.
+ *   topk_indices [B,G,ceil(L/32),max_topk_num] i32, head_mapping [G] i32.
+ *   rolling != 0 and seq_len > 128: tile t uses its first
+ *   128*ceil(max(floor(topk_percent*32t/100),128)/128) indices, else max_topk_num. */
+int kascade_prefill_reuse_call(const kascade_half* Q, const kascade_half* K, const kascade_half* V,
+                               const int32_t* topk_indices, const int32_t* head_mapping,
+                               float topk_percent, kascade_half* Output, int batch, int seq_len,
+                               int max_topk_num, int rolling, kascade_strides q_strides,
+                               kascade_strides kv_strides, void* stream);
+
+/* --------------------------------------------------------------- KV append */
+
+/* Writes n_new tokens per sequence into the paged cache at logical positions
+ * start_pos[b] .. start_pos[b]+n_new-1.  The reference has no counterpart (it
+ * re-materialises the whole cache every step: EfficientKascadeStrategy.py:149-150);
+ * this is the step right before the decode path.
+ *   k_new, v_new [B,n_new,G,D] with strides new_strides (b, l, h=g). */
+int kascade_paged_kv_append_call(kascade_half* K_pages, kascade_half* V_pages,
+                                 const kascade_half* k_new, const kascade_half* v_new,
+                                 const int32_t* start_pos, const int32_t* block_table, int batch,
+                                 int n_new, int max_pages, int page_size,
+                                 kascade_strides new_strides, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KASCADE_HIP_H */

@@ -1,0 +1,88 @@
+"""ctypes binding of libkascade_hip.so (the C ABI declared in include/kascade_hip.h).
+
+Loading fails loudly: there is no fallback implementation.  ``load()`` returns
+the library with argument types set; ``check(rc)`` turns a -1 return code into
+a ``KascadeError`` carrying ``kascade_get_last_error()``.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "libkascade_hip.so"
+
+
+class KascadeError(RuntimeError):
+    pass
+
+
+class Strides(C.Structure):
+    """kascade_strides: element strides (b, l, h) of a [B,L,H,D] view."""
+    _fields_ = [("b", C.c_int64), ("l", C.c_int64), ("h", C.c_int64)]
+
+
+_P = C.c_void_p
+_I = C.c_int
+_F = C.c_float
+_L = C.c_int64
+
+# name -> (restype, argtypes); must list every symbol of include/kascade_hip.h
+SIGNATURES = {
+    "kascade_init": (_I, []),
+    "kascade_get_last_error": (C.c_char_p, []),
+    "kascade_abi_version": (_I, []),
+    "kascade_device_cu_count": (_I, []),
+    "kascade_decode_reuse_call": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "kascade_decode_reuse_paged_call": (_I, [_P, _P, _P, _P, _P, _P, _F, _P, _P, _P, _I, _I, _I, _I,
+                                             _P, _I, _I, _P]),
+    "kascade_decode_dense_paged_call": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _I, _I, _P]),
+    "kascade_decode_recompute_paged_call": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I,
+                                                 _I, _I, _P, _I, _I, _P]),
+    "kascade_topk_workspace_bytes": (_L, [_I]),
+    "kascade_topk_call": (_I, [_P, _P, _I, _L, _I, _P, _P, _I, _I, _I, _P, _P]),
+    "kascade_prefill_dense_call": (_I, [_P, _P, _P, _P, _P, _I, _I, Strides, Strides, _I, _P]),
+    "kascade_prefill_aggregate_call": (_I, [_P, _P, _P, _P, _I, _I, Strides, Strides, _I, _P]),
+    "kascade_prefill_reuse_call": (_I, [_P, _P, _P, _P, _P, _F, _P, _I, _I, _I, _I, Strides, Strides,
+                                        _P]),
+    "kascade_paged_kv_append_call": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, Strides, _P]),
+}
+
+_lib = None
+_initialised = False
+
+
+def load() -> C.CDLL:
+    """dlopen the in-tree library and bind every declared symbol."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        raise KascadeError(
+            f"{LIB_PATH} is missing: build it with `python -m kascade_amd.build` "
+            "(there is no fallback path)")
+    lib = C.CDLL(str(LIB_PATH))
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)   # AttributeError if the symbol is not exported
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def last_error() -> str:
+    return load().kascade_get_last_error().decode("utf-8", "replace")
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        raise KascadeError(last_error())
+
+
+def init() -> C.CDLL:
+    """Load the library and run kascade_init() once on the current device."""
+    global _initialised
+    lib = load()
+    if not _initialised:
+        check(lib.kascade_init())
+        _initialised = True
+    return lib

@@ -1,0 +1,292 @@
+// extern "C" entry points of libkascade_hip.so: argument validation, launch
+// sequencing, error reporting.  No allocation happens here; every buffer is the
+// caller's.  Validation failures are reported before anything is launched, so
+// they can be exercised on a machine without a GPU.
+#include "../../include/kascade_hip.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "decode.h"
+#include "paged.h"
+#include "prefill.h"
+#include "topk.h"
+
+using namespace kascade;
+
+namespace {
+
+thread_local char g_err[1024] = "";
+int g_cu_count = 0;
+
+int fail(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return -1;
+}
+
+int check_hip(hipError_t e, const char* what) {
+    if (e == hipSuccess) return 0;
+    return fail("%s: %s", what, hipGetErrorString(e));
+}
+
+#define REQUIRE(cond, ...)                 \
+    do {                                   \
+        if (!(cond)) return fail(__VA_ARGS__); \
+    } while (0)
+
+inline const half_t* H(const kascade_half* p) { return reinterpret_cast<const half_t*>(p); }
+inline half_t* H(kascade_half* p) { return reinterpret_cast<half_t*>(p); }
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+int check_strides(const kascade_strides& s, const char* name) {
+    REQUIRE(s.b % 8 == 0 && s.l % 8 == 0 && s.h % 8 == 0,
+            "%s strides must be multiples of 8 elements (16-byte rows)", name);
+    REQUIRE(s.l > 0 && s.h > 0, "%s strides must be positive", name);
+    return 0;
+}
+
+int check_paging(const int32_t* block_table, int max_pages, int page_size, int* page_shift) {
+    if (!block_table) {
+        *page_shift = 0;
+        return 0;
+    }
+    int sh = ilog2_exact(page_size);
+    REQUIRE(sh >= 0, "page_size must be a power of two, got %d", page_size);
+    REQUIRE(max_pages > 0, "max_pages must be positive with a block table");
+    *page_shift = sh;
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int kascade_abi_version(void) { return 1; }
+
+const char* kascade_get_last_error(void) { return g_err; }
+
+int kascade_device_cu_count(void) { return g_cu_count; }
+
+int kascade_init(void) {
+    int dev = 0;
+    if (check_hip(hipGetDevice(&dev), "hipGetDevice")) return -1;
+    hipDeviceProp_t prop;
+    if (check_hip(hipGetDeviceProperties(&prop, dev), "hipGetDeviceProperties")) return -1;
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail("libkascade_hip is built for gfx950 only; device is %s", prop.gcnArchName);
+    g_cu_count = prop.multiProcessorCount;
+    return 0;
+}
+
+int kascade_decode_reuse_call(const kascade_half* Q, const kascade_half* K, const kascade_half* V,
+                              const int32_t* topk_indices, const int32_t* head_mapping,
+                              float* glse, float* Output_partial, kascade_half* Output, int batch,
+                              int kv_seqlen, int topk, int num_split, void* stream) {
+    return kascade_decode_reuse_paged_call(Q, K, V, nullptr, topk_indices, head_mapping, 0.f, glse,
+                                           Output_partial, Output, batch, kv_seqlen, topk,
+                                           num_split, nullptr, 0, 1, stream);
+}
+
+int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K,
+                                    const kascade_half* V, const int32_t* cache_seqlens,
+                                    const int32_t* topk_indices, const int32_t* head_mapping,
+                                    float topk_percent, float* glse, float* Output_partial,
+                                    kascade_half* Output, int batch, int kv_stride_tokens,
+                                    int topk, int num_split, const int32_t* block_table,
+                                    int max_pages, int page_size, void* stream) {
+    REQUIRE(Q && K && V && topk_indices && head_mapping && glse && Output_partial && Output,
+            "decode_reuse: null pointer argument");
+    REQUIRE(batch > 0 && topk > 0 && num_split > 0, "decode_reuse: batch, topk, num_split must be > 0");
+    REQUIRE(batch <= 65535, "decode_reuse: batch exceeds grid limit");
+    REQUIRE(block_table || kv_stride_tokens > 0, "decode_reuse: kv_stride_tokens must be > 0");
+    REQUIRE(!(topk_percent > 0.f) || cache_seqlens, "decode_reuse: topk_percent needs cache_seqlens");
+    REQUIRE(aligned16(Q) && aligned16(K) && aligned16(V), "decode_reuse: Q/K/V must be 16-byte aligned");
+    int shift;
+    if (check_paging(block_table, max_pages, page_size, &shift)) return -1;
+    DecodeParams p{};
+    p.Q = H(Q); p.K = H(K); p.V = H(V);
+    p.seqlens = cache_seqlens; p.idx = topk_indices; p.head_map = head_mapping;
+    p.block_table = block_table; p.glse = glse; p.opart = Output_partial; p.scores = nullptr;
+    p.max_pages = max_pages; p.page_shift = shift; p.kv_stride_tokens = kv_stride_tokens;
+    p.topk = topk; p.topk_percent = topk_percent; p.scores_stride = 0; p.num_split = num_split;
+    p.B = batch;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (check_hip(launch_decode_split(p, true, true, false, s), "decode_reuse split")) return -1;
+    return check_hip(launch_decode_combine(glse, Output_partial, H(Output), nullptr, batch,
+                                           num_split, true, s), "decode_reuse combine");
+}
+
+int kascade_decode_dense_paged_call(const kascade_half* Q, const kascade_half* K,
+                                    const kascade_half* V, const int32_t* cache_seqlens,
+                                    float* glse, float* Output_partial, kascade_half* Output,
+                                    int batch, int kv_stride_tokens, int num_split,
+                                    const int32_t* block_table, int max_pages, int page_size,
+                                    void* stream) {
+    REQUIRE(Q && K && V && glse && Output_partial && Output, "decode_dense: null pointer argument");
+    REQUIRE(batch > 0 && num_split > 0, "decode_dense: batch, num_split must be > 0");
+    REQUIRE(batch <= 65535, "decode_dense: batch exceeds grid limit");
+    REQUIRE(cache_seqlens || kv_stride_tokens > 0, "decode_dense: need cache_seqlens or kv_stride_tokens");
+    REQUIRE(block_table || kv_stride_tokens > 0, "decode_dense: kv_stride_tokens must be > 0");
+    REQUIRE(aligned16(Q) && aligned16(K) && aligned16(V), "decode_dense: Q/K/V must be 16-byte aligned");
+    int shift;
+    if (check_paging(block_table, max_pages, page_size, &shift)) return -1;
+    DecodeParams p{};
+    p.Q = H(Q); p.K = H(K); p.V = H(V);
+    p.seqlens = cache_seqlens; p.block_table = block_table; p.glse = glse; p.opart = Output_partial;
+    p.max_pages = max_pages; p.page_shift = shift; p.kv_stride_tokens = kv_stride_tokens;
+    p.num_split = num_split; p.B = batch;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (check_hip(launch_decode_split(p, false, true, false, s), "decode_dense split")) return -1;
+    return check_hip(launch_decode_combine(glse, Output_partial, H(Output), nullptr, batch,
+                                           num_split, true, s), "decode_dense combine");
+}
+
+int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_half* K,
+                                        const kascade_half* V, const int32_t* cache_seqlens,
+                                        float* glse, float* Output_partial, float* row_sums,
+                                        float* scores, kascade_half* Output,
+                                        kascade_half* aggregated_scores, int batch,
+                                        int kv_stride_tokens, int scores_stride, int num_split,
+                                        int with_output, const int32_t* block_table,
+                                        int max_pages, int page_size, void* stream) {
+    REQUIRE(Q && K && glse && row_sums && scores && aggregated_scores,
+            "decode_recompute: null pointer argument");
+    REQUIRE(!with_output || (V && Output && Output_partial),
+            "decode_recompute: with_output needs V, Output and Output_partial");
+    REQUIRE(batch > 0 && num_split > 0 && scores_stride > 0,
+            "decode_recompute: batch, num_split, scores_stride must be > 0");
+    REQUIRE(batch <= 65535, "decode_recompute: batch exceeds grid limit");
+    REQUIRE(cache_seqlens || (kv_stride_tokens > 0 && kv_stride_tokens <= scores_stride),
+            "decode_recompute: without cache_seqlens need 0 < kv_stride_tokens <= scores_stride");
+    REQUIRE(block_table || kv_stride_tokens > 0, "decode_recompute: kv_stride_tokens must be > 0");
+    REQUIRE(aligned16(Q) && aligned16(K) && (!with_output || aligned16(V)),
+            "decode_recompute: Q/K/V must be 16-byte aligned");
+    REQUIRE(aligned16(scores) && aligned16(aggregated_scores),
+            "decode_recompute: scores buffers must be 16-byte aligned");
+    int shift;
+    if (check_paging(block_table, max_pages, page_size, &shift)) return -1;
+    DecodeParams p{};
+    p.Q = H(Q); p.K = H(K); p.V = with_output ? H(V) : H(K);
+    p.seqlens = cache_seqlens; p.block_table = block_table; p.glse = glse; p.opart = Output_partial;
+    p.scores = scores; p.scores_stride = scores_stride;
+    p.max_pages = max_pages; p.page_shift = shift; p.kv_stride_tokens = kv_stride_tokens;
+    p.num_split = num_split; p.B = batch;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (check_hip(launch_decode_split(p, false, with_output != 0, true, s), "decode_recompute split"))
+        return -1;
+    if (check_hip(launch_decode_combine(glse, Output_partial, H(Output), row_sums, batch, num_split,
+                                        with_output != 0, s), "decode_recompute combine"))
+        return -1;
+    return check_hip(launch_decode_aggregate(scores, row_sums, cache_seqlens, H(aggregated_scores),
+                                             batch, scores_stride, kv_stride_tokens, s),
+                     "decode_recompute aggregate");
+}
+
+int64_t kascade_topk_workspace_bytes(int rows) {
+    (void)rows;
+    return 0;  // the single-workgroup-per-row selection keeps all state in LDS
+}
+
+int kascade_topk_call(const kascade_half* scores, int32_t* out_idx, int rows, int64_t row_stride,
+                      int uniform_len, const int32_t* valid_len, const int32_t* n_sel, int period,
+                      int k, int fill_value, void* workspace, void* stream) {
+    (void)workspace;
+    REQUIRE(scores && out_idx, "topk: null pointer argument");
+    REQUIRE(rows >= 0 && k > 0 && row_stride > 0, "topk: rows >= 0, k > 0, row_stride > 0 required");
+    REQUIRE(valid_len || (uniform_len >= 0 && uniform_len <= row_stride),
+            "topk: uniform_len must be within [0, row_stride]");
+    REQUIRE(!(valid_len || n_sel) || period > 0, "topk: period must be > 0 with per-row arrays");
+    if (period <= 0) period = 1;
+    return check_hip(launch_topk(H(scores), out_idx, rows, row_stride, uniform_len, valid_len, n_sel,
+                                 period, k, fill_value, static_cast<hipStream_t>(stream)),
+                     "topk");
+}
+
+int kascade_prefill_dense_call(const kascade_half* Q, const kascade_half* K, const kascade_half* V,
+                               float* log_sum, kascade_half* Output, int batch, int seq_len,
+                               kascade_strides q_strides, kascade_strides kv_strides,
+                               int with_output, void* stream) {
+    REQUIRE(Q && K, "prefill_dense: null pointer argument");
+    REQUIRE(!with_output || (V && Output), "prefill_dense: with_output needs V and Output");
+    REQUIRE(with_output || log_sum, "prefill_dense: nothing to compute (no Output, no log_sum)");
+    REQUIRE(batch > 0 && seq_len > 0 && batch <= 65535, "prefill_dense: bad batch/seq_len");
+    REQUIRE(aligned16(Q) && aligned16(K) && (!with_output || (aligned16(V) && aligned16(Output))),
+            "prefill_dense: tensors must be 16-byte aligned");
+    if (check_strides(q_strides, "Q") || check_strides(kv_strides, "K/V")) return -1;
+    PrefillParams p{};
+    p.Q = H(Q); p.K = H(K); p.V = with_output ? H(V) : H(K); p.log_sum = log_sum; p.O = H(Output);
+    p.q_sb = q_strides.b; p.q_sl = q_strides.l; p.q_sh = q_strides.h;
+    p.k_sb = kv_strides.b; p.k_sl = kv_strides.l; p.k_sh = kv_strides.h;
+    p.B = batch; p.L = seq_len; p.T = (seq_len + kTile - 1) / kTile;
+    return check_hip(launch_prefill_attn(p, false, with_output != 0, 2,
+                                         static_cast<hipStream_t>(stream)), "prefill_dense");
+}
+
+int kascade_prefill_aggregate_call(const kascade_half* Q, const kascade_half* K,
+                                   const float* log_sum, kascade_half* aggregate_scores, int batch,
+                                   int seq_len, kascade_strides q_strides,
+                                   kascade_strides kv_strides, int fill_invalid, void* stream) {
+    REQUIRE(Q && K && log_sum && aggregate_scores, "prefill_aggregate: null pointer argument");
+    REQUIRE(batch > 0 && seq_len > 0 && batch <= 65535, "prefill_aggregate: bad batch/seq_len");
+    REQUIRE(aligned16(Q) && aligned16(K), "prefill_aggregate: Q/K must be 16-byte aligned");
+    if (check_strides(q_strides, "Q") || check_strides(kv_strides, "K")) return -1;
+    PrefillParams p{};
+    p.Q = H(Q); p.K = H(K); p.V = H(K); p.log_sum_in = log_sum; p.agg = H(aggregate_scores);
+    p.q_sb = q_strides.b; p.q_sl = q_strides.l; p.q_sh = q_strides.h;
+    p.k_sb = kv_strides.b; p.k_sl = kv_strides.l; p.k_sh = kv_strides.h;
+    p.B = batch; p.L = seq_len; p.T = (seq_len + kTile - 1) / kTile; p.fill_invalid = fill_invalid;
+    return check_hip(launch_prefill_aggregate(p, static_cast<hipStream_t>(stream)),
+                     "prefill_aggregate");
+}
+
+int kascade_prefill_reuse_call(const kascade_half* Q, const kascade_half* K, const kascade_half* V,
+                               const int32_t* topk_indices, const int32_t* head_mapping,
+                               float topk_percent, kascade_half* Output, int batch, int seq_len,
+                               int max_topk_num, int rolling, kascade_strides q_strides,
+                               kascade_strides kv_strides, void* stream) {
+    REQUIRE(Q && K && V && topk_indices && head_mapping && Output,
+            "prefill_reuse: null pointer argument");
+    REQUIRE(batch > 0 && seq_len > 0 && batch <= 65535, "prefill_reuse: bad batch/seq_len");
+    REQUIRE(max_topk_num > 0, "prefill_reuse: max_topk_num must be > 0");
+    REQUIRE(!rolling || topk_percent > 0.f, "prefill_reuse: rolling needs topk_percent > 0");
+    REQUIRE(aligned16(Q) && aligned16(K) && aligned16(V) && aligned16(Output),
+            "prefill_reuse: tensors must be 16-byte aligned");
+    if (check_strides(q_strides, "Q") || check_strides(kv_strides, "K/V")) return -1;
+    PrefillParams p{};
+    p.Q = H(Q); p.K = H(K); p.V = H(V); p.idx = topk_indices; p.head_map = head_mapping;
+    p.O = H(Output); p.log_sum = nullptr;
+    p.q_sb = q_strides.b; p.q_sl = q_strides.l; p.q_sh = q_strides.h;
+    p.k_sb = kv_strides.b; p.k_sl = kv_strides.l; p.k_sh = kv_strides.h;
+    p.B = batch; p.L = seq_len; p.T = (seq_len + kTile - 1) / kTile;
+    p.max_topk = max_topk_num; p.rolling = rolling; p.topk_percent = topk_percent;
+    return check_hip(launch_prefill_attn(p, true, true, 1, static_cast<hipStream_t>(stream)),
+                     "prefill_reuse");
+}
+
+int kascade_paged_kv_append_call(kascade_half* K_pages, kascade_half* V_pages,
+                                 const kascade_half* k_new, const kascade_half* v_new,
+                                 const int32_t* start_pos, const int32_t* block_table, int batch,
+                                 int n_new, int max_pages, int page_size,
+                                 kascade_strides new_strides, void* stream) {
+    REQUIRE(K_pages && V_pages && k_new && v_new && start_pos && block_table,
+            "paged_kv_append: null pointer argument");
+    REQUIRE(batch > 0 && n_new >= 0, "paged_kv_append: bad batch/n_new");
+    int shift;
+    if (check_paging(block_table, max_pages, page_size, &shift)) return -1;
+    REQUIRE(new_strides.b % 8 == 0 && new_strides.l % 8 == 0 && new_strides.h % 8 == 0,
+            "paged_kv_append: strides must be multiples of 8 elements");
+    REQUIRE(aligned16(K_pages) && aligned16(V_pages) && aligned16(k_new) && aligned16(v_new),
+            "paged_kv_append: tensors must be 16-byte aligned");
+    return check_hip(launch_paged_kv_append(H(K_pages), H(V_pages), H(k_new), H(v_new), start_pos,
+                                            block_table, batch, n_new, max_pages, shift,
+                                            new_strides.b, new_strides.l, new_strides.h,
+                                            static_cast<hipStream_t>(stream)),
+                     "paged_kv_append");
+}
+
+}  // extern "C"

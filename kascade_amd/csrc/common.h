@@ -1,0 +1,62 @@
+// Shared device/host helpers for the gfx950 kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace kascade {
+
+constexpr int kHeads = 32;     // query heads
+constexpr int kGroups = 8;     // KV heads
+constexpr int kGroupSize = 4;  // query heads per KV head
+constexpr int kDim = 128;      // head dimension
+constexpr int kTile = 32;      // prefill query tile
+// D^-0.5 * log2(e): softmax is evaluated as exp2(s*kScaleLog2 - m*kScaleLog2)
+constexpr float kScaleLog2 = 0.12751743082459868f;
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+
+union Pack16 {  // one 16-byte global/LDS transaction seen as 8 halves
+    uint4_t u;
+    half8_t h8;
+    half2_t h2[4];
+    half_t h[8];
+};
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// Sum over the 16 lanes of a DPP row; every lane of the row receives the total.
+__device__ __forceinline__ float row16_sum(float x) {
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, false));   // quad_perm [1,0,3,2]
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, false));   // quad_perm [2,3,0,1]
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x141, 0xF, 0xF, false));  // row_half_mirror
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x140, 0xF, 0xF, false));  // row_mirror
+    return x;
+}
+
+__device__ __forceinline__ float dot8(const Pack16& a, const Pack16& b, float acc) {
+    acc = __builtin_amdgcn_fdot2(a.h2[0], b.h2[0], acc, false);
+    acc = __builtin_amdgcn_fdot2(a.h2[1], b.h2[1], acc, false);
+    acc = __builtin_amdgcn_fdot2(a.h2[2], b.h2[2], acc, false);
+    acc = __builtin_amdgcn_fdot2(a.h2[3], b.h2[3], acc, false);
+    return acc;
+}
+
+__device__ __forceinline__ uint4_t ld_global_16(const void* p) {
+    return *reinterpret_cast<const uint4_t*>(p);
+}
+
+inline int ilog2_exact(int x) {  // host: log2 of a power of two, -1 otherwise
+    if (x <= 0 || (x & (x - 1))) return -1;
+    int s = 0;
+    while ((1 << s) < x) ++s;
+    return s;
+}
+
+}  // namespace kascade

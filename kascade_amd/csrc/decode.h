@@ -1,0 +1,37 @@
+// Host-visible launchers of the decode kernels (decode.hip).
+#pragma once
+#include "common.h"
+
+namespace kascade {
+
+struct DecodeParams {
+    const half_t* Q;        // [B,H,D]
+    const half_t* K;        // pages [P,page,G,D] or contiguous [B,stride,G,D]
+    const half_t* V;
+    const int* seqlens;     // [B] or null
+    const int* idx;         // [B,G,topk] logical token ids (gather mode)
+    const int* head_map;    // [G] (gather mode)
+    const int* block_table; // [B,max_pages] or null
+    float* glse;            // [B,H,num_split]
+    float* opart;           // [B,H,num_split,D]
+    float* scores;          // [B,H,scores_stride] raw q.k (anchor mode)
+    int max_pages;
+    int page_shift;
+    int kv_stride_tokens;
+    int topk;
+    float topk_percent;
+    int scores_stride;
+    int num_split;
+    int B;
+};
+
+hipError_t launch_decode_split(const DecodeParams& p, bool gather, bool with_v, bool write_scores,
+                               hipStream_t stream);
+hipError_t launch_decode_combine(const float* glse, const float* opart, half_t* out,
+                                 float* row_sums, int batch, int num_split, bool with_v,
+                                 hipStream_t stream);
+hipError_t launch_decode_aggregate(const float* scores, const float* row_sums, const int* seqlens,
+                                   half_t* agg, int batch, int scores_stride, int uniform_len,
+                                   hipStream_t stream);
+
+}  // namespace kascade

@@ -1,0 +1,355 @@
+// Decode-step attention kernels for gfx950: bandwidth-bound split-K streaming of
+// K/V rows (gathered through a top-k index list, or dense), log-sum merge, and
+// pooled post-softmax scores for anchor layers.
+//
+// Work decomposition (one launch = all sequences, KV heads and splits):
+//   grid  (num_split, G, B), 256 threads = 4 wavefronts.
+//   A wavefront is four row-groups of 16 lanes; lane d-slice dl = lane%16 owns
+//   halves [8*dl, 8*dl+8) of every row it touches, so one 16-byte load per lane
+//   fetches four complete 256-byte K (or V) rows per wavefront instruction.
+//   Each row-group keeps an independent online-softmax state (max, sum, 4x8
+//   output accumulators per lane); the 16 states of a workgroup are merged once
+//   at the end, the splits by the combine kernel.
+//   q.k dot products run on v_dot2_f32_f16 + a 4-step DPP row reduction; p.v on
+//   fp32 FMAs.  2 flop/byte is far below the machine balance, so no MFMA here.
+#include "decode.h"
+
+namespace kascade {
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 8;                    // rows per row-group per iteration
+constexpr int kRowsPerIter = 16 * kUnroll;    // rows per workgroup iteration (128)
+constexpr int kSubChunk = 2048;               // rows whose physical ids are staged in LDS at once
+
+struct MergeState {  // one per wavefront after the in-wave merge
+    float m[kGroupSize];
+    float l[kGroupSize];
+    float acc[kGroupSize][kDim];
+};
+
+template <bool GATHER, bool WITH_V, bool WRITE_SCORES>
+__global__ __launch_bounds__(kThreads) void decode_split_kernel(DecodeParams p) {
+    __shared__ int s_row[kSubChunk];
+    __shared__ MergeState s_merge[4];
+
+    const int split = blockIdx.x;
+    const int g = blockIdx.y;
+    const int b = blockIdx.z;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int rg = lane >> 4;   // row group within the wavefront
+    const int dl = lane & 15;   // 16-byte slice of the 256-byte row
+
+    const int seqlen = p.seqlens ? p.seqlens[b] : p.kv_stride_tokens;
+    int n;  // rows this (b, g) pair attends to
+    if (GATHER) {
+        if (p.topk_percent > 0.f) {
+            long long fl = (long long)floor((double)p.topk_percent * (double)seqlen / 100.0);
+            n = (int)(((fl + 127) / 128) * 128);
+        } else {
+            n = p.topk;
+        }
+        n = min(n, p.topk);
+    } else {
+        n = seqlen;
+    }
+    // contiguous range of this split, multiple of 64 rows
+    int rps = (n + p.num_split - 1) / p.num_split;
+    rps = ((rps + 63) / 64) * 64;
+    const long long r0l = (long long)split * rps;
+    const int r0 = (int)min((long long)n, r0l);
+    const int r1 = (int)min((long long)n, r0l + rps);
+
+    // q fragments: 4 heads x 8 halves of this lane's d-slice
+    Pack16 qf[kGroupSize];
+#pragma unroll
+    for (int h = 0; h < kGroupSize; ++h)
+        qf[h].u = ld_global_16(p.Q + ((size_t)b * kHeads + g * kGroupSize + h) * kDim + dl * 8);
+
+    float m[kGroupSize], l[kGroupSize], acc[kGroupSize][8];
+#pragma unroll
+    for (int h = 0; h < kGroupSize; ++h) {
+        m[h] = -INFINITY;
+        l[h] = 0.f;
+#pragma unroll
+        for (int d = 0; d < 8; ++d) acc[h][d] = 0.f;
+    }
+
+    const int* idx_row = nullptr;
+    if (GATHER) idx_row = p.idx + ((size_t)b * kGroups + p.head_map[g]) * p.topk;
+    const int page_mask = (1 << p.page_shift) - 1;
+    const size_t head_off = (size_t)g * kDim + dl * 8;
+
+    for (int c0 = r0; c0 < r1; c0 += kSubChunk) {
+        const int cn = min(kSubChunk, r1 - c0);
+        __syncthreads();
+        // stage physical row ids of this sub-chunk
+        for (int i = tid; i < cn; i += kThreads) {
+            int tok = GATHER ? idx_row[c0 + i] : (c0 + i);
+            int row;
+            if (p.block_table) {
+                int pg = p.block_table[(size_t)b * p.max_pages + (tok >> p.page_shift)];
+                row = (pg << p.page_shift) + (tok & page_mask);
+            } else {
+                row = b * p.kv_stride_tokens + tok;
+            }
+            s_row[i] = row;
+        }
+        __syncthreads();
+
+        for (int it = 0; it < cn; it += kRowsPerIter) {
+            // wave covers 32 consecutive rows of the iteration: row = it + wave*32 + u*4 + rg
+            const int rbase = it + wave * 32 + rg;
+            Pack16 kf[kUnroll];
+            Pack16 vf[kUnroll];
+            bool valid[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                int r = rbase + u * 4;
+                valid[u] = r < cn;
+                int row = s_row[valid[u] ? r : (cn - 1)];
+                size_t off = (size_t)row * (kGroups * kDim) + head_off;
+                kf[u].u = ld_global_16(p.K + off);
+                if (WITH_V) vf[u].u = ld_global_16(p.V + off);
+            }
+            float s[kUnroll][kGroupSize];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+                for (int h = 0; h < kGroupSize; ++h) {
+                    float d = dot8(kf[u], qf[h], 0.f);
+                    d = row16_sum(d);
+                    s[u][h] = valid[u] ? d : -INFINITY;
+                }
+            }
+            if (WRITE_SCORES) {
+                // lanes dl < 8 write the four heads of row u = dl: for a fixed head the
+                // wavefront stores 32 consecutive tokens.
+                float w[kGroupSize] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+                    for (int h = 0; h < kGroupSize; ++h) w[h] = (u == dl) ? s[u][h] : w[h];
+                }
+                const int r = rbase + dl * 4;
+                if (dl < kUnroll && r < cn) {
+                    const int tok = c0 + r;  // dense mode only: token id == row number
+                    float* sp = p.scores + ((size_t)b * kHeads + g * kGroupSize) * p.scores_stride + tok;
+#pragma unroll
+                    for (int h = 0; h < kGroupSize; ++h) sp[(size_t)h * p.scores_stride] = w[h];
+                }
+            }
+#pragma unroll
+            for (int h = 0; h < kGroupSize; ++h) {
+                float mx = m[h];
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u) mx = fmaxf(mx, s[u][h]);
+                const float mref = (mx == -INFINITY) ? 0.f : mx * kScaleLog2;
+                const float corr = fast_exp2(m[h] * kScaleLog2 - mref);  // m=-inf -> 0
+                m[h] = mx;
+                float ps[kUnroll];
+                float sum = 0.f;
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u) {
+                    ps[u] = fast_exp2(s[u][h] * kScaleLog2 - mref);
+                    sum += ps[u];
+                }
+                l[h] = l[h] * corr + sum;
+                if (WITH_V) {
+#pragma unroll
+                    for (int d = 0; d < 8; ++d) {
+                        float a = acc[h][d] * corr;
+#pragma unroll
+                        for (int u = 0; u < kUnroll; ++u) a = fmaf(ps[u], (float)vf[u].h[d], a);
+                        acc[h][d] = a;
+                    }
+                }
+            }
+        }
+    }
+
+    // ---- merge the four row-groups of the wavefront (lanes l, l^16, l^32) ----
+#pragma unroll
+    for (int h = 0; h < kGroupSize; ++h) {
+#pragma unroll
+        for (int sh = 16; sh <= 32; sh <<= 1) {
+            float mo = __shfl_xor(m[h], sh);
+            float lo = __shfl_xor(l[h], sh);
+            float mx = fmaxf(m[h], mo);
+            float mref = (mx == -INFINITY) ? 0.f : mx * kScaleLog2;
+            float ca = fast_exp2(m[h] * kScaleLog2 - mref);
+            float cb = fast_exp2(mo * kScaleLog2 - mref);
+            l[h] = l[h] * ca + lo * cb;
+            if (WITH_V) {
+#pragma unroll
+                for (int d = 0; d < 8; ++d) {
+                    float ao = __shfl_xor(acc[h][d], sh);
+                    acc[h][d] = acc[h][d] * ca + ao * cb;
+                }
+            }
+            m[h] = mx;
+        }
+    }
+    if (rg == 0) {
+#pragma unroll
+        for (int h = 0; h < kGroupSize; ++h) {
+            if (dl == 0) {
+                s_merge[wave].m[h] = m[h];
+                s_merge[wave].l[h] = l[h];
+            }
+            if (WITH_V) {
+#pragma unroll
+                for (int d = 0; d < 8; ++d) s_merge[wave].acc[h][dl * 8 + d] = acc[h][d];
+            }
+        }
+    }
+    __syncthreads();
+    // ---- merge the four wavefronts; thread -> (head, two d's) ----
+    {
+        const int h = tid >> 6;
+        const int d0 = (tid & 63) * 2;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) mx = fmaxf(mx, s_merge[w].m[h]);
+        const float mref = (mx == -INFINITY) ? 0.f : mx * kScaleLog2;
+        float L = 0.f, o0 = 0.f, o1 = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            float c = fast_exp2(s_merge[w].m[h] * kScaleLog2 - mref);
+            L += s_merge[w].l[h] * c;
+            if (WITH_V) {
+                o0 += s_merge[w].acc[h][d0] * c;
+                o1 += s_merge[w].acc[h][d0 + 1] * c;
+            }
+        }
+        const size_t ph = ((size_t)b * kHeads + g * kGroupSize + h) * p.num_split + split;
+        if ((tid & 63) == 0) p.glse[ph] = (L > 0.f) ? (fast_log2(L) + mref) : -INFINITY;
+        if (WITH_V) {
+            const float inv = (L > 0.f) ? 1.f / L : 0.f;
+            float2 o = make_float2(o0 * inv, o1 * inv);
+            *reinterpret_cast<float2*>(p.opart + ph * kDim + d0) = o;
+        }
+    }
+}
+
+// Merge the per-split log-sums (and partial outputs) of one (b, head).
+// grid (H, B), 128 threads = one per output dimension.
+template <bool WITH_V>
+__global__ __launch_bounds__(128) void decode_combine_kernel(const float* __restrict__ glse,
+                                                            const float* __restrict__ opart,
+                                                            half_t* __restrict__ out,
+                                                            float* __restrict__ row_sums,
+                                                            int num_split) {
+    const int h = blockIdx.x;
+    const int b = blockIdx.y;
+    const int d = threadIdx.x;
+    const size_t base = ((size_t)b * kHeads + h) * num_split;
+    float mx = -INFINITY;
+    for (int s = 0; s < num_split; ++s) mx = fmaxf(mx, glse[base + s]);
+    const float mref = (mx == -INFINITY) ? 0.f : mx;
+    float sum = 0.f;
+    for (int s = 0; s < num_split; ++s) sum += fast_exp2(glse[base + s] - mref);
+    const float lse = (sum > 0.f) ? fast_log2(sum) + mref : -INFINITY;
+    if (row_sums && d == 0) row_sums[(size_t)b * kHeads + h] = lse;
+    if (WITH_V) {
+        float o = 0.f;
+        for (int s = 0; s < num_split; ++s) {
+            float w = fast_exp2(glse[base + s] - ((lse == -INFINITY) ? 0.f : lse));
+            if (w > 0.f) o += w * opart[(base + s) * kDim + d];
+        }
+        out[((size_t)b * kHeads + h) * kDim + d] = (half_t)o;
+    }
+}
+
+// agg[b,g,j] = fp16( sum_h exp2(s[b,4g+h,j]*scale - lse[b,4g+h]) ), 0 beyond the sequence.
+// grid (ceil(stride/2048), G, B), 256 threads x 8 tokens.
+__global__ __launch_bounds__(256) void decode_aggregate_kernel(const float* __restrict__ scores,
+                                                              const float* __restrict__ row_sums,
+                                                              const int* __restrict__ seqlens,
+                                                              half_t* __restrict__ agg,
+                                                              int scores_stride, int uniform_len) {
+    const int g = blockIdx.y;
+    const int b = blockIdx.z;
+    const int len = seqlens ? seqlens[b] : uniform_len;
+    const int j0 = (blockIdx.x * 256 + threadIdx.x) * 8;
+    if (j0 >= scores_stride) return;
+    float lse[kGroupSize];
+#pragma unroll
+    for (int h = 0; h < kGroupSize; ++h) lse[h] = row_sums[(size_t)b * kHeads + g * kGroupSize + h];
+    float sum[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sum[e] = 0.f;
+    const bool full = (j0 + 8 <= scores_stride) && ((scores_stride & 3) == 0);
+#pragma unroll
+    for (int h = 0; h < kGroupSize; ++h) {
+        const float* sp = scores + ((size_t)b * kHeads + g * kGroupSize + h) * scores_stride + j0;
+        float v[8];
+        if (full && j0 + 8 <= len) {
+            float4 a = *reinterpret_cast<const float4*>(sp);
+            float4 c = *reinterpret_cast<const float4*>(sp + 4);
+            v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+            v[4] = c.x; v[5] = c.y; v[6] = c.z; v[7] = c.w;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = (j0 + e < len) ? sp[e] : -INFINITY;
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sum[e] += fast_exp2(v[e] * kScaleLog2 - lse[h]);
+    }
+    half_t* ap = agg + ((size_t)b * kGroups + g) * scores_stride + j0;
+    if (full && ((scores_stride & 7) == 0)) {
+        Pack16 o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o.h[e] = (j0 + e < len) ? (half_t)sum[e] : (half_t)0.f;
+        *reinterpret_cast<uint4_t*>(ap) = o.u;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            if (j0 + e < scores_stride) ap[e] = (j0 + e < len) ? (half_t)sum[e] : (half_t)0.f;
+    }
+}
+
+}  // namespace
+
+hipError_t launch_decode_split(const DecodeParams& p, bool gather, bool with_v, bool write_scores,
+                               hipStream_t stream) {
+    dim3 grid(p.num_split, kGroups, p.B), block(kThreads);
+    if (gather) {
+        hipLaunchKernelGGL((decode_split_kernel<true, true, false>), grid, block, 0, stream, p);
+    } else if (write_scores) {
+        if (with_v)
+            hipLaunchKernelGGL((decode_split_kernel<false, true, true>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((decode_split_kernel<false, false, true>), grid, block, 0, stream, p);
+    } else {
+        hipLaunchKernelGGL((decode_split_kernel<false, true, false>), grid, block, 0, stream, p);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_decode_combine(const float* glse, const float* opart, half_t* out,
+                                 float* row_sums, int batch, int num_split, bool with_v,
+                                 hipStream_t stream) {
+    dim3 grid(kHeads, batch), block(128);
+    if (with_v)
+        hipLaunchKernelGGL((decode_combine_kernel<true>), grid, block, 0, stream, glse, opart, out,
+                           row_sums, num_split);
+    else
+        hipLaunchKernelGGL((decode_combine_kernel<false>), grid, block, 0, stream, glse, opart, out,
+                           row_sums, num_split);
+    return hipGetLastError();
+}
+
+hipError_t launch_decode_aggregate(const float* scores, const float* row_sums, const int* seqlens,
+                                   half_t* agg, int batch, int scores_stride, int uniform_len,
+                                   hipStream_t stream) {
+    dim3 grid((scores_stride + 2047) / 2048, kGroups, batch), block(256);
+    hipLaunchKernelGGL(decode_aggregate_kernel, grid, block, 0, stream, scores, row_sums, seqlens,
+                       agg, scores_stride, uniform_len);
+    return hipGetLastError();
+}
+
+}  // namespace kascade

@@ -1,0 +1,12 @@
+// Host-visible launcher of the paged KV append kernel (paged.hip).
+#pragma once
+#include "common.h"
+
+namespace kascade {
+
+hipError_t launch_paged_kv_append(half_t* Kp, half_t* Vp, const half_t* k_new, const half_t* v_new,
+                                  const int* start_pos, const int* block_table, int batch,
+                                  int n_new, int max_pages, int page_shift, long long sb,
+                                  long long sl, long long sh, hipStream_t stream);
+
+}  // namespace kascade

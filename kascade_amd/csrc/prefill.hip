@@ -1,0 +1,435 @@
+// Prefill attention kernels for gfx950 (fp16 MFMA 32x32x16, fp32 softmax).
+//
+// prefill_attn_kernel -- flash attention over one (query block, KV head, batch)
+//   per workgroup; 4 wavefronts, wavefront w owns q-head 4g+w and 32*NQB queries,
+//   so the four heads of a KV head share every K/V tile staged in LDS.
+//   Three key regimes (REUSE): dense causal, gathered top-k rows through the
+//   tile's index list, and the within-tile causal diagonal.
+//
+//   The kernel works on S^T = K Q^T so that each lane owns one query column:
+//   row max / row sum are in-lane reductions plus one cross-half exchange, and
+//   the exponentiated scores are already in the B-operand layout of the second
+//   product O^T = V^T P^T -- P never leaves registers.  K rows are stored in LDS
+//   at a bit-swapped slot (bits 2 and 3 exchanged) which makes the accumulator
+//   registers of one lane cover 8 consecutive key positions, i.e. one 16-byte
+//   read of the transposed V tile per MFMA operand.  V is transposed on its way
+//   into LDS (4 keys x 8 d per thread, eight 8-byte writes) with a 16-byte-chunk
+//   XOR swizzle that keeps both the transposing writes and the operand reads
+//   spread over the banks.
+//
+// prefill_aggregate_kernel -- pooled tile scores: S = Q_tile K^T with the 128
+//   (query, head) rows of a tile held as A operands in registers by every
+//   wavefront; each wavefront takes 32 keys of a 128-key tile, so pooling over
+//   rows is an in-lane sum over accumulator registers.
+#include "prefill.h"
+
+namespace kascade {
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kKT = 64;            // keys per tile (attention kernel)
+constexpr int kKStride = 136;      // halves per K row in LDS (128 + 8 pad)
+constexpr int kAggKT = 128;        // keys per tile (aggregate kernel)
+
+__device__ __forceinline__ int swap_bits23(int x) {
+    return (x & ~0xC) | ((x & 4) << 1) | ((x & 8) >> 1);
+}
+
+__device__ __forceinline__ int rolling_budget(float pct, int tile_start) {
+    long long fl = (long long)floor((double)pct * (double)tile_start / 100.0);
+    if (fl < 128) fl = 128;
+    return (int)(((fl + 127) / 128) * 128);
+}
+
+template <int NQB, bool REUSE, bool WITH_V>
+__global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillParams p) {
+    __shared__ __attribute__((aligned(16))) half_t sK[kKT * kKStride];
+    __shared__ __attribute__((aligned(16))) half_t sV[kDim * kKT];
+
+    constexpr int QT = 32 * NQB;
+    const int L = p.L;
+    const int nqt = (L + QT - 1) / QT;
+    const int tq = nqt - 1 - (int)blockIdx.x;   // long (late) query blocks first
+    const int g = blockIdx.y;
+    const int b = blockIdx.z;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int li = lane & 31;
+    const int lg = lane >> 5;
+    const int q0 = tq * QT;
+    const int head = g * kGroupSize + wave;
+
+    // ---- Q fragments (B operand of S^T): query li (+32 qb), d chunk 16*ks + 8*lg ----
+    half8_t qf[NQB][8];
+#pragma unroll
+    for (int qb = 0; qb < NQB; ++qb) {
+        const int q = q0 + 32 * qb + li;
+        const bool ok = q < L;
+        const half_t* qp = p.Q + (long long)b * p.q_sb + (long long)min(q, L - 1) * p.q_sl +
+                           (long long)head * p.q_sh + lg * 8;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            Pack16 t;
+            t.u = ld_global_16(qp + ks * 16);
+            if (!ok) t.u = uint4_t{0, 0, 0, 0};
+            qf[qb][ks] = t.h8;
+        }
+    }
+
+    // ---- key regime of this block ----
+    bool sparse = false;
+    int n = 0, ng = 0;
+    const int* idx_row = nullptr;
+    if (REUSE) {
+        n = (p.rolling && L > 128) ? rolling_budget(p.topk_percent, q0) : p.max_topk;
+        n = min(n, p.max_topk);
+        if (q0 > n) {
+            sparse = true;
+            ng = (n + kKT - 1) / kKT;
+            idx_row = p.idx + (((long long)b * kGroups + p.head_map[g]) * p.T + tq) * p.max_topk;
+        }
+    }
+    const int ntiles = sparse ? ng + 1 : (min(q0 + QT, L) + kKT - 1) / kKT;
+
+    const int krow = tid >> 4;   // K: key position krow + 16 i, 16-byte column kcol
+    const int kcol = tid & 15;
+    const half_t* kbase = p.K + (long long)b * p.k_sb + (long long)g * p.k_sh + kcol * 8;
+    const half_t* vbase = p.V + (long long)b * p.k_sb + (long long)g * p.k_sh + kcol * 8;
+
+    int nk[4], nv[4];       // key ids of the tile to be loaded next
+    uint4_t kr[4], vr[4];   // tile data in flight
+    auto fetch_ids = [&](int ti) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int pk = krow + 16 * i;       // K position of chunk i
+            const int pv = 4 * krow + i;        // V position of chunk i
+            if (!sparse) {
+                nk[i] = min(ti * kKT + pk, L - 1);
+                nv[i] = min(ti * kKT + pv, L - 1);
+            } else if (ti < ng) {
+                nk[i] = idx_row[min(ti * kKT + pk, n - 1)];
+                nv[i] = idx_row[min(ti * kKT + pv, n - 1)];
+            } else {
+                nk[i] = min(q0 + pk, L - 1);
+                nv[i] = min(q0 + pv, L - 1);
+            }
+        }
+    };
+    auto issue_loads = [&]() {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) kr[i] = ld_global_16(kbase + (long long)nk[i] * p.k_sl);
+        if (WITH_V) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) vr[i] = ld_global_16(vbase + (long long)nv[i] * p.k_sl);
+        }
+    };
+
+    float m[NQB], l[NQB];
+    float16_t oT[NQB][4];
+#pragma unroll
+    for (int qb = 0; qb < NQB; ++qb) {
+        m[qb] = -INFINITY;
+        l[qb] = 0.f;
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) oT[qb][db][v] = 0.f;
+    }
+
+    fetch_ids(0);
+    issue_loads();
+    if (ntiles > 1) fetch_ids(1);
+
+    for (int ti = 0; ti < ntiles; ++ti) {
+        __syncthreads();
+        // ---- registers -> LDS ----
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int slot = swap_bits23(krow + 16 * i);
+            *reinterpret_cast<uint4_t*>(&sK[slot * kKStride + kcol * 8]) = kr[i];
+        }
+        if (WITH_V) {
+            Pack16 v0, v1, v2, v3;
+            v0.u = vr[0]; v1.u = vr[1]; v2.u = vr[2]; v3.u = vr[3];
+            const int kq = krow;   // keys 4*kq .. 4*kq+3
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                const int d = kcol * 8 + r;
+                const int sw = (r ^ kcol) & 7;
+                half4_t w = {v0.h[r], v1.h[r], v2.h[r], v3.h[r]};
+                *reinterpret_cast<half4_t*>(&sV[d * kKT + (((kq >> 1) ^ sw) * 8) + (kq & 1) * 4]) = w;
+            }
+        }
+        __syncthreads();
+        if (ti + 1 < ntiles) {
+            issue_loads();
+            if (ti + 2 < ntiles) fetch_ids(ti + 2);
+        }
+
+        // ---- S^T = K_tile Q^T ----
+        const bool diag_tile = sparse && (ti == ng);
+        const int nkb = (diag_tile && QT == 32) ? 1 : 2;
+        float16_t sT[NQB][2];
+#pragma unroll
+        for (int qb = 0; qb < NQB; ++qb)
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) sT[qb][kb][v] = 0.f;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            if (kb < nkb) {
+#pragma unroll
+                for (int ks = 0; ks < 8; ++ks) {
+                    half8_t a = *reinterpret_cast<const half8_t*>(
+                        &sK[(32 * kb + li) * kKStride + ks * 16 + lg * 8]);
+#pragma unroll
+                    for (int qb = 0; qb < NQB; ++qb)
+                        sT[qb][kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[qb][ks], sT[qb][kb], 0, 0, 0);
+                }
+            }
+        }
+        // ---- masks: accumulator v of key block kb is tile position 32kb + 16(v/8) + 8lg + v%8 ----
+        if (!sparse || diag_tile) {
+            const int kstart = diag_tile ? q0 : ti * kKT;
+            if (kstart + kKT - 1 > q0 || kstart + kKT > L) {
+#pragma unroll
+                for (int qb = 0; qb < NQB; ++qb) {
+                    const int q = q0 + 32 * qb + li;
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const int key = kstart + 32 * kb + 16 * (v >> 3) + 8 * lg + (v & 7);
+                            if (key > q || key >= L) sT[qb][kb][v] = -INFINITY;
+                        }
+                }
+            }
+        } else if ((ti + 1) * kKT > n) {
+#pragma unroll
+            for (int qb = 0; qb < NQB; ++qb)
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int pos = ti * kKT + 32 * kb + 16 * (v >> 3) + 8 * lg + (v & 7);
+                        if (pos >= n) sT[qb][kb][v] = -INFINITY;
+                    }
+        }
+        if (nkb == 1) {
+#pragma unroll
+            for (int qb = 0; qb < NQB; ++qb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) sT[qb][1][v] = -INFINITY;
+        }
+        // ---- online softmax (one query column per lane) ----
+        half8_t pf[NQB][4];
+#pragma unroll
+        for (int qb = 0; qb < NQB; ++qb) {
+            float mx = -INFINITY;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) mx = fmaxf(mx, sT[qb][kb][v]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const float mnew = fmaxf(m[qb], mx);
+            const float mref = (mnew == -INFINITY) ? 0.f : mnew * kScaleLog2;
+            const float corr = fast_exp2(m[qb] * kScaleLog2 - mref);
+            m[qb] = mnew;
+            float sum = 0.f;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const float e = fast_exp2(sT[qb][kb][v] * kScaleLog2 - mref);
+                    sT[qb][kb][v] = e;
+                    sum += e;
+                }
+            l[qb] = l[qb] * corr + sum;   // per-lane partial sum (own key positions)
+            if (WITH_V) {
+#pragma unroll
+                for (int db = 0; db < 4; ++db)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) oT[qb][db][v] *= corr;
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    half8_t t;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) t[e] = (half_t)sT[qb][s >> 1][8 * (s & 1) + e];
+                    pf[qb][s] = t;
+                }
+            }
+        }
+        // ---- O^T += V^T P^T ----
+        if (WITH_V) {
+#pragma unroll
+            for (int db = 0; db < 4; ++db) {
+                const int d = 32 * db + li;
+                const int sw = ((d & 7) ^ (d >> 3)) & 7;
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    if (s < 2 * nkb) {
+                        half8_t a = *reinterpret_cast<const half8_t*>(
+                            &sV[d * kKT + (((2 * s + lg) ^ sw) * 8)]);
+#pragma unroll
+                        for (int qb = 0; qb < NQB; ++qb)
+                            oT[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pf[qb][s], oT[qb][db], 0, 0, 0);
+                    }
+                }
+            }
+        }
+    }
+
+    // ---- epilogue ----
+#pragma unroll
+    for (int qb = 0; qb < NQB; ++qb) {
+        const int q = q0 + 32 * qb + li;
+        const float lt = l[qb] + __shfl_xor(l[qb], 32);
+        if (q < L) {
+            if (p.log_sum && lg == 0)
+                p.log_sum[((long long)b * L + q) * kHeads + head] = fast_log2(lt) + m[qb] * kScaleLog2;
+            if (WITH_V) {
+                const float inv = 1.f / lt;
+                half_t* op = p.O + (((long long)b * L + q) * kHeads + head) * kDim;
+#pragma unroll
+                for (int db = 0; db < 4; ++db)
+#pragma unroll
+                    for (int v4 = 0; v4 < 4; ++v4) {
+                        half4_t o = {(half_t)(oT[qb][db][4 * v4 + 0] * inv), (half_t)(oT[qb][db][4 * v4 + 1] * inv),
+                                     (half_t)(oT[qb][db][4 * v4 + 2] * inv), (half_t)(oT[qb][db][4 * v4 + 3] * inv)};
+                        *reinterpret_cast<half4_t*>(op + 32 * db + 8 * v4 + 4 * lg) = o;
+                    }
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void prefill_aggregate_kernel(PrefillParams p) {
+    __shared__ __attribute__((aligned(16))) half_t sK[kAggKT * kKStride];
+    __shared__ __attribute__((aligned(16))) float s_lse[128];
+
+    const int L = p.L;
+    const int t = p.T - 1 - (int)blockIdx.x;
+    const int g = blockIdx.y;
+    const int b = blockIdx.z;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int li = lane & 31;
+    const int lg = lane >> 5;
+    const int ts = t * kTile;
+    half_t* out = p.agg + (((long long)b * kGroups + g) * p.T + t) * L;
+    const half_t neg_inf = (half_t)(-INFINITY);
+
+    const int ntiles = (ts + kAggKT - 1) / kAggKT;
+    if (ntiles > 0) {
+        // A operands: row block rb = q-head 4g+rb, row li = query ts+li
+        half8_t qa[kGroupSize][8];
+#pragma unroll
+        for (int rb = 0; rb < kGroupSize; ++rb) {
+            const int q = ts + li;
+            const bool ok = q < L;
+            const half_t* qp = p.Q + (long long)b * p.q_sb + (long long)min(q, L - 1) * p.q_sl +
+                               (long long)(g * kGroupSize + rb) * p.q_sh + lg * 8;
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) {
+                Pack16 x;
+                x.u = ld_global_16(qp + ks * 16);
+                if (!ok) x.u = uint4_t{0, 0, 0, 0};
+                qa[rb][ks] = x.h8;
+            }
+        }
+        if (tid < 128) {
+            const int q = ts + (tid & 31);
+            s_lse[tid] = (q < L) ? p.log_sum_in[((long long)b * L + q) * kHeads + g * kGroupSize + (tid >> 5)]
+                                 : INFINITY;
+        }
+        const int krow = tid >> 4, kcol = tid & 15;
+        const half_t* kbase = p.K + (long long)b * p.k_sb + (long long)g * p.k_sh + kcol * 8;
+        uint4_t kr[8];
+        auto issue_loads = [&](int ti) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int key = min(ti * kAggKT + krow + 16 * i, L - 1);
+                kr[i] = ld_global_16(kbase + (long long)key * p.k_sl);
+            }
+        };
+        issue_loads(0);
+        for (int ti = 0; ti < ntiles; ++ti) {
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                *reinterpret_cast<uint4_t*>(&sK[(krow + 16 * i) * kKStride + kcol * 8]) = kr[i];
+            __syncthreads();
+            if (ti + 1 < ntiles) issue_loads(ti + 1);
+
+            float16_t acc[kGroupSize];
+#pragma unroll
+            for (int rb = 0; rb < kGroupSize; ++rb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[rb][v] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) {
+                half8_t bf = *reinterpret_cast<const half8_t*>(
+                    &sK[(32 * wave + li) * kKStride + ks * 16 + lg * 8]);
+#pragma unroll
+                for (int rb = 0; rb < kGroupSize; ++rb)
+                    acc[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa[rb][ks], bf, acc[rb], 0, 0, 0);
+            }
+            // accumulator v of row block rb is query row 8(v/4) + 4lg + v%4, column = key li
+            float sum = 0.f;
+#pragma unroll
+            for (int rb = 0; rb < kGroupSize; ++rb)
+#pragma unroll
+                for (int v4 = 0; v4 < 4; ++v4) {
+                    const float4_t ls = *reinterpret_cast<const float4_t*>(&s_lse[rb * 32 + 8 * v4 + 4 * lg]);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        sum += fast_exp2(acc[rb][4 * v4 + e] * kScaleLog2 - ls[e]);
+                }
+            sum += __shfl_xor(sum, 32);
+            const int key = ti * kAggKT + 32 * wave + li;
+            if (lg == 0 && key < L) {
+                if (key < ts)
+                    out[key] = (half_t)sum;
+                else if (p.fill_invalid)
+                    out[key] = neg_inf;
+            }
+        }
+    }
+    if (p.fill_invalid) {
+        for (int key = ntiles * kAggKT + tid; key < L; key += kThreads) out[key] = neg_inf;
+    }
+}
+
+}  // namespace
+
+hipError_t launch_prefill_attn(const PrefillParams& p, bool reuse, bool with_v, int nqb,
+                               hipStream_t stream) {
+    const int qt = 32 * nqb;
+    dim3 grid((p.L + qt - 1) / qt, kGroups, p.B), block(kThreads);
+    if (reuse) {
+        hipLaunchKernelGGL((prefill_attn_kernel<1, true, true>), grid, block, 0, stream, p);
+    } else if (nqb == 2) {
+        if (with_v)
+            hipLaunchKernelGGL((prefill_attn_kernel<2, false, true>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((prefill_attn_kernel<2, false, false>), grid, block, 0, stream, p);
+    } else {
+        if (with_v)
+            hipLaunchKernelGGL((prefill_attn_kernel<1, false, true>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((prefill_attn_kernel<1, false, false>), grid, block, 0, stream, p);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_prefill_aggregate(const PrefillParams& p, hipStream_t stream) {
+    dim3 grid(p.T, kGroups, p.B), block(kThreads);
+    hipLaunchKernelGGL(prefill_aggregate_kernel, grid, block, 0, stream, p);
+    return hipGetLastError();
+}
+
+}  // namespace kascade

@@ -1,0 +1,297 @@
+"""Python callables over the C ABI, shaped like the reference's kernel objects.
+
+The reference reaches its kernels through tilelang ``JITKernel`` callables that
+take the non-output tensors positionally, allocate the tensors listed in
+``out_idx`` with ``torch.empty`` and return them, read dynamic sizes from the
+tensor shapes and launch on the current torch stream
+(EfficientKascadeStrategy.py:24-70, kernel_utils.py:50-81).  The functions here
+keep those call shapes; each one names the reference callable it stands for.
+
+PyTorch is used for device memory and the stream handle only.  Every function
+raises ``KascadeError`` when libkascade_hip.so is missing or a call fails.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import Strides, KascadeError
+from . import budgets
+
+H, G, D, TILE = 32, 8, 128, 32
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _req(t: torch.Tensor, dtype, name: str, contiguous: bool = True):
+    if not t.is_cuda:
+        raise KascadeError(f"{name} must be a device tensor")
+    if t.dtype != dtype:
+        raise KascadeError(f"{name} must be {dtype}, got {t.dtype}")
+    if contiguous and not t.is_contiguous():
+        raise KascadeError(f"{name} must be contiguous")
+
+
+def _blhd_strides(t: torch.Tensor, name: str) -> Strides:
+    """Strides of a [B,L,heads,D] view whose innermost dimension is contiguous."""
+    if t.dim() != 4 or t.shape[-1] != D or t.stride(-1) != 1:
+        raise KascadeError(f"{name} must be [B,L,heads,{D}] with a contiguous last dimension")
+    return Strides(t.stride(0), t.stride(1), t.stride(2))
+
+
+def default_num_split(rows_per_seq: int, pairs: int) -> int:
+    """Split count for a decode launch: enough workgroups to cover the device several
+    times over while keeping at least 256 rows per split."""
+    cus = _lib.init().kascade_device_cu_count() or 256
+    want = max(1, (8 * cus + pairs - 1) // pairs)
+    by_rows = max(1, rows_per_seq // 256)
+    return int(max(1, min(want, by_rows, 256)))
+
+
+# ---------------------------------------------------------------- decode
+def decode_reuse(Q, K, V, topk_indices, head_mapping, glse, Output_partial) -> torch.Tensor:
+    """``decode_reuse_kernel(Q, K, V, topk_indices, head_mapping, glse, Output_partial) -> O``
+    (out_idx=[7]; EfficientKascadeStrategy.py:30-38, 113, 122).  Contiguous cache
+    K,V [B,L,G,D]; the split count is glse.shape[2]."""
+    lib = _lib.init()
+    B, Hq, Dq = Q.shape
+    L = K.shape[1]
+    _req(Q, torch.float16, "Q"); _req(K, torch.float16, "K"); _req(V, torch.float16, "V")
+    _req(topk_indices, torch.int32, "topk_indices"); _req(head_mapping, torch.int32, "head_mapping")
+    _req(glse, torch.float32, "glse"); _req(Output_partial, torch.float32, "Output_partial")
+    if (Hq, Dq, K.shape[2]) != (H, D, G):
+        raise KascadeError("decode_reuse supports H=32, G=8, D=128 only")
+    ns = glse.shape[2]
+    if tuple(glse.shape) != (B, H, ns) or tuple(Output_partial.shape) != (B, H, ns, D):
+        raise KascadeError("glse must be [B,H,S] and Output_partial [B,H,S,D]")
+    out = torch.empty(B, H, D, device=Q.device, dtype=torch.float16)
+    _lib.check(lib.kascade_decode_reuse_call(
+        _ptr(Q), _ptr(K), _ptr(V), _ptr(topk_indices), _ptr(head_mapping), _ptr(glse),
+        _ptr(Output_partial), _ptr(out), B, L, topk_indices.shape[-1], ns, _stream()))
+    return out
+
+
+def decode_reuse_paged(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_percent, glse,
+                       Output_partial, block_table=None, page_size: int = 16) -> torch.Tensor:
+    """``reuse kvcache kernel(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_percent,
+    glse, Output_partial) -> O`` (out_idx=[9]; reuse_kascade_gqa_decode_with_kvcache.py:160-173)
+    with an optional block table.  Without one K,V are the padded [B,maxL,G,D] cache;
+    with one they are pages [P,page_size,G,D]."""
+    lib = _lib.init()
+    B = Q.shape[0]
+    _req(Q, torch.float16, "Q"); _req(K, torch.float16, "K"); _req(V, torch.float16, "V")
+    _req(topk_indices, torch.int32, "topk_indices"); _req(head_mapping, torch.int32, "head_mapping")
+    _req(glse, torch.float32, "glse"); _req(Output_partial, torch.float32, "Output_partial")
+    if cache_seqlens is not None:
+        _req(cache_seqlens, torch.int32, "cache_seqlens")
+    ns = glse.shape[2]
+    if block_table is not None:
+        _req(block_table, torch.int32, "block_table")
+        stride_tokens, max_pages = 0, block_table.shape[1]
+    else:
+        stride_tokens, max_pages = K.shape[1], 0
+    out = torch.empty(B, H, D, device=Q.device, dtype=torch.float16)
+    _lib.check(lib.kascade_decode_reuse_paged_call(
+        _ptr(Q), _ptr(K), _ptr(V), _ptr(cache_seqlens), _ptr(topk_indices), _ptr(head_mapping),
+        float(topk_percent), _ptr(glse), _ptr(Output_partial), _ptr(out), B, stride_tokens,
+        topk_indices.shape[-1], ns, _ptr(block_table), max_pages, page_size, _stream()))
+    return out
+
+
+def decode_dense_paged(Q, K, V, cache_seqlens, glse, Output_partial, block_table=None,
+                       page_size: int = 16, kv_len: Optional[int] = None) -> torch.Tensor:
+    """Dense split-K decode, the baseline of gqa_decode.py / gqa_decode_with_kvcache.py:
+    ``kernel(Q, K, V, [cache_seqlens,] glse, Output_partial) -> O``."""
+    lib = _lib.init()
+    B = Q.shape[0]
+    _req(Q, torch.float16, "Q"); _req(K, torch.float16, "K"); _req(V, torch.float16, "V")
+    _req(glse, torch.float32, "glse"); _req(Output_partial, torch.float32, "Output_partial")
+    ns = glse.shape[2]
+    if block_table is not None:
+        _req(block_table, torch.int32, "block_table")
+        stride_tokens, max_pages = (kv_len or 0), block_table.shape[1]
+    else:
+        stride_tokens, max_pages = K.shape[1], 0
+    out = torch.empty(B, H, D, device=Q.device, dtype=torch.float16)
+    _lib.check(lib.kascade_decode_dense_paged_call(
+        _ptr(Q), _ptr(K), _ptr(V), _ptr(cache_seqlens), _ptr(glse), _ptr(Output_partial), _ptr(out),
+        B, stride_tokens, ns, _ptr(block_table), max_pages, page_size, _stream()))
+    return out
+
+
+def decode_recompute(Q, K, V, glse, Output_partial, row_sums, scores, layer: int,
+                     cache_seqlens=None, block_table=None, page_size: int = 16,
+                     kv_len: Optional[int] = None) -> Tuple[Optional[torch.Tensor], torch.Tensor]:
+    """``decode_recomp{0,1}_kernel(Q, K, V, glse, Output_partial, row_sums, scores) -> (O, agg)``
+    (out_idx=[7,8]; EfficientKascadeStrategy.py:24-28, 107-110) and its kvcache form
+    (recompute_kascade_gqa_decode_with_kvcache.py:302-333).  ``scores`` is fp32 scratch
+    [B,H,stride]; agg is [B,G,stride] fp16.  layer == 0 also computes the dense output;
+    otherwise O is None."""
+    lib = _lib.init()
+    B = Q.shape[0]
+    _req(Q, torch.float16, "Q"); _req(K, torch.float16, "K")
+    _req(glse, torch.float32, "glse"); _req(row_sums, torch.float32, "row_sums")
+    _req(scores, torch.float32, "scores")
+    with_out = 1 if layer == 0 else 0
+    ns = glse.shape[2]
+    stride = scores.shape[2]
+    if block_table is not None:
+        _req(block_table, torch.int32, "block_table")
+        stride_tokens, max_pages = (kv_len or 0), block_table.shape[1]
+    else:
+        stride_tokens, max_pages = K.shape[1], 0
+    out = torch.empty(B, H, D, device=Q.device, dtype=torch.float16) if with_out else None
+    agg = torch.empty(B, G, stride, device=Q.device, dtype=torch.float16)
+    _lib.check(lib.kascade_decode_recompute_paged_call(
+        _ptr(Q), _ptr(K), _ptr(V), _ptr(cache_seqlens), _ptr(glse), _ptr(Output_partial),
+        _ptr(row_sums), _ptr(scores), _ptr(out), _ptr(agg), B, stride_tokens, stride, ns, with_out,
+        _ptr(block_table), max_pages, page_size, _stream()))
+    return out, agg
+
+
+# ----------------------------------------------------------------- top-k
+def topk_indices(scores: torch.Tensor, k: int, valid_len=None, n_sel=None,
+                 uniform_len: Optional[int] = None, fill_value: Optional[int] = None
+                 ) -> torch.Tensor:
+    """Stands for ``torch.topk(scores, k, dim=-1).indices.to(int32)``
+    (EfficientKascadeStrategy.py:82, 111) as an exact selection: row r delivers the
+    n_sel largest of its first valid_len entries in slots [0, n_sel), ascending by
+    index; remaining slots hold fill_value.  valid_len / n_sel are int32 device
+    tensors indexed by (row % len) or None for uniform rows."""
+    lib = _lib.init()
+    _req(scores, torch.float16, "scores", contiguous=False)
+    if scores.stride(-1) != 1:
+        raise KascadeError("scores rows must be contiguous")
+    Lrow = scores.shape[-1]
+    lead = scores.shape[:-1]
+    rows = int(math.prod(lead)) if len(lead) else 1
+    # rows must be evenly strided
+    flat = scores.reshape(rows, Lrow) if scores.is_contiguous() else None
+    if flat is None:
+        row_stride = scores.stride(-2)
+        exp = row_stride
+        for dim in range(scores.dim() - 2, -1, -1):
+            if scores.stride(dim) != exp and scores.shape[dim] != 1:
+                raise KascadeError("scores must have uniformly strided rows")
+            exp *= scores.shape[dim]
+    else:
+        row_stride = Lrow
+    period = 1
+    if valid_len is not None:
+        _req(valid_len, torch.int32, "valid_len"); period = valid_len.numel()
+    if n_sel is not None:
+        _req(n_sel, torch.int32, "n_sel")
+        if valid_len is not None and n_sel.numel() != period:
+            raise KascadeError("valid_len and n_sel must have the same length")
+        period = n_sel.numel()
+    out = torch.empty(*lead, k, device=scores.device, dtype=torch.int32)
+    _lib.check(lib.kascade_topk_call(
+        _ptr(scores), _ptr(out), rows, row_stride, Lrow if uniform_len is None else uniform_len,
+        _ptr(valid_len), _ptr(n_sel), period, k, (Lrow - 1) if fill_value is None else fill_value,
+        None, _stream()))
+    return out
+
+
+# --------------------------------------------------------------- prefill
+def prefill_recompute0(Q, K, V) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``prefill_recomp0_kernel(Q, K, V) -> (log_sum, O)`` (out_idx=[3,4];
+    EfficientKascadeStrategy.py:40-43, 78).  Q [B,L,H,D], K,V [B,L,G,D] (strided views allowed)."""
+    lib = _lib.init()
+    _req(Q, torch.float16, "Q", False); _req(K, torch.float16, "K", False); _req(V, torch.float16, "V", False)
+    B, L = Q.shape[0], Q.shape[1]
+    qs, ks = _blhd_strides(Q, "Q"), _blhd_strides(K, "K")
+    if tuple(V.stride()) != tuple(K.stride()):
+        raise KascadeError("K and V must share strides")
+    log_sum = torch.empty(B, L, H, device=Q.device, dtype=torch.float32)
+    out = torch.empty(B, L, H, D, device=Q.device, dtype=torch.float16)
+    _lib.check(lib.kascade_prefill_dense_call(_ptr(Q), _ptr(K), _ptr(V), _ptr(log_sum), _ptr(out),
+                                              B, L, qs, ks, 1, _stream()))
+    return log_sum, out
+
+
+def prefill_recompute1(Q, K) -> torch.Tensor:
+    """``prefill_recomp1_kernel(Q, K) -> log_sum`` (out_idx=[2]; EfficientKascadeStrategy.py:44-47, 80)."""
+    lib = _lib.init()
+    _req(Q, torch.float16, "Q", False); _req(K, torch.float16, "K", False)
+    B, L = Q.shape[0], Q.shape[1]
+    qs, ks = _blhd_strides(Q, "Q"), _blhd_strides(K, "K")
+    log_sum = torch.empty(B, L, H, device=Q.device, dtype=torch.float32)
+    _lib.check(lib.kascade_prefill_dense_call(_ptr(Q), _ptr(K), None, _ptr(log_sum), None,
+                                              B, L, qs, ks, 0, _stream()))
+    return log_sum
+
+
+def prefill_dense(Q, K, V) -> torch.Tensor:
+    """Dense causal prefill baseline (example_gqa_fwd_bshd_wgmma_pipelined.py:121-166):
+    ``kernel(Q, K, V) -> O``; no log-sum is written."""
+    lib = _lib.init()
+    _req(Q, torch.float16, "Q", False); _req(K, torch.float16, "K", False); _req(V, torch.float16, "V", False)
+    B, L = Q.shape[0], Q.shape[1]
+    qs, ks = _blhd_strides(Q, "Q"), _blhd_strides(K, "K")
+    if tuple(V.stride()) != tuple(K.stride()):
+        raise KascadeError("K and V must share strides")
+    out = torch.empty(B, L, H, D, device=Q.device, dtype=torch.float16)
+    _lib.check(lib.kascade_prefill_dense_call(_ptr(Q), _ptr(K), _ptr(V), None, _ptr(out),
+                                              B, L, qs, ks, 1, _stream()))
+    return out
+
+
+def prefill_aggregate(Q, K, log_sum, scores, fill_invalid: bool = False) -> None:
+    """``aggregate_kernel(Q, K, log_sum, scores)`` (out_idx=None; in place;
+    EfficientKascadeStrategy.py:49-59, 81).  scores [B,G,ceil(L/32),L] fp16."""
+    lib = _lib.init()
+    _req(Q, torch.float16, "Q", False); _req(K, torch.float16, "K", False)
+    _req(log_sum, torch.float32, "log_sum"); _req(scores, torch.float16, "scores")
+    B, L = Q.shape[0], Q.shape[1]
+    T = (L + TILE - 1) // TILE
+    if tuple(scores.shape) != (B, G, T, L) or tuple(log_sum.shape) != (B, L, H):
+        raise KascadeError("scores must be [B,G,ceil(L/32),L] and log_sum [B,L,H]")
+    qs, ks = _blhd_strides(Q, "Q"), _blhd_strides(K, "K")
+    _lib.check(lib.kascade_prefill_aggregate_call(_ptr(Q), _ptr(K), _ptr(log_sum), _ptr(scores), B, L,
+                                                  qs, ks, 1 if fill_invalid else 0, _stream()))
+
+
+def prefill_reuse(Q, K, V, topk_idx, head_mapping, topk_percent, rolling: bool) -> torch.Tensor:
+    """``prefill_reuse_kernel(Q, K, V, topk_indices, head_mapping, topk_percent) -> O``
+    (out_idx=[6]; EfficientKascadeStrategy.py:61-70, 92, 97); ``rolling`` selects between the
+    reference's two compiled objects."""
+    lib = _lib.init()
+    _req(Q, torch.float16, "Q", False); _req(K, torch.float16, "K", False); _req(V, torch.float16, "V", False)
+    _req(topk_idx, torch.int32, "topk_indices"); _req(head_mapping, torch.int32, "head_mapping")
+    B, L = Q.shape[0], Q.shape[1]
+    T = (L + TILE - 1) // TILE
+    if tuple(topk_idx.shape[:3]) != (B, G, T):
+        raise KascadeError("topk_indices must be [B,G,ceil(L/32),max_topk]")
+    qs, ks = _blhd_strides(Q, "Q"), _blhd_strides(K, "K")
+    if tuple(V.stride()) != tuple(K.stride()):
+        raise KascadeError("K and V must share strides")
+    out = torch.empty(B, L, H, D, device=Q.device, dtype=torch.float16)
+    _lib.check(lib.kascade_prefill_reuse_call(
+        _ptr(Q), _ptr(K), _ptr(V), _ptr(topk_idx), _ptr(head_mapping), float(topk_percent), _ptr(out),
+        B, L, topk_idx.shape[-1], 1 if rolling else 0, qs, ks, _stream()))
+    return out
+
+
+# ------------------------------------------------------------- KV append
+def paged_kv_append(K_pages, V_pages, k_new, v_new, start_pos, block_table, page_size: int = 16):
+    """Write k_new/v_new [B,n_new,G,D] into the paged cache at positions start_pos[b]+t."""
+    lib = _lib.init()
+    _req(K_pages, torch.float16, "K_pages"); _req(V_pages, torch.float16, "V_pages")
+    _req(k_new, torch.float16, "k_new", False); _req(v_new, torch.float16, "v_new", False)
+    _req(start_pos, torch.int32, "start_pos"); _req(block_table, torch.int32, "block_table")
+    if tuple(k_new.stride()) != tuple(v_new.stride()):
+        raise KascadeError("k_new and v_new must share strides")
+    B, n_new = k_new.shape[0], k_new.shape[1]
+    st = _blhd_strides(k_new, "k_new")
+    _lib.check(lib.kascade_paged_kv_append_call(
+        _ptr(K_pages), _ptr(V_pages), _ptr(k_new), _ptr(v_new), _ptr(start_pos), _ptr(block_table),
+        B, n_new, block_table.shape[1], page_size, st, _stream()))

@@ -1,0 +1,213 @@
+"""GPU parity of the decode kernels (through the C ABI) against the CPU oracle."""
+import pytest
+import torch
+
+from oracle import kascade_oracle as orc
+from tests.helpers import assert_close, check_topk_rows
+
+pytestmark = pytest.mark.gpu
+
+H, G, D = 32, 8, 128
+
+
+def _scratch(B, ns, dev):
+    return (torch.empty(B, H, ns, device=dev, dtype=torch.float32),
+            torch.empty(B, H, ns, D, device=dev, dtype=torch.float32))
+
+
+def _rand_idx(B, L, k, gen):
+    rows = [torch.stack([torch.randperm(L, generator=gen)[:k] for _ in range(G)]) for _ in range(B)]
+    return torch.stack(rows).to(torch.int32)
+
+
+@pytest.mark.parametrize("L,k,ns", [(1000, 256, 8), (777, 300, 3), (4096, 1024, 1), (130, 130, 8)])
+def test_decode_reuse_contiguous(cuda, L, k, ns):
+    from kascade_amd import kernels
+    gen = torch.Generator().manual_seed(L + k)
+    B = 2
+    q = torch.randn(B, H, D, generator=gen).half()
+    kk = torch.randn(B, L, G, D, generator=gen).half()
+    vv = torch.randn(B, L, G, D, generator=gen).half()
+    idx = _rand_idx(B, L, k, gen)
+    hm = torch.randint(0, G, (G,), generator=gen).to(torch.int32)
+    want = orc.reuse_decode(q, kk, vv, idx, hm.tolist())
+    glse, part = _scratch(B, ns, cuda)
+    got = kernels.decode_reuse(q.to(cuda), kk.to(cuda), vv.to(cuda), idx.to(cuda), hm.to(cuda), glse, part)
+    torch.cuda.synchronize()
+    assert_close(got, want, f"decode_reuse L={L} k={k} ns={ns}")
+    # gather == scatter formulation (distinct indices)
+    assert_close(got, orc.reuse_decode_scatter(q, kk, vv, idx, hm.tolist()), "decode_reuse vs scatter form")
+
+
+def test_decode_reuse_all_keys_is_dense(cuda):
+    from kascade_amd import kernels
+    gen = torch.Generator().manual_seed(5)
+    B, L = 1, 640
+    q = torch.randn(B, H, D, generator=gen).half()
+    kk = torch.randn(B, L, G, D, generator=gen).half()
+    vv = torch.randn(B, L, G, D, generator=gen).half()
+    idx = torch.stack([torch.randperm(L, generator=gen) for _ in range(G)]).unsqueeze(0).to(torch.int32)
+    hm = torch.arange(G, dtype=torch.int32)
+    glse, part = _scratch(B, 4, cuda)
+    got = kernels.decode_reuse(q.to(cuda), kk.to(cuda), vv.to(cuda), idx.to(cuda), hm.to(cuda), glse, part)
+    want, _ = orc.dense_decode(q, kk, vv)
+    assert_close(got, want, "decode_reuse with k=L")
+
+
+def _paged_case(seqlens, seed, peaked=True):
+    from kascade_amd import workloads
+    return workloads.paged_decode_inputs(seqlens, seed=seed, device="cpu", peaked=peaked)
+
+
+@pytest.mark.parametrize("seqlens,ns", [([300, 1000, 515], 4), ([2048, 64], 7), ([4500], 16)])
+def test_decode_dense_paged(cuda, seqlens, ns):
+    from kascade_amd import kernels
+    w = _paged_case(seqlens, seed=len(seqlens))
+    kc = orc.paged_to_contiguous(w.k_pages, w.block_table, seqlens)
+    vc = orc.paged_to_contiguous(w.v_pages, w.block_table, seqlens)
+    want, _ = orc.dense_decode(w.q, kc, vc, seqlens)
+    B = len(seqlens)
+    glse, part = _scratch(B, ns, cuda)
+    got = kernels.decode_dense_paged(w.q.to(cuda), w.k_pages.to(cuda), w.v_pages.to(cuda),
+                                     w.seqlens.to(cuda), glse, part, w.block_table.to(cuda), w.page_size)
+    assert_close(got, want, f"decode_dense_paged {seqlens}")
+
+
+@pytest.mark.parametrize("layer", [0, 1])
+@pytest.mark.parametrize("seqlens", [[1500, 700, 2048], [3000]])
+def test_decode_recompute_paged(cuda, seqlens, layer):
+    """Anchor decode: pooled scores, global log-sum, indices and output vs the oracle."""
+    from kascade_amd import kernels, budgets
+    p = 10
+    w = _paged_case(seqlens, seed=11 + layer)
+    B, Lmax = len(seqlens), max(seqlens)
+    kc = orc.paged_to_contiguous(w.k_pages, w.block_table, seqlens)
+    vc = orc.paged_to_contiguous(w.v_pages, w.block_table, seqlens)
+    o_want, idx_want, agg_want = orc.anchor_decode(w.q, kc, vc, p, layer == 0, seqlens)
+    ns = 6
+    glse, part = _scratch(B, ns, cuda)
+    row_sums = torch.empty(B, H, device=cuda, dtype=torch.float32)
+    stride = ((Lmax + 7) // 8) * 8
+    scores = torch.empty(B, H, stride, device=cuda, dtype=torch.float32)
+    o, agg = kernels.decode_recompute(w.q.to(cuda), w.k_pages.to(cuda), w.v_pages.to(cuda), glse, part,
+                                      row_sums, scores, layer, cache_seqlens=w.seqlens.to(cuda),
+                                      block_table=w.block_table.to(cuda), page_size=w.page_size)
+    torch.cuda.synchronize()
+    agg_c = agg.cpu()[:, :, :Lmax]
+    # pooled probabilities: fp16 values, allow 2 fp16 ulps + tiny absolute slack
+    assert_close(agg_c, agg_want, "agg", atol=2e-6, rtol=2e-3)
+    for b, n in enumerate(seqlens):
+        assert float(agg_c[b, :, n:].abs().max()) == 0.0 if n < Lmax else True
+        assert abs(float(agg_c[b, :, :n].float().sum(-1).mean()) - 4.0) < 2e-2
+    _, lse = orc.dense_decode(w.q, kc, vc, seqlens)
+    assert_close(row_sums, lse * orc.LOG2E, "row_sums", atol=2e-3, rtol=1e-4)
+    # selection
+    K = orc.max_topk_kvcache(Lmax, p)
+    counts = torch.tensor([budgets.decode_budget(n, p) for n in seqlens], dtype=torch.int32)
+    assert counts.tolist() == [orc.n_kvcache(n, p) for n in seqlens]
+    valid = w.seqlens.to(cuda)
+    nsel = counts.to(cuda)
+    # rows are (b, g): per-row arrays are indexed by row % period, so expand to B*G entries
+    idx = kernels.topk_indices(agg[:, :, :Lmax], K, valid_len=valid.repeat_interleave(G),
+                               n_sel=nsel.repeat_interleave(G), fill_value=0)
+    torch.cuda.synchronize()
+    idx_c = idx.cpu()
+    # exact on the kernel's own scores, tie-aware (1 ulp) on the oracle's
+    check_topk_rows(agg_c.reshape(B * G, Lmax), idx_c.reshape(B * G, K),
+                    lambda r: counts[r // G], lambda r: seqlens[r // G], "topk(own scores)")
+    own = [orc.topk_agreement(agg_c.reshape(B * G, Lmax)[r], idx_c.reshape(B * G, K)[r],
+                              int(counts[r // G]), seqlens[r // G], ulps=0.0)[0] for r in range(B * G)]
+    assert all(own), "selection is not exact on the kernel's own scores"
+    check_topk_rows(agg_want.reshape(B * G, Lmax), idx_c.reshape(B * G, K),
+                    lambda r: counts[r // G], lambda r: seqlens[r // G], "topk(oracle scores)")
+    if layer == 0:
+        assert_close(o, o_want, "anchor-0 decode output")
+    else:
+        assert o is None
+        # anchor > 0: reuse pass with its own indices and the identity map
+        hm = torch.arange(G, dtype=torch.int32, device=cuda)
+        glse2, part2 = _scratch(B, ns, cuda)
+        o2 = kernels.decode_reuse_paged(w.q.to(cuda), w.k_pages.to(cuda), w.v_pages.to(cuda),
+                                        w.seqlens.to(cuda), idx, hm, float(p), glse2, part2,
+                                        block_table=w.block_table.to(cuda), page_size=w.page_size)
+        want2 = orc.reuse_decode(w.q, kc, vc, idx_c, list(range(G)), counts.tolist())
+        assert_close(o2, want2, "anchor decode sparse output (own indices)")
+
+
+def test_decode_reuse_paged_ragged_head_mapping(cuda):
+    """Reuse layer on a ragged paged batch through a random head map, indices from the oracle anchor."""
+    from kascade_amd import kernels
+    p = 10
+    seqlens = [1400, 2600, 1290]
+    w = _paged_case(seqlens, seed=3)
+    kc = orc.paged_to_contiguous(w.k_pages, w.block_table, seqlens)
+    vc = orc.paged_to_contiguous(w.v_pages, w.block_table, seqlens)
+    _, idx, _ = orc.anchor_decode(w.q, kc, vc, p, True, seqlens)
+    kr = orc.paged_to_contiguous(w.k_pages_reuse, w.block_table, seqlens)
+    counts = [orc.n_kvcache(n, p) for n in seqlens]
+    want = orc.reuse_decode(w.q_reuse, kr, vc, idx, w.head_mapping, counts)
+    B = len(seqlens)
+    outs = []
+    for ns in (1, 5):
+        glse, part = _scratch(B, ns, cuda)
+        got = kernels.decode_reuse_paged(
+            w.q_reuse.to(cuda), w.k_pages_reuse.to(cuda), w.v_pages.to(cuda), w.seqlens.to(cuda),
+            idx.to(cuda), torch.tensor(w.head_mapping, dtype=torch.int32, device=cuda), float(p),
+            glse, part, block_table=w.block_table.to(cuda), page_size=w.page_size)
+        assert_close(got, want, f"decode_reuse_paged ns={ns}")
+        outs.append(got.cpu())
+    # head-map identity: mapping m on idx == identity map on idx[:, m]
+    glse, part = _scratch(B, 5, cuda)
+    got_id = kernels.decode_reuse_paged(
+        w.q_reuse.to(cuda), w.k_pages_reuse.to(cuda), w.v_pages.to(cuda), w.seqlens.to(cuda),
+        idx[:, w.head_mapping].contiguous().to(cuda), torch.arange(G, dtype=torch.int32, device=cuda),
+        float(p), glse, part, block_table=w.block_table.to(cuda), page_size=w.page_size)
+    assert torch.equal(got_id.cpu(), outs[1]), "head_mapping is not a pure row gather"
+
+
+def test_block_table_permutation_invariance(cuda):
+    """Any placement of the same logical cache gives bit-identical results."""
+    from kascade_amd import kernels
+    seqlens = [900, 333]
+    w = _paged_case(seqlens, seed=9)
+    B = len(seqlens)
+    kc = orc.paged_to_contiguous(w.k_pages, w.block_table, seqlens)   # [B,Lmax,G,D], zero padded
+    vc = orc.paged_to_contiguous(w.v_pages, w.block_table, seqlens)
+    Lmax = kc.shape[1]
+    lens = w.seqlens.to(cuda)
+    glse, part = _scratch(B, 4, cuda)
+    a = kernels.decode_dense_paged(w.q.to(cuda), w.k_pages.to(cuda), w.v_pages.to(cuda), lens, glse, part,
+                                   w.block_table.to(cuda), w.page_size)
+    b = kernels.decode_dense_paged(w.q.to(cuda), kc.to(cuda), vc.to(cuda), lens, glse.clone(), part.clone())
+    assert torch.equal(a.cpu(), b.cpu())
+    gen = torch.Generator().manual_seed(1)
+    idx = _rand_idx(B, min(seqlens), 256, gen)
+    hm = torch.arange(G, dtype=torch.int32, device=cuda)
+    c = kernels.decode_reuse_paged(w.q.to(cuda), w.k_pages.to(cuda), w.v_pages.to(cuda), lens, idx.to(cuda), hm,
+                                   0.0, glse, part, block_table=w.block_table.to(cuda), page_size=w.page_size)
+    d = kernels.decode_reuse_paged(w.q.to(cuda), kc.to(cuda), vc.to(cuda), lens, idx.to(cuda), hm, 0.0,
+                                   glse.clone(), part.clone())
+    assert torch.equal(c.cpu(), d.cpu())
+    assert Lmax == max(seqlens)
+
+
+def test_kv_append_roundtrip(cuda):
+    from kascade_amd import kernels
+    gen = torch.Generator().manual_seed(2)
+    B, page, n_new, P = 3, 16, 5, 40
+    Kp = torch.zeros(P, page, G, D, dtype=torch.float16, device=cuda)
+    Vp = torch.zeros_like(Kp)
+    bt = torch.randperm(P, generator=gen)[:B * 4].view(B, 4).to(torch.int32)
+    start = torch.tensor([0, 13, 30], dtype=torch.int32)
+    kn = torch.randn(B, n_new, G, D, generator=gen).half()
+    vn = torch.randn(B, n_new, G, D, generator=gen).half()
+    kernels.paged_kv_append(Kp, Vp, kn.to(cuda), vn.to(cuda), start.to(cuda), bt.to(cuda), page)
+    torch.cuda.synchronize()
+    Kc, Vc = Kp.cpu(), Vp.cpu()
+    for b in range(B):
+        for t in range(n_new):
+            tok = int(start[b]) + t
+            pg = int(bt[b, tok // page])
+            assert torch.equal(Kc[pg, tok % page], kn[b, t])
+            assert torch.equal(Vc[pg, tok % page], vn[b, t])
+    assert int((Kc != 0).any(dim=-1).any(dim=-1).sum()) == B * n_new

@@ -1,0 +1,367 @@
+"""Pins the CPU oracle with mathematics that does not restate its formulas:
+library routines (SDPA, logsumexp, topk), brute-force loops on tiny inputs,
+closed forms, invariants and equivalences between independent formulations."""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import kascade_oracle as orc
+
+torch.manual_seed(0)
+
+
+def _qkv(B, L, H, G, D, seed=0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(B, L, H, D, generator=g).to(dtype),
+            torch.randn(B, L, G, D, generator=g).to(dtype),
+            torch.randn(B, L, G, D, generator=g).to(dtype))
+
+
+# ------------------------------------------------------------------ budgets
+def test_budget_table():
+    """Values listed for the benchmark lengths (p = 10, tile 32)."""
+    want = {2048: (256, 172), 16384: (1664, None), 32768: (3328, 3244), 65536: (6656, None),
+            131072: (13184, None), 196608: (19712, None), 262144: (26240, None), 524288: (52480, None)}
+    for L, (kk, ks) in want.items():
+        assert orc.k_kern(L, 10) == kk
+        if ks is not None:
+            assert orc.k_strat(L, 10, 32) == ks
+    assert [orc.n_kvcache(n, 10) for n in (131072, 196608, 262144, 524288)] == [13184, 19712, 26240, 52480]
+    # small and capped cases
+    assert orc.k_kern(100, 10) == 100 and orc.k_kern(129, 10) == 128 and orc.k_kern(1000, 50) == 512
+    assert orc.k_kern(200, 90) == 200
+    assert orc.n_kern(0, 10) == 128 and orc.n_kern(1280, 10) == 128 and orc.n_kern(1312, 10) == 256
+    assert orc.n_strat(0, 10, 172) == 128 and orc.n_strat(32 * 60, 10, 172) == 172
+
+
+def test_budget_integer_vs_float_forms():
+    """For p = 10 the integer floor equals the reference's double and float32 expressions
+    (int((p/100)*x) on the host, int32((p/100)*x) on the device) for all tile starts < 2^20."""
+    x = np.arange(0, 1 << 20, 32, dtype=np.int64)
+    exact = (10 * x) // 100
+    assert np.array_equal(exact, np.floor((10 / 100) * x.astype(np.float64)).astype(np.int64))
+    f32 = (np.float32(10) / np.float32(100)) * x.astype(np.float32)
+    assert np.array_equal(exact, f32.astype(np.int32).astype(np.int64))
+    assert orc.pct_floor(10, 65536) == 6553 and orc.pct_floor(12.5, 1000) == 125
+
+
+def test_rolling_budget_within_row_width():
+    """n_kern(t) <= k_kern(L') for every sparse-regime tile of every prompt length L' > 32 t:
+    chunked and one-shot prefill consume identical index prefixes."""
+    for Lp in list(range(129, 4000, 37)) + [16384]:
+        K = orc.k_kern(Lp, 10)
+        for t in range(math.ceil(Lp / 32)):
+            n = orc.n_kern(32 * t, 10)
+            if 32 * t > n:
+                assert n <= K, (Lp, t, n, K)
+
+
+# --------------------------------------------------------------------- masks
+@pytest.mark.parametrize("Lq,start,Lk", [(96, 0, 96), (70, 0, 70), (64, 64, 200), (45, 32, 130)])
+def test_tile_mask_roll_equals_closed_form(Lq, start, Lk):
+    tile = 32
+    m = orc.causal_additive_mask(Lq, Lk, torch.float32, q_offset=start)
+    rolled = orc.tile_mask_roll(m, tile, start)[0, 0]
+    T = math.ceil(Lq / tile)
+    if T < 2:
+        pytest.skip("construction needs two tiles")
+    closed = orc.tile_mask_closed_form(T, Lk, tile, start)
+    assert torch.equal(rolled == 0, closed)
+
+
+# --------------------------------------------------------- dense attention
+@pytest.mark.parametrize("L", [33, 128, 300])
+def test_dense_prefill_vs_sdpa(L):
+    B, H, G, D = 2, 8, 2, 16
+    q, k, v = _qkv(B, L, H, G, D, seed=L)
+    o, lse2 = orc.dense_prefill(q, k, v, block=64)
+    kk = k.permute(0, 2, 1, 3).repeat_interleave(H // G, dim=1)
+    vv = v.permute(0, 2, 1, 3).repeat_interleave(H // G, dim=1)
+    ref = F.scaled_dot_product_attention(q.permute(0, 2, 1, 3), kk, vv, is_causal=True).permute(0, 2, 1, 3)
+    assert torch.allclose(o, ref, atol=1e-5, rtol=1e-5)
+    # log-sum: exp2 domain, sums to one
+    s = torch.einsum("blhd,bmhd->bhlm", q, kk.permute(0, 2, 1, 3)) * D ** -0.5
+    s = s.masked_fill(torch.triu(torch.ones(L, L, dtype=torch.bool), 1), float("-inf"))
+    assert torch.allclose(lse2, (torch.logsumexp(s, -1) * orc.LOG2E).permute(0, 2, 1), atol=1e-4)
+    total = torch.exp2(s * orc.LOG2E - lse2.permute(0, 2, 1).unsqueeze(-1)).sum(-1)
+    assert torch.allclose(total, torch.ones_like(total), atol=1e-4)
+
+
+def test_dense_decode_vs_sdpa_and_masking():
+    B, H, G, D, L = 3, 8, 2, 16, 50
+    g = torch.Generator().manual_seed(1)
+    q = torch.randn(B, H, D, generator=g)
+    k = torch.randn(B, L, G, D, generator=g)
+    v = torch.randn(B, L, G, D, generator=g)
+    lens = [50, 17, 1]
+    o, lse = orc.dense_decode(q, k, v, lens)
+    for b, n in enumerate(lens):
+        kk = k[b, :n].permute(1, 0, 2).repeat_interleave(H // G, dim=0)
+        vv = v[b, :n].permute(1, 0, 2).repeat_interleave(H // G, dim=0)
+        ref = F.scaled_dot_product_attention(q[b].unsqueeze(1), kk, vv).squeeze(1)
+        assert torch.allclose(o[b], ref, atol=1e-5)
+    assert torch.allclose(o[2], v[2, 0].repeat_interleave(H // G, dim=0), atol=1e-6)
+
+
+# ------------------------------------------------------------ pooled scores
+def _pooled_brute(q, k, tile):
+    B, L, H, D = q.shape
+    G = k.shape[2]
+    rep = H // G
+    T = math.ceil(L / tile)
+    out = torch.full((B, G, T, L), float("-inf"), dtype=torch.float64)
+    for b in range(B):
+        P = torch.zeros(H, L, L, dtype=torch.float64)
+        for h in range(H):
+            for i in range(L):
+                s = (k[b, :i + 1, h // rep].double() @ q[b, i, h].double()) / math.sqrt(D)
+                P[h, i, :i + 1] = torch.softmax(s, 0)
+        for g in range(G):
+            for t in range(T):
+                for j in range(min(t * tile, L)):
+                    out[b, g, t, j] = P[g * rep:(g + 1) * rep, t * tile:(t + 1) * tile, j].sum()
+    return out
+
+
+@pytest.mark.parametrize("L,tile", [(70, 32), (64, 16), (50, 32)])
+def test_pooled_prefill_scores_brute_force(L, tile):
+    q, k, _ = _qkv(1, L, 4, 2, 8, seed=L)
+    got = orc.pooled_prefill_scores(q, k, tile, block_tiles=1, out_dtype=torch.float32)
+    want = _pooled_brute(q, k, tile)
+    assert torch.equal(torch.isfinite(got), torch.isfinite(want))
+    fin = torch.isfinite(want)
+    assert torch.allclose(got[fin].double(), want[fin], atol=1e-6)
+    assert not torch.isfinite(got[:, :, 0]).any()            # tile 0 sees nothing
+    assert float(got[fin].min()) >= 0
+    # blocking does not change the result
+    got2 = orc.pooled_prefill_scores(q, k, tile, block_tiles=7, out_dtype=torch.float32)
+    assert torch.allclose(got2[fin], got[fin], atol=1e-6)
+    # fp16 cast is the last step
+    assert torch.equal(orc.pooled_prefill_scores(q, k, tile)[fin], got[fin].half())
+
+
+def test_pooled_decode_scores_properties():
+    B, H, G, D, L = 2, 8, 2, 16, 200
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn(B, H, D, generator=g)
+    k = torch.randn(B, L, G, D, generator=g)
+    lens = [200, 77]
+    agg = orc.pooled_decode_scores(q, k, lens)
+    assert agg.dtype == torch.float16 and tuple(agg.shape) == (B, G, L)
+    assert torch.allclose(agg.float().sum(-1), torch.full((B, G), float(H // G)), atol=5e-3)
+    assert float(agg[1, :, 77:].abs().max()) == 0
+    # definition, by loops
+    for b, n in enumerate(lens):
+        for gg in range(G):
+            acc = torch.zeros(n, dtype=torch.float64)
+            for h in range(gg * (H // G), (gg + 1) * (H // G)):
+                acc += torch.softmax(k[b, :n, gg].double() @ q[b, h].double() / math.sqrt(D), 0)
+            assert torch.allclose(agg[b, gg, :n].double(), acc, atol=1e-3, rtol=1e-3)
+
+
+# ---------------------------------------------------------------- reuse
+def _reuse_prefill_brute(q, k, v, idx, hm, tile, rolling, p):
+    B, L, H, D = q.shape
+    G = k.shape[2]
+    rep = H // G
+    K = idx.shape[-1]
+    out = torch.zeros(B, L, H, D, dtype=torch.float64)
+    for b in range(B):
+        for i in range(L):
+            t = i // tile
+            n = orc.prefill_budget(t, tile, L, p, rolling, K)
+            for h in range(H):
+                g = h // rep
+                if t * tile <= n:
+                    keys = set(range(i + 1))
+                else:
+                    keys = set(int(x) for x in idx[b, hm[g], t, :n]) | set(range(t * tile, i + 1))
+                    keys = {j for j in keys if j <= i}
+                ks = sorted(keys)
+                s = (k[b, ks, g].double() @ q[b, i, h].double()) / math.sqrt(D)
+                out[b, i, h] = torch.softmax(s, 0) @ v[b, ks, g].double()
+    return out
+
+
+@pytest.mark.parametrize("rolling", [False, True])
+def test_reuse_prefill_brute_force(rolling):
+    L, tile, p = 400, 32, 10
+    q, k, v = _qkv(1, L, 4, 2, 8, seed=9)
+    K = 160     # sparse regime from tile 6 (192 > 160) when not rolling, tile 5 when rolling (n=128)
+    pooled = orc.pooled_prefill_scores(q, k, tile)
+    idx = orc.topk_rows(pooled, K)
+    hm = [1, 0]
+    got = orc.reuse_prefill(q, k, v, idx, hm, tile, rolling, p, block_tiles=3)
+    want = _reuse_prefill_brute(q, k, v, idx, hm, tile, rolling, p)
+    assert torch.allclose(got.double(), want, atol=1e-5)
+
+
+def test_reuse_prefill_special_cases():
+    L, tile = 200, 32
+    q, k, v = _qkv(1, L, 4, 2, 8, seed=4)
+    dense, _ = orc.dense_prefill(q, k, v)
+    T = math.ceil(L / tile)
+    # every tile in the dense regime
+    idx = torch.zeros(1, 2, T, L, dtype=torch.int32)
+    assert torch.allclose(orc.reuse_prefill(q, k, v, idx, [0, 1], tile, False, 10), dense, atol=1e-6)
+    # index rows listing all earlier keys == dense, whatever the regime (budget 64 < tile start)
+    K = 64
+    idx = torch.zeros(1, 2, T, K, dtype=torch.int32)
+    kk = k.clone()
+    for t in range(T):
+        idx[:, :, t] = torch.arange(K) % max(1, t * tile) if t * tile <= K else torch.arange(K)
+    # keys beyond the 64 selected get -inf scores through a huge negative key; instead compare
+    # against the masked definition on a case where selected ∪ diagonal covers everything:
+    L2 = 96
+    q2, k2, v2 = _qkv(1, L2, 4, 2, 8, seed=5)
+    idx2 = torch.arange(64, dtype=torch.int32).view(1, 1, 1, 64).expand(1, 2, 3, 64).contiguous()
+    d2, _ = orc.dense_prefill(q2, k2, v2)
+    # tile 2 starts at 64 == budget -> dense regime by the "<=" rule; tile 0,1 dense as well
+    assert torch.allclose(orc.reuse_prefill(q2, k2, v2, idx2, [0, 1], 32, False, 10), d2, atol=1e-6)
+    # head map identity: map m on idx == identity on idx[:, m]
+    pooled = orc.pooled_prefill_scores(q, k, tile)
+    idx = orc.topk_rows(pooled, 96)
+    a = orc.reuse_prefill(q, k, v, idx, [1, 1], tile, False, 10)
+    b = orc.reuse_prefill(q, k, v, idx[:, [1, 1]].contiguous(), [0, 1], tile, False, 10)
+    assert torch.equal(a, b)
+
+
+def test_reuse_decode_forms_agree():
+    B, H, G, D, L, K = 2, 8, 2, 16, 300, 64
+    g = torch.Generator().manual_seed(6)
+    q = torch.randn(B, H, D, generator=g)
+    k = torch.randn(B, L, G, D, generator=g)
+    v = torch.randn(B, L, G, D, generator=g)
+    idx = torch.stack([torch.stack([torch.randperm(L, generator=g)[:K] for _ in range(G)]) for _ in range(B)]).int()
+    hm = [1, 0]
+    a = orc.reuse_decode(q, k, v, idx, hm)
+    b = orc.reuse_decode_scatter(q, k, v, idx, hm)
+    assert torch.allclose(a, b, atol=1e-5)
+    # per-sequence prefix
+    a2 = orc.reuse_decode(q, k, v, idx, hm, counts=[64, 20])
+    b2 = orc.reuse_decode_scatter(q, k, v, idx, hm, counts=[64, 20])
+    assert torch.allclose(a2, b2, atol=1e-5) and not torch.allclose(a2[1], a[1], atol=1e-5)
+    # all keys selected == dense decode
+    full = torch.arange(L, dtype=torch.int32).view(1, 1, L).expand(B, G, L).contiguous()
+    d, _ = orc.dense_decode(q, k, v)
+    assert torch.allclose(orc.reuse_decode(q, k, v, full, [0, 1]), d, atol=1e-5)
+    # duplicates: idempotent in the scatter form, double-counted in the gather form
+    dup = idx.clone()
+    dup[:, :, 1] = dup[:, :, 0]
+    assert not torch.allclose(orc.reuse_decode(q, k, v, dup, hm), orc.reuse_decode_scatter(q, k, v, dup, hm), atol=1e-6)
+
+
+def test_anchor_decode_observables():
+    B, H, G, D, L = 2, 8, 2, 16, 1500
+    g = torch.Generator().manual_seed(8)
+    q = torch.randn(B, H, D, generator=g)
+    k = torch.randn(B, L, G, D, generator=g)
+    v = torch.randn(B, L, G, D, generator=g)
+    o, idx, agg = orc.anchor_decode(q, k, v, 10, layer0=True)
+    assert tuple(idx.shape) == (B, G, orc.k_kern(L, 10)) and idx.dtype == torch.int32
+    assert torch.allclose(o, orc.dense_decode(q, k, v)[0])
+    vals = torch.gather(agg.float(), 2, idx.long())
+    assert bool((vals[..., :-1] >= vals[..., 1:]).all())             # sorted descending
+    rest = agg.float().clone().scatter_(2, idx.long(), -1.0)
+    assert bool((rest.max(-1).values <= vals[..., -1]).all())        # nothing larger left out
+    o1, idx1, _ = orc.anchor_decode(q, k, v, 10, layer0=False)
+    assert torch.allclose(o1, orc.reuse_decode(q, k, v, idx1, [0, 1]))
+    # ragged
+    lens = [1500, 640]
+    o2, idx2, agg2 = orc.anchor_decode(q, k, v, 10, layer0=False, seqlens=lens)
+    assert idx2.shape[-1] == orc.max_topk_kvcache(1500, 10) == 256
+    n1 = orc.n_kvcache(640, 10)
+    assert n1 == 128 and int(idx2[1, :, :n1].max()) < 640
+
+
+def test_topk_agreement_metric():
+    s = torch.tensor([0.5, 0.1, 0.5, 0.3, 0.0, 0.3, 0.2])
+    ok, rec, _ = orc.topk_agreement(s, torch.tensor([0, 2, 3]), 3, 7)
+    assert ok and rec == 1.0
+    ok, _, _ = orc.topk_agreement(s, torch.tensor([0, 2, 5]), 3, 7)       # tie at the threshold
+    assert ok
+    ok, _, _ = orc.topk_agreement(s, torch.tensor([0, 3, 5]), 3, 7)       # misses a strict member
+    assert not ok
+    ok, _, _ = orc.topk_agreement(s, torch.tensor([0, 2, 6]), 3, 7, ulps=0)  # below the threshold
+    assert not ok
+    ok, _, _ = orc.topk_agreement(s, torch.tensor([0, 0, 2]), 3, 7)       # duplicate
+    assert not ok
+    ok, _, _ = orc.topk_agreement(s, torch.tensor([0, 2, 6]), 3, 6)       # out of the valid range
+    assert not ok
+
+
+# ----------------------------------------------------- strategy semantics
+def _strategy_case(L=256, B=1, H=8, G=2, D=16, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, H, L, D, generator=g)
+    k = torch.randn(B, G, L, D, generator=g)
+    v = torch.randn(B, G, L, D, generator=g)
+    return q, k, v
+
+
+@pytest.mark.parametrize("rolling", [False, True])
+def test_strategy_oracle_layer0_dense_and_reuse_definition(rolling):
+    L, tile, p = 512, 32, 30
+    q, k, v = _strategy_case(L)
+    mask = orc.causal_additive_mask(L, L, torch.float32)
+    st = orc.StrategyOracle([0], [[0, 1], [1, 0]], k=p, tile_size=tile, rolling_prefill=rolling, block_size=128)
+    o0 = st.attention_forward(0, q, k, v, mask, 16 ** -0.5)
+    dense, _ = orc.dense_prefill(q.permute(0, 2, 1, 3), k.permute(0, 2, 1, 3), v.permute(0, 2, 1, 3))
+    assert torch.allclose(o0, dense, atol=1e-5)
+    kw = orc.k_strat(L, p, tile)
+    assert tuple(st._topk_to_reuse.shape) == (1, 2, L, kw)
+    # rows are constant within a tile
+    tt = st._topk_to_reuse.view(1, 2, L // tile, tile, kw)
+    assert bool((tt == tt[:, :, :, :1]).all())
+    # one-shot == blocked
+    st1 = orc.StrategyOracle([0], [[0, 1], [1, 0]], k=p, tile_size=tile, rolling_prefill=rolling, block_size=12288)
+    o0b = st1.attention_forward(0, q, k, v, mask, 16 ** -0.5)
+    assert torch.allclose(o0, o0b, atol=1e-6) and torch.equal(st._topk_to_reuse, st1._topk_to_reuse)
+    # reuse layer: masked attention over (stored indices ∪ in-tile diagonal), by loops
+    q1 = q + 0.3 * torch.randn(q.shape, generator=torch.Generator().manual_seed(5))
+    o1 = st.attention_forward(1, q1, k, v, mask, 16 ** -0.5)
+    idx = st._topk_to_reuse
+    want = torch.zeros_like(o1)
+    for i in range(0, L, 37):
+        for h in range(8):
+            g = h // 4
+            keys = {int(x) for x in idx[0, [1, 0][g], i]} | set(range((i // tile) * tile, i + 1))
+            ks = sorted(j for j in keys if j <= i)
+            s = (k[0, g, ks] @ q1[0, h, i]) * 16 ** -0.5
+            want[0, i, h] = torch.softmax(s, 0) @ v[0, g, ks]
+            assert torch.allclose(o1[0, i, h], want[0, i, h], atol=1e-5), (i, h)
+
+
+def test_strategy_oracle_decode_step():
+    L, p = 700, 20
+    q, k, v = _strategy_case(L, seed=2)
+    st = orc.StrategyOracle([0], [[0, 1], [1, 1]], k=p, tile_size=32, rolling_prefill=False)
+    qd = q[:, :, -1:]
+    mask = torch.zeros(1, 1, 1, L)
+    o0 = st.attention_forward(0, qd, k, v, mask, 16 ** -0.5)
+    dd, _ = orc.dense_decode(qd[:, :, 0], k.permute(0, 2, 1, 3), v.permute(0, 2, 1, 3))
+    assert torch.allclose(o0[:, 0], dd, atol=1e-5)
+    kw = orc.k_strat(L, p, 32)
+    assert tuple(st._topk_to_reuse.shape) == (1, 2, 1, kw)
+    o1 = st.attention_forward(1, qd, k, v, mask, 16 ** -0.5)
+    want = orc.reuse_decode(qd[:, :, 0], k.permute(0, 2, 1, 3), v.permute(0, 2, 1, 3),
+                            st._topk_to_reuse[:, :, 0], [1, 1])
+    assert torch.allclose(o1[:, 0], want, atol=1e-5)
+
+
+# ------------------------------------------------------------ data fixtures
+def test_head_mapping_fixtures():
+    root = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "kascade_amd", "head_mappings")
+    specs = {"Meta-Llama-3.1-8B-Instruct_layers_0_2_8_13_14.npy": (32, [0, 2, 8, 13, 14]),
+             "DeepSeek-R1-Distill-Llama-8B_layers_0_2_8_13_14.npy": (32, [0, 2, 8, 13, 14]),
+             "Qwen3-8B_layers_0_2_7_14_23.npy": (36, [0, 2, 7, 14, 23])}
+    for name, (layers, anchors) in specs.items():
+        a = np.load(os.path.join(root, name), allow_pickle=False)
+        assert a.shape == (layers, 8) and a.dtype == np.int32
+        assert a.min() >= 0 and a.max() <= 7
+        for l in anchors:
+            assert a[l].tolist() == list(range(8))
