@@ -84,7 +84,9 @@ int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K
 
 /* Dense split-K decode (the reference's TileLang dense baseline, gqa_decode.py:117-254 and
  * gqa_decode_with_kvcache.py:118-257), same cache conventions as above.
- * cache_seqlens may be NULL (all sequences have kv_stride_tokens tokens). */
+ * cache_seqlens may be NULL (all sequences have kv_stride_tokens tokens).  With a block
+ * table kv_stride_tokens is an upper bound on the sequence lengths (0: max_pages*page_size);
+ * it sizes the splits. */
 int kascade_decode_dense_paged_call(const kascade_half* Q, const kascade_half* K,
                                     const kascade_half* V, const int32_t* cache_seqlens,
                                     float* glse, float* Output_partial, kascade_half* Output,

@@ -50,6 +50,11 @@ int check_strides(const kascade_strides& s, const char* name) {
     return 0;
 }
 
+int rows_per_split(long long max_rows, int num_split) {
+    long long r = (max_rows + num_split - 1) / num_split;
+    return (int)(((r + 63) / 64) * 64);
+}
+
 int check_paging(const int32_t* block_table, int max_pages, int page_size, int* page_shift) {
     if (!block_table) {
         *page_shift = 0;
@@ -114,6 +119,7 @@ int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K
     p.block_table = block_table; p.glse = glse; p.opart = Output_partial; p.scores = nullptr;
     p.max_pages = max_pages; p.page_shift = shift; p.kv_stride_tokens = kv_stride_tokens;
     p.topk = topk; p.topk_percent = topk_percent; p.scores_stride = 0; p.num_split = num_split;
+    p.rows_per_split = rows_per_split(topk, num_split);
     p.B = batch;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (check_hip(launch_decode_split(p, true, true, false, s), "decode_reuse split")) return -1;
@@ -140,6 +146,8 @@ int kascade_decode_dense_paged_call(const kascade_half* Q, const kascade_half* K
     p.seqlens = cache_seqlens; p.block_table = block_table; p.glse = glse; p.opart = Output_partial;
     p.max_pages = max_pages; p.page_shift = shift; p.kv_stride_tokens = kv_stride_tokens;
     p.num_split = num_split; p.B = batch;
+    const long long max_rows = kv_stride_tokens > 0 ? kv_stride_tokens : (long long)max_pages * page_size;
+    p.rows_per_split = rows_per_split(max_rows, num_split);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (check_hip(launch_decode_split(p, false, true, false, s), "decode_dense split")) return -1;
     return check_hip(launch_decode_combine(glse, Output_partial, H(Output), nullptr, batch,
@@ -176,6 +184,9 @@ int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_hal
     p.scores = scores; p.scores_stride = scores_stride;
     p.max_pages = max_pages; p.page_shift = shift; p.kv_stride_tokens = kv_stride_tokens;
     p.num_split = num_split; p.B = batch;
+    long long max_rows = kv_stride_tokens > 0 ? kv_stride_tokens : (long long)max_pages * page_size;
+    if (max_rows > scores_stride) max_rows = scores_stride;
+    p.rows_per_split = rows_per_split(max_rows, num_split);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (check_hip(launch_decode_split(p, false, with_output != 0, true, s), "decode_recompute split"))
         return -1;

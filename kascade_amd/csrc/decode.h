@@ -22,6 +22,7 @@ struct DecodeParams {
     float topk_percent;
     int scores_stride;
     int num_split;
+    int rows_per_split;     // multiple of 64; num_split*rows_per_split >= longest row list
     int B;
 };
 

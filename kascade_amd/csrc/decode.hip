@@ -19,7 +19,10 @@ namespace kascade {
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kUnroll = 8;                    // rows per row-group per iteration
+#ifndef KASCADE_DECODE_UNROLL
+#define KASCADE_DECODE_UNROLL 8
+#endif
+constexpr int kUnroll = KASCADE_DECODE_UNROLL;  // rows per row-group per iteration
 constexpr int kRowsPerIter = 16 * kUnroll;    // rows per workgroup iteration (128)
 constexpr int kSubChunk = 2048;               // rows whose physical ids are staged in LDS at once
 
@@ -56,12 +59,11 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(DecodeParams p) 
     } else {
         n = seqlen;
     }
-    // contiguous range of this split, multiple of 64 rows
-    int rps = (n + p.num_split - 1) / p.num_split;
-    rps = ((rps + 63) / 64) * 64;
-    const long long r0l = (long long)split * rps;
+    // contiguous range of this split; every split covers rows_per_split rows, sequences
+    // shorter than num_split*rows_per_split leave their last splits empty
+    const long long r0l = (long long)split * p.rows_per_split;
     const int r0 = (int)min((long long)n, r0l);
-    const int r1 = (int)min((long long)n, r0l + rps);
+    const int r1 = (int)min((long long)n, r0l + p.rows_per_split);
 
     // q fragments: 4 heads x 8 halves of this lane's d-slice
     Pack16 qf[kGroupSize];
@@ -83,6 +85,82 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(DecodeParams p) 
     const int page_mask = (1 << p.page_shift) - 1;
     const size_t head_off = (size_t)g * kDim + dl * 8;
 
+    struct Batch {
+        Pack16 k[kUnroll];
+        Pack16 v[kUnroll];
+    };
+    // wave covers 32 consecutive rows of an iteration: row = it + wave*32 + u*4 + rg
+    auto load_batch = [&](int it, int cn, Batch& bt) {
+        if (it >= cn) return;
+        const int rbase = it + wave * (4 * kUnroll) + rg;
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const int r = rbase + u * 4;
+            const int row = s_row[r < cn ? r : (cn - 1)];
+            const size_t off = (size_t)row * (kGroups * kDim) + head_off;
+            bt.k[u].u = ld_global_16(p.K + off);
+            if (WITH_V) bt.v[u].u = ld_global_16(p.V + off);
+        }
+    };
+    auto compute_batch = [&](int it, int cn, int c0, const Batch& bt) {
+        if (it >= cn) return;
+        const int rbase = it + wave * (4 * kUnroll) + rg;
+        float s[kUnroll][kGroupSize];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const bool valid = (rbase + u * 4) < cn;
+#pragma unroll
+            for (int h = 0; h < kGroupSize; ++h) {
+                float d = dot8(bt.k[u], qf[h], 0.f);
+                d = row16_sum(d);
+                s[u][h] = valid ? d : -INFINITY;
+            }
+        }
+        if (WRITE_SCORES) {
+            // lanes dl < kUnroll write the four heads of row u = dl: for a fixed head the
+            // wavefront stores 4*kUnroll consecutive tokens.
+            float w[kGroupSize] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+                for (int h = 0; h < kGroupSize; ++h) w[h] = (u == dl) ? s[u][h] : w[h];
+            }
+            const int r = rbase + dl * 4;
+            if (dl < kUnroll && r < cn) {
+                const int tok = c0 + r;  // dense mode only: token id == row number
+                float* sp = p.scores + ((size_t)b * kHeads + g * kGroupSize) * p.scores_stride + tok;
+#pragma unroll
+                for (int h = 0; h < kGroupSize; ++h) sp[(size_t)h * p.scores_stride] = w[h];
+            }
+        }
+#pragma unroll
+        for (int h = 0; h < kGroupSize; ++h) {
+            float mx = m[h];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) mx = fmaxf(mx, s[u][h]);
+            const float mref = (mx == -INFINITY) ? 0.f : mx * kScaleLog2;
+            const float corr = fast_exp2(m[h] * kScaleLog2 - mref);  // m=-inf -> 0
+            m[h] = mx;
+            float ps[kUnroll];
+            float sum = 0.f;
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                ps[u] = fast_exp2(s[u][h] * kScaleLog2 - mref);
+                sum += ps[u];
+            }
+            l[h] = l[h] * corr + sum;
+            if (WITH_V) {
+#pragma unroll
+                for (int d = 0; d < 8; ++d) {
+                    float a = acc[h][d] * corr;
+#pragma unroll
+                    for (int u = 0; u < kUnroll; ++u) a = fmaf(ps[u], (float)bt.v[u].h[d], a);
+                    acc[h][d] = a;
+                }
+            }
+        }
+    };
+
     for (int c0 = r0; c0 < r1; c0 += kSubChunk) {
         const int cn = min(kSubChunk, r1 - c0);
         __syncthreads();
@@ -100,74 +178,14 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(DecodeParams p) 
         }
         __syncthreads();
 
-        for (int it = 0; it < cn; it += kRowsPerIter) {
-            // wave covers 32 consecutive rows of the iteration: row = it + wave*32 + u*4 + rg
-            const int rbase = it + wave * 32 + rg;
-            Pack16 kf[kUnroll];
-            Pack16 vf[kUnroll];
-            bool valid[kUnroll];
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
-                int r = rbase + u * 4;
-                valid[u] = r < cn;
-                int row = s_row[valid[u] ? r : (cn - 1)];
-                size_t off = (size_t)row * (kGroups * kDim) + head_off;
-                kf[u].u = ld_global_16(p.K + off);
-                if (WITH_V) vf[u].u = ld_global_16(p.V + off);
-            }
-            float s[kUnroll][kGroupSize];
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
-#pragma unroll
-                for (int h = 0; h < kGroupSize; ++h) {
-                    float d = dot8(kf[u], qf[h], 0.f);
-                    d = row16_sum(d);
-                    s[u][h] = valid[u] ? d : -INFINITY;
-                }
-            }
-            if (WRITE_SCORES) {
-                // lanes dl < 8 write the four heads of row u = dl: for a fixed head the
-                // wavefront stores 32 consecutive tokens.
-                float w[kGroupSize] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int u = 0; u < kUnroll; ++u) {
-#pragma unroll
-                    for (int h = 0; h < kGroupSize; ++h) w[h] = (u == dl) ? s[u][h] : w[h];
-                }
-                const int r = rbase + dl * 4;
-                if (dl < kUnroll && r < cn) {
-                    const int tok = c0 + r;  // dense mode only: token id == row number
-                    float* sp = p.scores + ((size_t)b * kHeads + g * kGroupSize) * p.scores_stride + tok;
-#pragma unroll
-                    for (int h = 0; h < kGroupSize; ++h) sp[(size_t)h * p.scores_stride] = w[h];
-                }
-            }
-#pragma unroll
-            for (int h = 0; h < kGroupSize; ++h) {
-                float mx = m[h];
-#pragma unroll
-                for (int u = 0; u < kUnroll; ++u) mx = fmaxf(mx, s[u][h]);
-                const float mref = (mx == -INFINITY) ? 0.f : mx * kScaleLog2;
-                const float corr = fast_exp2(m[h] * kScaleLog2 - mref);  // m=-inf -> 0
-                m[h] = mx;
-                float ps[kUnroll];
-                float sum = 0.f;
-#pragma unroll
-                for (int u = 0; u < kUnroll; ++u) {
-                    ps[u] = fast_exp2(s[u][h] * kScaleLog2 - mref);
-                    sum += ps[u];
-                }
-                l[h] = l[h] * corr + sum;
-                if (WITH_V) {
-#pragma unroll
-                    for (int d = 0; d < 8; ++d) {
-                        float a = acc[h][d] * corr;
-#pragma unroll
-                        for (int u = 0; u < kUnroll; ++u) a = fmaf(ps[u], (float)vf[u].h[d], a);
-                        acc[h][d] = a;
-                    }
-                }
-            }
+        // software pipeline: the loads of iteration i+1 are in flight while iteration i computes
+        Batch ba, bb;
+        load_batch(0, cn, ba);
+        for (int it = 0; it < cn; it += 2 * kRowsPerIter) {
+            load_batch(it + kRowsPerIter, cn, bb);
+            compute_batch(it, cn, c0, ba);
+            load_batch(it + 2 * kRowsPerIter, cn, ba);
+            compute_batch(it + kRowsPerIter, cn, c0, bb);
         }
     }
 

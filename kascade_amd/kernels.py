@@ -48,13 +48,16 @@ def _blhd_strides(t: torch.Tensor, name: str) -> Strides:
     return Strides(t.stride(0), t.stride(1), t.stride(2))
 
 
-def default_num_split(rows_per_seq: int, pairs: int) -> int:
-    """Split count for a decode launch: enough workgroups to cover the device several
-    times over while keeping at least 256 rows per split."""
+def default_num_split(total_rows: int, max_rows: int, wgs_per_cu: int = 2, min_rows: int = 512) -> int:
+    """Split count for a decode launch.  Every split covers the same number of rows
+    (ceil(max_rows/num_split)), so the number of non-empty workgroups is about
+    total_rows / rows_per_split; aim at wgs_per_cu of them per compute unit without
+    dropping below min_rows rows per workgroup (per-workgroup set-up is not free).
+    total_rows = sum over (sequence, KV head) of the rows visited; max_rows = longest list."""
     cus = _lib.init().kascade_device_cu_count() or 256
-    want = max(1, (8 * cus + pairs - 1) // pairs)
-    by_rows = max(1, rows_per_seq // 256)
-    return int(max(1, min(want, by_rows, 256)))
+    target_wgs = wgs_per_cu * cus
+    rows_per_split = max(min_rows, -(-total_rows // target_wgs))
+    return int(max(1, min(256, -(-max_rows // rows_per_split))))
 
 
 # ---------------------------------------------------------------- decode
