@@ -1,0 +1,295 @@
+#!/usr/bin/env python3
+"""Benchmark of the Kascade attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Timed region ("step"): one prefill attention pass of a 32-layer Llama-3.1-8B-shaped stack at
+32K tokens (batch 1, 32 q-heads / 8 KV heads, head_dim 128, fp16, tile 32, top-k 10 %,
+rolling prefill): 1 anchor-0 layer, 4 anchor layers, 27 reuse layers -- the layer mix the
+reference's own table weights its columns by.  ``value`` is the layer-weighted mean attention
+time per layer in ms (= ms_per_step / 32), inputs resident in HBM.
+
+Outside the timed region the same process measures, with HIP events on the launch stream:
+each kernel of the step on its own (roofline figures), the dense prefill baseline, paged
+decode (dense / anchor-0 / anchor / reuse, rotating over several distinct layer caches so that
+every call finds its K/V cold in HBM) and a bounded CPU run of the oracle (reported baseline).
+
+One JSON line is printed on stdout; progress goes to stderr.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+H, G, D, TILE = 32, 8, 128, 32
+PCT = 10
+ANCHORS = (0, 2, 8, 13, 14)
+N_LAYERS = 32
+HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
+MFMA_PEAK_TFLOPS = 2500.0      # MI355X published dense fp16 MFMA rate
+H100_PREFILL_32K_MS = 6.42     # reference's published Kascade prefill ms @32768 (H100)
+
+
+def log(msg):
+    print(msg, file=sys.stderr, flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--seq-len", type=int, default=32768)
+    ap.add_argument("--skip-decode", action="store_true")
+    ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--decode-only", action="store_true", help="skip the per-kernel prefill section")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from kascade_amd import _lib, kernels, budgets, workloads
+    from kascade_amd.strategy import EfficientKascadeStrategy, PagedKascadeDecoder, get_head_mapping
+
+    _lib.init()   # no fallback: raises if libkascade_hip.so is missing
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    def ev_time(fn, n=5, warm=1):
+        """Median duration (us) of fn() measured with events on the stream the kernels launch on."""
+        for _ in range(warm):
+            fn()
+        ts = []
+        for _ in range(n):
+            s = torch.cuda.Event(enable_timing=True)
+            e = torch.cuda.Event(enable_timing=True)
+            s.record()
+            fn()
+            e.record()
+            e.synchronize()
+            ts.append(s.elapsed_time(e) * 1e3)
+        ts.sort()
+        return ts[len(ts) // 2]
+
+    head_map = get_head_mapping("Meta-Llama-3.1-8B-Instruct", list(ANCHORS))
+
+    # ------------------------------------------------------------------ prefill, 32K
+    L = args.seq_len
+    log(f"[bench] generating prefill inputs L={L}")
+    w = workloads.prefill_inputs(1, L, seed=0, device=dev)
+    strat = EfficientKascadeStrategy(list(ANCHORS), None, k=PCT, tile_size=TILE, rolling_prefill=True,
+                                     head_mapping=head_map, register=False)
+    width = budgets.topk_width(L, PCT)
+    T = math.ceil(L / TILE)
+
+    def prefill_layer(layer):
+        if layer in ANCHORS:
+            return strat._prefill_recomp_forward(w.q, w.k, w.v, width, TILE, layer, PCT)
+        return strat._prefill_reuse_forward(w.q_reuse, w.k_reuse, w.v, PCT, layer)
+
+    def prefill_step():
+        for layer in range(N_LAYERS):
+            prefill_layer(layer)
+
+    log("[bench] warmup")
+    for _ in range(args.warmup):
+        prefill_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        prefill_step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    value = ms_per_step / N_LAYERS
+    log(f"[bench] prefill step {ms_per_step:.2f} ms -> {value:.3f} ms/layer")
+
+    # ---- per-kernel timings of the same workload (HIP events, current stream) ----
+    kern = {}
+    flop_dense = 2.0 * H * L * L * D               # causal QK^T + PV
+    flop_qk = 1.0 * H * L * L * D                  # causal QK^T only
+    sum_m = 0
+    gathered = 0
+    for t in range(T):
+        n = budgets.rolling_budget(t * TILE, PCT)
+        if t * TILE <= n:
+            sum_m += min((t + 1) * TILE, L)
+        else:
+            sum_m += n + TILE
+            gathered += n
+    flop_reuse = 4.0 * D * (H // G) * TILE * G * sum_m
+    if not args.decode_only:
+        t_dense = ev_time(lambda: kernels.prefill_dense(w.q, w.k, w.v), n=3)
+        t_p0 = ev_time(lambda: kernels.prefill_recompute0(w.q, w.k, w.v), n=3)
+        t_p1 = ev_time(lambda: kernels.prefill_recompute1(w.q, w.k), n=3)
+        log_sum = kernels.prefill_recompute1(w.q, w.k)
+        scores = torch.empty(1, G, T, L, device=dev, dtype=torch.float16)
+        t_agg = ev_time(lambda: kernels.prefill_aggregate(w.q, w.k, log_sum, scores), n=3)
+        valid, nsel = strat._tile_budgets(L, width, dev)
+        t_topk = ev_time(lambda: kernels.topk_indices(scores, width, valid_len=valid, n_sel=nsel), n=3)
+        idx = kernels.topk_indices(scores, width, valid_len=valid, n_sel=nsel)
+        hm = strat._hm(1, dev)
+        t_reuse = ev_time(lambda: kernels.prefill_reuse(w.q_reuse, w.k_reuse, w.v, idx, hm, float(PCT), True), n=5)
+        del scores, idx, log_sum
+
+        def mfma(flop, us):
+            a = flop / us / 1e6
+            return {"bound": "mfma", "achieved": round(a, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(a / MFMA_PEAK_TFLOPS, 4), "us": round(us, 1)}
+        kern["prefill_attn_dense(QK+PV+lse)"] = mfma(flop_dense, t_p0)
+        kern["prefill_attn_dense(baseline, no lse)"] = mfma(flop_dense, t_dense)
+        kern["prefill_attn_scores(QK only)"] = mfma(flop_qk, t_p1)
+        kern["prefill_aggregate"] = mfma(flop_qk, t_agg)
+        kern["prefill_attn_reuse"] = mfma(flop_reuse, t_reuse)
+        kern["prefill_attn_reuse"]["gathered_GBps"] = round(gathered * G * D * 2 * 2 / t_reuse / 1e3, 1)
+        sel_bytes = G * sum(32 * t for t in range(T)) * 2
+        kern["topk_select(prefill)"] = {"bound": "hbm", "achieved": round(sel_bytes / t_topk / 1e3, 1),
+                                        "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                        "frac": round(sel_bytes / t_topk / 1e3 / HBM_PEAK_GBS, 4),
+                                        "us": round(t_topk, 1)}
+        t_a0 = t_p0 + t_agg + t_topk
+        t_a = t_p1 + t_agg + t_topk + t_reuse
+        prefill = {"seq_len": L, "dense_ms": round(t_dense / 1e3, 3), "anchor0_ms": round(t_a0 / 1e3, 3),
+                   "anchor_ms": round(t_a / 1e3, 3), "reuse_ms": round(t_reuse / 1e3, 3),
+                   "kascade_ms_per_layer": round(value, 3),
+                   "speedup_vs_dense": round(t_dense / 1e3 / value, 3)}
+        # dominant kernel of the timed step = largest total time
+        totals = {"prefill_attn_reuse": 31 * t_reuse, "prefill_aggregate": 5 * t_agg,
+                  "prefill_attn_dense(QK+PV+lse)": t_p0, "prefill_attn_scores(QK only)": 4 * t_p1}
+        dom = max(totals, key=totals.get)
+        roofline = dict(kern[dom])
+        roofline["kernel"] = dom
+        roofline["traffic"] = None
+    else:
+        prefill, roofline = {}, {"bound": "mfma", "achieved": None, "peak": MFMA_PEAK_TFLOPS,
+                                 "unit": "TFLOP/s", "frac": None, "traffic": None}
+    del w
+    torch.cuda.empty_cache()
+
+    # ------------------------------------------------------------------ paged decode
+    decode = {}
+    if not args.skip_decode:
+        cases = [("cfg2_B16_L65536", [65536] * 16, False, 4),
+                 ("B16_L131072", [131072] * 16, False, 3),
+                 ("cfg3_ragged_B4", [131072, 196608, 262144, 524288], True, 4)]
+        for name, seqlens, ragged, n_caches in cases:
+            log(f"[bench] decode {name}: generating {n_caches} layer caches")
+            B, max_len = len(seqlens), max(seqlens)
+            caches = [workloads.paged_decode_inputs(seqlens, seed=10 + i, device=dev, reuse_keys=False)
+                      for i in range(n_caches)]
+            c0 = caches[0]
+            dec = PagedKascadeDecoder(PCT, head_map, ANCHORS, B, max_len, page_size=16, device=dev)
+            calls = [0]
+
+            def cache():
+                calls[0] += 1
+                return caches[calls[0] % n_caches]
+
+            def dense_layer():
+                c = cache()
+                return dec.dense(c.q, c.k_pages, c.v_pages, c0.block_table, c0.seqlens, max_len)
+
+            def kascade_layer(layer):
+                c = cache()
+                return dec.forward(layer, c.q, c.k_pages, c.v_pages, c0.block_table, c0.seqlens, max_len,
+                                   ragged=ragged)
+
+            def kascade_step():
+                for layer in range(N_LAYERS):
+                    kascade_layer(layer)
+
+            def dense_step():
+                for _ in range(N_LAYERS):
+                    dense_layer()
+
+            t_dense = ev_time(dense_step, n=3) / N_LAYERS
+            t_kas = ev_time(kascade_step, n=3) / N_LAYERS
+            t_a0 = ev_time(lambda: kascade_layer(0), n=5)
+            t_a = ev_time(lambda: kascade_layer(2), n=5)
+            kascade_layer(0)
+            t_r = ev_time(lambda: kascade_layer(1), n=9)
+            counts = [budgets.decode_budget(n, PCT) if ragged else budgets.topk_width(n, PCT) for n in seqlens]
+            reuse_bytes = sum(G * n * D * 2 * 2 + G * n * 4 for n in counts) + 2 * B * H * D * 2
+            dense_bytes = sum(n * G * D * 2 * 2 for n in seqlens)
+            decode[name] = {
+                "dense_us": round(t_dense, 1), "anchor0_us": round(t_a0, 1), "anchor_us": round(t_a, 1),
+                "reuse_us": round(t_r, 1), "kascade_us_per_layer": round(t_kas, 1),
+                "speedup_vs_dense": round(t_dense / t_kas, 3),
+                "reuse_GBps": round(reuse_bytes / t_r / 1e3, 1),
+                "reuse_frac_hbm": round(reuse_bytes / t_r / 1e3 / HBM_PEAK_GBS, 4),
+                "dense_GBps": round(dense_bytes / t_dense / 1e3, 1),
+                "dense_frac_hbm": round(dense_bytes / t_dense / 1e3 / HBM_PEAK_GBS, 4),
+                "num_split_dense": dec.ns_dense, "num_split_reuse": dec.ns_reuse,
+            }
+            log(f"[bench] decode {name}: {decode[name]}")
+            del caches, c0, dec
+            torch.cuda.empty_cache()
+
+    # ------------------------------------------------------------------ CPU baseline (oracle)
+    cpu = None
+    if not args.skip_cpu:
+        from oracle import kascade_oracle as orc
+        nthreads = torch.get_num_threads()
+        Lc = args.seq_len
+        log(f"[bench] cpu baseline: oracle on {nthreads} threads (os.cpu_count()={os.cpu_count()})")
+        wc = workloads.prefill_inputs(1, Lc, seed=0, device="cpu")
+        nblk, rows = 4, 256
+        est = {"anchor0": 0.0, "anchor": 0.0, "reuse": 0.0}
+        idx_full = None
+        for i in range(nblk):
+            s = int((i + 0.5) * Lc / nblk) // TILE * TILE
+            e = min(s + rows, Lc)
+            ta, tb = s // TILE, math.ceil(e / TILE)
+            weight = (Lc / nblk) / (e - s)
+            t0 = time.perf_counter()
+            orc.dense_prefill(wc.q, wc.k, wc.v, rows=(s, e))
+            t_dense_blk = time.perf_counter() - t0
+            t0 = time.perf_counter()
+            pooled = orc.pooled_prefill_scores(wc.q, wc.k, TILE, tiles=(ta, tb))
+            idx_blk = orc.topk_rows(pooled, budgets.topk_width(Lc, PCT))
+            t_pool_blk = time.perf_counter() - t0
+            idx_full = torch.zeros(1, G, math.ceil(Lc / TILE), idx_blk.shape[-1], dtype=torch.int32)
+            idx_full[:, :, ta:tb] = idx_blk
+            t0 = time.perf_counter()
+            orc.reuse_prefill(wc.q_reuse, wc.k_reuse, wc.v, idx_full, wc.head_mapping, TILE, True, PCT,
+                              tiles=(ta, tb))
+            t_reuse_blk = time.perf_counter() - t0
+            est["anchor0"] += weight * (t_dense_blk + t_pool_blk)
+            est["anchor"] += weight * (t_pool_blk + t_reuse_blk)
+            est["reuse"] += weight * t_reuse_blk
+            log(f"[bench] cpu block {i}: rows {s}..{e}: dense {t_dense_blk:.2f}s pool+topk {t_pool_blk:.2f}s "
+                f"reuse {t_reuse_blk:.2f}s")
+        cpu_ms = (est["anchor0"] + 4 * est["anchor"] + 27 * est["reuse"]) / N_LAYERS * 1e3
+        cpu = {"value": round(cpu_ms, 1), "unit": "ms", "cores": nthreads, "kind": "port",
+               "sample": f"oracle (dense-matrix PyTorch, fp32) on {nblk} blocks of {rows} query rows centred in "
+                         f"each quarter of the {Lc}-token prompt, extrapolated by rows; layer mix 1/4/27",
+               "per_layer_ms": {k: round(v * 1e3, 1) for k, v in est.items()}}
+
+    out = {
+        "metric": "kascade prefill attn ms/layer @32K (value) & decode attn us/layer @64K/128K/ragged (decode), "
+                  "top-k 10%; % MFMA/HBM roofline",
+        "value": round(value, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 3), "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": round(value / H100_PREFILL_32K_MS, 4) if L == 32768 else None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "configs[1]: Llama-3.1-8B-shaped causal prefill attention, batch 1, seq 32768, "
+                               "32 q-heads / 8 KV heads, head_dim 128, tile 32, top-k 10%, rolling; one step = "
+                               "32 layers (1 anchor-0, 4 anchor, 27 reuse)",
+                   "seq_len": L, "layers_per_step": N_LAYERS,
+                   "baseline_note": "vs_baseline = value / 6.42 ms, the reference's published H100 figure"},
+        "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "decode": decode, "kernels": kern,
+    }
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

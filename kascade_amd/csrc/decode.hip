@@ -20,7 +20,7 @@ namespace {
 
 constexpr int kThreads = 256;
 #ifndef KASCADE_DECODE_UNROLL
-#define KASCADE_DECODE_UNROLL 8
+#define KASCADE_DECODE_UNROLL 4
 #endif
 constexpr int kUnroll = KASCADE_DECODE_UNROLL;  // rows per row-group per iteration
 constexpr int kRowsPerIter = 16 * kUnroll;    // rows per workgroup iteration (128)
@@ -56,6 +56,7 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(DecodeParams p) 
             n = p.topk;
         }
         n = min(n, p.topk);
+        if (p.seqlens) n = min(n, seqlen);   // never more rows than the sequence holds
     } else {
         n = seqlen;
     }
@@ -167,6 +168,7 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(DecodeParams p) 
         // stage physical row ids of this sub-chunk
         for (int i = tid; i < cn; i += kThreads) {
             int tok = GATHER ? idx_row[c0 + i] : (c0 + i);
+            tok = max(0, min(tok, seqlen - 1));   // a corrupt index must not leave the sequence
             int row;
             if (p.block_table) {
                 int pg = p.block_table[(size_t)b * p.max_pages + (tok >> p.page_shift)];

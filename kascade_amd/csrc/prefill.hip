@@ -109,8 +109,8 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillParams p)
                 nk[i] = min(ti * kKT + pk, L - 1);
                 nv[i] = min(ti * kKT + pv, L - 1);
             } else if (ti < ng) {
-                nk[i] = idx_row[min(ti * kKT + pk, n - 1)];
-                nv[i] = idx_row[min(ti * kKT + pv, n - 1)];
+                nk[i] = max(0, min(idx_row[min(ti * kKT + pk, n - 1)], L - 1));
+                nv[i] = max(0, min(idx_row[min(ti * kKT + pv, n - 1)], L - 1));
             } else {
                 nk[i] = min(q0 + pk, L - 1);
                 nv[i] = min(q0 + pv, L - 1);

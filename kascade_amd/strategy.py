@@ -1,0 +1,291 @@
+"""Host side of the Kascade hot path: the ``efficient_kascade`` attention strategy.
+
+``EfficientKascadeStrategy`` keeps the reference class's constructor, attributes,
+method seams and HF registration (src/strategies/EfficientKascadeStrategy.py:16-168,
+parents KascadeStrategy.py:11-16, 174-183 and Strategy.py:8-11), with the HIP
+kernels of libkascade_hip.so behind the seams:
+
+    attention_forward(module, query[B,H,Lq,D], key[B,G,Lk,D], value, mask, scaling)
+        -> (attn_output[B,Lq,H,D], None)
+    _prefill_recomp_forward / _prefill_reuse_forward
+    _decode_recomp_forward  / _decode_reuse_forward
+
+Differences, all inside the seams: strided [B,L,H,D] views of HF's [B,H,L,D]
+tensors go to the prefill kernels as they are (no copy); the anchor's top-k is an
+exact selection kernel that delivers each row's consumed prefix instead of a full
+sort; the decode split count adapts to the device instead of the fixed 8.
+
+``PagedKascadeDecoder`` is the paged-cache decode backend (block table, per
+sequence lengths) with the reference's kvcache call order
+(recompute_kascade_gqa_decode_with_kvcache.py:368-377).
+"""
+from __future__ import annotations
+
+import math
+import os
+from pathlib import Path
+from typing import List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from . import budgets, kernels
+from ._lib import KascadeError
+
+H, G, D, TILE = 32, 8, 128, 32
+
+
+def get_head_mapping(model_name: str, recompute_layers: Sequence[int],
+                     search_dirs: Optional[Sequence[os.PathLike]] = None) -> List[List[int]]:
+    """int32 [num_layers][G] head maps (KascadeStrategy.py:174-183).  Looked up as
+    ``{basename}_layers_{a_b_c}.npy`` in ./results/head_mappings (the reference's cwd-relative
+    location) and then in the package's own head_mappings directory."""
+    base = model_name.split("/")[-1]
+    fname = f"{base}_layers_{'_'.join(map(str, recompute_layers))}.npy"
+    dirs = list(search_dirs or []) + [Path("./results/head_mappings"),
+                                      Path(__file__).resolve().parent / "head_mappings"]
+    for d in dirs:
+        path = Path(d) / fname
+        if path.exists():
+            return np.load(path, allow_pickle=False).tolist()
+    raise ValueError(f"Head mapping file not found for model {model_name} with layers {list(recompute_layers)}.")
+
+
+class EfficientKascadeStrategy:
+    """Drop-in for the reference's EfficientKascadeStrategy (name ``efficient_kascade``)."""
+
+    def __init__(self, recompute_layers: List[int], model_name: Optional[str], k=1, tile_size=1,
+                 rolling_prefill=False, block_size=12288, head_mapping: Optional[List[List[int]]] = None,
+                 register: bool = True):
+        if recompute_layers is None:
+            raise ValueError("recompute_layers cannot be None for KascadeStrategy")
+        if not (0 <= k <= 100):
+            raise ValueError(f"Invalid k: {k}. It should be between 0 and 100%.")
+        if tile_size != TILE:
+            raise KascadeError(f"the kernels are specialised to tile_size={TILE}, got {tile_size}")
+        if 0 not in recompute_layers:
+            raise KascadeError("layer 0 must be a recompute (anchor) layer for the efficient path")
+        self.name = "efficient_kascade"
+        self.k = k
+        self.tile_size = tile_size
+        self.rolling_prefill = rolling_prefill
+        self.recompute_layers = list(recompute_layers)
+        self._block_size = block_size
+        self._head_mapping = head_mapping if head_mapping is not None else \
+            get_head_mapping(model_name, self.recompute_layers)
+        self._heads, self._dim, self._groups = H, D, G
+        self._topk_to_reuse = None
+        self._hm_cache = {}
+        self._budget_cache = {}
+        if register:
+            self.register_attention()
+
+    # ------------------------------------------------------------------ helpers
+    def _hm(self, layer, device) -> torch.Tensor:
+        key = (layer, str(device))
+        if key not in self._hm_cache:
+            row = list(range(G)) if layer is None else self._head_mapping[layer]
+            self._hm_cache[key] = torch.tensor(row, device=device, dtype=torch.int32)
+        return self._hm_cache[key]
+
+    def _tile_budgets(self, L, width, device):
+        key = (L, width, self.rolling_prefill, float(self.k), str(device))
+        if key not in self._budget_cache:
+            valid, nsel = budgets.prefill_tile_budgets(L, self.tile_size, self.k, self.rolling_prefill, width)
+            self._budget_cache[key] = (torch.tensor(valid, device=device, dtype=torch.int32),
+                                       torch.tensor(nsel, device=device, dtype=torch.int32))
+        return self._budget_cache[key]
+
+    # ------------------------------------------------------------------ prefill
+    def _prefill_recomp_forward(self, Q, K, V, topk, tile_size, layer, topk_percent):
+        """Anchor prefill (EfficientKascadeStrategy.py:72-93): log-sum pass (+ dense output on
+        layer 0), pooled tile scores, per-tile selection, and on layers > 0 the sparse pass with
+        the fresh indices and the identity head map."""
+        B, L = Q.shape[:2]
+        T = math.ceil(L / tile_size)
+        if layer == 0:
+            log_sum, o = kernels.prefill_recompute0(Q, K, V)
+        else:
+            log_sum = kernels.prefill_recompute1(Q, K)
+        scores = torch.empty((B, G, T, L), device=Q.device, dtype=torch.float16)
+        kernels.prefill_aggregate(Q, K, log_sum, scores)
+        valid, nsel = self._tile_budgets(L, topk, Q.device)
+        self._topk_to_reuse = kernels.topk_indices(scores, topk, valid_len=valid, n_sel=nsel)
+        if layer != 0:
+            o = kernels.prefill_reuse(Q, K, V, self._topk_to_reuse, self._hm(None, Q.device), topk_percent,
+                                      self.rolling_prefill)
+        return o
+
+    def _prefill_reuse_forward(self, Q, K, V, topk_percent, layer):
+        """Reuse prefill (EfficientKascadeStrategy.py:95-98)."""
+        return kernels.prefill_reuse(Q, K, V, self._topk_to_reuse, self._hm(layer, Q.device), topk_percent,
+                                     self.rolling_prefill)
+
+    # ------------------------------------------------------------------- decode
+    def _decode_scratch(self, B, ns, device):
+        return (torch.empty(B, H, ns, device=device, dtype=torch.float32),
+                torch.empty(B, H, ns, D, device=device, dtype=torch.float32))
+
+    def _decode_recomp_forward(self, Q, K, V, topk, layer):
+        """Anchor decode (EfficientKascadeStrategy.py:100-115) over a contiguous [B,L,G,D] cache."""
+        B, L = K.shape[:2]
+        ns = kernels.default_num_split(B * G * L, L)
+        glse, part = self._decode_scratch(B, ns, Q.device)
+        row_sums = torch.empty(B, H, device=Q.device, dtype=torch.float32)
+        stride = ((L + 7) // 8) * 8
+        scores = torch.empty(B, H, stride, device=Q.device, dtype=torch.float32)
+        o, agg = kernels.decode_recompute(Q, K, V, glse, part, row_sums, scores, layer)
+        self._topk_to_reuse = kernels.topk_indices(agg[:, :, :L], topk, fill_value=0)
+        if layer != 0:
+            ns = kernels.default_num_split(B * G * topk, topk)
+            glse, part = self._decode_scratch(B, ns, Q.device)
+            o = kernels.decode_reuse(Q, K, V, self._topk_to_reuse, self._hm(None, Q.device), glse, part)
+        return o
+
+    def _decode_reuse_forward(self, Q, K, V, layer):
+        """Reuse decode (EfficientKascadeStrategy.py:117-123)."""
+        B = Q.shape[0]
+        topk = self._topk_to_reuse.shape[-1]
+        ns = kernels.default_num_split(B * G * topk, topk)
+        glse, part = self._decode_scratch(B, ns, Q.device)
+        return kernels.decode_reuse(Q, K, V, self._topk_to_reuse, self._hm(layer, Q.device), glse, part)
+
+    # --------------------------------------------------------------- HF boundary
+    def attention_forward(self, module, query, key, value, attention_mask, scaling, dropout=0.0, **kwargs):
+        """EfficientKascadeStrategy.py:126-161.  query [B,H,Lq,D], key/value [B,G,Lk,D]."""
+        if key.shape[-2] <= 128:
+            from transformers.modeling_utils import ALL_ATTENTION_FUNCTIONS
+            return ALL_ATTENTION_FUNCTIONS["sdpa"](module, query, key, value, attention_mask,
+                                                   scaling=scaling, dropout=dropout, **kwargs)
+        if query.shape[1] != H or key.shape[1] != G or query.shape[-1] != D or query.dtype != torch.float16:
+            raise KascadeError("efficient_kascade supports fp16 with 32 query heads, 8 KV heads, head_dim 128")
+        is_decode = (query.shape[2] == 1)
+        Lk = key.shape[-2]
+        rounded_k = budgets.topk_width(Lk, self.k)
+        query = query.transpose(1, 2)   # B, L, H, D (strided view)
+        key = key.transpose(1, 2)
+        value = value.transpose(1, 2)
+        layer = module.layer_idx
+        if is_decode:
+            query = query.squeeze(1).contiguous()
+            key = key.contiguous()
+            value = value.contiguous()
+            if layer in self.recompute_layers:
+                o = self._decode_recomp_forward(query, key, value, rounded_k, layer)
+            else:
+                o = self._decode_reuse_forward(query, key, value, layer)
+            o = o.unsqueeze(1)
+        else:
+            if query.shape[1] != Lk:
+                raise KascadeError("prefill needs Lq == Lk (no cached prefix), as in the reference kernels")
+            if layer in self.recompute_layers:
+                o = self._prefill_recomp_forward(query, key, value, rounded_k, self.tile_size, layer, self.k)
+            else:
+                o = self._prefill_reuse_forward(query, key, value, self.k, layer)
+        return o, None
+
+    def register_attention(self):
+        """EfficientKascadeStrategy.py:163-168."""
+        from transformers.modeling_utils import ALL_ATTENTION_FUNCTIONS
+        from transformers.masking_utils import ALL_MASK_ATTENTION_FUNCTIONS
+
+        def _attention_forward(module, query, key, value, attention_mask, scaling, dropout=0.0, **kwargs):
+            return self.attention_forward(module, query, key, value, attention_mask, scaling,
+                                          dropout=dropout, **kwargs)
+        ALL_MASK_ATTENTION_FUNCTIONS.register(self.name, ALL_MASK_ATTENTION_FUNCTIONS["sdpa"])
+        ALL_ATTENTION_FUNCTIONS.register(self.name, _attention_forward)
+
+
+class PagedKascadeDecoder:
+    """Paged decode backend: anchor and reuse decode over K/V pages [P,page,G,D] with a block
+    table [B,max_pages] and per-sequence lengths.  Scratch is allocated once for a maximum
+    batch / context and reused by every call (the C ABI never allocates).
+
+    Call order per decode step follows the reference's kvcache ``full_kernel``
+    (recompute_kascade_gqa_decode_with_kvcache.py:368-377): anchor -> selection over
+    agg[:, :, :max_len] with row width max_topk -> (layers > 0) reuse with the identity map;
+    reuse layers read rows head_mapping[layer] of the last anchor's indices."""
+
+    def __init__(self, k: float, head_mapping: List[List[int]], recompute_layers: Sequence[int],
+                 max_batch: int, max_seqlen: int, page_size: int = 16, device="cuda",
+                 num_split_dense: Optional[int] = None, num_split_reuse: Optional[int] = None):
+        self.k = k
+        self.page_size = page_size
+        self.recompute_layers = list(recompute_layers)
+        self._head_mapping = head_mapping
+        self.device = torch.device(device)
+        self.max_batch, self.max_seqlen = max_batch, max_seqlen
+        self.stride = ((max_seqlen + 7) // 8) * 8
+        self.max_topk = budgets.decode_budget(max_seqlen, k)
+        self.ns_dense = num_split_dense or kernels.default_num_split(max_batch * G * max_seqlen, max_seqlen)
+        self.ns_reuse = num_split_reuse or kernels.default_num_split(max_batch * G * self.max_topk, self.max_topk)
+        ns = max(self.ns_dense, self.ns_reuse)
+        dev = self.device
+        self._glse = torch.empty(max_batch * H * ns, device=dev, dtype=torch.float32)
+        self._part = torch.empty(max_batch * H * ns * D, device=dev, dtype=torch.float32)
+        self._row_sums = torch.empty(max_batch, H, device=dev, dtype=torch.float32)
+        self._scores = torch.empty(max_batch * H * self.stride, device=dev, dtype=torch.float32)
+        self._hm = {None: torch.arange(G, device=dev, dtype=torch.int32)}
+        for l, row in enumerate(head_mapping):
+            self._hm[l] = torch.tensor(row, device=dev, dtype=torch.int32)
+        self._topk_to_reuse = None
+        self._counts = None
+
+    def _scratch(self, B, ns):
+        return self._glse[:B * H * ns].view(B, H, ns), self._part[:B * H * ns * D].view(B, H, ns, D)
+
+    def dense(self, q, k_pages, v_pages, block_table, seqlens, max_len: int):
+        B = q.shape[0]
+        glse, part = self._scratch(B, self.ns_dense)
+        return kernels.decode_dense_paged(q, k_pages, v_pages, seqlens, glse, part, block_table,
+                                          self.page_size, kv_len=max_len)
+
+    def anchor(self, layer, q, k_pages, v_pages, block_table, seqlens, max_len: int,
+               ragged: bool = True):
+        """Anchor layer: returns the attention output [B,H,D]; keeps indices for reuse layers."""
+        B = q.shape[0]
+        stride = ((max_len + 7) // 8) * 8
+        glse, part = self._scratch(B, self.ns_dense)
+        scores = self._scores[:B * H * stride].view(B, H, stride)
+        o, agg = kernels.decode_recompute(q, k_pages, v_pages, glse, part, self._row_sums[:B], scores, layer,
+                                          cache_seqlens=seqlens, block_table=block_table,
+                                          page_size=self.page_size, kv_len=max_len)
+        if ragged:
+            width = budgets.decode_budget(max_len, self.k)
+            lens_rows = seqlens.repeat_interleave(G)
+            counts = self._decode_counts(seqlens).repeat_interleave(G)
+            self._topk_to_reuse = kernels.topk_indices(agg[:, :, :max_len], width, valid_len=lens_rows,
+                                                       n_sel=counts, fill_value=0)
+            self._pct = float(self.k)
+        else:
+            width = budgets.topk_width(max_len, self.k)
+            self._topk_to_reuse = kernels.topk_indices(agg[:, :, :max_len], width, fill_value=0)
+            self._pct = 0.0
+        if layer != 0:
+            o = self._reuse(q, k_pages, v_pages, block_table, seqlens, self._hm[None])
+        return o
+
+    def _decode_counts(self, seqlens: torch.Tensor) -> torch.Tensor:
+        # 128*ceil(floor(k*len/100)/128) on the device, exact integer arithmetic for integer k
+        if float(self.k).is_integer():
+            fl = (seqlens.to(torch.int64) * int(self.k)) // 100
+        else:
+            fl = torch.floor(seqlens.to(torch.float64) * float(self.k) / 100.0).to(torch.int64)
+        return (((fl + 127) // 128) * 128).to(torch.int32)
+
+    def _reuse(self, q, k_pages, v_pages, block_table, seqlens, hm):
+        B = q.shape[0]
+        glse, part = self._scratch(B, self.ns_reuse)
+        return kernels.decode_reuse_paged(q, k_pages, v_pages, seqlens, self._topk_to_reuse, hm, self._pct,
+                                          glse, part, block_table=block_table, page_size=self.page_size)
+
+    def reuse(self, layer, q, k_pages, v_pages, block_table, seqlens):
+        """Reuse layer: attends to rows head_mapping[layer] of the last anchor's indices."""
+        if self._topk_to_reuse is None:
+            raise KascadeError("reuse layer called before any anchor layer")
+        return self._reuse(q, k_pages, v_pages, block_table, seqlens, self._hm[layer])
+
+    def forward(self, layer, q, k_pages, v_pages, block_table, seqlens, max_len: int, ragged: bool = True):
+        if layer in self.recompute_layers:
+            return self.anchor(layer, q, k_pages, v_pages, block_table, seqlens, max_len, ragged)
+        return self.reuse(layer, q, k_pages, v_pages, block_table, seqlens)

@@ -103,33 +103,35 @@ def _expand_kv(x: torch.Tensor, rep: int) -> torch.Tensor:
     return x.permute(0, 2, 1, 3).repeat_interleave(rep, dim=1)
 
 
-def dense_prefill(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, block: int = 1024
-                  ) -> Tuple[torch.Tensor, torch.Tensor]:
+def dense_prefill(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, block: int = 1024,
+                  rows: Optional[Tuple[int, int]] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """Dense causal GQA attention and the log2-domain log-sum the anchor kernels
     emit (recompute_kascade_gqa_prefill.py:225-274: O = softmax(QK^T/sqrt(D)) V,
     log_sum = log2(sum) + max*scale with scale = D^-0.5*log2(e)).
 
     q [B,L,H,D]; k,v [B,L,G,D]  ->  O [B,L,H,D] fp32, log_sum [B,L,H] fp32.
-    Row-blocked so long sequences fit in host memory."""
+    Row-blocked so long sequences fit in host memory.  ``rows=(s, e)`` computes only
+    query rows s..e-1 (outputs then have e-s rows)."""
     B, L, H, D = q.shape
+    r0, r1 = (0, L) if rows is None else rows
     G = k.shape[2]
     rep = H // G
     c = D ** -0.5
     kf = _expand_kv(k.float(), rep)            # [B,H,L,D]
     vf = _expand_kv(v.float(), rep)
     qf = q.float().permute(0, 2, 1, 3)          # [B,H,L,D]
-    out = torch.empty(B, H, L, D, dtype=torch.float32)
-    lse2 = torch.empty(B, H, L, dtype=torch.float32)
-    for s in range(0, L, block):
-        e = min(s + block, L)
+    out = torch.empty(B, H, r1 - r0, D, dtype=torch.float32)
+    lse2 = torch.empty(B, H, r1 - r0, dtype=torch.float32)
+    for s in range(r0, r1, block):
+        e = min(s + block, r1)
         sc = torch.matmul(qf[:, :, s:e], kf[:, :, :e].transpose(2, 3)) * c   # [B,H,blk,e]
         i = torch.arange(s, e).view(-1, 1)
         j = torch.arange(e).view(1, -1)
         sc.masked_fill_(j > i, float("-inf"))
         lse = torch.logsumexp(sc, dim=-1)
         p = torch.exp(sc - lse.unsqueeze(-1))
-        out[:, :, s:e] = torch.matmul(p, vf[:, :, :e])
-        lse2[:, :, s:e] = lse * LOG2E
+        out[:, :, s - r0:e - r0] = torch.matmul(p, vf[:, :, :e])
+        lse2[:, :, s - r0:e - r0] = lse * LOG2E
     return out.permute(0, 2, 1, 3).contiguous(), lse2.permute(0, 2, 1).contiguous()
 
 
@@ -156,24 +158,27 @@ def dense_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
 # anchor layers (kernel semantics)
 # --------------------------------------------------------------------------
 def pooled_prefill_scores(q: torch.Tensor, k: torch.Tensor, tile: int, block_tiles: int = 32,
-                          out_dtype: torch.dtype = torch.float16) -> torch.Tensor:
+                          out_dtype: torch.dtype = torch.float16,
+                          tiles: Optional[Tuple[int, int]] = None) -> torch.Tensor:
     """Post-softmax scores pooled over the q-heads of each KV head and the
     ``tile`` queries of each tile; keys at or after the tile start are -inf.
     Follows ref_program_correct_recompute (recompute_kascade_gqa_prefill.py:
     363-394): fp32 softmax, fp32 sums, one final cast to fp16, and the aggregate
     kernel's validity rule ``j < tile_start`` (same file :182-189).
 
-    q [B,L,H,D], k [B,L,G,D] -> [B,G,ceil(L/tile),L] (out_dtype)."""
+    q [B,L,H,D], k [B,L,G,D] -> [B,G,ceil(L/tile),L] (out_dtype).  ``tiles=(a, b)``
+    computes only tile rows a..b-1 (output then has b-a tile rows)."""
     B, L, H, D = q.shape
     G = k.shape[2]
     rep = H // G
     T = math.ceil(L / tile)
+    ta, tb = (0, T) if tiles is None else tiles
     c = D ** -0.5
     kf = _expand_kv(k.float(), rep)
     qf = q.float().permute(0, 2, 1, 3)
-    pooled = torch.full((B, G, T, L), float("-inf"), dtype=torch.float32)
-    for t0 in range(0, T, block_tiles):
-        t1 = min(t0 + block_tiles, T)
+    pooled = torch.full((B, G, tb - ta, L), float("-inf"), dtype=torch.float32)
+    for t0 in range(ta, tb, block_tiles):
+        t1 = min(t0 + block_tiles, tb)
         s, e = t0 * tile, min(t1 * tile, L)
         sc = torch.matmul(qf[:, :, s:e], kf[:, :, :e].transpose(2, 3)) * c
         i = torch.arange(s, e).view(-1, 1)
@@ -185,7 +190,7 @@ def pooled_prefill_scores(q: torch.Tensor, k: torch.Tensor, tile: int, block_til
             rs, re = t * tile - s, min((t + 1) * tile, L) - s
             ts = t * tile
             if ts > 0:
-                pooled[:, :, t, :ts] = p[:, :, rs:re, :ts].sum(dim=2)
+                pooled[:, :, t - ta, :ts] = p[:, :, rs:re, :ts].sum(dim=2)
     return pooled.to(out_dtype)
 
 
@@ -198,7 +203,7 @@ def topk_rows(scores: torch.Tensor, k: int) -> torch.Tensor:
 
 def reuse_prefill(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, idx: torch.Tensor,
                   head_mapping: Sequence[int], tile: int, rolling: bool, p: float,
-                  block_tiles: int = 32) -> torch.Tensor:
+                  block_tiles: int = 32, tiles: Optional[Tuple[int, int]] = None) -> torch.Tensor:
     """Sparse causal attention of a reuse layer, kernel semantics
     (reuse_kascade_gqa_prefill.py:58-77, 147-198 and the PyTorch twin
     recompute_kascade_gqa_prefill.py:403-457).
@@ -207,20 +212,23 @@ def reuse_prefill(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, idx: torch.
       all keys j <= i                         if tile*t <= n(t)   (dense regime)
       idx[b, head_mapping[g], t, :n(t)]  U  {tile*t <= j <= i}     otherwise,
     n(t) = n_kern(tile*t) when rolling and L > 128, else idx.shape[-1].
-    q [B,L,H,D]; k,v [B,L,G,D]; idx [B,G,T,K] int32 -> O [B,L,H,D] fp32."""
+    q [B,L,H,D]; k,v [B,L,G,D]; idx [B,G,T,K] int32 -> O [B,L,H,D] fp32.
+    ``tiles=(a, b)`` computes only the queries of tiles a..b-1."""
     B, L, H, D = q.shape
     G = k.shape[2]
     rep = H // G
     T = math.ceil(L / tile)
+    ta, tb = (0, T) if tiles is None else tiles
+    row0 = ta * tile
     K = idx.shape[-1]
     c = D ** -0.5
     kf = _expand_kv(k.float(), rep)
     vf = _expand_kv(v.float(), rep)
     qf = q.float().permute(0, 2, 1, 3)
     hm = torch.as_tensor(list(head_mapping), dtype=torch.long)
-    out = torch.empty(B, H, L, D, dtype=torch.float32)
-    for t0 in range(0, T, block_tiles):
-        t1 = min(t0 + block_tiles, T)
+    out = torch.empty(B, H, min(tb * tile, L) - row0, D, dtype=torch.float32)
+    for t0 in range(ta, tb, block_tiles):
+        t1 = min(t0 + block_tiles, tb)
         s, e = t0 * tile, min(t1 * tile, L)
         sc = torch.matmul(qf[:, :, s:e], kf[:, :, :e].transpose(2, 3)) * c     # [B,H,rows,e]
         allow = torch.zeros(B, G, e - s, e, dtype=torch.bool)
@@ -243,7 +251,7 @@ def reuse_prefill(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, idx: torch.
         allow_h = allow.repeat_interleave(rep, dim=1)
         sc.masked_fill_(~allow_h, float("-inf"))
         pr = torch.softmax(sc, dim=-1)
-        out[:, :, s:e] = torch.matmul(pr, vf[:, :, :e])
+        out[:, :, s - row0:e - row0] = torch.matmul(pr, vf[:, :, :e])
     return out.permute(0, 2, 1, 3).contiguous()
 
 
