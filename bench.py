@@ -187,7 +187,8 @@ def main():
             caches = [workloads.paged_decode_inputs(seqlens, seed=10 + i, device=dev, reuse_keys=False)
                       for i in range(n_caches)]
             c0 = caches[0]
-            dec = PagedKascadeDecoder(PCT, head_map, ANCHORS, B, max_len, page_size=16, device=dev)
+            dec = PagedKascadeDecoder(PCT, head_map, ANCHORS, B, max_len, page_size=16, device=dev,
+                                      total_tokens=sum(seqlens))
             calls = [0]
 
             def cache():

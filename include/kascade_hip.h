@@ -125,8 +125,12 @@ int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_hal
  * lower index), ordered by ascending index; when fewer than n entries are valid
  * all valid ones are emitted followed by the first invalid positions, as
  * torch.topk does for -inf padding.  Slots [n, k) are set to fill_value.
- *   workspace: device scratch of at least kascade_topk_workspace_bytes(rows) bytes. */
-int64_t kascade_topk_workspace_bytes(int rows);
+ * uniform_len is also the upper bound of every valid_len entry (longer entries are clamped).
+ *   workspace: NULL, or device scratch of kascade_topk_workspace_bytes(rows, uniform_len)
+ *   bytes.  With a workspace, long rows (that function returns > 0) are selected by several
+ *   workgroups per row -- coarse histograms merged with atomics, per-chunk counts, ordered
+ *   compaction -- with identical results; without one, one workgroup handles each row. */
+int64_t kascade_topk_workspace_bytes(int rows, int64_t row_len);
 int kascade_topk_call(const kascade_half* scores, int32_t* out_idx, int rows, int64_t row_stride,
                       int uniform_len, const int32_t* valid_len, const int32_t* n_sel, int period,
                       int k, int fill_value, void* workspace, void* stream);

@@ -15,6 +15,10 @@
 
 using namespace kascade;
 
+#ifndef KASCADE_DENSE_NQB
+#define KASCADE_DENSE_NQB 1   // 32-query blocks per wavefront in the dense prefill kernels
+#endif
+
 namespace {
 
 thread_local char g_err[1024] = "";
@@ -198,24 +202,26 @@ int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_hal
                      "decode_recompute aggregate");
 }
 
-int64_t kascade_topk_workspace_bytes(int rows) {
-    (void)rows;
-    return 0;  // the single-workgroup-per-row selection keeps all state in LDS
+int64_t kascade_topk_workspace_bytes(int rows, int64_t row_len) {
+    return topk_split_workspace_bytes(rows, row_len);
 }
 
 int kascade_topk_call(const kascade_half* scores, int32_t* out_idx, int rows, int64_t row_stride,
                       int uniform_len, const int32_t* valid_len, const int32_t* n_sel, int period,
                       int k, int fill_value, void* workspace, void* stream) {
-    (void)workspace;
     REQUIRE(scores && out_idx, "topk: null pointer argument");
     REQUIRE(rows >= 0 && k > 0 && row_stride > 0, "topk: rows >= 0, k > 0, row_stride > 0 required");
-    REQUIRE(valid_len || (uniform_len >= 0 && uniform_len <= row_stride),
+    REQUIRE(uniform_len >= 0 && uniform_len <= row_stride,
             "topk: uniform_len must be within [0, row_stride]");
     REQUIRE(!(valid_len || n_sel) || period > 0, "topk: period must be > 0 with per-row arrays");
     if (period <= 0) period = 1;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (workspace && topk_split_workspace_bytes(rows, uniform_len) > 0)
+        return check_hip(launch_topk_split(H(scores), out_idx, rows, row_stride, uniform_len,
+                                           uniform_len, valid_len, n_sel, period, k, fill_value,
+                                           workspace, s), "topk (split)");
     return check_hip(launch_topk(H(scores), out_idx, rows, row_stride, uniform_len, valid_len, n_sel,
-                                 period, k, fill_value, static_cast<hipStream_t>(stream)),
-                     "topk");
+                                 period, k, fill_value, s), "topk");
 }
 
 int kascade_prefill_dense_call(const kascade_half* Q, const kascade_half* K, const kascade_half* V,
@@ -234,7 +240,7 @@ int kascade_prefill_dense_call(const kascade_half* Q, const kascade_half* K, con
     p.q_sb = q_strides.b; p.q_sl = q_strides.l; p.q_sh = q_strides.h;
     p.k_sb = kv_strides.b; p.k_sl = kv_strides.l; p.k_sh = kv_strides.h;
     p.B = batch; p.L = seq_len; p.T = (seq_len + kTile - 1) / kTile;
-    return check_hip(launch_prefill_attn(p, false, with_output != 0, 2,
+    return check_hip(launch_prefill_attn(p, false, with_output != 0, with_output ? KASCADE_DENSE_NQB : 2,
                                          static_cast<hipStream_t>(stream)), "prefill_dense");
 }
 

@@ -13,9 +13,10 @@
 //   at a bit-swapped slot (bits 2 and 3 exchanged) which makes the accumulator
 //   registers of one lane cover 8 consecutive key positions, i.e. one 16-byte
 //   read of the transposed V tile per MFMA operand.  V is transposed on its way
-//   into LDS (4 keys x 8 d per thread, eight 8-byte writes) with a 16-byte-chunk
-//   XOR swizzle that keeps both the transposing writes and the operand reads
-//   spread over the banks.
+//   into LDS (4 keys x 8 d per thread, eight 8-byte writes) with the 16-byte chunks
+//   of each row XOR-swizzled by (d & 7) ^ (d >> 3); of the layouts measured with the
+//   LDS bank-conflict counter this one conflicts least (K rows padded to 272 bytes
+//   show no conflicts at all).
 //
 // prefill_aggregate_kernel -- pooled tile scores: S = Q_tile K^T with the 128
 //   (query, head) rows of a tile held as A operands in registers by every
@@ -30,6 +31,7 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kKT = 64;            // keys per tile (attention kernel)
 constexpr int kKStride = 136;      // halves per K row in LDS (128 + 8 pad)
+constexpr int kVStride = 64;       // halves per V^T row in LDS (one 64-key tile)
 constexpr int kAggKT = 128;        // keys per tile (aggregate kernel)
 
 __device__ __forceinline__ int swap_bits23(int x) {
@@ -43,9 +45,7 @@ __device__ __forceinline__ int rolling_budget(float pct, int tile_start) {
 }
 
 template <int NQB, bool REUSE, bool WITH_V>
-__global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillParams p) {
-    __shared__ __attribute__((aligned(16))) half_t sK[kKT * kKStride];
-    __shared__ __attribute__((aligned(16))) half_t sV[kDim * kKT];
+__device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t* sK, half_t* sV) {
 
     constexpr int QT = 32 * NQB;
     const int L = p.L;
@@ -157,9 +157,9 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillParams p)
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
                 const int d = kcol * 8 + r;
-                const int sw = (r ^ kcol) & 7;
+                const int sw = (r ^ kcol) & 7;    // = ((d & 7) ^ (d >> 3)) & 7
                 half4_t w = {v0.h[r], v1.h[r], v2.h[r], v3.h[r]};
-                *reinterpret_cast<half4_t*>(&sV[d * kKT + (((kq >> 1) ^ sw) * 8) + (kq & 1) * 4]) = w;
+                *reinterpret_cast<half4_t*>(&sV[d * kVStride + (((kq >> 1) ^ sw) * 8) + (kq & 1) * 4]) = w;
             }
         }
         __syncthreads();
@@ -249,10 +249,12 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillParams p)
                 }
             l[qb] = l[qb] * corr + sum;   // per-lane partial sum (own key positions)
             if (WITH_V) {
+                if (__any(corr != 1.f)) {   // wavefront-uniform: skip when no maximum moved
 #pragma unroll
-                for (int db = 0; db < 4; ++db)
+                    for (int db = 0; db < 4; ++db)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) oT[qb][db][v] *= corr;
+                        for (int v = 0; v < 16; ++v) oT[qb][db][v] *= corr;
+                }
 #pragma unroll
                 for (int s = 0; s < 4; ++s) {
                     half8_t t;
@@ -272,7 +274,7 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillParams p)
                 for (int s = 0; s < 4; ++s) {
                     if (s < 2 * nkb) {
                         half8_t a = *reinterpret_cast<const half8_t*>(
-                            &sV[d * kKT + (((2 * s + lg) ^ sw) * 8)]);
+                            &sV[d * kVStride + (((2 * s + lg) ^ sw) * 8)]);
 #pragma unroll
                         for (int qb = 0; qb < NQB; ++qb)
                             oT[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pf[qb][s], oT[qb][db], 0, 0, 0);
@@ -304,6 +306,28 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillParams p)
             }
         }
     }
+}
+
+#ifndef KASCADE_PREFILL_WAVES_NQB1
+#define KASCADE_PREFILL_WAVES_NQB1 2
+#endif
+
+// 32 queries per wavefront: register budget capped so that two workgroups share a
+// compute unit and hide each other's LDS staging and gather latency.
+template <bool REUSE, bool WITH_V>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(KASCADE_PREFILL_WAVES_NQB1)))
+void prefill_attn_kernel_q32(PrefillParams p) {
+    __shared__ __attribute__((aligned(16))) half_t sK[kKT * kKStride];
+    __shared__ __attribute__((aligned(16))) half_t sV[kDim * kVStride];
+    prefill_attn_body<1, REUSE, WITH_V>(p, sK, sV);
+}
+
+// 64 queries per wavefront: one wavefront per SIMD with the whole register file.
+template <bool WITH_V>
+__global__ __launch_bounds__(kThreads) void prefill_attn_kernel_q64(PrefillParams p) {
+    __shared__ __attribute__((aligned(16))) half_t sK[kKT * kKStride];
+    __shared__ __attribute__((aligned(16))) half_t sV[kDim * kVStride];
+    prefill_attn_body<2, false, WITH_V>(p, sK, sV);
 }
 
 __global__ __launch_bounds__(kThreads) void prefill_aggregate_kernel(PrefillParams p) {
@@ -411,17 +435,17 @@ hipError_t launch_prefill_attn(const PrefillParams& p, bool reuse, bool with_v, 
     const int qt = 32 * nqb;
     dim3 grid((p.L + qt - 1) / qt, kGroups, p.B), block(kThreads);
     if (reuse) {
-        hipLaunchKernelGGL((prefill_attn_kernel<1, true, true>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((prefill_attn_kernel_q32<true, true>), grid, block, 0, stream, p);
     } else if (nqb == 2) {
         if (with_v)
-            hipLaunchKernelGGL((prefill_attn_kernel<2, false, true>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((prefill_attn_kernel_q64<true>), grid, block, 0, stream, p);
         else
-            hipLaunchKernelGGL((prefill_attn_kernel<2, false, false>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((prefill_attn_kernel_q64<false>), grid, block, 0, stream, p);
     } else {
         if (with_v)
-            hipLaunchKernelGGL((prefill_attn_kernel<1, false, true>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((prefill_attn_kernel_q32<false, true>), grid, block, 0, stream, p);
         else
-            hipLaunchKernelGGL((prefill_attn_kernel<1, false, false>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((prefill_attn_kernel_q32<false, false>), grid, block, 0, stream, p);
     }
     return hipGetLastError();
 }

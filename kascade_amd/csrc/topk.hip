@@ -16,6 +16,10 @@ constexpr int kThreads = 1024;
 constexpr int kWaves = kThreads / 64;
 constexpr int kChunk = kThreads * 8;
 constexpr int kBins1 = 2048;
+}  // namespace
+constexpr int kSplitMinLen = 32768;   // rows at least this long take the multi-workgroup path
+constexpr int kSplitMaxRows = 4096;   // workspace is 8 KB per row for the coarse histogram
+namespace {
 
 __device__ __forceinline__ uint32_t order_key(uint16_t bits) {
     // monotone map fp16 -> u16: negatives below positives, -inf lowest finite order
@@ -77,7 +81,7 @@ __global__ __launch_bounds__(kThreads) void topk_select_kernel(
     const int tid = threadIdx.x;
     const long long row = blockIdx.x;
     const int pr = (int)(row % period);
-    const int len = valid_len ? valid_len[pr] : uniform_len;
+    const int len = valid_len ? min(valid_len[pr], uniform_len) : uniform_len;
     int n = n_sel ? n_sel[pr] : k;
     n = max(0, min(n, k));
     const uint16_t* src = scores + row * row_stride;
@@ -181,7 +185,274 @@ __global__ __launch_bounds__(kThreads) void topk_select_kernel(
     for (int i = n + tid; i < k; i += kThreads) dst[i] = fill;
 }
 
+
+// --------------------------------------------------------------------------
+// Long rows: the same radix select spread over several workgroups per row.
+// Every workgroup owns one chunk of kSplitChunk entries of one row; per-row state
+// lives in a caller-provided workspace:
+//   hist1 [rows][2048]            coarse histogram (atomically merged)
+//   sel   [rows][8]               {mode, b1, cum_above, T, r, n, len}
+//   cinfo [rows][chunks][34]      per chunk: fine histogram of bin b1 (32) and the
+//                                 number of entries in bins above b1
+//   coff  [rows][chunks][2]       per chunk: selected-greater / equal counts before it
+// Launch sequence: zero -> hist1 -> scan1 -> hist2 -> scan2 -> write.
+// --------------------------------------------------------------------------
+constexpr int kSplitChunk = 16384;
+constexpr int kSelWords = 8;
+constexpr int kInfoWords = 34;
+
+struct SplitWs {
+    uint32_t* hist1;
+    uint32_t* sel;
+    uint32_t* cinfo;
+    uint32_t* coff;
+};
+
+__device__ __forceinline__ void row_params(const int* valid_len, const int* n_sel, int period,
+                                           int uniform_len, int k, long long row, int& len, int& n) {
+    const int pr = (int)(row % period);
+    len = valid_len ? min(valid_len[pr], uniform_len) : uniform_len;
+    n = n_sel ? n_sel[pr] : k;
+    n = max(0, min(n, k));
+}
+
+__global__ __launch_bounds__(256) void topk_zero_kernel(uint32_t* p, long long n) {
+    long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+__global__ __launch_bounds__(kThreads) void topk_split_hist1_kernel(
+    const uint16_t* __restrict__ scores, long long row_stride, int uniform_len,
+    const int* __restrict__ valid_len, const int* __restrict__ n_sel, int period, int k, SplitWs ws) {
+    __shared__ uint32_t s_hist[kBins1];
+    const int tid = threadIdx.x;
+    const long long row = blockIdx.y;
+    int len, n;
+    row_params(valid_len, n_sel, period, uniform_len, k, row, len, n);
+    const int c0 = blockIdx.x * kSplitChunk;
+    if (len <= n || n == 0 || c0 >= len) return;
+    const int c1 = min(len, c0 + kSplitChunk);
+    const uint16_t* src = scores + row * row_stride;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(src) & 15) == 0);
+    for (int i = tid; i < kBins1; i += kThreads) s_hist[i] = 0;
+    __syncthreads();
+    for (int base = c0 + tid * 8; base < c1; base += kChunk) {
+        uint32_t keys[8];
+        int nv = load_keys(src, aligned, base, c1, keys);
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            if (e < nv) atomicAdd(&s_hist[keys[e] >> 5], 1u);
+    }
+    __syncthreads();
+    uint32_t* gh = ws.hist1 + row * kBins1;
+    for (int i = tid; i < kBins1; i += kThreads) {
+        uint32_t c = s_hist[i];
+        if (c) atomicAdd(&gh[i], c);
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void topk_split_scan1_kernel(
+    int uniform_len, const int* __restrict__ valid_len, const int* __restrict__ n_sel, int period,
+    int k, SplitWs ws) {
+    __shared__ uint32_t s_wave[kWaves];
+    const int tid = threadIdx.x;
+    const long long row = blockIdx.x;
+    int len, n;
+    row_params(valid_len, n_sel, period, uniform_len, k, row, len, n);
+    uint32_t* sel = ws.sel + row * kSelWords;
+    if (len <= n || n == 0) {
+        if (tid == 0) { sel[0] = 0; sel[5] = (uint32_t)n; sel[6] = (uint32_t)len; }
+        return;
+    }
+    const uint32_t* gh = ws.hist1 + row * kBins1;
+    const int rb0 = kBins1 - 1 - 2 * tid;
+    const uint32_t c0 = gh[rb0], c1 = gh[rb0 - 1];
+    uint32_t total;
+    const uint32_t above0 = block_excl_scan(c0 + c1, s_wave, &total);
+    const uint32_t above1 = above0 + c0;
+    const uint32_t un = (uint32_t)n;
+    if (above0 < un && un <= above0 + c0) {
+        sel[1] = rb0; sel[2] = above0;
+    } else if (above1 < un && un <= above1 + c1) {
+        sel[1] = rb0 - 1; sel[2] = above1;
+    }
+    if (tid == 0) { sel[0] = 1; sel[5] = (uint32_t)n; sel[6] = (uint32_t)len; }
+}
+
+__global__ __launch_bounds__(kThreads) void topk_split_hist2_kernel(
+    const uint16_t* __restrict__ scores, long long row_stride, int max_chunks, SplitWs ws) {
+    __shared__ uint32_t s_hist2[32];
+    __shared__ uint32_t s_gt1;
+    const int tid = threadIdx.x;
+    const long long row = blockIdx.y;
+    const uint32_t* sel = ws.sel + row * kSelWords;
+    const int len = (int)sel[6];
+    const int c0 = blockIdx.x * kSplitChunk;
+    if (sel[0] == 0 || c0 >= len) return;
+    const int c1 = min(len, c0 + kSplitChunk);
+    const uint32_t b1 = sel[1];
+    const uint16_t* src = scores + row * row_stride;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(src) & 15) == 0);
+    if (tid < 32) s_hist2[tid] = 0;
+    if (tid == 32) s_gt1 = 0;
+    __syncthreads();
+    uint32_t gt1 = 0;
+    for (int base = c0 + tid * 8; base < c1; base += kChunk) {
+        uint32_t keys[8];
+        int nv = load_keys(src, aligned, base, c1, keys);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            if (e < nv) {
+                const uint32_t hb = keys[e] >> 5;
+                if (hb == b1) atomicAdd(&s_hist2[keys[e] & 31u], 1u);
+                gt1 += (hb > b1);
+            }
+        }
+    }
+    if (gt1) atomicAdd(&s_gt1, gt1);
+    __syncthreads();
+    uint32_t* info = ws.cinfo + (row * max_chunks + blockIdx.x) * kInfoWords;
+    if (tid < 32) info[tid] = s_hist2[tid];
+    if (tid == 32) info[32] = s_gt1;
+}
+
+__global__ __launch_bounds__(64) void topk_split_scan2_kernel(int max_chunks, SplitWs ws) {
+    const long long row = blockIdx.x;
+    uint32_t* sel = ws.sel + row * kSelWords;
+    if (sel[0] == 0) return;
+    const int lane = threadIdx.x;
+    const int len = (int)sel[6];
+    const uint32_t n = sel[5];
+    const int nchunks = (len + kSplitChunk - 1) / kSplitChunk;
+    const uint32_t* info = ws.cinfo + row * max_chunks * kInfoWords;
+    // lanes 0..31: total fine histogram
+    uint32_t h = 0;
+    if (lane < 32)
+        for (int c = 0; c < nchunks; ++c) h += info[c * kInfoWords + lane];
+    // suffix scan over the 32 bins (descending), done by every lane redundantly through shuffles
+    uint32_t above = sel[2];
+    int b2 = 31;
+    for (; b2 > 0; --b2) {
+        const uint32_t c = __shfl(h, b2);
+        if (above + c >= n) break;
+        above += c;
+    }
+    const uint32_t r = n - above;
+    if (lane == 0) { sel[3] = (sel[1] << 5) | (uint32_t)b2; sel[4] = r; }
+    // per-chunk counts and their exclusive prefix (chunks are few: serial over c, parallel over bins)
+    uint32_t gt_run = 0, eq_run = 0;
+    uint32_t* off = ws.coff + row * max_chunks * 2;
+    for (int c = 0; c < nchunks; ++c) {
+        uint32_t v = (lane < 32 && lane > b2) ? info[c * kInfoWords + lane] : 0u;
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) v += __shfl_xor(v, o);
+        const uint32_t gt = info[c * kInfoWords + 32] + v;
+        const uint32_t eq = info[c * kInfoWords + b2];
+        if (lane == 0) { off[2 * c] = gt_run; off[2 * c + 1] = eq_run; }
+        gt_run += gt;
+        eq_run += eq;
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void topk_split_write_kernel(
+    const uint16_t* __restrict__ scores, int* __restrict__ out, long long row_stride, int k,
+    int fill, int max_chunks, SplitWs ws) {
+    __shared__ uint32_t s_wave[kWaves];
+    const int tid = threadIdx.x;
+    const long long row = blockIdx.y;
+    const uint32_t* sel = ws.sel + row * kSelWords;
+    const int len = (int)sel[6];
+    const int n = (int)sel[5];
+    int* dst = out + row * (long long)k;
+    const int c0 = blockIdx.x * kSplitChunk;
+    if (blockIdx.x == 0) {
+        if (sel[0] == 0) {
+            for (int i = tid; i < k; i += kThreads) dst[i] = (i < n) ? i : fill;
+            return;
+        }
+        for (int i = n + tid; i < k; i += kThreads) dst[i] = fill;
+    }
+    if (sel[0] == 0 || c0 >= len) return;
+    const int c1 = min(len, c0 + kSplitChunk);
+    const uint32_t T = sel[3];
+    const uint32_t r = sel[4];
+    const uint32_t* off = ws.coff + (row * max_chunks + blockIdx.x) * 2;
+    uint32_t gt_base = off[0], eq_base = off[1];
+    const uint16_t* src = scores + row * row_stride;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(src) & 15) == 0);
+    for (int cbase = c0; cbase < c1; cbase += kChunk) {
+        const int base = cbase + tid * 8;
+        uint32_t keys[8];
+        int nv = (base < c1) ? load_keys(src, aligned, base, c1, keys) : 0;
+        uint32_t gt = 0, eq = 0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            if (e < nv) {
+                gt += (keys[e] > T);
+                eq += (keys[e] == T);
+            }
+        }
+        uint32_t total;
+        const uint32_t ex = block_excl_scan(gt | (eq << 16), s_wave, &total);
+        uint32_t my_gt = gt_base + (ex & 0xFFFFu);
+        uint32_t my_eq = eq_base + (ex >> 16);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            if (e < nv) {
+                if (keys[e] > T) {
+                    dst[my_gt + min(my_eq, r)] = base + e;
+                    ++my_gt;
+                } else if (keys[e] == T) {
+                    if (my_eq < r) dst[my_gt + my_eq] = base + e;
+                    ++my_eq;
+                }
+            }
+        }
+        gt_base += total & 0xFFFFu;
+        eq_base += total >> 16;
+    }
+}
+
+SplitWs carve_ws(void* workspace, int rows, int max_chunks) {
+    SplitWs ws;
+    uint32_t* p = reinterpret_cast<uint32_t*>(workspace);
+    ws.hist1 = p; p += (size_t)rows * kBins1;
+    ws.sel = p;   p += (size_t)rows * kSelWords;
+    ws.cinfo = p; p += (size_t)rows * max_chunks * kInfoWords;
+    ws.coff = p;
+    return ws;
+}
+
 }  // namespace
+
+long long topk_split_workspace_bytes(int rows, long long row_len) {
+    if (row_len < kSplitMinLen || rows > kSplitMaxRows) return 0;
+    const long long chunks = (row_len + kSplitChunk - 1) / kSplitChunk;
+    return 4ll * rows * (kBins1 + kSelWords + chunks * (kInfoWords + 2));
+}
+
+hipError_t launch_topk_split(const half_t* scores, int* out_idx, int rows, long long row_stride,
+                             int max_len, int uniform_len, const int* valid_len, const int* n_sel,
+                             int period, int k, int fill, void* workspace, hipStream_t stream) {
+    if (rows == 0) return hipSuccess;
+    const int max_chunks = (max_len + kSplitChunk - 1) / kSplitChunk;
+    SplitWs ws = carve_ws(workspace, rows, max_chunks);
+    const uint16_t* src = reinterpret_cast<const uint16_t*>(scores);
+    const long long nz = (long long)rows * kBins1;
+    hipLaunchKernelGGL(topk_zero_kernel, dim3((unsigned)((nz + 255) / 256)), dim3(256), 0, stream,
+                       ws.hist1, nz);
+    dim3 grid(max_chunks, rows);
+    hipLaunchKernelGGL(topk_split_hist1_kernel, grid, dim3(kThreads), 0, stream, src, row_stride,
+                       uniform_len, valid_len, n_sel, period, k, ws);
+    hipLaunchKernelGGL(topk_split_scan1_kernel, dim3(rows), dim3(kThreads), 0, stream, uniform_len,
+                       valid_len, n_sel, period, k, ws);
+    hipLaunchKernelGGL(topk_split_hist2_kernel, grid, dim3(kThreads), 0, stream, src, row_stride,
+                       max_chunks, ws);
+    hipLaunchKernelGGL(topk_split_scan2_kernel, dim3(rows), dim3(64), 0, stream, max_chunks, ws);
+    hipLaunchKernelGGL(topk_split_write_kernel, grid, dim3(kThreads), 0, stream, src, out_idx,
+                       row_stride, k, fill, max_chunks, ws);
+    return hipGetLastError();
+}
 
 hipError_t launch_topk(const half_t* scores, int* out_idx, int rows, long long row_stride,
                        int uniform_len, const int* valid_len, const int* n_sel, int period, int k,

@@ -162,6 +162,19 @@ def decode_recompute(Q, K, V, glse, Output_partial, row_sums, scores, layer: int
 
 
 # ----------------------------------------------------------------- top-k
+_TOPK_WS = {}
+
+
+def _topk_workspace(nbytes: int, device) -> torch.Tensor:
+    """Scratch for the multi-workgroup selection, grown on demand and kept per device."""
+    key = str(device)
+    ws = _TOPK_WS.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(nbytes, device=device, dtype=torch.uint8)
+        _TOPK_WS[key] = ws
+    return ws
+
+
 def topk_indices(scores: torch.Tensor, k: int, valid_len=None, n_sel=None,
                  uniform_len: Optional[int] = None, fill_value: Optional[int] = None
                  ) -> torch.Tensor:
@@ -197,10 +210,13 @@ def topk_indices(scores: torch.Tensor, k: int, valid_len=None, n_sel=None,
             raise KascadeError("valid_len and n_sel must have the same length")
         period = n_sel.numel()
     out = torch.empty(*lead, k, device=scores.device, dtype=torch.int32)
+    ulen = Lrow if uniform_len is None else uniform_len
+    ws_bytes = lib.kascade_topk_workspace_bytes(rows, ulen)
+    ws = _topk_workspace(ws_bytes, scores.device) if ws_bytes > 0 else None
     _lib.check(lib.kascade_topk_call(
-        _ptr(scores), _ptr(out), rows, row_stride, Lrow if uniform_len is None else uniform_len,
+        _ptr(scores), _ptr(out), rows, row_stride, ulen,
         _ptr(valid_len), _ptr(n_sel), period, k, (Lrow - 1) if fill_value is None else fill_value,
-        None, _stream()))
+        _ptr(ws), _stream()))
     return out
 
 

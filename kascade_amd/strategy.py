@@ -208,7 +208,11 @@ class PagedKascadeDecoder:
 
     def __init__(self, k: float, head_mapping: List[List[int]], recompute_layers: Sequence[int],
                  max_batch: int, max_seqlen: int, page_size: int = 16, device="cuda",
-                 num_split_dense: Optional[int] = None, num_split_reuse: Optional[int] = None):
+                 num_split_dense: Optional[int] = None, num_split_reuse: Optional[int] = None,
+                 total_tokens: Optional[int] = None):
+        """total_tokens: expected sum of the sequence lengths of a batch (default
+        max_batch*max_seqlen); with ragged batches it sizes the splits so that the non-empty
+        workgroups, not the grid, cover the device about twice."""
         self.k = k
         self.page_size = page_size
         self.recompute_layers = list(recompute_layers)
@@ -217,8 +221,10 @@ class PagedKascadeDecoder:
         self.max_batch, self.max_seqlen = max_batch, max_seqlen
         self.stride = ((max_seqlen + 7) // 8) * 8
         self.max_topk = budgets.decode_budget(max_seqlen, k)
-        self.ns_dense = num_split_dense or kernels.default_num_split(max_batch * G * max_seqlen, max_seqlen)
-        self.ns_reuse = num_split_reuse or kernels.default_num_split(max_batch * G * self.max_topk, self.max_topk)
+        total = total_tokens if total_tokens is not None else max_batch * max_seqlen
+        self.ns_dense = num_split_dense or kernels.default_num_split(G * total, max_seqlen)
+        self.ns_reuse = num_split_reuse or kernels.default_num_split(
+            G * budgets.decode_budget(total, k), self.max_topk)
         ns = max(self.ns_dense, self.ns_reuse)
         dev = self.device
         self._glse = torch.empty(max_batch * H * ns, device=dev, dtype=torch.float32)

@@ -1,0 +1,84 @@
+"""GPU tests of the exact top-n selection (C ABI kascade_topk_call), single- and multi-workgroup."""
+import pytest
+import torch
+
+from oracle import kascade_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _scores(rows, L, seed, ties=True):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.rand(rows, L, generator=g) ** 4          # many small values
+    if ties:
+        x = (x * 64).round() / 64 * (torch.rand(rows, L, generator=g) < 0.7) + x * 1e-3
+    return x.half()
+
+
+def _check(scores_c, idx_c, n_of, valid_of, K, fill):
+    for r in range(scores_c.shape[0]):
+        n, valid = int(n_of(r)), int(valid_of(r))
+        row = idx_c[r]
+        if valid <= min(n, K):
+            assert torch.equal(row[:min(n, K)], torch.arange(min(n, K), dtype=torch.int32)), f"row {r}"
+        else:
+            ok, _, msg = orc.topk_agreement(scores_c[r], row, n, valid, ulps=0.0)
+            assert ok, f"row {r}: {msg}"
+            m = min(n, K)
+            if m >= 2:
+                assert bool((row[1:m] > row[:m - 1]).all()), f"row {r}: not ascending"
+        assert bool((row[min(n, K):] == fill).all()), f"row {r}: tail not filled"
+
+
+@pytest.mark.parametrize("rows,L,K", [(5, 1000, 128), (3, 8200, 1024), (4, 70001, 7040), (2, 140000, 13184)])
+def test_topk_uniform_rows(cuda, rows, L, K):
+    from kascade_amd import kernels
+    sc = _scores(rows, L, seed=L)
+    idx = kernels.topk_indices(sc.to(cuda), K, fill_value=7)
+    torch.cuda.synchronize()
+    _check(sc, idx.cpu(), lambda r: K, lambda r: L, K, 7)
+
+
+def test_topk_split_equals_single_workgroup(cuda):
+    """Long ragged rows: the multi-workgroup path and the one-workgroup kernel agree bit for bit."""
+    from kascade_amd import kernels, _lib
+    rows, L, K = 6, 100000, 9984
+    sc = _scores(rows, L, seed=3)
+    sc[1, 500:900] = float("-inf")
+    sc[2] = 0.25                                     # one value everywhere: pure tie-breaking
+    valid = torch.tensor([100000, 64000, 33000, 5000, 9984, 99999], dtype=torch.int32)
+    nsel = torch.tensor([9984, 6400, 3328, 512, 9984, 0], dtype=torch.int32)
+    d, dvalid, dnsel = sc.to(cuda), valid.to(cuda), nsel.to(cuda)
+    split = kernels.topk_indices(d, K, valid_len=dvalid, n_sel=dnsel, fill_value=-1)
+    lib = _lib.init()
+    assert lib.kascade_topk_workspace_bytes(rows, L) > 0
+    single = torch.empty(rows, K, dtype=torch.int32, device=cuda)
+    _lib.check(lib.kascade_topk_call(d.data_ptr(), single.data_ptr(), rows, L, L, dvalid.data_ptr(),
+                                     dnsel.data_ptr(), rows, K, -1, None,
+                                     torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert torch.equal(split.cpu(), single.cpu())
+    _check(sc, split.cpu(), lambda r: nsel[r], lambda r: valid[r], K, -1)
+    # all-equal row: the lowest indices win
+    assert torch.equal(split[2, :3328].cpu(), torch.arange(3328, dtype=torch.int32))
+
+
+def test_topk_strided_unaligned_rows(cuda):
+    from kascade_amd import kernels
+    rows, stride, L, K = 7, 1003, 999, 100          # odd stride: rows are not 16-byte aligned
+    base = _scores(rows, stride, seed=9).to(cuda)
+    view = base[:, :L]
+    idx = kernels.topk_indices(view, K, fill_value=0)
+    torch.cuda.synchronize()
+    _check(base.cpu()[:, :L], idx.cpu(), lambda r: K, lambda r: L, K, 0)
+
+
+def test_topk_matches_torch_topk_sets_when_no_ties(cuda):
+    from kascade_amd import kernels
+    g = torch.Generator().manual_seed(4)
+    rows, L, K = 8, 5000, 640
+    perm = torch.stack([torch.randperm(L, generator=g) for _ in range(rows)])
+    sc = (perm + 0x3000).to(torch.int16).view(torch.float16)   # distinct positive bit patterns
+    idx = kernels.topk_indices(sc.to(cuda), K)
+    want = torch.topk(sc.float(), K, dim=-1).indices.sort(dim=-1).values.int()
+    assert torch.equal(idx.cpu(), want)
