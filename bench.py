@@ -42,6 +42,62 @@ def log(msg):
     print(msg, file=sys.stderr, flush=True)
 
 
+SINGLE_KERNELS = ("prefill_dense", "prefill_scores", "prefill_aggregate", "prefill_topk", "prefill_reuse",
+                  "decode_dense", "decode_anchor0", "decode_anchor", "decode_topk", "decode_reuse")
+
+
+def run_single_kernel(name, iters, seq_len, dev, head_map):
+    """Profiling mode (rocprofv3 -- python3 bench.py --kernel NAME): the named kernel alone on its
+    benchmark workload -- prefill kernels on config 1 (32K), decode kernels on config 2 (B=16,
+    L=65536, paged) rotating over three layer caches so the K/V rows come from HBM."""
+    import torch
+    from kascade_amd import kernels, budgets, workloads
+    from kascade_amd.strategy import PagedKascadeDecoder
+    if name.startswith("prefill"):
+        L = seq_len
+        T = math.ceil(L / TILE)
+        w = workloads.prefill_inputs(1, L, seed=0, device=dev)
+        width = budgets.topk_width(L, PCT)
+        valid, nsel = budgets.prefill_tile_budgets(L, TILE, PCT, True, width)
+        valid = torch.tensor(valid, dtype=torch.int32, device=dev)
+        nsel = torch.tensor(nsel, dtype=torch.int32, device=dev)
+        log_sum = kernels.prefill_recompute1(w.q, w.k)
+        scores = torch.empty(1, G, T, L, device=dev, dtype=torch.float16)
+        kernels.prefill_aggregate(w.q, w.k, log_sum, scores)
+        idx = kernels.topk_indices(scores, width, valid_len=valid, n_sel=nsel)
+        hm = torch.tensor(head_map[1], dtype=torch.int32, device=dev)
+        fn = {"prefill_dense": lambda: kernels.prefill_recompute0(w.q, w.k, w.v),
+              "prefill_scores": lambda: kernels.prefill_recompute1(w.q, w.k),
+              "prefill_aggregate": lambda: kernels.prefill_aggregate(w.q, w.k, log_sum, scores),
+              "prefill_topk": lambda: kernels.topk_indices(scores, width, valid_len=valid, n_sel=nsel),
+              "prefill_reuse": lambda: kernels.prefill_reuse(w.q_reuse, w.k_reuse, w.v, idx, hm, float(PCT), True),
+              }[name]
+        for _ in range(iters):
+            fn()
+    else:
+        seqlens = [65536] * 16
+        caches = [workloads.paged_decode_inputs(seqlens, seed=10 + i, device=dev, reuse_keys=False)
+                  for i in range(3)]
+        c0 = caches[0]
+        dec = PagedKascadeDecoder(PCT, head_map, ANCHORS, 16, 65536, device=dev)
+        dec.anchor(0, c0.q, c0.k_pages, c0.v_pages, c0.block_table, c0.seqlens, 65536, ragged=False)
+        agg = torch.rand(16, G, 65536, device=dev).half()
+        for i in range(iters):
+            c = caches[i % 3]
+            if name == "decode_dense":
+                dec.dense(c.q, c.k_pages, c.v_pages, c0.block_table, c0.seqlens, 65536)
+            elif name == "decode_anchor0":
+                dec.anchor(0, c.q, c.k_pages, c.v_pages, c0.block_table, c0.seqlens, 65536, ragged=False)
+            elif name == "decode_anchor":
+                dec.anchor(2, c.q, c.k_pages, c.v_pages, c0.block_table, c0.seqlens, 65536, ragged=False)
+            elif name == "decode_topk":
+                kernels.topk_indices(agg, budgets.topk_width(65536, PCT), fill_value=0)
+            else:
+                dec.reuse(1, c.q, c.k_pages, c.v_pages, c0.block_table, c0.seqlens)
+    torch.cuda.synchronize()
+    print(json.dumps({"kernel": name, "iters": iters}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -51,6 +107,9 @@ def main():
     ap.add_argument("--skip-decode", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--decode-only", action="store_true", help="skip the per-kernel prefill section")
+    ap.add_argument("--kernel", choices=sorted(SINGLE_KERNELS), default=None,
+                    help="profiling mode: run only this kernel --iters times on its benchmark workload")
+    ap.add_argument("--iters", type=int, default=5)
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
@@ -82,6 +141,10 @@ def main():
         return ts[len(ts) // 2]
 
     head_map = get_head_mapping("Meta-Llama-3.1-8B-Instruct", list(ANCHORS))
+
+    if args.kernel:
+        run_single_kernel(args.kernel, args.iters, args.seq_len, dev, head_map)
+        return
 
     # ------------------------------------------------------------------ prefill, 32K
     L = args.seq_len

@@ -56,8 +56,10 @@ def default_num_split(total_rows: int, max_rows: int, wgs_per_cu: int = 2, min_r
     total_rows = sum over (sequence, KV head) of the rows visited; max_rows = longest list."""
     cus = _lib.init().kascade_device_cu_count() or 256
     target_wgs = wgs_per_cu * cus
-    rows_per_split = max(min_rows, -(-total_rows // target_wgs))
-    return int(max(1, min(256, -(-max_rows // rows_per_split))))
+    rows_per_split = max(min_rows, total_rows / target_wgs)
+    # round to nearest: one workgroup more than a whole number per compute unit costs a
+    # full extra wave of workgroups on a few units (tail), one fewer costs nothing
+    return int(max(1, min(256, round(max_rows / rows_per_split))))
 
 
 # ---------------------------------------------------------------- decode

@@ -1,0 +1,103 @@
+"""CPU-only checks of the C ABI: the library loads, exports every symbol the header declares,
+and rejects bad arguments before touching a GPU (return code -1 + message)."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "kascade_hip.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from kascade_amd import _lib
+    if not _lib.LIB_PATH.exists():
+        from kascade_amd import build
+        build.build()
+    return _lib.load()
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(kascade_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_bound(lib):
+    from kascade_amd import _lib
+    names = _declared_functions()
+    assert len(names) >= 14
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/kascade_hip.h but not exported"
+        assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
+    assert sorted(_lib.SIGNATURES) == names
+
+
+def test_abi_version_and_error_buffer(lib):
+    assert lib.kascade_abi_version() >= 1
+    assert isinstance(lib.kascade_get_last_error(), bytes)
+
+
+def test_topk_workspace_sizing(lib):
+    assert lib.kascade_topk_workspace_bytes(128, 1000) == 0          # short rows: one workgroup per row
+    assert lib.kascade_topk_workspace_bytes(8192, 32768) == 0        # too many rows for the workspace
+    n = lib.kascade_topk_workspace_bytes(32, 524288)
+    assert n == 4 * 32 * (2048 + 8 + 32 * 36)
+
+
+def _err(lib):
+    return lib.kascade_get_last_error().decode()
+
+
+def test_null_pointers_are_rejected(lib):
+    from kascade_amd._lib import Strides
+    s = Strides(8, 8, 8)
+    assert lib.kascade_decode_reuse_call(None, None, None, None, None, None, None, None, 1, 128, 128, 8, None) == -1
+    assert "null pointer" in _err(lib)
+    assert lib.kascade_decode_dense_paged_call(None, None, None, None, None, None, None, 1, 128, 8, None, 0, 16, None) == -1
+    assert "null pointer" in _err(lib)
+    assert lib.kascade_decode_recompute_paged_call(None, None, None, None, None, None, None, None, None, None,
+                                                   1, 128, 128, 8, 1, None, 0, 16, None) == -1
+    assert lib.kascade_topk_call(None, None, 1, 10, 10, None, None, 1, 4, 0, None, None) == -1
+    assert lib.kascade_prefill_dense_call(None, None, None, None, None, 1, 64, s, s, 1, None) == -1
+    assert lib.kascade_prefill_aggregate_call(None, None, None, None, 1, 64, s, s, 0, None) == -1
+    assert lib.kascade_prefill_reuse_call(None, None, None, None, None, 10.0, None, 1, 64, 128, 1, s, s, None) == -1
+    assert lib.kascade_paged_kv_append_call(None, None, None, None, None, None, 1, 1, 1, 16, s, None) == -1
+
+
+def test_bad_sizes_are_rejected(lib):
+    from kascade_amd._lib import Strides
+    buf = (C.c_char * 4096)()
+    p = C.addressof(buf) & ~15          # fake, 16-byte aligned, never dereferenced: validation fails first
+    p += 16
+    assert lib.kascade_decode_reuse_paged_call(p, p, p, None, p, p, 0.0, p, p, p, 0, 128, 128, 8, None, 0, 16, None) == -1
+    assert "batch" in _err(lib)
+    assert lib.kascade_decode_reuse_paged_call(p, p, p, None, p, p, 10.0, p, p, p, 1, 128, 128, 8, None, 0, 16, None) == -1
+    assert "cache_seqlens" in _err(lib)
+    assert lib.kascade_decode_dense_paged_call(p, p, p, None, p, p, p, 1, 128, 8, p, 4, 12, None) == -1
+    assert "power of two" in _err(lib)
+    assert lib.kascade_decode_dense_paged_call(p + 2, p, p, None, p, p, p, 1, 128, 8, None, 0, 16, None) == -1
+    assert "aligned" in _err(lib)
+    assert lib.kascade_topk_call(p, p, 4, 100, 200, None, None, 1, 8, 0, None, None) == -1
+    assert "uniform_len" in _err(lib)
+    bad = Strides(100, 4, 128)          # not multiples of 8 elements
+    ok = Strides(4096 * 128, 4096, 128)
+    assert lib.kascade_prefill_dense_call(p, p, p, p, p, 1, 64, bad, ok, 1, None) == -1
+    assert "strides" in _err(lib)
+    assert lib.kascade_prefill_reuse_call(p, p, p, p, p, 0.0, p, 1, 64, 128, 1, ok, ok, None) == -1
+    assert "rolling" in _err(lib)
+    assert lib.kascade_prefill_reuse_call(p, p, p, p, p, 10.0, p, 1, 64, 0, 0, ok, ok, None) == -1
+    assert "max_topk_num" in _err(lib)
+
+
+def test_python_wrappers_fail_loudly_without_gpu():
+    import torch
+    from kascade_amd import kernels
+    from kascade_amd._lib import KascadeError
+    if torch.cuda.is_available():
+        pytest.skip("GPU present")
+    q = torch.zeros(1, 32, 128, dtype=torch.float16)
+    with pytest.raises((KascadeError, RuntimeError)):
+        kernels.decode_reuse(q, q, q, q, q, q, q)
