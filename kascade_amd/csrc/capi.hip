@@ -172,6 +172,7 @@ int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_hal
             "decode_recompute: with_output needs V, Output and Output_partial");
     REQUIRE(batch > 0 && num_split > 0 && scores_stride > 0,
             "decode_recompute: batch, num_split, scores_stride must be > 0");
+    REQUIRE(scores_stride % 8 == 0, "decode_recompute: scores_stride must be a multiple of 8");
     REQUIRE(batch <= 65535, "decode_recompute: batch exceeds grid limit");
     REQUIRE(cache_seqlens || (kv_stride_tokens > 0 && kv_stride_tokens <= scores_stride),
             "decode_recompute: without cache_seqlens need 0 < kv_stride_tokens <= scores_stride");

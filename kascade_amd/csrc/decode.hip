@@ -14,17 +14,24 @@
 //   fp32 FMAs.  2 flop/byte is far below the machine balance, so no MFMA here.
 #include "decode.h"
 
+#include <type_traits>
+
 namespace kascade {
 
 namespace {
 
 constexpr int kThreads = 256;
+// The instruction scheduler otherwise sinks every prefetch load down to its first use (to save
+// registers), which serialises load -> wait -> use and removes all memory-level parallelism.
+#define KASCADE_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
 #ifndef KASCADE_DECODE_UNROLL
 #define KASCADE_DECODE_UNROLL 4
 #endif
 constexpr int kUnroll = KASCADE_DECODE_UNROLL;  // rows per row-group per iteration
 constexpr int kRowsPerIter = 16 * kUnroll;    // rows per workgroup iteration (128)
-constexpr int kSubChunk = 2048;               // rows whose physical ids are staged in LDS at once
+constexpr int kScoreBatches = 16;             // batches between two score flushes (anchor mode)
+constexpr int kStripRows = 16 * kScoreBatches;  // rows a wavefront owns per super-iteration
+constexpr int kSubChunk = 1024;               // rows whose physical ids are staged in LDS at once
 
 struct MergeState {  // one per wavefront after the in-wave merge
     float m[kGroupSize];
@@ -33,12 +40,14 @@ struct MergeState {  // one per wavefront after the in-wave merge
 };
 
 template <bool GATHER, bool WITH_V, bool WRITE_SCORES>
-__global__ __launch_bounds__(kThreads) void decode_split_kernel(DecodeParams p) {
-    __shared__ int s_row[kSubChunk];
+__global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decode_split_kernel(DecodeParams p) {
+    __shared__ int s_row[GATHER ? kSubChunk : 1];
     __shared__ MergeState s_merge[4];
+    // anchor mode: two buffers of four wavefront strips (4 heads x kStripRows raw scores)
+    __shared__ __attribute__((aligned(16))) float s_sc[WRITE_SCORES ? 2 : 1][WRITE_SCORES ? 4 : 1][kGroupSize][WRITE_SCORES ? kStripRows : 4];
 
-    const int split = blockIdx.x;
-    const int g = blockIdx.y;
+    const int g = blockIdx.x;       // the 8 KV heads of one token range are adjacent in dispatch order
+    const int split = blockIdx.y;
     const int b = blockIdx.z;
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
@@ -90,22 +99,20 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(DecodeParams p) 
         Pack16 k[kUnroll];
         Pack16 v[kUnroll];
     };
-    // wave covers 32 consecutive rows of an iteration: row = it + wave*32 + u*4 + rg
-    auto load_batch = [&](int it, int cn, Batch& bt) {
-        if (it >= cn) return;
-        const int rbase = it + wave * (4 * kUnroll) + rg;
+    // A wavefront covers 4*kUnroll consecutive rows of an iteration: row = it + wave*4U + u*4 + rg.
+    // `rows` are physical row numbers (page*page_size + slot, or b*stride + token).
+    auto issue_loads = [&](const int (&rows)[kUnroll], Batch& bt) {
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-            const int r = rbase + u * 4;
-            const int row = s_row[r < cn ? r : (cn - 1)];
-            const size_t off = (size_t)row * (kGroups * kDim) + head_off;
+            const size_t off = (size_t)rows[u] * (kGroups * kDim) + head_off;
             bt.k[u].u = ld_global_16(p.K + off);
             if (WITH_V) bt.v[u].u = ld_global_16(p.V + off);
         }
     };
-    auto compute_batch = [&](int it, int cn, int c0, const Batch& bt) {
-        if (it >= cn) return;
-        const int rbase = it + wave * (4 * kUnroll) + rg;
+    // Straight-line on purpose (no early exit, loads never skipped): a branch between issuing
+    // a batch and consuming it makes the compiler wait for every outstanding load.
+    // rbase: first row (relative to c0) of this lane's row-group in the batch, rows rbase + 4u.
+    auto compute_batch = [&](int rbase, int cn, int c0, int phase, int buf, const Batch& bt) {
         float s[kUnroll][kGroupSize];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
@@ -118,21 +125,23 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(DecodeParams p) 
             }
         }
         if (WRITE_SCORES) {
-            // lanes dl < kUnroll write the four heads of row u = dl: for a fixed head the
-            // wavefront stores 4*kUnroll consecutive tokens.
-            float w[kGroupSize] = {0.f, 0.f, 0.f, 0.f};
+            // Raw scores are parked in LDS strips (per wavefront: 4 heads x kStripRows tokens)
+            // and written to HBM by a fifth wavefront that streams nothing.  A store issued by
+            // a streaming wavefront costs it dearly: loads and stores complete in order on one
+            // counter, so every younger K/V load is held back until the store is acknowledged.
+            static_assert(!WRITE_SCORES || kUnroll == 4, "score staging assumes 4 rows per row-group");
+            const int usel = dl & 3, hsel = dl >> 2;
+            float w[kGroupSize];
 #pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
+            for (int h = 0; h < kGroupSize; ++h) {
+                w[h] = s[0][h];
 #pragma unroll
-                for (int h = 0; h < kGroupSize; ++h) w[h] = (u == dl) ? s[u][h] : w[h];
+                for (int u = 1; u < kUnroll; ++u) w[h] = (usel == u) ? s[u][h] : w[h];
             }
-            const int r = rbase + dl * 4;
-            if (dl < kUnroll && r < cn) {
-                const int tok = c0 + r;  // dense mode only: token id == row number
-                float* sp = p.scores + ((size_t)b * kHeads + g * kGroupSize) * p.scores_stride + tok;
+            float val = w[0];
 #pragma unroll
-                for (int h = 0; h < kGroupSize; ++h) sp[(size_t)h * p.scores_stride] = w[h];
-            }
+            for (int h = 1; h < kGroupSize; ++h) val = (hsel == h) ? w[h] : val;
+            s_sc[buf][wave][hsel][phase * 16 + usel * 4 + rg] = val;
         }
 #pragma unroll
         for (int h = 0; h < kGroupSize; ++h) {
@@ -162,33 +171,140 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(DecodeParams p) 
         }
     };
 
-    for (int c0 = r0; c0 < r1; c0 += kSubChunk) {
-        const int cn = min(kSubChunk, r1 - c0);
-        __syncthreads();
-        // stage physical row ids of this sub-chunk
-        for (int i = tid; i < cn; i += kThreads) {
-            int tok = GATHER ? idx_row[c0 + i] : (c0 + i);
-            tok = max(0, min(tok, seqlen - 1));   // a corrupt index must not leave the sequence
-            int row;
-            if (p.block_table) {
-                int pg = p.block_table[(size_t)b * p.max_pages + (tok >> p.page_shift)];
-                row = (pg << p.page_shift) + (tok & page_mask);
-            } else {
-                row = b * p.kv_stride_tokens + tok;
+    if (GATHER) {
+        // Index list -> block table -> physical row, staged in LDS one sub-chunk at a time.
+        for (int c0 = r0; c0 < r1; c0 += kSubChunk) {
+            const int cn = min(kSubChunk, r1 - c0);
+            __syncthreads();
+            for (int i = tid; i < cn; i += kThreads) {
+                int tok = idx_row[c0 + i];
+                tok = max(0, min(tok, seqlen - 1));   // a corrupt index must not leave the sequence
+                int row;
+                if (p.block_table) {
+                    int pg = p.block_table[(size_t)b * p.max_pages + (tok >> p.page_shift)];
+                    row = (pg << p.page_shift) + (tok & page_mask);
+                } else {
+                    row = b * p.kv_stride_tokens + tok;
+                }
+                s_row[i] = row;
             }
-            s_row[i] = row;
+            __syncthreads();
+            auto staged_rows = [&](int it, int (&rows)[kUnroll]) {
+                const int rbase = it + wave * (4 * kUnroll) + rg;
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u) rows[u] = s_row[min(rbase + u * 4, cn - 1)];
+            };
+            // software pipeline: the loads of iteration i+1 are in flight while iteration i computes
+            Batch ba, bb;
+            int rows[kUnroll];
+            staged_rows(0, rows);
+            issue_loads(rows, ba);
+            for (int it = 0; it < cn; it += 2 * kRowsPerIter) {
+                staged_rows(it + kRowsPerIter, rows);      // rows past the end are clamped and masked
+                issue_loads(rows, bb);
+                KASCADE_SCHED_FENCE();
+                compute_batch(it + wave * (4 * kUnroll) + rg, cn, c0, 0, 0, ba);
+                KASCADE_SCHED_FENCE();
+                staged_rows(it + 2 * kRowsPerIter, rows);
+                issue_loads(rows, ba);
+                KASCADE_SCHED_FENCE();
+                compute_batch(it + kRowsPerIter + wave * (4 * kUnroll) + rg, cn, c0, 0, 0, bb);
+                KASCADE_SCHED_FENCE();
+            }
         }
-        __syncthreads();
-
-        // software pipeline: the loads of iteration i+1 are in flight while iteration i computes
-        Batch ba, bb;
-        load_batch(0, cn, ba);
-        for (int it = 0; it < cn; it += 2 * kRowsPerIter) {
-            load_batch(it + kRowsPerIter, cn, bb);
-            compute_batch(it, cn, c0, ba);
-            load_batch(it + 2 * kRowsPerIter, cn, ba);
-            compute_batch(it + kRowsPerIter, cn, c0, bb);
+    } else {
+        // Dense range [r0, r1): no staging and no barriers.  Three-stage pipeline: block-table
+        // entries two iterations ahead, K/V rows one iteration ahead, arithmetic on the current.
+        const int cn = r1 - r0;
+        const int* bt_row = p.block_table ? p.block_table + (size_t)b * p.max_pages : nullptr;
+        // A wavefront owns kStripRows consecutive rows of every super-iteration of
+        // 4*kStripRows rows and walks them in kScoreBatches batches of 16 (batch number
+        // q = it / kRowsPerIter, phase q % kScoreBatches).
+        auto rbase_of = [&](int it) {
+            const int q = it / kRowsPerIter;
+            return (q / kScoreBatches) * (4 * kStripRows) + wave * kStripRows + (q % kScoreBatches) * 16 + rg;
+        };
+        // Writer wavefront: stores the four strips of super-iteration `sup` (buffer sup & 1), one
+        // 16-byte store per lane per instruction, 1 KB contiguous per (strip, head).
+        auto flush_scores = [&](int sup) {
+            constexpr int kVecPerStrip = kGroupSize * kStripRows / 4;   // float4 per strip
+#pragma unroll 4
+            for (int i = 0; i < 4 * kVecPerStrip / 64; ++i) {
+                const int idx = i * 64 + lane;
+                const int w = idx / kVecPerStrip, rem = idx % kVecPerStrip;
+                const int h = rem / (kStripRows / 4), t4 = (rem % (kStripRows / 4)) * 4;
+                const float4_t v = *reinterpret_cast<const float4_t*>(&s_sc[sup & 1][w][h][t4]);
+                const int r = sup * (4 * kStripRows) + w * kStripRows + t4;
+                float* dst = p.scores + ((size_t)b * kHeads + g * kGroupSize + h) * p.scores_stride + r0 + r;
+                if (r + 3 < cn) {
+                    *reinterpret_cast<float4_t*>(dst) = v;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (r + e < cn) dst[e] = v[e];
+                }
+            }
+        };
+        auto tok_of = [&](int it, int u) { return min(r0 + rbase_of(it) + u * 4, r1 - 1); };
+        // The paged / contiguous choice is hoisted out of the loop as a compile-time tag: a
+        // per-load "table ? table[i] : 0" turns into a branch whose join waits for every load
+        // in flight.
+        auto run = [&](auto paged_tag) {
+        constexpr bool PAGED = decltype(paged_tag)::value;
+        auto fetch_pages = [&](int it, int (&pg)[kUnroll]) {
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) pg[u] = PAGED ? bt_row[tok_of(it, u) >> p.page_shift] : 0;
+        };
+        auto rows_of = [&](int it, const int (&pg)[kUnroll], int (&rows)[kUnroll]) {
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                const int tok = tok_of(it, u);
+                rows[u] = PAGED ? (pg[u] << p.page_shift) + (tok & page_mask) : b * p.kv_stride_tokens + tok;
+            }
+        };
+        if (cn > 0) {
+            // Block-table entries are fetched *before* the K/V loads of the preceding batch in
+            // program order: loads complete in order, so waiting for a younger table entry would
+            // otherwise drain the K/V loads in flight.
+            Batch ba, bb;
+            int pga[kUnroll], pgb[kUnroll], rows[kUnroll];
+            fetch_pages(0, pga);
+            rows_of(0, pga, rows);
+            issue_loads(rows, ba);
+            fetch_pages(kRowsPerIter, pgb);
+            // every wavefront runs the same number of batches: enough for the longest strip
+            const int full = cn / (4 * kStripRows), rem = cn - full * (4 * kStripRows);
+            const int nbatch = full * kScoreBatches + min(kScoreBatches, (rem + 15) / 16);
+            const int it_end = ((nbatch + 1) & ~1) * kRowsPerIter;   // the loop body handles two batches
+            if (WRITE_SCORES && wave == 4) {
+                // one barrier per super-iteration, matched by the streaming wavefronts below
+                const int nsup = (it_end / kRowsPerIter + kScoreBatches - 1) / kScoreBatches;
+                for (int sup = 0; sup < nsup; ++sup) {
+                    __syncthreads();
+                    flush_scores(sup);
+                }
+            } else {
+            for (int it = 0; it < it_end; it += 2 * kRowsPerIter) {
+                const int q = it / kRowsPerIter;
+                fetch_pages(it + 2 * kRowsPerIter, pga);   // tokens past the end are clamped and masked
+                rows_of(it + kRowsPerIter, pgb, rows);
+                issue_loads(rows, bb);
+                KASCADE_SCHED_FENCE();
+                compute_batch(rbase_of(it), cn, r0, q % kScoreBatches, (q / kScoreBatches) & 1, ba);
+                KASCADE_SCHED_FENCE();
+                fetch_pages(it + 3 * kRowsPerIter, pgb);
+                rows_of(it + 2 * kRowsPerIter, pga, rows);
+                issue_loads(rows, ba);
+                KASCADE_SCHED_FENCE();
+                compute_batch(rbase_of(it + kRowsPerIter), cn, r0, (q + 1) % kScoreBatches, (q / kScoreBatches) & 1, bb);
+                KASCADE_SCHED_FENCE();
+                if (WRITE_SCORES && ((q + 2) % kScoreBatches == 0 || it + 2 * kRowsPerIter >= it_end))
+                    __syncthreads();   // strips of this super-iteration are complete: hand them to the writer
+            }
+            }
         }
+        };
+        if (bt_row) run(std::true_type{}); else run(std::false_type{});
     }
 
     // ---- merge the four row-groups of the wavefront (lanes l, l^16, l^32) ----
@@ -213,7 +329,7 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(DecodeParams p) 
             m[h] = mx;
         }
     }
-    if (rg == 0) {
+    if (rg == 0 && wave < 4) {   // the writer wavefront of the anchor variants holds no state
 #pragma unroll
         for (int h = 0; h < kGroupSize; ++h) {
             if (dl == 0) {
@@ -228,7 +344,7 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(DecodeParams p) 
     }
     __syncthreads();
     // ---- merge the four wavefronts; thread -> (head, two d's) ----
-    {
+    if (tid < kThreads) {
         const int h = tid >> 6;
         const int d0 = (tid & 63) * 2;
         float mx = -INFINITY;
@@ -336,7 +452,7 @@ __global__ __launch_bounds__(256) void decode_aggregate_kernel(const float* __re
 
 hipError_t launch_decode_split(const DecodeParams& p, bool gather, bool with_v, bool write_scores,
                                hipStream_t stream) {
-    dim3 grid(p.num_split, kGroups, p.B), block(kThreads);
+    dim3 grid(kGroups, p.num_split, p.B), block(write_scores ? kThreads + 64 : kThreads);
     if (gather) {
         hipLaunchKernelGGL((decode_split_kernel<true, true, false>), grid, block, 0, stream, p);
     } else if (write_scores) {
