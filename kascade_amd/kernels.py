@@ -316,3 +316,69 @@ def paged_kv_append(K_pages, V_pages, k_new, v_new, start_pos, block_table, page
     _lib.check(lib.kascade_paged_kv_append_call(
         _ptr(K_pages), _ptr(V_pages), _ptr(k_new), _ptr(v_new), _ptr(start_pos), _ptr(block_table),
         B, n_new, block_table.shape[1], page_size, st, _stream()))
+
+
+# ------------------------------------------------- benchmark / correctness glue
+def prefill_full_kernel(Q, K, V, topk, tile_size=TILE, layer=0, topk_percent=10, rolling=False,
+                        fill_invalid=True):
+    """``full_kernel(recompute_kernel, aggregate_kernel, reuse_kernel, Q, K, V, topk, tile_size,
+    layer, topk_percent)`` of recompute_kascade_gqa_prefill.py:340-361: runs an anchor layer and
+    returns the three observables the reference's correctness mode compares, (O, indices, scores).
+    scores holds -inf at and after each tile's start when fill_invalid is set."""
+    if tile_size != TILE:
+        raise KascadeError(f"tile_size must be {TILE}")
+    B, L = Q.shape[:2]
+    T = (L + TILE - 1) // TILE
+    if layer == 0:
+        log_sum, o = prefill_recompute0(Q, K, V)
+    else:
+        log_sum = prefill_recompute1(Q, K)
+    scores = torch.empty(B, G, T, L, device=Q.device, dtype=torch.float16)
+    prefill_aggregate(Q, K, log_sum, scores, fill_invalid=fill_invalid)
+    valid, nsel = budgets.prefill_tile_budgets(L, TILE, topk_percent, rolling, topk)
+    indices = topk_indices(scores, topk,
+                           valid_len=torch.tensor(valid, dtype=torch.int32, device=Q.device),
+                           n_sel=torch.tensor(nsel, dtype=torch.int32, device=Q.device))
+    if layer != 0:
+        o = prefill_reuse(Q, K, V, indices, torch.arange(G, device=Q.device, dtype=torch.int32),
+                          topk_percent, rolling)
+    return o, indices, scores
+
+
+def decode_full_kernel(Q, K, V, topk, glse, Output_partial, row_sums, scores, layer=0):
+    """``full_kernel(recompute_kernel, reuse_kernel, Q, K, V, topk, glse, Output_partial, row_sums,
+    scores, layer)`` of recompute_kascade_gqa_decode.py:396-402 over a contiguous cache:
+    returns (O, topk_indices, aggregated scores)."""
+    L = K.shape[1]
+    o, agg = decode_recompute(Q, K, V, glse, Output_partial, row_sums, scores, layer)
+    indices = topk_indices(agg[:, :, :L], topk, fill_value=0)
+    if layer != 0:
+        o = decode_reuse(Q, K, V, indices, torch.arange(G, device=Q.device, dtype=torch.int32), glse,
+                         Output_partial)
+    return o, indices, agg[:, :, :L]
+
+
+def decode_full_kernel_kvcache(Q, K, V, cache_seqlens, topk_percent, glse, Output_partial, row_sums, scores,
+                               layer=0, block_table=None, page_size: int = 16, max_seqlen: Optional[int] = None):
+    """kvcache ``full_kernel`` of recompute_kascade_gqa_decode_with_kvcache.py:368-377 over a padded
+    or paged cache: anchor pass, selection over agg[:, :, :max_seqlen] with row width
+    128*ceil(floor(p*max_seqlen/100)/128), per-sequence prefix budgets, and on layers > 0 the
+    reuse pass with the identity head map.  max_seqlen avoids a device->host copy of the lengths."""
+    if max_seqlen is None:
+        max_seqlen = int(cache_seqlens.max().item())
+    o, agg = decode_recompute(Q, K, V, glse, Output_partial, row_sums, scores, layer,
+                              cache_seqlens=cache_seqlens, block_table=block_table, page_size=page_size,
+                              kv_len=max_seqlen)
+    width = budgets.decode_budget(max_seqlen, topk_percent)
+    if float(topk_percent).is_integer():
+        fl = (cache_seqlens.to(torch.int64) * int(topk_percent)) // 100
+    else:
+        fl = torch.floor(cache_seqlens.to(torch.float64) * float(topk_percent) / 100.0).to(torch.int64)
+    counts = (((fl + 127) // 128) * 128).to(torch.int32)
+    indices = topk_indices(agg[:, :, :max_seqlen], width, valid_len=cache_seqlens.repeat_interleave(G),
+                           n_sel=counts.repeat_interleave(G), fill_value=0)
+    if layer != 0:
+        o = decode_reuse_paged(Q, K, V, cache_seqlens, indices,
+                               torch.arange(G, device=Q.device, dtype=torch.int32), topk_percent, glse,
+                               Output_partial, block_table=block_table, page_size=page_size)
+    return o, indices, agg[:, :, :max_seqlen]

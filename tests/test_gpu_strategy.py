@@ -1,0 +1,121 @@
+"""GPU tests of the host-side mirror: EfficientKascadeStrategy.attention_forward through the HF
+calling convention (query [B,H,Lq,D], key/value [B,G,Lk,D]) and the full_kernel glue, against the
+CPU oracle."""
+import pytest
+import torch
+
+from oracle import kascade_oracle as orc
+from tests.helpers import assert_close, check_topk_rows
+
+pytestmark = pytest.mark.gpu
+
+H, G, D, TILE = 32, 8, 128, 32
+
+
+class _Module(torch.nn.Module):
+    def __init__(self, layer_idx):
+        super().__init__()
+        self.layer_idx = layer_idx
+        self.num_key_value_groups = H // G
+
+
+def _hf(x):   # [B,L,h,D] -> HF layout [B,h,L,D] (contiguous in that layout)
+    return x.permute(0, 2, 1, 3).contiguous()
+
+
+@pytest.mark.parametrize("rolling", [True, False])
+def test_strategy_prefill_three_layer_kinds(cuda, rolling):
+    from kascade_amd import workloads
+    from kascade_amd.strategy import EfficientKascadeStrategy
+    L, p = 1300, 10
+    w = workloads.prefill_inputs(1, L, seed=5, device="cpu")
+    hm = [list(range(G)), w.head_mapping, list(range(G)), w.head_mapping]
+    s = EfficientKascadeStrategy([0, 2], None, k=p, tile_size=TILE, rolling_prefill=rolling,
+                                 head_mapping=hm, register=False)
+    scaling = D ** -0.5
+    K = orc.k_kern(L, p)
+    # layer 0: dense output + indices
+    o0, none = s.attention_forward(_Module(0), _hf(w.q).to(cuda), _hf(w.k).to(cuda), _hf(w.v).to(cuda), None, scaling)
+    assert none is None and tuple(o0.shape) == (1, L, H, D)
+    want0, _ = orc.dense_prefill(w.q, w.k, w.v)
+    assert_close(o0, want0, "layer 0 output")
+    idx0 = s._topk_to_reuse.cpu()
+    assert tuple(idx0.shape) == (1, G, (L + TILE - 1) // TILE, K)
+    pooled = orc.pooled_prefill_scores(w.q, w.k, TILE)
+    T = pooled.shape[2]
+    nsel = [min(K, orc.prefill_budget(t, TILE, L, p, rolling, K)) for t in range(T)]
+    check_topk_rows(pooled.reshape(G * T, L), idx0.reshape(G * T, K), lambda r: nsel[r % T],
+                    lambda r: (r % T) * TILE, "layer-0 indices")
+    # layer 1: reuse through its head map
+    o1, _ = s.attention_forward(_Module(1), _hf(w.q_reuse).to(cuda), _hf(w.k_reuse).to(cuda), _hf(w.v).to(cuda), None, scaling)
+    want1 = orc.reuse_prefill(w.q_reuse, w.k_reuse, w.v, idx0, w.head_mapping, TILE, rolling, p)
+    assert_close(o1, want1, "reuse layer output")
+    # layer 2: anchor > 0, sparse with its own fresh indices
+    o2, _ = s.attention_forward(_Module(2), _hf(w.q_reuse).to(cuda), _hf(w.k_reuse).to(cuda), _hf(w.v).to(cuda), None, scaling)
+    idx2 = s._topk_to_reuse.cpu()
+    want2 = orc.reuse_prefill(w.q_reuse, w.k_reuse, w.v, idx2, list(range(G)), TILE, rolling, p)
+    assert_close(o2, want2, "anchor>0 output")
+    assert not torch.equal(idx2, idx0)
+
+
+def test_strategy_decode_layers(cuda):
+    from kascade_amd.strategy import EfficientKascadeStrategy
+    g = torch.Generator().manual_seed(3)
+    B, L, p = 2, 2000, 10
+    q = torch.randn(B, H, 1, D, generator=g).half()
+    k = (torch.randn(B, G, L, D, generator=g) * 1.5).half()
+    v = torch.randn(B, G, L, D, generator=g).half()
+    hm = [list(range(G)), [3, 3, 0, 1, 7, 6, 5, 2], list(range(G))]
+    s = EfficientKascadeStrategy([0, 2], None, k=p, tile_size=TILE, head_mapping=hm, register=False)
+    kc, vc = k.permute(0, 2, 1, 3).contiguous(), v.permute(0, 2, 1, 3).contiguous()
+    o0, _ = s.attention_forward(_Module(0), q.to(cuda), k.to(cuda), v.to(cuda), None, D ** -0.5)
+    assert tuple(o0.shape) == (B, 1, H, D)
+    want0, _ = orc.dense_decode(q[:, :, 0], kc, vc)
+    assert_close(o0[:, 0], want0, "decode layer 0")
+    idx = s._topk_to_reuse.cpu()
+    K = orc.k_kern(L, p)
+    assert tuple(idx.shape) == (B, G, K)
+    agg = orc.pooled_decode_scores(q[:, :, 0], kc)
+    check_topk_rows(agg.reshape(B * G, L), idx.reshape(B * G, K), lambda r: K, lambda r: L, "decode indices")
+    o1, _ = s.attention_forward(_Module(1), q.to(cuda), k.to(cuda), v.to(cuda), None, D ** -0.5)
+    assert_close(o1[:, 0], orc.reuse_decode(q[:, :, 0], kc, vc, idx, hm[1]), "decode reuse layer")
+    o2, _ = s.attention_forward(_Module(2), q.to(cuda), k.to(cuda), v.to(cuda), None, D ** -0.5)
+    idx2 = s._topk_to_reuse.cpu()
+    assert_close(o2[:, 0], orc.reuse_decode(q[:, :, 0], kc, vc, idx2, list(range(G))), "decode anchor>0")
+
+
+def test_full_kernel_observables(cuda):
+    """(O, indices, scores) of the anchor glue functions, as the reference's correctness mode compares them."""
+    from kascade_amd import kernels, workloads
+    L, p = 900, 20
+    w = workloads.prefill_inputs(1, L, seed=8, device="cpu", peaked=False)
+    K = orc.k_kern(L, p)
+    for layer in (0, 1):
+        o, idx, sc = kernels.prefill_full_kernel(w.q.to(cuda), w.k.to(cuda), w.v.to(cuda), K, TILE, layer, p, rolling=False)
+        o_w, idx_w, sc_w = orc.anchor_prefill(w.q, w.k, w.v, p, TILE, layer == 0, False)
+        fin = torch.isfinite(sc_w)
+        assert torch.equal(torch.isfinite(sc.cpu()), fin)
+        assert_close(torch.where(fin, sc.cpu(), torch.zeros(())), torch.where(fin, sc_w, torch.zeros(())).float(),
+                     "scores", atol=2e-6, rtol=2e-3)
+        if layer == 0:
+            assert_close(o, o_w, "O layer 0")
+        else:
+            assert_close(o, orc.reuse_prefill(w.q, w.k, w.v, idx.cpu(), list(range(G)), TILE, False, p), "O layer 1")
+    # decode, ragged + paged
+    seqlens = [1800, 1333]
+    pw = workloads.paged_decode_inputs(seqlens, seed=4, device="cpu")
+    B, ns, Lmax = 2, 3, 1800
+    glse = torch.empty(B, H, ns, device=cuda)
+    part = torch.empty(B, H, ns, D, device=cuda)
+    rs = torch.empty(B, H, device=cuda)
+    sc = torch.empty(B, H, 1800, device=cuda)
+    o, idx, agg = kernels.decode_full_kernel_kvcache(pw.q.to(cuda), pw.k_pages.to(cuda), pw.v_pages.to(cuda),
+                                                     pw.seqlens.to(cuda), 10, glse, part, rs, sc, layer=1,
+                                                     block_table=pw.block_table.to(cuda), max_seqlen=Lmax)
+    kc = orc.paged_to_contiguous(pw.k_pages, pw.block_table, seqlens)
+    vc = orc.paged_to_contiguous(pw.v_pages, pw.block_table, seqlens)
+    _, idx_w, agg_w = orc.anchor_decode(pw.q, kc, vc, 10, False, seqlens)
+    assert tuple(idx.shape) == tuple(idx_w.shape)
+    assert_close(agg.cpu(), agg_w, "agg", atol=2e-6, rtol=2e-3)
+    counts = [orc.n_kvcache(n, 10) for n in seqlens]
+    assert_close(o, orc.reuse_decode(pw.q, kc, vc, idx.cpu(), list(range(G)), counts), "kvcache full_kernel O")
