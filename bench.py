@@ -36,13 +36,15 @@ N_LAYERS = 32
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 MFMA_PEAK_TFLOPS = 2500.0      # MI355X published dense fp16 MFMA rate
 H100_PREFILL_32K_MS = 6.42     # reference's published Kascade prefill ms @32768 (H100)
+# rocprofv3 FETCH_SIZE*2.0 + WRITE_SIZE*1.0 per launch at config 1 (profiles/prefill_reuse.md)
+MEASURED_TRAFFIC_BYTES = {"prefill_attn_reuse": 1.376e9}
 
 
 def log(msg):
     print(msg, file=sys.stderr, flush=True)
 
 
-SINGLE_KERNELS = ("prefill_dense", "prefill_scores", "prefill_aggregate", "prefill_topk", "prefill_reuse",
+SINGLE_KERNELS = ("membw_copy", "prefill_dense", "prefill_scores", "prefill_aggregate", "prefill_topk", "prefill_reuse",
                   "decode_dense", "decode_anchor0", "decode_anchor", "decode_topk", "decode_reuse")
 
 
@@ -53,6 +55,15 @@ def run_single_kernel(name, iters, seq_len, dev, head_map):
     import torch
     from kascade_amd import kernels, budgets, workloads
     from kascade_amd.strategy import PagedKascadeDecoder
+    if name == "membw_copy":
+        # calibration for the FETCH_SIZE / WRITE_SIZE counters: a plain device copy of exactly 1 GiB
+        x = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        y = torch.empty_like(x)
+        for _ in range(iters):
+            y.copy_(x)
+        torch.cuda.synchronize()
+        print(json.dumps({"kernel": name, "iters": iters, "bytes_per_copy": 1 << 30}), flush=True)
+        return
     if name.startswith("prefill"):
         L = seq_len
         T = math.ceil(L / TILE)
@@ -231,7 +242,9 @@ def main():
         dom = max(totals, key=totals.get)
         roofline = dict(kern[dom])
         roofline["kernel"] = dom
-        roofline["traffic"] = None
+        # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of the same kernel
+        # on this workload (scaled by the plain-copy calibration): summaries under profiles/.
+        roofline["traffic"] = MEASURED_TRAFFIC_BYTES.get(dom) if L == 32768 else None
     else:
         prefill, roofline = {}, {"bound": "mfma", "achieved": None, "peak": MFMA_PEAK_TFLOPS,
                                  "unit": "TFLOP/s", "frac": None, "traffic": None}
