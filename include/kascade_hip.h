@@ -192,6 +192,52 @@ int kascade_paged_kv_append_call(kascade_half* K_pages, kascade_half* V_pages,
                                  int n_new, int max_pages, int page_size,
                                  kascade_strides new_strides, void* stream);
 
+/* ------------------------------------------- chunked prefill over the paged cache */
+
+/* The reference prefills a prompt in one call over contiguous K/V
+ * (EfficientKascadeStrategy.py:110-147).  A serving engine prefills in chunks: the chunk's K/V
+ * are appended to the paged cache first, then its queries attend to everything cached so far.
+ * These three calls are the three prefill kernels above with
+ *   - queries Q [B,q_len,H,D] (strides q_strides) at global positions q_start .. q_start+q_len-1,
+ *     q_start a multiple of 32 and the same for every sequence of the batch;
+ *   - keys = cache positions 0 .. q_start+q_len-1, read from K_pages/V_pages
+ *     [num_pages,page_size,G,D] through block_table [B,max_pages];
+ *   - outputs indexed by the chunk's own rows: log_sum [B,q_len,H], Output [B,q_len,H,D],
+ *     aggregate_scores [B,G,ceil(q_len/32),q_start+q_len].
+ * With q_start = 0 and q_len = L they compute what the whole-prompt calls compute; a prompt
+ * processed in 32-aligned chunks gives bit-identical rows.  No counterpart in the reference. */
+int kascade_prefill_chunk_dense_call(const kascade_half* Q, const kascade_half* K_pages,
+                                     const kascade_half* V_pages, float* log_sum,
+                                     kascade_half* Output, int batch, int q_start, int q_len,
+                                     kascade_strides q_strides, const int32_t* block_table,
+                                     int max_pages, int page_size, int num_pages, int with_output,
+                                     void* stream);
+
+int kascade_prefill_chunk_aggregate_call(const kascade_half* Q, const kascade_half* K_pages,
+                                         const float* log_sum, kascade_half* aggregate_scores,
+                                         int batch, int q_start, int q_len,
+                                         kascade_strides q_strides, const int32_t* block_table,
+                                         int max_pages, int page_size, int num_pages,
+                                         int fill_invalid, void* stream);
+
+/* physical_rows [B,G,ceil(q_len/32),max_topk_num]: the tile's top-k tokens already translated
+ * to rows of the paged cache (kascade_translate_indices_call), so that the gather needs no
+ * second dependent load. */
+int kascade_prefill_chunk_reuse_call(const kascade_half* Q, const kascade_half* K_pages,
+                                     const kascade_half* V_pages, const int32_t* physical_rows,
+                                     const int32_t* head_mapping, float topk_percent,
+                                     kascade_half* Output, int batch, int q_start, int q_len,
+                                     int max_topk_num, int rolling, kascade_strides q_strides,
+                                     const int32_t* block_table, int max_pages, int page_size,
+                                     int num_pages, void* stream);
+
+/* physical_rows[b,i] = block_table[b, t / page_size] * page_size + t % page_size with
+ * t = clamp(token_idx[b,i], 0, kv_len-1), i < per_sequence.  physical_rows may alias token_idx.
+ * No counterpart in the reference (its prefill never sees a paged cache). */
+int kascade_translate_indices_call(const int32_t* token_idx, int32_t* physical_rows,
+                                   const int32_t* block_table, int batch, int64_t per_sequence,
+                                   int max_pages, int page_size, int kv_len, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -49,6 +49,13 @@ SIGNATURES = {
     "kascade_prefill_reuse_call": (_I, [_P, _P, _P, _P, _P, _F, _P, _I, _I, _I, _I, Strides, Strides,
                                         _P]),
     "kascade_paged_kv_append_call": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, Strides, _P]),
+    "kascade_prefill_chunk_dense_call": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, Strides, _P, _I, _I, _I,
+                                              _I, _P]),
+    "kascade_prefill_chunk_aggregate_call": (_I, [_P, _P, _P, _P, _I, _I, _I, Strides, _P, _I, _I, _I,
+                                                  _I, _P]),
+    "kascade_prefill_chunk_reuse_call": (_I, [_P, _P, _P, _P, _P, _F, _P, _I, _I, _I, _I, _I, Strides,
+                                              _P, _I, _I, _I, _P]),
+    "kascade_translate_indices_call": (_I, [_P, _P, _P, _I, C.c_int64, _I, _I, _I, _P]),
 }
 
 _lib = None

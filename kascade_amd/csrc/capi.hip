@@ -240,7 +240,7 @@ int kascade_prefill_dense_call(const kascade_half* Q, const kascade_half* K, con
     p.Q = H(Q); p.K = H(K); p.V = with_output ? H(V) : H(K); p.log_sum = log_sum; p.O = H(Output);
     p.q_sb = q_strides.b; p.q_sl = q_strides.l; p.q_sh = q_strides.h;
     p.k_sb = kv_strides.b; p.k_sl = kv_strides.l; p.k_sh = kv_strides.h;
-    p.B = batch; p.L = seq_len; p.T = (seq_len + kTile - 1) / kTile;
+    p.B = batch; p.L = seq_len; p.Lq = seq_len; p.T = (seq_len + kTile - 1) / kTile;
     return check_hip(launch_prefill_attn(p, false, with_output != 0, with_output ? KASCADE_DENSE_NQB : 2,
                                          static_cast<hipStream_t>(stream)), "prefill_dense");
 }
@@ -257,7 +257,7 @@ int kascade_prefill_aggregate_call(const kascade_half* Q, const kascade_half* K,
     p.Q = H(Q); p.K = H(K); p.V = H(K); p.log_sum_in = log_sum; p.agg = H(aggregate_scores);
     p.q_sb = q_strides.b; p.q_sl = q_strides.l; p.q_sh = q_strides.h;
     p.k_sb = kv_strides.b; p.k_sl = kv_strides.l; p.k_sh = kv_strides.h;
-    p.B = batch; p.L = seq_len; p.T = (seq_len + kTile - 1) / kTile; p.fill_invalid = fill_invalid;
+    p.B = batch; p.L = seq_len; p.Lq = seq_len; p.T = (seq_len + kTile - 1) / kTile; p.fill_invalid = fill_invalid;
     return check_hip(launch_prefill_aggregate(p, static_cast<hipStream_t>(stream)),
                      "prefill_aggregate");
 }
@@ -280,7 +280,7 @@ int kascade_prefill_reuse_call(const kascade_half* Q, const kascade_half* K, con
     p.O = H(Output); p.log_sum = nullptr;
     p.q_sb = q_strides.b; p.q_sl = q_strides.l; p.q_sh = q_strides.h;
     p.k_sb = kv_strides.b; p.k_sl = kv_strides.l; p.k_sh = kv_strides.h;
-    p.B = batch; p.L = seq_len; p.T = (seq_len + kTile - 1) / kTile;
+    p.B = batch; p.L = seq_len; p.Lq = seq_len; p.T = (seq_len + kTile - 1) / kTile;
     p.max_topk = max_topk_num; p.rolling = rolling; p.topk_percent = topk_percent;
     return check_hip(launch_prefill_attn(p, true, true, 1, static_cast<hipStream_t>(stream)),
                      "prefill_reuse");
@@ -305,6 +305,112 @@ int kascade_paged_kv_append_call(kascade_half* K_pages, kascade_half* V_pages,
                                             new_strides.b, new_strides.l, new_strides.h,
                                             static_cast<hipStream_t>(stream)),
                      "paged_kv_append");
+}
+
+// ---- chunked prefill over the paged cache ----
+
+static int chunk_params(PrefillParams& p, const char* what, const kascade_half* Q, int batch,
+                        int q_start, int q_len, kascade_strides q_strides,
+                        const int32_t* block_table, int max_pages, int page_size, int num_pages) {
+    REQUIRE(block_table, "prefill_chunk: block_table is required");
+    REQUIRE(batch > 0 && batch <= 65535 && q_len > 0, "prefill_chunk: bad batch/q_len");
+    REQUIRE(q_start >= 0 && q_start % kTile == 0, "prefill_chunk: q_start must be a multiple of 32");
+    REQUIRE(aligned16(Q), "prefill_chunk: Q must be 16-byte aligned");
+    if (check_strides(q_strides, "Q")) return -1;
+    int shift;
+    if (check_paging(block_table, max_pages, page_size, &shift)) return -1;
+    REQUIRE(num_pages > 0 && (long long)num_pages * page_size < (1LL << 31),
+            "prefill_chunk: num_pages out of range");
+    REQUIRE((long long)max_pages * page_size >= (long long)q_start + q_len,
+            "prefill_chunk: block table shorter than q_start + q_len");
+    (void)what;
+    p.Q = H(Q);
+    p.q_sb = q_strides.b; p.q_sl = q_strides.l; p.q_sh = q_strides.h;
+    p.B = batch; p.L = q_start + q_len; p.Lq = q_len; p.q_start = q_start;
+    p.T = (q_len + kTile - 1) / kTile;
+    p.block_table = block_table; p.max_pages = max_pages; p.page_shift = shift;
+    p.num_pages = num_pages;
+    return 0;
+}
+
+int kascade_prefill_chunk_dense_call(const kascade_half* Q, const kascade_half* K_pages,
+                                     const kascade_half* V_pages, float* log_sum,
+                                     kascade_half* Output, int batch, int q_start, int q_len,
+                                     kascade_strides q_strides, const int32_t* block_table,
+                                     int max_pages, int page_size, int num_pages, int with_output,
+                                     void* stream) {
+    REQUIRE(Q && K_pages, "prefill_chunk_dense: null pointer argument");
+    REQUIRE(!with_output || (V_pages && Output), "prefill_chunk_dense: with_output needs V and Output");
+    REQUIRE(with_output || log_sum, "prefill_chunk_dense: nothing to compute (no Output, no log_sum)");
+    REQUIRE(aligned16(K_pages) && (!with_output || (aligned16(V_pages) && aligned16(Output))),
+            "prefill_chunk_dense: tensors must be 16-byte aligned");
+    PrefillParams p{};
+    if (chunk_params(p, "dense", Q, batch, q_start, q_len, q_strides, block_table, max_pages,
+                     page_size, num_pages))
+        return -1;
+    p.K = H(K_pages); p.V = with_output ? H(V_pages) : H(K_pages);
+    p.log_sum = log_sum; p.O = H(Output);
+    return check_hip(launch_prefill_attn(p, false, with_output != 0, 1,
+                                         static_cast<hipStream_t>(stream)), "prefill_chunk_dense");
+}
+
+int kascade_prefill_chunk_aggregate_call(const kascade_half* Q, const kascade_half* K_pages,
+                                         const float* log_sum, kascade_half* aggregate_scores,
+                                         int batch, int q_start, int q_len,
+                                         kascade_strides q_strides, const int32_t* block_table,
+                                         int max_pages, int page_size, int num_pages,
+                                         int fill_invalid, void* stream) {
+    REQUIRE(Q && K_pages && log_sum && aggregate_scores,
+            "prefill_chunk_aggregate: null pointer argument");
+    REQUIRE(aligned16(K_pages), "prefill_chunk_aggregate: K must be 16-byte aligned");
+    PrefillParams p{};
+    if (chunk_params(p, "aggregate", Q, batch, q_start, q_len, q_strides, block_table, max_pages,
+                     page_size, num_pages))
+        return -1;
+    p.K = H(K_pages); p.V = H(K_pages); p.log_sum_in = log_sum; p.agg = H(aggregate_scores);
+    p.fill_invalid = fill_invalid;
+    return check_hip(launch_prefill_aggregate(p, static_cast<hipStream_t>(stream)),
+                     "prefill_chunk_aggregate");
+}
+
+int kascade_prefill_chunk_reuse_call(const kascade_half* Q, const kascade_half* K_pages,
+                                     const kascade_half* V_pages, const int32_t* physical_rows,
+                                     const int32_t* head_mapping, float topk_percent,
+                                     kascade_half* Output, int batch, int q_start, int q_len,
+                                     int max_topk_num, int rolling, kascade_strides q_strides,
+                                     const int32_t* block_table, int max_pages, int page_size,
+                                     int num_pages, void* stream) {
+    REQUIRE(Q && K_pages && V_pages && physical_rows && head_mapping && Output,
+            "prefill_chunk_reuse: null pointer argument");
+    REQUIRE(max_topk_num > 0, "prefill_chunk_reuse: max_topk_num must be > 0");
+    REQUIRE(!rolling || topk_percent > 0.f, "prefill_chunk_reuse: rolling needs topk_percent > 0");
+    REQUIRE(aligned16(K_pages) && aligned16(V_pages) && aligned16(Output),
+            "prefill_chunk_reuse: tensors must be 16-byte aligned");
+    PrefillParams p{};
+    if (chunk_params(p, "reuse", Q, batch, q_start, q_len, q_strides, block_table, max_pages,
+                     page_size, num_pages))
+        return -1;
+    p.K = H(K_pages); p.V = H(V_pages); p.idx = physical_rows; p.head_map = head_mapping;
+    p.O = H(Output); p.log_sum = nullptr;
+    p.max_topk = max_topk_num; p.rolling = rolling; p.topk_percent = topk_percent;
+    return check_hip(launch_prefill_attn(p, true, true, 1, static_cast<hipStream_t>(stream)),
+                     "prefill_chunk_reuse");
+}
+
+int kascade_translate_indices_call(const int32_t* token_idx, int32_t* physical_rows,
+                                   const int32_t* block_table, int batch, int64_t per_sequence,
+                                   int max_pages, int page_size, int kv_len, void* stream) {
+    REQUIRE(token_idx && physical_rows && block_table, "translate_indices: null pointer argument");
+    REQUIRE(batch > 0 && batch <= 65535 && per_sequence >= 0 && kv_len > 0,
+            "translate_indices: bad batch/per_sequence/kv_len");
+    int shift;
+    if (check_paging(block_table, max_pages, page_size, &shift)) return -1;
+    REQUIRE((long long)max_pages * page_size >= kv_len,
+            "translate_indices: block table shorter than kv_len");
+    return check_hip(launch_translate_indices(token_idx, physical_rows, block_table, batch,
+                                              per_sequence, max_pages, shift, kv_len,
+                                              static_cast<hipStream_t>(stream)),
+                     "translate_indices");
 }
 
 }  // extern "C"

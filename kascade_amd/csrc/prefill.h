@@ -5,18 +5,23 @@
 namespace kascade {
 
 struct PrefillParams {
-    const half_t* Q;          // [B,L,H,D] through (q_sb, q_sl, q_sh)
-    const half_t* K;          // [B,L,G,D] through (k_sb, k_sl, k_sh); V shares the strides
-    const half_t* V;
-    const int* idx;           // [B,G,T,max_topk] (reuse)
+    // Queries are rows [0, Lq) of Q at global positions q_start + row; keys are positions
+    // [0, L), L = q_start + Lq.  A whole-prompt call has q_start = 0 and Lq = L.
+    const half_t* Q;          // [B,Lq,H,D] through (q_sb, q_sl, q_sh)
+    const half_t* K;          // [B,L,G,D] through (k_sb, k_sl, k_sh); V shares the strides.
+    const half_t* V;          //   Paged: [num_pages, page, G, D] contiguous, strides unused
+    const int* idx;           // [B,G,T,max_topk] (reuse); physical rows when paged
     const int* head_map;      // [G] (reuse)
-    const float* log_sum_in;  // [B,L,H] (aggregate)
-    float* log_sum;           // [B,L,H] or null (attention kernel output)
-    half_t* O;                // [B,L,H,D] contiguous
+    const float* log_sum_in;  // [B,Lq,H] (aggregate)
+    float* log_sum;           // [B,Lq,H] or null (attention kernel output)
+    half_t* O;                // [B,Lq,H,D] contiguous
     half_t* agg;              // [B,G,T,L] (aggregate)
+    const int* block_table;   // [B,max_pages] or null (strided K/V)
     long long q_sb, q_sl, q_sh;
     long long k_sb, k_sl, k_sh;
-    int B, L, T;
+    int B, L, T;              // T = ceil(Lq / 32) query tiles of this call
+    int Lq, q_start;
+    int max_pages, page_shift, num_pages;
     int max_topk;
     int rolling;
     float topk_percent;
@@ -26,5 +31,9 @@ struct PrefillParams {
 hipError_t launch_prefill_attn(const PrefillParams& p, bool reuse, bool with_v, int nqb,
                                hipStream_t stream);
 hipError_t launch_prefill_aggregate(const PrefillParams& p, hipStream_t stream);
+// out[b,i] = physical cache row of token idx[b,i] (clamped to [0, L)); out may alias idx.
+hipError_t launch_translate_indices(const int* idx, int* out, const int* block_table, int B,
+                                    long long per_seq, int max_pages, int page_shift, int L,
+                                    hipStream_t stream);
 
 }  // namespace kascade

@@ -24,6 +24,8 @@
 //   rows is an in-lane sum over accumulator registers.
 #include "prefill.h"
 
+#include <algorithm>
+
 namespace kascade {
 
 namespace {
@@ -44,12 +46,16 @@ __device__ __forceinline__ int rolling_budget(float pct, int tile_start) {
     return (int)(((fl + 127) / 128) * 128);
 }
 
-template <int NQB, bool REUSE, bool WITH_V>
+// Queries are rows [0, Lq) of Q at global positions q_start + row (q_start a multiple of 32);
+// keys are positions [0, L) with L = q_start + Lq.  PAGED: K/V are pages [P, page, G, D]
+// addressed through the block table, and gathered index rows hold physical row numbers.
+template <int NQB, bool REUSE, bool WITH_V, bool PAGED>
 __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t* sK, half_t* sV) {
 
     constexpr int QT = 32 * NQB;
     const int L = p.L;
-    const int nqt = (L + QT - 1) / QT;
+    const int Lq = p.Lq;
+    const int nqt = (Lq + QT - 1) / QT;
     const int tq = nqt - 1 - (int)blockIdx.x;   // long (late) query blocks first
     const int g = blockIdx.y;
     const int b = blockIdx.z;
@@ -58,16 +64,17 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
     const int lane = tid & 63;
     const int li = lane & 31;
     const int lg = lane >> 5;
-    const int q0 = tq * QT;
+    const int q0l = tq * QT;            // first query row of this block
+    const int q0 = p.q_start + q0l;     // its global position
     const int head = g * kGroupSize + wave;
 
     // ---- Q fragments (B operand of S^T): query li (+32 qb), d chunk 16*ks + 8*lg ----
     half8_t qf[NQB][8];
 #pragma unroll
     for (int qb = 0; qb < NQB; ++qb) {
-        const int q = q0 + 32 * qb + li;
-        const bool ok = q < L;
-        const half_t* qp = p.Q + (long long)b * p.q_sb + (long long)min(q, L - 1) * p.q_sl +
+        const int ql = q0l + 32 * qb + li;
+        const bool ok = ql < Lq;
+        const half_t* qp = p.Q + (long long)b * p.q_sb + (long long)min(ql, Lq - 1) * p.q_sl +
                            (long long)head * p.q_sh + lg * 8;
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
@@ -95,34 +102,66 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
 
     const int krow = tid >> 4;   // K: key position krow + 16 i, 16-byte column kcol
     const int kcol = tid & 15;
-    const half_t* kbase = p.K + (long long)b * p.k_sb + (long long)g * p.k_sh + kcol * 8;
-    const half_t* vbase = p.V + (long long)b * p.k_sb + (long long)g * p.k_sh + kcol * 8;
+    const half_t* kbase = PAGED ? p.K + (long long)g * kDim + kcol * 8
+                                : p.K + (long long)b * p.k_sb + (long long)g * p.k_sh + kcol * 8;
+    const half_t* vbase = PAGED ? p.V + (long long)g * kDim + kcol * 8
+                                : p.V + (long long)b * p.k_sb + (long long)g * p.k_sh + kcol * 8;
+    const int* bt_row = PAGED ? p.block_table + (long long)b * p.max_pages : nullptr;
+    const int page_mask = (1 << p.page_shift) - 1;
+    const int max_row = PAGED ? (p.num_pages << p.page_shift) - 1 : 0;
 
-    int nk[4], nv[4];       // key ids of the tile to be loaded next
+    // key position `pos` of tile `ti` -> key id (contiguous and diagonal tiles)
+    auto tile_key = [&](int ti, int pos) {
+        return min((sparse ? q0 : ti * kKT) + pos, L - 1);
+    };
+    // nk/nv: what the next tile's loads need.  Strided K/V: key ids.  PAGED: block-table
+    // entries for contiguous keys (combined with the key's slot when the loads are issued, so
+    // that nothing waits on the table load here) or physical rows for gathered tiles.
+    int nk[4], nv[4];
+    int pend_ti = 0;        // tile the ids belong to
     uint4_t kr[4], vr[4];   // tile data in flight
     auto fetch_ids = [&](int ti) {
+        pend_ti = ti;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int pk = krow + 16 * i;       // K position of chunk i
             const int pv = 4 * krow + i;        // V position of chunk i
-            if (!sparse) {
-                nk[i] = min(ti * kKT + pk, L - 1);
-                nv[i] = min(ti * kKT + pv, L - 1);
-            } else if (ti < ng) {
-                nk[i] = max(0, min(idx_row[min(ti * kKT + pk, n - 1)], L - 1));
-                nv[i] = max(0, min(idx_row[min(ti * kKT + pv, n - 1)], L - 1));
+            if (sparse && ti < ng) {
+                const int a = idx_row[min(ti * kKT + pk, n - 1)];
+                const int c = idx_row[min(ti * kKT + pv, n - 1)];
+                nk[i] = max(0, min(a, PAGED ? max_row : L - 1));
+                nv[i] = max(0, min(c, PAGED ? max_row : L - 1));
+            } else if (PAGED) {
+                nk[i] = bt_row[tile_key(ti, pk) >> p.page_shift];
+                nv[i] = bt_row[tile_key(ti, pv) >> p.page_shift];
             } else {
-                nk[i] = min(q0 + pk, L - 1);
-                nv[i] = min(q0 + pv, L - 1);
+                nk[i] = tile_key(ti, pk);
+                nv[i] = tile_key(ti, pv);
             }
         }
     };
     auto issue_loads = [&]() {
+        if (PAGED) {
+            const bool gathered = sparse && pend_ti < ng;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) kr[i] = ld_global_16(kbase + (long long)nk[i] * p.k_sl);
-        if (WITH_V) {
+            for (int i = 0; i < 4; ++i) {
+                const int rk = gathered ? nk[i] : (nk[i] << p.page_shift) + (tile_key(pend_ti, krow + 16 * i) & page_mask);
+                kr[i] = ld_global_16(kbase + (long long)rk * (kGroups * kDim));
+            }
+            if (WITH_V) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) vr[i] = ld_global_16(vbase + (long long)nv[i] * p.k_sl);
+                for (int i = 0; i < 4; ++i) {
+                    const int rv = gathered ? nv[i] : (nv[i] << p.page_shift) + (tile_key(pend_ti, 4 * krow + i) & page_mask);
+                    vr[i] = ld_global_16(vbase + (long long)rv * (kGroups * kDim));
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) kr[i] = ld_global_16(kbase + (long long)nk[i] * p.k_sl);
+            if (WITH_V) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) vr[i] = ld_global_16(vbase + (long long)nv[i] * p.k_sl);
+            }
         }
     };
 
@@ -197,7 +236,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
             if (kstart + kKT - 1 > q0 || kstart + kKT > L) {
 #pragma unroll
                 for (int qb = 0; qb < NQB; ++qb) {
-                    const int q = q0 + 32 * qb + li;
+                    const int q = q0 + 32 * qb + li;   // global position
 #pragma unroll
                     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -284,17 +323,17 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
         }
     }
 
-    // ---- epilogue ----
+    // ---- epilogue (rows are local to this call) ----
 #pragma unroll
     for (int qb = 0; qb < NQB; ++qb) {
-        const int q = q0 + 32 * qb + li;
+        const int ql = q0l + 32 * qb + li;
         const float lt = l[qb] + __shfl_xor(l[qb], 32);
-        if (q < L) {
+        if (ql < Lq) {
             if (p.log_sum && lg == 0)
-                p.log_sum[((long long)b * L + q) * kHeads + head] = fast_log2(lt) + m[qb] * kScaleLog2;
+                p.log_sum[((long long)b * Lq + ql) * kHeads + head] = fast_log2(lt) + m[qb] * kScaleLog2;
             if (WITH_V) {
                 const float inv = 1.f / lt;
-                half_t* op = p.O + (((long long)b * L + q) * kHeads + head) * kDim;
+                half_t* op = p.O + (((long long)b * Lq + ql) * kHeads + head) * kDim;
 #pragma unroll
                 for (int db = 0; db < 4; ++db)
 #pragma unroll
@@ -314,12 +353,12 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
 
 // 32 queries per wavefront: register budget capped so that two workgroups share a
 // compute unit and hide each other's LDS staging and gather latency.
-template <bool REUSE, bool WITH_V>
+template <bool REUSE, bool WITH_V, bool PAGED>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(KASCADE_PREFILL_WAVES_NQB1)))
 void prefill_attn_kernel_q32(PrefillParams p) {
     __shared__ __attribute__((aligned(16))) half_t sK[kKT * kKStride];
     __shared__ __attribute__((aligned(16))) half_t sV[kDim * kVStride];
-    prefill_attn_body<1, REUSE, WITH_V>(p, sK, sV);
+    prefill_attn_body<1, REUSE, WITH_V, PAGED>(p, sK, sV);
 }
 
 // 64 queries per wavefront: one wavefront per SIMD with the whole register file.
@@ -327,14 +366,18 @@ template <bool WITH_V>
 __global__ __launch_bounds__(kThreads) void prefill_attn_kernel_q64(PrefillParams p) {
     __shared__ __attribute__((aligned(16))) half_t sK[kKT * kKStride];
     __shared__ __attribute__((aligned(16))) half_t sV[kDim * kVStride];
-    prefill_attn_body<2, false, WITH_V>(p, sK, sV);
+    prefill_attn_body<2, false, WITH_V, false>(p, sK, sV);
 }
 
+// Pooled tile scores: out[b,g,t,key] = sum over the 32 queries of tile t and the 4 q-heads of g
+// of exp2(s*scale - log_sum), for keys before the tile's first (global) position.
+template <bool PAGED>
 __global__ __launch_bounds__(kThreads) void prefill_aggregate_kernel(PrefillParams p) {
     __shared__ __attribute__((aligned(16))) half_t sK[kAggKT * kKStride];
     __shared__ __attribute__((aligned(16))) float s_lse[128];
 
     const int L = p.L;
+    const int Lq = p.Lq;
     const int t = p.T - 1 - (int)blockIdx.x;
     const int g = blockIdx.y;
     const int b = blockIdx.z;
@@ -343,19 +386,20 @@ __global__ __launch_bounds__(kThreads) void prefill_aggregate_kernel(PrefillPara
     const int lane = tid & 63;
     const int li = lane & 31;
     const int lg = lane >> 5;
-    const int ts = t * kTile;
+    const int tl = t * kTile;            // first query row of the tile
+    const int ts = p.q_start + tl;       // its global position
     half_t* out = p.agg + (((long long)b * kGroups + g) * p.T + t) * L;
     const half_t neg_inf = (half_t)(-INFINITY);
 
     const int ntiles = (ts + kAggKT - 1) / kAggKT;
     if (ntiles > 0) {
-        // A operands: row block rb = q-head 4g+rb, row li = query ts+li
+        // A operands: row block rb = q-head 4g+rb, row li = query tl+li
         half8_t qa[kGroupSize][8];
 #pragma unroll
         for (int rb = 0; rb < kGroupSize; ++rb) {
-            const int q = ts + li;
-            const bool ok = q < L;
-            const half_t* qp = p.Q + (long long)b * p.q_sb + (long long)min(q, L - 1) * p.q_sl +
+            const int q = tl + li;
+            const bool ok = q < Lq;
+            const half_t* qp = p.Q + (long long)b * p.q_sb + (long long)min(q, Lq - 1) * p.q_sl +
                                (long long)(g * kGroupSize + rb) * p.q_sh + lg * 8;
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks) {
@@ -366,28 +410,45 @@ __global__ __launch_bounds__(kThreads) void prefill_aggregate_kernel(PrefillPara
             }
         }
         if (tid < 128) {
-            const int q = ts + (tid & 31);
-            s_lse[tid] = (q < L) ? p.log_sum_in[((long long)b * L + q) * kHeads + g * kGroupSize + (tid >> 5)]
-                                 : INFINITY;
+            const int q = tl + (tid & 31);
+            s_lse[tid] = (q < Lq) ? p.log_sum_in[((long long)b * Lq + q) * kHeads + g * kGroupSize + (tid >> 5)]
+                                  : INFINITY;
         }
         const int krow = tid >> 4, kcol = tid & 15;
-        const half_t* kbase = p.K + (long long)b * p.k_sb + (long long)g * p.k_sh + kcol * 8;
+        const half_t* kbase = PAGED ? p.K + (long long)g * kDim + kcol * 8
+                                    : p.K + (long long)b * p.k_sb + (long long)g * p.k_sh + kcol * 8;
+        const int* bt_row = PAGED ? p.block_table + (long long)b * p.max_pages : nullptr;
+        const int page_mask = (1 << p.page_shift) - 1;
         uint4_t kr[8];
+        int pg[8];   // block-table entries of the tile after the one in flight (paged)
+        auto fetch_pages = [&](int ti) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                pg[i] = bt_row[min(ti * kAggKT + krow + 16 * i, L - 1) >> p.page_shift];
+        };
         auto issue_loads = [&](int ti) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const int key = min(ti * kAggKT + krow + 16 * i, L - 1);
-                kr[i] = ld_global_16(kbase + (long long)key * p.k_sl);
+                if (PAGED)
+                    kr[i] = ld_global_16(kbase + (long long)((pg[i] << p.page_shift) + (key & page_mask)) * (kGroups * kDim));
+                else
+                    kr[i] = ld_global_16(kbase + (long long)key * p.k_sl);
             }
         };
+        if (PAGED) fetch_pages(0);
         issue_loads(0);
+        if (PAGED && ntiles > 1) fetch_pages(1);
         for (int ti = 0; ti < ntiles; ++ti) {
             __syncthreads();
 #pragma unroll
             for (int i = 0; i < 8; ++i)
                 *reinterpret_cast<uint4_t*>(&sK[(krow + 16 * i) * kKStride + kcol * 8]) = kr[i];
             __syncthreads();
-            if (ti + 1 < ntiles) issue_loads(ti + 1);
+            if (ti + 1 < ntiles) {
+                issue_loads(ti + 1);
+                if (PAGED && ti + 2 < ntiles) fetch_pages(ti + 2);
+            }
 
             float16_t acc[kGroupSize];
 #pragma unroll
@@ -433,9 +494,17 @@ __global__ __launch_bounds__(kThreads) void prefill_aggregate_kernel(PrefillPara
 hipError_t launch_prefill_attn(const PrefillParams& p, bool reuse, bool with_v, int nqb,
                                hipStream_t stream) {
     const int qt = 32 * nqb;
-    dim3 grid((p.L + qt - 1) / qt, kGroups, p.B), block(kThreads);
-    if (reuse) {
-        hipLaunchKernelGGL((prefill_attn_kernel_q32<true, true>), grid, block, 0, stream, p);
+    const bool paged = p.block_table != nullptr;
+    dim3 grid((p.Lq + qt - 1) / qt, kGroups, p.B), block(kThreads);
+    if (paged) {
+        if (reuse)
+            hipLaunchKernelGGL((prefill_attn_kernel_q32<true, true, true>), grid, block, 0, stream, p);
+        else if (with_v)
+            hipLaunchKernelGGL((prefill_attn_kernel_q32<false, true, true>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((prefill_attn_kernel_q32<false, false, true>), grid, block, 0, stream, p);
+    } else if (reuse) {
+        hipLaunchKernelGGL((prefill_attn_kernel_q32<true, true, false>), grid, block, 0, stream, p);
     } else if (nqb == 2) {
         if (with_v)
             hipLaunchKernelGGL((prefill_attn_kernel_q64<true>), grid, block, 0, stream, p);
@@ -443,16 +512,43 @@ hipError_t launch_prefill_attn(const PrefillParams& p, bool reuse, bool with_v, 
             hipLaunchKernelGGL((prefill_attn_kernel_q64<false>), grid, block, 0, stream, p);
     } else {
         if (with_v)
-            hipLaunchKernelGGL((prefill_attn_kernel_q32<false, true>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((prefill_attn_kernel_q32<false, true, false>), grid, block, 0, stream, p);
         else
-            hipLaunchKernelGGL((prefill_attn_kernel_q32<false, false>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((prefill_attn_kernel_q32<false, false, false>), grid, block, 0, stream, p);
     }
     return hipGetLastError();
 }
 
 hipError_t launch_prefill_aggregate(const PrefillParams& p, hipStream_t stream) {
     dim3 grid(p.T, kGroups, p.B), block(kThreads);
-    hipLaunchKernelGGL(prefill_aggregate_kernel, grid, block, 0, stream, p);
+    if (p.block_table)
+        hipLaunchKernelGGL(prefill_aggregate_kernel<true>, grid, block, 0, stream, p);
+    else
+        hipLaunchKernelGGL(prefill_aggregate_kernel<false>, grid, block, 0, stream, p);
+    return hipGetLastError();
+}
+
+// idx[i] (token position) -> physical row of the paged cache, in place or to another buffer.
+__global__ void translate_indices_kernel(const int* __restrict__ idx, int* __restrict__ out,
+                                         const int* __restrict__ block_table, long long per_seq,
+                                         int max_pages, int page_shift, int L) {
+    const int b = blockIdx.y;
+    const int* bt = block_table + (long long)b * max_pages;
+    const int mask = (1 << page_shift) - 1;
+    for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < per_seq;
+         i += (long long)gridDim.x * blockDim.x) {
+        const int tok = max(0, min(idx[b * per_seq + i], L - 1));
+        out[b * per_seq + i] = (bt[tok >> page_shift] << page_shift) + (tok & mask);
+    }
+}
+
+hipError_t launch_translate_indices(const int* idx, int* out, const int* block_table, int B,
+                                    long long per_seq, int max_pages, int page_shift, int L,
+                                    hipStream_t stream) {
+    if (per_seq <= 0 || B <= 0) return hipSuccess;
+    const int blocks = (int)std::min<long long>((per_seq + 255) / 256, 4096);
+    hipLaunchKernelGGL(translate_indices_kernel, dim3(blocks, B), dim3(256), 0, stream, idx, out,
+                       block_table, per_seq, max_pages, page_shift, L);
     return hipGetLastError();
 }
 

@@ -318,6 +318,84 @@ def paged_kv_append(K_pages, V_pages, k_new, v_new, start_pos, block_table, page
         B, n_new, block_table.shape[1], page_size, st, _stream()))
 
 
+# ------------------------------------------- chunked prefill over the paged cache
+def _chunk_args(Q, K_pages, block_table, q_start: int, page_size: int):
+    _req(Q, torch.float16, "Q", False); _req(K_pages, torch.float16, "K_pages")
+    _req(block_table, torch.int32, "block_table")
+    if K_pages.dim() != 4 or K_pages.shape[1] != page_size or tuple(K_pages.shape[2:]) != (G, D):
+        raise KascadeError(f"pages must be [num_pages,{page_size},{G},{D}]")
+    if q_start % TILE:
+        raise KascadeError(f"q_start must be a multiple of {TILE}")
+    return Q.shape[0], Q.shape[1], _blhd_strides(Q, "Q")
+
+
+def prefill_chunk_dense(Q, K_pages, V_pages, block_table, q_start: int, page_size: int = 16,
+                        with_output: bool = True) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Dense causal attention of a chunk's queries (global positions q_start..q_start+Lq-1) over
+    cache positions [0, q_start+Lq): the chunked form of ``prefill_recomp0_kernel`` /
+    ``prefill_recomp1_kernel`` (EfficientKascadeStrategy.py:78, 80).  Returns (log_sum, O);
+    O is None without with_output."""
+    lib = _lib.init()
+    B, Lq, qs = _chunk_args(Q, K_pages, block_table, q_start, page_size)
+    log_sum = torch.empty(B, Lq, H, device=Q.device, dtype=torch.float32)
+    out = torch.empty(B, Lq, H, D, device=Q.device, dtype=torch.float16) if with_output else None
+    if with_output:
+        _req(V_pages, torch.float16, "V_pages")
+    _lib.check(lib.kascade_prefill_chunk_dense_call(
+        _ptr(Q), _ptr(K_pages), _ptr(V_pages) if with_output else None, _ptr(log_sum), _ptr(out), B,
+        q_start, Lq, qs, _ptr(block_table), block_table.shape[1], page_size, K_pages.shape[0],
+        1 if with_output else 0, _stream()))
+    return log_sum, out
+
+
+def prefill_chunk_aggregate(Q, K_pages, log_sum, scores, block_table, q_start: int,
+                            page_size: int = 16, fill_invalid: bool = False) -> None:
+    """Chunked ``aggregate_kernel`` (EfficientKascadeStrategy.py:81): scores
+    [B,G,ceil(Lq/32),q_start+Lq] fp16, row t valid for keys < q_start + 32 t."""
+    lib = _lib.init()
+    B, Lq, qs = _chunk_args(Q, K_pages, block_table, q_start, page_size)
+    _req(log_sum, torch.float32, "log_sum"); _req(scores, torch.float16, "scores")
+    T = (Lq + TILE - 1) // TILE
+    if tuple(scores.shape) != (B, G, T, q_start + Lq) or tuple(log_sum.shape) != (B, Lq, H):
+        raise KascadeError("scores must be [B,G,ceil(Lq/32),q_start+Lq] and log_sum [B,Lq,H]")
+    _lib.check(lib.kascade_prefill_chunk_aggregate_call(
+        _ptr(Q), _ptr(K_pages), _ptr(log_sum), _ptr(scores), B, q_start, Lq, qs, _ptr(block_table),
+        block_table.shape[1], page_size, K_pages.shape[0], 1 if fill_invalid else 0, _stream()))
+
+
+def translate_indices(token_idx, block_table, kv_len: int, page_size: int = 16, out=None):
+    """Token positions [B, ...] -> rows of the paged cache (block_table[b, t // page] * page +
+    t % page), what the chunked reuse kernel gathers from."""
+    lib = _lib.init()
+    _req(token_idx, torch.int32, "token_idx"); _req(block_table, torch.int32, "block_table")
+    B = token_idx.shape[0]
+    if out is None:
+        out = torch.empty_like(token_idx)
+    _lib.check(lib.kascade_translate_indices_call(
+        _ptr(token_idx), _ptr(out), _ptr(block_table), B, token_idx.numel() // B,
+        block_table.shape[1], page_size, kv_len, _stream()))
+    return out
+
+
+def prefill_chunk_reuse(Q, K_pages, V_pages, physical_rows, head_mapping, topk_percent,
+                        rolling: bool, block_table, q_start: int, page_size: int = 16) -> torch.Tensor:
+    """Chunked ``prefill_reuse_kernel`` (EfficientKascadeStrategy.py:92, 97): physical_rows
+    [B,G,ceil(Lq/32),max_topk] comes from ``translate_indices``."""
+    lib = _lib.init()
+    B, Lq, qs = _chunk_args(Q, K_pages, block_table, q_start, page_size)
+    _req(V_pages, torch.float16, "V_pages")
+    _req(physical_rows, torch.int32, "physical_rows"); _req(head_mapping, torch.int32, "head_mapping")
+    T = (Lq + TILE - 1) // TILE
+    if tuple(physical_rows.shape[:3]) != (B, G, T):
+        raise KascadeError("physical_rows must be [B,G,ceil(Lq/32),max_topk]")
+    out = torch.empty(B, Lq, H, D, device=Q.device, dtype=torch.float16)
+    _lib.check(lib.kascade_prefill_chunk_reuse_call(
+        _ptr(Q), _ptr(K_pages), _ptr(V_pages), _ptr(physical_rows), _ptr(head_mapping),
+        float(topk_percent), _ptr(out), B, q_start, Lq, physical_rows.shape[-1], 1 if rolling else 0,
+        qs, _ptr(block_table), block_table.shape[1], page_size, K_pages.shape[0], _stream()))
+    return out
+
+
 # ------------------------------------------------- benchmark / correctness glue
 def prefill_full_kernel(Q, K, V, topk, tile_size=TILE, layer=0, topk_percent=10, rolling=False,
                         fill_invalid=True):

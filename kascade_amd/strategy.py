@@ -17,7 +17,8 @@ sort; the decode split count adapts to the device instead of the fixed 8.
 
 ``PagedKascadeDecoder`` is the paged-cache decode backend (block table, per
 sequence lengths) with the reference's kvcache call order
-(recompute_kascade_gqa_decode_with_kvcache.py:368-377).
+(recompute_kascade_gqa_decode_with_kvcache.py:368-377).  ``PagedKascadePrefill`` is
+the chunked-prefill backend over the same paged cache.
 """
 from __future__ import annotations
 
@@ -295,3 +296,85 @@ class PagedKascadeDecoder:
         if layer in self.recompute_layers:
             return self.anchor(layer, q, k_pages, v_pages, block_table, seqlens, max_len, ragged)
         return self.reuse(layer, q, k_pages, v_pages, block_table, seqlens)
+
+
+class PagedKascadePrefill:
+    """Chunked prefill backend over the paged cache: a prompt arrives in 32-aligned chunks, each
+    chunk's K/V are appended to the cache (``kernels.paged_kv_append``) and its queries then
+    attend to every cached position.  Per chunk the layer sequence is the reference's prefill
+    sequence (EfficientKascadeStrategy.py:72-98): an anchor layer runs the log-sum pass (dense
+    output on layer 0), pools tile scores, selects each tile's top-k and, on layers > 0, runs
+    its own sparse pass with the identity head map; reuse layers gather rows
+    head_mapping[layer] of the last anchor's indices.  A prompt processed this way gives the
+    rows a whole-prompt call gives."""
+
+    def __init__(self, k: float, head_mapping: List[List[int]], recompute_layers: Sequence[int],
+                 page_size: int = 16, rolling_prefill: bool = True, device="cuda"):
+        self.k = k
+        self.page_size = page_size
+        self.rolling_prefill = rolling_prefill
+        self.recompute_layers = list(recompute_layers)
+        self.device = torch.device(device)
+        self._hm = {None: torch.arange(G, device=self.device, dtype=torch.int32)}
+        for l, row in enumerate(head_mapping):
+            self._hm[l] = torch.tensor(row, device=self.device, dtype=torch.int32)
+        self._rows_to_reuse = None      # physical rows [B,G,T,width] of the last anchor
+        self._topk_to_reuse = None      # the same selection as token positions
+        self._budget_cache = {}
+        self._scores = None
+
+    def _tile_budgets(self, q_start: int, Lq: int, width: int):
+        key = (q_start, Lq, width)
+        hit = self._budget_cache.get(key)
+        if hit is None:
+            Lk = q_start + Lq
+            T = (Lq + TILE - 1) // TILE
+            valid = [q_start + TILE * t for t in range(T)]
+            if self.rolling_prefill and Lk > budgets.CHUNK:
+                nsel = [min(budgets.rolling_budget(s, self.k), width) for s in valid]
+            else:
+                nsel = [width] * T
+            hit = (torch.tensor(valid, dtype=torch.int32, device=self.device),
+                   torch.tensor(nsel, dtype=torch.int32, device=self.device))
+            self._budget_cache[key] = hit
+        return hit
+
+    def _score_buffer(self, B, T, Lk):
+        n = B * G * T * Lk
+        if self._scores is None or self._scores.numel() < n:
+            self._scores = torch.empty(n, device=self.device, dtype=torch.float16)
+        return self._scores[:n].view(B, G, T, Lk)
+
+    def anchor(self, layer, q, k_pages, v_pages, block_table, q_start: int):
+        B, Lq = q.shape[:2]
+        Lk = q_start + Lq
+        T = (Lq + TILE - 1) // TILE
+        width = budgets.topk_width(Lk, self.k)
+        log_sum, o = kernels.prefill_chunk_dense(q, k_pages, v_pages, block_table, q_start,
+                                                 self.page_size, with_output=(layer == 0))
+        scores = self._score_buffer(B, T, Lk)
+        kernels.prefill_chunk_aggregate(q, k_pages, log_sum, scores, block_table, q_start, self.page_size)
+        valid, nsel = self._tile_budgets(q_start, Lq, width)
+        self._topk_to_reuse = kernels.topk_indices(scores, width, valid_len=valid, n_sel=nsel)
+        self._rows_to_reuse = kernels.translate_indices(self._topk_to_reuse, block_table, Lk, self.page_size)
+        if layer != 0:
+            o = self._reuse(q, k_pages, v_pages, block_table, q_start, self._hm[None])
+        return o
+
+    def _reuse(self, q, k_pages, v_pages, block_table, q_start, hm):
+        return kernels.prefill_chunk_reuse(q, k_pages, v_pages, self._rows_to_reuse, hm, float(self.k),
+                                           self.rolling_prefill, block_table, q_start, self.page_size)
+
+    def reuse(self, layer, q, k_pages, v_pages, block_table, q_start: int):
+        if self._rows_to_reuse is None:
+            raise KascadeError("reuse layer called before any anchor layer")
+        return self._reuse(q, k_pages, v_pages, block_table, q_start, self._hm[layer])
+
+    def dense(self, q, k_pages, v_pages, block_table, q_start: int):
+        return kernels.prefill_chunk_dense(q, k_pages, v_pages, block_table, q_start, self.page_size)[1]
+
+    def forward(self, layer, q, k_pages, v_pages, block_table, q_start: int):
+        """q [B,Lq,H,D] at global positions q_start.. (K/V of the chunk already in the cache)."""
+        if layer in self.recompute_layers:
+            return self.anchor(layer, q, k_pages, v_pages, block_table, q_start)
+        return self.reuse(layer, q, k_pages, v_pages, block_table, q_start)
