@@ -117,6 +117,7 @@ def main():
     ap.add_argument("--seq-len", type=int, default=32768)
     ap.add_argument("--skip-decode", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--skip-stack", action="store_true", help="skip the 36-layer chunked-prefill + decode stack")
     ap.add_argument("--decode-only", action="store_true", help="skip the per-kernel prefill section")
     ap.add_argument("--kernel", choices=sorted(SINGLE_KERNELS), default=None,
                     help="profiling mode: run only this kernel --iters times on its benchmark workload")
@@ -311,6 +312,82 @@ def main():
             del caches, c0, dec
             torch.cuda.empty_cache()
 
+    # ------------------------------------------------- 36-layer stack, chunked prefill + decode
+    stack_res = {}
+    if not args.skip_stack:
+        from kascade_amd.stack import KascadeAttentionStack
+        n_layers, anchors = 36, [0, 2, 8, 13, 14]
+        prompt, chunk, steps = 16384, 2048, 256
+        n_tok = prompt + steps
+        log(f"[bench] stack: {n_layers} layers, prompt {prompt} in chunks of {chunk}, {steps} decode steps")
+        maps = [list(range(G)) if l in anchors else workloads.random_head_mapping(500 + l) for l in range(n_layers)]
+        base = workloads.prefill_inputs(1, n_tok, seed=4, device=dev)
+        qs, ks, vs = [], [], []
+        for l in range(n_layers):
+            if l in anchors:
+                qs.append(workloads.perturb(base.q, seed=600 + l)); ks.append(workloads.perturb(base.k, seed=700 + l))
+            else:   # correlated with the preceding anchor
+                a = max(x for x in anchors if x < l)
+                qs.append(workloads.perturb(qs[a], seed=600 + l)); ks.append(workloads.perturb(ks[a], seed=700 + l))
+            vs.append(workloads.gaussian((1, n_tok, G, D), seed=800 + l, device=dev))
+        del base
+        dq = torch.stack([x[:, prompt:] for x in qs]).permute(2, 0, 1, 3, 4).contiguous()        # [steps,layers,1,H,D]
+        dk = torch.stack([x[:, prompt:] for x in ks]).permute(2, 0, 1, 3, 4).unsqueeze(3).contiguous()
+        dv = torch.stack([x[:, prompt:] for x in vs]).permute(2, 0, 1, 3, 4).unsqueeze(3).contiguous()
+        chunks = [([q[:, s:s + chunk] for q in qs], [k[:, s:s + chunk] for k in ks], [v[:, s:s + chunk] for v in vs])
+                  for s in range(0, prompt, chunk)]
+
+        def wall(fn):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) * 1e3
+
+        for name, dense in (("kascade", False), ("dense", True)):
+            st = KascadeAttentionStack(n_layers, anchors, maps, PCT, n_tok, batch=1, page_size=16,
+                                       rolling_prefill=True, device=dev, table_seed=2, dense=dense)
+
+            def run_prefill():
+                st.reset()
+                for cq, ck, cv in chunks:
+                    st.prefill_chunk(cq, ck, cv)
+
+            run_prefill()                                   # warm-up
+            t_pre = min(wall(run_prefill) for _ in range(3))
+
+            def run_decode_eager():
+                st.reset(prompt)
+                for s in range(steps):
+                    st.decode_step(dq[s], dk[s], dv[s])
+
+            def run_decode_graph():
+                st.reset(prompt)
+                for s in range(steps):
+                    st.graph_q.copy_(dq[s]); st.graph_k.copy_(dk[s]); st.graph_v.copy_(dv[s])
+                    st.replay_decode()
+
+            t_eager = wall(run_decode_eager)
+            st.reset(prompt)
+            st.capture_decode()
+            run_decode_graph()
+            t_graph = min(wall(run_decode_graph) for _ in range(2))
+            stack_res[name] = {"prefill_ms": round(t_pre, 2), "decode_ms_graph": round(t_graph, 2),
+                               "decode_ms_eager": round(t_eager, 2),
+                               "decode_us_per_step_per_layer": round(t_graph * 1e3 / steps / n_layers, 2),
+                               "us_per_token": round((t_pre + t_graph) * 1e3 / n_tok, 2)}
+            log(f"[bench] stack {name}: {stack_res[name]}")
+            del st
+            torch.cuda.empty_cache()
+        stack_res["speedup_prefill"] = round(stack_res["dense"]["prefill_ms"] / stack_res["kascade"]["prefill_ms"], 3)
+        stack_res["speedup_decode"] = round(stack_res["dense"]["decode_ms_graph"] / stack_res["kascade"]["decode_ms_graph"], 3)
+        stack_res["speedup_per_token"] = round(stack_res["dense"]["us_per_token"] / stack_res["kascade"]["us_per_token"], 3)
+        stack_res["workload"] = ("configs[4]: 36 attention layers, anchors {0,2,8,13,14}, 16384-token prompt in 2048-token "
+                                 "chunks over a paged cache (page 16), then 256 decode steps replayed as one HIP graph "
+                                 "per step; attention only, per-layer Q/K/V synthetic")
+        del qs, ks, vs, dq, dk, dv, chunks
+        torch.cuda.empty_cache()
+
     # ------------------------------------------------------------------ CPU baseline (oracle)
     cpu = None
     if not args.skip_cpu:
@@ -363,7 +440,8 @@ def main():
                                "32 layers (1 anchor-0, 4 anchor, 27 reuse)",
                    "seq_len": L, "layers_per_step": N_LAYERS,
                    "baseline_note": "vs_baseline = value / 6.42 ms, the reference's published H100 figure"},
-        "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "decode": decode, "kernels": kern,
+        "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "decode": decode, "stack": stack_res,
+        "kernels": kern,
     }
     print(json.dumps(out), flush=True)
 

@@ -372,29 +372,65 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
 }
 
 // Merge the per-split log-sums (and partial outputs) of one (b, head).
-// grid (H, B), 128 threads = one per output dimension.
+// grid (H, B), 128 threads: the splits are spread over the threads for the two reductions,
+// then thread d accumulates output dimension d with the weights staged in LDS.
+constexpr int kCombineLds = 512;   // splits whose weights fit the LDS buffer
+
+__device__ __forceinline__ float combine_reduce(float x, bool is_max, float* s_red) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+        const float y = __shfl_xor(x, o);
+        x = is_max ? fmaxf(x, y) : x + y;
+    }
+    __syncthreads();   // s_red may still be read from the previous reduction
+    if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = x;
+    __syncthreads();
+    return is_max ? fmaxf(s_red[0], s_red[1]) : s_red[0] + s_red[1];
+}
+
 template <bool WITH_V>
 __global__ __launch_bounds__(128) void decode_combine_kernel(const float* __restrict__ glse,
                                                             const float* __restrict__ opart,
                                                             half_t* __restrict__ out,
                                                             float* __restrict__ row_sums,
                                                             int num_split) {
+    __shared__ float s_w[kCombineLds];
+    __shared__ float s_red[2];
     const int h = blockIdx.x;
     const int b = blockIdx.y;
     const int d = threadIdx.x;
     const size_t base = ((size_t)b * kHeads + h) * num_split;
     float mx = -INFINITY;
-    for (int s = 0; s < num_split; ++s) mx = fmaxf(mx, glse[base + s]);
+    for (int s = d; s < num_split; s += 128) mx = fmaxf(mx, glse[base + s]);
+    mx = combine_reduce(mx, true, s_red);
     const float mref = (mx == -INFINITY) ? 0.f : mx;
     float sum = 0.f;
-    for (int s = 0; s < num_split; ++s) sum += fast_exp2(glse[base + s] - mref);
+    for (int s = d; s < num_split; s += 128) sum += fast_exp2(glse[base + s] - mref);
+    sum = combine_reduce(sum, false, s_red);
     const float lse = (sum > 0.f) ? fast_log2(sum) + mref : -INFINITY;
     if (row_sums && d == 0) row_sums[(size_t)b * kHeads + h] = lse;
     if (WITH_V) {
+        const float lref = (lse == -INFINITY) ? 0.f : lse;
+        for (int s = d; s < min(num_split, kCombineLds); s += 128) s_w[s] = fast_exp2(glse[base + s] - lref);
+        __syncthreads();
+        const float* op = opart + base * kDim + d;
         float o = 0.f;
-        for (int s = 0; s < num_split; ++s) {
-            float w = fast_exp2(glse[base + s] - ((lse == -INFINITY) ? 0.f : lse));
-            if (w > 0.f) o += w * opart[(base + s) * kDim + d];
+        int s = 0;
+        // a split that saw no rows leaves its partial output unwritten: select, never multiply
+        for (; s + 8 <= min(num_split, kCombineLds); s += 8) {
+            float x[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = op[(size_t)(s + e) * kDim];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float w = s_w[s + e];
+                o += (w > 0.f) ? w * x[e] : 0.f;
+            }
+        }
+        for (; s < num_split; ++s) {
+            const float w = (s < kCombineLds) ? s_w[s] : fast_exp2(glse[base + s] - lref);
+            const float x = op[(size_t)s * kDim];
+            o += (w > 0.f) ? w * x : 0.f;
         }
         out[((size_t)b * kHeads + h) * kDim + d] = (half_t)o;
     }

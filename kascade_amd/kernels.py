@@ -57,12 +57,26 @@ def default_num_split(total_rows: int, max_rows: int, wgs_per_cu: int = 2, min_r
     cus = _lib.init().kascade_device_cu_count() or 256
     target_wgs = wgs_per_cu * cus
     rows_per_split = max(min_rows, total_rows / target_wgs)
+    if total_rows / rows_per_split < cus:
+        # small launch (short lists, small batch): latency, not set-up, is what counts, so
+        # spread down to 128 rows per workgroup to put one workgroup on every compute unit
+        rows_per_split = max(min(128, min_rows), total_rows / cus)
     # round to nearest: one workgroup more than a whole number per compute unit costs a
     # full extra wave of workgroups on a few units (tail), one fewer costs nothing
     return int(max(1, min(256, round(max_rows / rows_per_split))))
 
 
 # ---------------------------------------------------------------- decode
+def _out_buffer(out, B, device) -> torch.Tensor:
+    """The caller's [B,H,D] fp16 output buffer, or a fresh one."""
+    if out is None:
+        return torch.empty(B, H, D, device=device, dtype=torch.float16)
+    _req(out, torch.float16, "out")
+    if tuple(out.shape) != (B, H, D):
+        raise KascadeError(f"out must be [{B},{H},{D}]")
+    return out
+
+
 def decode_reuse(Q, K, V, topk_indices, head_mapping, glse, Output_partial) -> torch.Tensor:
     """``decode_reuse_kernel(Q, K, V, topk_indices, head_mapping, glse, Output_partial) -> O``
     (out_idx=[7]; EfficientKascadeStrategy.py:30-38, 113, 122).  Contiguous cache
@@ -86,7 +100,7 @@ def decode_reuse(Q, K, V, topk_indices, head_mapping, glse, Output_partial) -> t
 
 
 def decode_reuse_paged(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_percent, glse,
-                       Output_partial, block_table=None, page_size: int = 16) -> torch.Tensor:
+                       Output_partial, block_table=None, page_size: int = 16, out=None) -> torch.Tensor:
     """``reuse kvcache kernel(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_percent,
     glse, Output_partial) -> O`` (out_idx=[9]; reuse_kascade_gqa_decode_with_kvcache.py:160-173)
     with an optional block table.  Without one K,V are the padded [B,maxL,G,D] cache;
@@ -104,7 +118,7 @@ def decode_reuse_paged(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_
         stride_tokens, max_pages = 0, block_table.shape[1]
     else:
         stride_tokens, max_pages = K.shape[1], 0
-    out = torch.empty(B, H, D, device=Q.device, dtype=torch.float16)
+    out = _out_buffer(out, B, Q.device)
     _lib.check(lib.kascade_decode_reuse_paged_call(
         _ptr(Q), _ptr(K), _ptr(V), _ptr(cache_seqlens), _ptr(topk_indices), _ptr(head_mapping),
         float(topk_percent), _ptr(glse), _ptr(Output_partial), _ptr(out), B, stride_tokens,
@@ -113,7 +127,7 @@ def decode_reuse_paged(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_
 
 
 def decode_dense_paged(Q, K, V, cache_seqlens, glse, Output_partial, block_table=None,
-                       page_size: int = 16, kv_len: Optional[int] = None) -> torch.Tensor:
+                       page_size: int = 16, kv_len: Optional[int] = None, out=None) -> torch.Tensor:
     """Dense split-K decode, the baseline of gqa_decode.py / gqa_decode_with_kvcache.py:
     ``kernel(Q, K, V, [cache_seqlens,] glse, Output_partial) -> O``."""
     lib = _lib.init()
@@ -126,7 +140,7 @@ def decode_dense_paged(Q, K, V, cache_seqlens, glse, Output_partial, block_table
         stride_tokens, max_pages = (kv_len or 0), block_table.shape[1]
     else:
         stride_tokens, max_pages = K.shape[1], 0
-    out = torch.empty(B, H, D, device=Q.device, dtype=torch.float16)
+    out = _out_buffer(out, B, Q.device)
     _lib.check(lib.kascade_decode_dense_paged_call(
         _ptr(Q), _ptr(K), _ptr(V), _ptr(cache_seqlens), _ptr(glse), _ptr(Output_partial), _ptr(out),
         B, stride_tokens, ns, _ptr(block_table), max_pages, page_size, _stream()))
@@ -135,7 +149,7 @@ def decode_dense_paged(Q, K, V, cache_seqlens, glse, Output_partial, block_table
 
 def decode_recompute(Q, K, V, glse, Output_partial, row_sums, scores, layer: int,
                      cache_seqlens=None, block_table=None, page_size: int = 16,
-                     kv_len: Optional[int] = None) -> Tuple[Optional[torch.Tensor], torch.Tensor]:
+                     kv_len: Optional[int] = None, out=None) -> Tuple[Optional[torch.Tensor], torch.Tensor]:
     """``decode_recomp{0,1}_kernel(Q, K, V, glse, Output_partial, row_sums, scores) -> (O, agg)``
     (out_idx=[7,8]; EfficientKascadeStrategy.py:24-28, 107-110) and its kvcache form
     (recompute_kascade_gqa_decode_with_kvcache.py:302-333).  ``scores`` is fp32 scratch
@@ -154,7 +168,7 @@ def decode_recompute(Q, K, V, glse, Output_partial, row_sums, scores, layer: int
         stride_tokens, max_pages = (kv_len or 0), block_table.shape[1]
     else:
         stride_tokens, max_pages = K.shape[1], 0
-    out = torch.empty(B, H, D, device=Q.device, dtype=torch.float16) if with_out else None
+    out = _out_buffer(out, B, Q.device) if with_out else None
     agg = torch.empty(B, G, stride, device=Q.device, dtype=torch.float16)
     _lib.check(lib.kascade_decode_recompute_paged_call(
         _ptr(Q), _ptr(K), _ptr(V), _ptr(cache_seqlens), _ptr(glse), _ptr(Output_partial),

@@ -1,0 +1,146 @@
+"""A stack of attention layers over one paged KV cache per layer: chunked prefill of a prompt,
+then token-by-token decode, with the anchor / reuse layer schedule of the ``efficient_kascade``
+strategy (EfficientKascadeStrategy.py:126-161 decides per call between the four kernels; here
+the same decision is made per layer of a chunk or of a decode step).
+
+Only attention runs here: the caller supplies each layer's Q and the new K/V rows (in a model
+they come from the layer's projections).  Every layer has its own pages; all layers share the
+sequence's block table, so an anchor layer's selection, translated once to cache rows, serves
+the reuse layers that follow it.
+
+A decode step is a fixed launch sequence whose only varying inputs live in device memory (the
+new rows and the sequence lengths), so it can be captured once into a HIP graph and replayed:
+at short contexts the step is launch-bound and the graph removes the host from the loop.
+"""
+from __future__ import annotations
+
+import math
+from typing import List, Optional, Sequence
+
+import torch
+
+from . import kernels
+from ._lib import KascadeError
+from .strategy import PagedKascadeDecoder, PagedKascadePrefill
+
+H, G, D, TILE = 32, 8, 128, 32
+
+
+class KascadeAttentionStack:
+    def __init__(self, num_layers: int, recompute_layers: Sequence[int], head_mapping: List[List[int]],
+                 k: float, max_seqlen: int, batch: int = 1, page_size: int = 16,
+                 rolling_prefill: bool = True, device="cuda", table_seed: int = 0,
+                 dense: bool = False):
+        """dense=True runs every layer as dense attention over the same caches (the baseline)."""
+        if 0 not in recompute_layers and not dense:
+            raise KascadeError("layer 0 must be an anchor layer")
+        self.num_layers, self.batch, self.page_size = num_layers, batch, page_size
+        self.recompute_layers = list(recompute_layers)
+        self.dense_only = dense
+        self.device = torch.device(device)
+        self.max_seqlen = max_seqlen
+        pages_per_seq = math.ceil(max_seqlen / page_size)
+        n_pages = batch * pages_per_seq
+        gen = torch.Generator().manual_seed(table_seed)
+        self.block_table = torch.randperm(n_pages, generator=gen).to(torch.int32).view(batch, pages_per_seq) \
+            .to(self.device)
+        self.k_pages = [torch.zeros(n_pages, page_size, G, D, device=self.device, dtype=torch.float16)
+                        for _ in range(num_layers)]
+        self.v_pages = [torch.zeros_like(p) for p in self.k_pages]
+        self.length = 0                                                 # host copy of the common length
+        self.seqlens = torch.zeros(batch, device=self.device, dtype=torch.int32)
+        self._next = torch.zeros_like(self.seqlens)                     # lengths after the append
+        self.prefill = PagedKascadePrefill(k, head_mapping, recompute_layers, page_size, rolling_prefill,
+                                           self.device)
+        self.decoder = PagedKascadeDecoder(k, head_mapping, recompute_layers, batch, max_seqlen, page_size,
+                                           self.device)
+        self._graph = None
+
+    def reset(self, length: int = 0):
+        """Forget everything cached beyond ``length`` tokens (the pages keep their contents)."""
+        self.length = length
+        self.seqlens.fill_(length)
+
+    # ------------------------------------------------------------------ prefill
+    def prefill_chunk(self, q: Sequence[torch.Tensor], k_new: Sequence[torch.Tensor],
+                      v_new: Sequence[torch.Tensor]) -> List[torch.Tensor]:
+        """One chunk through all layers.  q[l] [B,Lq,H,D], k_new[l]/v_new[l] [B,Lq,G,D]; the chunk
+        starts at the current length, which must be a multiple of 32.  Returns O[l] [B,Lq,H,D]."""
+        Lq = q[0].shape[1]
+        q_start = self.length
+        if q_start % TILE:
+            raise KascadeError("a prefill chunk must start at a multiple of 32 tokens")
+        if q_start + Lq > self.max_seqlen:
+            raise KascadeError("chunk exceeds max_seqlen")
+        outs = []
+        for l in range(self.num_layers):
+            kernels.paged_kv_append(self.k_pages[l], self.v_pages[l], k_new[l], v_new[l], self.seqlens,
+                                    self.block_table, self.page_size)
+            if self.dense_only:
+                outs.append(self.prefill.dense(q[l], self.k_pages[l], self.v_pages[l], self.block_table, q_start))
+            else:
+                outs.append(self.prefill.forward(l, q[l], self.k_pages[l], self.v_pages[l], self.block_table,
+                                                 q_start))
+        self.length += Lq
+        self.seqlens += Lq
+        return outs
+
+    # ------------------------------------------------------------------- decode
+    def _decode_layers(self, q, k_new, v_new, out):
+        """The launch sequence of one decode step; lengths are read from device memory."""
+        torch.add(self.seqlens, 1, out=self._next)
+        for l in range(self.num_layers):
+            kernels.paged_kv_append(self.k_pages[l], self.v_pages[l], k_new[l], v_new[l], self.seqlens,
+                                    self.block_table, self.page_size)
+            if self.dense_only:
+                self.decoder.dense(q[l], self.k_pages[l], self.v_pages[l], self.block_table, self._next,
+                                   self.max_seqlen, out=out[l])
+            else:
+                self.decoder.forward(l, q[l], self.k_pages[l], self.v_pages[l], self.block_table,
+                                     self._next, self.max_seqlen, ragged=True, out=out[l])
+        self.seqlens.copy_(self._next)
+
+    def decode_step(self, q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor,
+                    out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """q [layers,B,H,D], k_new/v_new [layers,B,1,G,D] -> O [layers,B,H,D] (eager launches)."""
+        if self.length + 1 > self.max_seqlen:
+            raise KascadeError("decode step exceeds max_seqlen")
+        if out is None:
+            out = torch.empty(self.num_layers, self.batch, H, D, device=self.device, dtype=torch.float16)
+        self._decode_layers(q, k_new, v_new, out)
+        self.length += 1
+        return out
+
+    def capture_decode(self):
+        """Capture one decode step into a HIP graph over static input/output buffers
+        (``graph_q``, ``graph_k``, ``graph_v`` -> ``graph_out``).  The warm-up run before the
+        capture appends one (zero) token; the lengths are restored afterwards, so that slot is
+        simply overwritten by the first replay."""
+        n, B, dev = self.num_layers, self.batch, self.device
+        self.graph_q = torch.zeros(n, B, H, D, device=dev, dtype=torch.float16)
+        self.graph_k = torch.zeros(n, B, 1, G, D, device=dev, dtype=torch.float16)
+        self.graph_v = torch.zeros_like(self.graph_k)
+        self.graph_out = torch.zeros(n, B, H, D, device=dev, dtype=torch.float16)
+        if self.length + 1 > self.max_seqlen:
+            raise KascadeError("no room to capture a decode step")
+        saved = self.seqlens.clone()
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side):      # warm-up on the side stream: allocator and workspaces settle
+            self._decode_layers(self.graph_q, self.graph_k, self.graph_v, self.graph_out)
+            self.seqlens.copy_(saved)
+        torch.cuda.current_stream(dev).wait_stream(side)
+        torch.cuda.synchronize(dev)
+        self._graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self._graph):
+            self._decode_layers(self.graph_q, self.graph_k, self.graph_v, self.graph_out)
+
+    def replay_decode(self) -> torch.Tensor:
+        """Replay the captured step on the inputs currently in the static buffers."""
+        if self._graph is None:
+            raise KascadeError("capture_decode() first")
+        if self.length + 1 > self.max_seqlen:
+            raise KascadeError("decode step exceeds max_seqlen")
+        self._graph.replay()
+        self.length += 1
+        return self.graph_out

@@ -241,26 +241,26 @@ class PagedKascadeDecoder:
     def _scratch(self, B, ns):
         return self._glse[:B * H * ns].view(B, H, ns), self._part[:B * H * ns * D].view(B, H, ns, D)
 
-    def dense(self, q, k_pages, v_pages, block_table, seqlens, max_len: int):
+    def dense(self, q, k_pages, v_pages, block_table, seqlens, max_len: int, out=None):
         B = q.shape[0]
         glse, part = self._scratch(B, self.ns_dense)
         return kernels.decode_dense_paged(q, k_pages, v_pages, seqlens, glse, part, block_table,
-                                          self.page_size, kv_len=max_len)
+                                          self.page_size, kv_len=max_len, out=out)
 
     def anchor(self, layer, q, k_pages, v_pages, block_table, seqlens, max_len: int,
-               ragged: bool = True):
-        """Anchor layer: returns the attention output [B,H,D]; keeps indices for reuse layers."""
+               ragged: bool = True, out=None):
+        """Anchor layer: returns the attention output [B,H,D] (written to ``out`` when given);
+        keeps indices for reuse layers."""
         B = q.shape[0]
         stride = ((max_len + 7) // 8) * 8
         glse, part = self._scratch(B, self.ns_dense)
         scores = self._scores[:B * H * stride].view(B, H, stride)
         o, agg = kernels.decode_recompute(q, k_pages, v_pages, glse, part, self._row_sums[:B], scores, layer,
                                           cache_seqlens=seqlens, block_table=block_table,
-                                          page_size=self.page_size, kv_len=max_len)
+                                          page_size=self.page_size, kv_len=max_len, out=out)
         if ragged:
             width = budgets.decode_budget(max_len, self.k)
-            lens_rows = seqlens.repeat_interleave(G)
-            counts = self._decode_counts(seqlens).repeat_interleave(G)
+            lens_rows, counts = self._row_budgets(seqlens)
             self._topk_to_reuse = kernels.topk_indices(agg[:, :, :max_len], width, valid_len=lens_rows,
                                                        n_sel=counts, fill_value=0)
             self._pct = float(self.k)
@@ -269,8 +269,18 @@ class PagedKascadeDecoder:
             self._topk_to_reuse = kernels.topk_indices(agg[:, :, :max_len], width, fill_value=0)
             self._pct = 0.0
         if layer != 0:
-            o = self._reuse(q, k_pages, v_pages, block_table, seqlens, self._hm[None])
+            o = self._reuse(q, k_pages, v_pages, block_table, seqlens, self._hm[None], out)
         return o
+
+    def _row_budgets(self, seqlens: torch.Tensor):
+        """Per (sequence, KV head) row: valid length and selection count.  The anchors of one
+        decode step see the same lengths, so the tensors are kept until seqlens is written again
+        (a dozen tiny launches otherwise, as long as an anchor pass at short contexts)."""
+        key = (seqlens.data_ptr(), seqlens._version, seqlens.numel())
+        if self._counts is None or self._counts[0] != key:
+            self._counts = (key, seqlens.repeat_interleave(G),
+                            self._decode_counts(seqlens).repeat_interleave(G))
+        return self._counts[1], self._counts[2]
 
     def _decode_counts(self, seqlens: torch.Tensor) -> torch.Tensor:
         # 128*ceil(floor(k*len/100)/128) on the device, exact integer arithmetic for integer k
@@ -280,22 +290,23 @@ class PagedKascadeDecoder:
             fl = torch.floor(seqlens.to(torch.float64) * float(self.k) / 100.0).to(torch.int64)
         return (((fl + 127) // 128) * 128).to(torch.int32)
 
-    def _reuse(self, q, k_pages, v_pages, block_table, seqlens, hm):
+    def _reuse(self, q, k_pages, v_pages, block_table, seqlens, hm, out=None):
         B = q.shape[0]
         glse, part = self._scratch(B, self.ns_reuse)
         return kernels.decode_reuse_paged(q, k_pages, v_pages, seqlens, self._topk_to_reuse, hm, self._pct,
-                                          glse, part, block_table=block_table, page_size=self.page_size)
+                                          glse, part, block_table=block_table, page_size=self.page_size, out=out)
 
-    def reuse(self, layer, q, k_pages, v_pages, block_table, seqlens):
+    def reuse(self, layer, q, k_pages, v_pages, block_table, seqlens, out=None):
         """Reuse layer: attends to rows head_mapping[layer] of the last anchor's indices."""
         if self._topk_to_reuse is None:
             raise KascadeError("reuse layer called before any anchor layer")
-        return self._reuse(q, k_pages, v_pages, block_table, seqlens, self._hm[layer])
+        return self._reuse(q, k_pages, v_pages, block_table, seqlens, self._hm[layer], out)
 
-    def forward(self, layer, q, k_pages, v_pages, block_table, seqlens, max_len: int, ragged: bool = True):
+    def forward(self, layer, q, k_pages, v_pages, block_table, seqlens, max_len: int, ragged: bool = True,
+                out=None):
         if layer in self.recompute_layers:
-            return self.anchor(layer, q, k_pages, v_pages, block_table, seqlens, max_len, ragged)
-        return self.reuse(layer, q, k_pages, v_pages, block_table, seqlens)
+            return self.anchor(layer, q, k_pages, v_pages, block_table, seqlens, max_len, ragged, out)
+        return self.reuse(layer, q, k_pages, v_pages, block_table, seqlens, out)
 
 
 class PagedKascadePrefill:

@@ -93,7 +93,10 @@ def test_default_num_split_heuristic(monkeypatch):
     rps = -(-52480 // ns)
     wgs = sum(-(-n // rps) for n in (13184, 19712, 26240, 52480)) * 8
     assert 400 <= wgs <= 640
-    assert kernels.default_num_split(8 * 300, 300) == 1
+    # launches too small to fill the device spread down to 128 rows per workgroup
+    assert kernels.default_num_split(8 * 300, 300) == 2
+    assert kernels.default_num_split(8 * 1664, 1664) == 13
+    assert kernels.default_num_split(8 * 100, 100) == 1
 
 
 def test_workloads_are_seeded_and_shaped():
