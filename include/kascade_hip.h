@@ -53,6 +53,16 @@ int kascade_device_cu_count(void);
 
 /* ------------------------------------------------------------------ decode */
 
+/* Every decode call splits each (sequence, KV head) row list over num_split workgroups that
+ * write partial results (glse, Output_partial) and then merges them.  sync_counters selects
+ * how (no counterpart in the reference, which always launches a second kernel):
+ *   NULL      a second (combine) launch merges the splits;
+ *   non-NULL  [batch*8] i32 in device memory, zero before the first call: the last split
+ *             workgroup of each (sequence, KV head) to finish merges that pair's splits inside
+ *             the same launch and sets its counter back to zero, so the array can be handed
+ *             to the next call as it is.  One launch fewer per layer, which matters at short
+ *             contexts.  Calls that overlap in time on one device must not share an array. */
+
 /* Reuse-layer decode, contiguous cache.  Same argument list as the reference's
  * `call` of dynamic_alllen_reuse_cp_async_dim128_gsize4_heads32_groups8.cu:260
  * (DSL: reuse_kascade_gqa_decode.py:180-191) plus the split count that the
@@ -63,7 +73,8 @@ int kascade_device_cu_count(void);
 int kascade_decode_reuse_call(const kascade_half* Q, const kascade_half* K, const kascade_half* V,
                               const int32_t* topk_indices, const int32_t* head_mapping,
                               float* glse, float* Output_partial, kascade_half* Output,
-                              int batch, int kv_seqlen, int topk, int num_split, void* stream);
+                              int batch, int kv_seqlen, int topk, int num_split,
+                              int32_t* sync_counters, void* stream);
 
 /* Reuse-layer decode over a padded or paged cache with per-sequence lengths.
  * Argument order follows the reference's kvcache `call`
@@ -80,7 +91,8 @@ int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K
                                     float topk_percent, float* glse, float* Output_partial,
                                     kascade_half* Output, int batch, int kv_stride_tokens,
                                     int topk, int num_split, const int32_t* block_table,
-                                    int max_pages, int page_size, void* stream);
+                                    int max_pages, int page_size, int32_t* sync_counters,
+                                    void* stream);
 
 /* Dense split-K decode (the reference's TileLang dense baseline, gqa_decode.py:117-254 and
  * gqa_decode_with_kvcache.py:118-257), same cache conventions as above.
@@ -92,7 +104,7 @@ int kascade_decode_dense_paged_call(const kascade_half* Q, const kascade_half* K
                                     float* glse, float* Output_partial, kascade_half* Output,
                                     int batch, int kv_stride_tokens, int num_split,
                                     const int32_t* block_table, int max_pages, int page_size,
-                                    void* stream);
+                                    int32_t* sync_counters, void* stream);
 
 /* Anchor-layer decode: split QK^T (+PV when with_output != 0), log-sum merge and
  * pooled post-softmax scores.  Replaces the three launches of the reference's
@@ -111,7 +123,8 @@ int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_hal
                                         kascade_half* aggregated_scores, int batch,
                                         int kv_stride_tokens, int scores_stride, int num_split,
                                         int with_output, const int32_t* block_table,
-                                        int max_pages, int page_size, void* stream);
+                                        int max_pages, int page_size, int32_t* sync_counters,
+                                        void* stream);
 
 /* ------------------------------------------------------------------- top-k */
 

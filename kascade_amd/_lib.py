@@ -36,12 +36,13 @@ SIGNATURES = {
     "kascade_get_last_error": (C.c_char_p, []),
     "kascade_abi_version": (_I, []),
     "kascade_device_cu_count": (_I, []),
-    "kascade_decode_reuse_call": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "kascade_decode_reuse_call": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _P]),
     "kascade_decode_reuse_paged_call": (_I, [_P, _P, _P, _P, _P, _P, _F, _P, _P, _P, _I, _I, _I, _I,
-                                             _P, _I, _I, _P]),
-    "kascade_decode_dense_paged_call": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _I, _I, _P]),
+                                             _P, _I, _I, _P, _P]),
+    "kascade_decode_dense_paged_call": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _I, _I, _P,
+                                             _P]),
     "kascade_decode_recompute_paged_call": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I,
-                                                 _I, _I, _P, _I, _I, _P]),
+                                                 _I, _I, _P, _I, _I, _P, _P]),
     "kascade_topk_workspace_bytes": (_L, [_I, _L]),
     "kascade_topk_call": (_I, [_P, _P, _I, _L, _I, _P, _P, _I, _I, _I, _P, _P]),
     "kascade_prefill_dense_call": (_I, [_P, _P, _P, _P, _P, _I, _I, Strides, Strides, _I, _P]),

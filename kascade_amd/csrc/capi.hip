@@ -75,7 +75,7 @@ int check_paging(const int32_t* block_table, int max_pages, int page_size, int* 
 
 extern "C" {
 
-int kascade_abi_version(void) { return 1; }
+int kascade_abi_version(void) { return 2; }
 
 const char* kascade_get_last_error(void) { return g_err; }
 
@@ -95,10 +95,11 @@ int kascade_init(void) {
 int kascade_decode_reuse_call(const kascade_half* Q, const kascade_half* K, const kascade_half* V,
                               const int32_t* topk_indices, const int32_t* head_mapping,
                               float* glse, float* Output_partial, kascade_half* Output, int batch,
-                              int kv_seqlen, int topk, int num_split, void* stream) {
+                              int kv_seqlen, int topk, int num_split, int32_t* sync_counters,
+                              void* stream) {
     return kascade_decode_reuse_paged_call(Q, K, V, nullptr, topk_indices, head_mapping, 0.f, glse,
                                            Output_partial, Output, batch, kv_seqlen, topk,
-                                           num_split, nullptr, 0, 1, stream);
+                                           num_split, nullptr, 0, 1, sync_counters, stream);
 }
 
 int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K,
@@ -107,7 +108,8 @@ int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K
                                     float topk_percent, float* glse, float* Output_partial,
                                     kascade_half* Output, int batch, int kv_stride_tokens,
                                     int topk, int num_split, const int32_t* block_table,
-                                    int max_pages, int page_size, void* stream) {
+                                    int max_pages, int page_size, int32_t* sync_counters,
+                                    void* stream) {
     REQUIRE(Q && K && V && topk_indices && head_mapping && glse && Output_partial && Output,
             "decode_reuse: null pointer argument");
     REQUIRE(batch > 0 && topk > 0 && num_split > 0, "decode_reuse: batch, topk, num_split must be > 0");
@@ -125,8 +127,10 @@ int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K
     p.topk = topk; p.topk_percent = topk_percent; p.scores_stride = 0; p.num_split = num_split;
     p.rows_per_split = rows_per_split(topk, num_split);
     p.B = batch;
+    p.counters = sync_counters; p.out = H(Output);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (check_hip(launch_decode_split(p, true, true, false, s), "decode_reuse split")) return -1;
+    if (sync_counters) return 0;   // the split kernel's last workgroups have combined
     return check_hip(launch_decode_combine(glse, Output_partial, H(Output), nullptr, batch,
                                            num_split, true, s), "decode_reuse combine");
 }
@@ -136,7 +140,7 @@ int kascade_decode_dense_paged_call(const kascade_half* Q, const kascade_half* K
                                     float* glse, float* Output_partial, kascade_half* Output,
                                     int batch, int kv_stride_tokens, int num_split,
                                     const int32_t* block_table, int max_pages, int page_size,
-                                    void* stream) {
+                                    int32_t* sync_counters, void* stream) {
     REQUIRE(Q && K && V && glse && Output_partial && Output, "decode_dense: null pointer argument");
     REQUIRE(batch > 0 && num_split > 0, "decode_dense: batch, num_split must be > 0");
     REQUIRE(batch <= 65535, "decode_dense: batch exceeds grid limit");
@@ -152,8 +156,10 @@ int kascade_decode_dense_paged_call(const kascade_half* Q, const kascade_half* K
     p.num_split = num_split; p.B = batch;
     const long long max_rows = kv_stride_tokens > 0 ? kv_stride_tokens : (long long)max_pages * page_size;
     p.rows_per_split = rows_per_split(max_rows, num_split);
+    p.counters = sync_counters; p.out = H(Output);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (check_hip(launch_decode_split(p, false, true, false, s), "decode_dense split")) return -1;
+    if (sync_counters) return 0;
     return check_hip(launch_decode_combine(glse, Output_partial, H(Output), nullptr, batch,
                                            num_split, true, s), "decode_dense combine");
 }
@@ -165,7 +171,8 @@ int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_hal
                                         kascade_half* aggregated_scores, int batch,
                                         int kv_stride_tokens, int scores_stride, int num_split,
                                         int with_output, const int32_t* block_table,
-                                        int max_pages, int page_size, void* stream) {
+                                        int max_pages, int page_size, int32_t* sync_counters,
+                                        void* stream) {
     REQUIRE(Q && K && glse && row_sums && scores && aggregated_scores,
             "decode_recompute: null pointer argument");
     REQUIRE(!with_output || (V && Output && Output_partial),
@@ -192,10 +199,12 @@ int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_hal
     long long max_rows = kv_stride_tokens > 0 ? kv_stride_tokens : (long long)max_pages * page_size;
     if (max_rows > scores_stride) max_rows = scores_stride;
     p.rows_per_split = rows_per_split(max_rows, num_split);
+    p.counters = sync_counters; p.out = H(Output); p.row_sums = row_sums;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (check_hip(launch_decode_split(p, false, with_output != 0, true, s), "decode_recompute split"))
         return -1;
-    if (check_hip(launch_decode_combine(glse, Output_partial, H(Output), row_sums, batch, num_split,
+    if (!sync_counters &&
+        check_hip(launch_decode_combine(glse, Output_partial, H(Output), row_sums, batch, num_split,
                                         with_output != 0, s), "decode_recompute combine"))
         return -1;
     return check_hip(launch_decode_aggregate(scores, row_sums, cache_seqlens, H(aggregated_scores),

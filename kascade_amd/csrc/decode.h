@@ -15,6 +15,12 @@ struct DecodeParams {
     float* glse;            // [B,H,num_split]
     float* opart;           // [B,H,num_split,D]
     float* scores;          // [B,H,scores_stride] raw q.k (anchor mode)
+    // Fused combine: with counters != null ([B*G] ints, zero before the first launch and zero
+    // again after every launch) the last split workgroup of each (b, g) merges the splits into
+    // out [B,H,D] and row_sums [B,H] (either may be null), and no combine launch is needed.
+    int* counters;
+    half_t* out;
+    float* row_sums;
     int max_pages;
     int page_shift;
     int kv_stride_tokens;

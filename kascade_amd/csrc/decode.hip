@@ -33,6 +33,26 @@ constexpr int kScoreBatches = 16;             // batches between two score flush
 constexpr int kStripRows = 16 * kScoreBatches;  // rows a wavefront owns per super-iteration
 constexpr int kSubChunk = 1024;               // rows whose physical ids are staged in LDS at once
 
+// Device-coherent accesses (relaxed atomics at agent scope) for data that one workgroup writes
+// and another workgroup of the same launch reads.
+__device__ __forceinline__ void store_device(float* p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_device2(float* p, float a, float b) {
+    union { float f[2]; unsigned long long u; } x;
+    x.f[0] = a; x.f[1] = b;
+    __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), x.u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_device(const float* p) {
+    return __hip_atomic_load(const_cast<float*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float2 load_device2(const float* p) {
+    union { float f[2]; unsigned long long u; } x;
+    x.u = __hip_atomic_load(reinterpret_cast<unsigned long long*>(const_cast<float*>(p)), __ATOMIC_RELAXED,
+                            __HIP_MEMORY_SCOPE_AGENT);
+    return make_float2(x.f[0], x.f[1]);
+}
+
 struct MergeState {  // one per wavefront after the in-wave merge
     float m[kGroupSize];
     float l[kGroupSize];
@@ -43,6 +63,7 @@ template <bool GATHER, bool WITH_V, bool WRITE_SCORES>
 __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decode_split_kernel(DecodeParams p) {
     __shared__ int s_row[GATHER ? kSubChunk : 1];
     __shared__ MergeState s_merge[4];
+    __shared__ int s_last;
     // anchor mode: two buffers of four wavefront strips (4 heads x kStripRows raw scores)
     __shared__ __attribute__((aligned(16))) float s_sc[WRITE_SCORES ? 2 : 1][WRITE_SCORES ? 4 : 1][kGroupSize][WRITE_SCORES ? kStripRows : 4];
 
@@ -362,11 +383,83 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
             }
         }
         const size_t ph = ((size_t)b * kHeads + g * kGroupSize + h) * p.num_split + split;
-        if ((tid & 63) == 0) p.glse[ph] = (L > 0.f) ? (fast_log2(L) + mref) : -INFINITY;
+        const float lse_part = (L > 0.f) ? (fast_log2(L) + mref) : -INFINITY;
+        const float inv = (L > 0.f) ? 1.f / L : 0.f;
+        if (p.counters == nullptr) {
+            if ((tid & 63) == 0) p.glse[ph] = lse_part;
+            if (WITH_V) *reinterpret_cast<float2*>(p.opart + ph * kDim + d0) = make_float2(o0 * inv, o1 * inv);
+        } else {
+            // read by another workgroup of this launch: device-coherent stores
+            if ((tid & 63) == 0) store_device(p.glse + ph, lse_part);
+            if (WITH_V) store_device2(p.opart + ph * kDim + d0, o0 * inv, o1 * inv);
+        }
+    }
+    // ---- fused combine: the last workgroup of (b, g) to arrive merges the splits ----
+    // The partial results above are written through to device-coherent memory and the barrier
+    // waits for those stores before thread 0 counts this workgroup in; the merging workgroup
+    // reads them back with device-coherent loads.  No device-wide fence is involved: one per
+    // workgroup would write back and invalidate the L2 that the K/V stream lives in.
+    if (p.counters == nullptr) return;
+    __syncthreads();
+    if (tid == 0) {
+        const int arrived = __hip_atomic_fetch_add(&p.counters[b * kGroups + g], 1, __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT);
+        s_last = (arrived == p.num_split - 1);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    if (tid == 0)   // ready for the next launch
+        __hip_atomic_store(&p.counters[b * kGroups + g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid < kThreads) {
+        // wavefront -> head; lanes over the splits for the reductions, then two d's per lane
+        const int head = g * kGroupSize + wave;
+        const int ns = p.num_split;
+        const size_t base = ((size_t)b * kHeads + head) * ns;
+        const float* gl = p.glse + base;
+        const float* op = p.opart + base * kDim + lane * 2;
+        // the first partial outputs are requested together with the log-sums, so that short
+        // split lists cost one trip to memory, not two
+        constexpr int kEarly = 16;
+        float2 xe[kEarly];
         if (WITH_V) {
-            const float inv = (L > 0.f) ? 1.f / L : 0.f;
-            float2 o = make_float2(o0 * inv, o1 * inv);
-            *reinterpret_cast<float2*>(p.opart + ph * kDim + d0) = o;
+#pragma unroll
+            for (int j = 0; j < kEarly; ++j) xe[j] = load_device2(op + (size_t)min(j, ns - 1) * kDim);
+        }
+        const float g0 = (lane < ns) ? load_device(gl + lane) : -INFINITY;   // splits [0, 64)
+        float mx = g0;
+        for (int s = lane + 64; s < ns; s += 64) mx = fmaxf(mx, load_device(gl + s));
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+        const float mref = (mx == -INFINITY) ? 0.f : mx;
+        float sum = fast_exp2(g0 - mref);
+        for (int s = lane + 64; s < ns; s += 64) sum += fast_exp2(load_device(gl + s) - mref);
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
+        const float lse = (sum > 0.f) ? fast_log2(sum) + mref : -INFINITY;
+        if (p.row_sums && lane == 0) p.row_sums[(size_t)b * kHeads + head] = lse;
+        if (WITH_V) {
+            const float lref = (lse == -INFINITY) ? 0.f : lse;
+            float o0 = 0.f, o1 = 0.f;
+            float wl = fast_exp2(g0 - lref);   // 0 in lanes beyond the split count
+#pragma unroll
+            for (int j = 0; j < kEarly; ++j) {
+                const float w = __shfl(wl, j);
+                o0 += w * xe[j].x;
+                o1 += w * xe[j].y;
+            }
+            for (int s0 = 0; s0 < ns; s0 += 64) {
+                if (s0 > 0) wl = (s0 + lane < ns) ? fast_exp2(load_device(gl + s0 + lane) - lref) : 0.f;
+                const int cnt = min(64, ns - s0);
+#pragma unroll 8
+                for (int j = (s0 == 0 ? kEarly : 0); j < cnt; ++j) {
+                    const float w = __shfl(wl, j);
+                    const float2 x = load_device2(op + (size_t)(s0 + j) * kDim);
+                    o0 += w * x.x;
+                    o1 += w * x.y;
+                }
+            }
+            half2_t o = {(half_t)o0, (half_t)o1};
+            *reinterpret_cast<half2_t*>(p.out + ((size_t)b * kHeads + head) * kDim + lane * 2) = o;
         }
     }
 }

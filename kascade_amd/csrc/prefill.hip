@@ -371,8 +371,11 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel_q64(PrefillParam
 
 // Pooled tile scores: out[b,g,t,key] = sum over the 32 queries of tile t and the 4 q-heads of g
 // of exp2(s*scale - log_sum), for keys before the tile's first (global) position.
+// Two workgroups per compute unit (register budget 256): one wavefront's exponentials run
+// under the other's matrix instructions.
 template <bool PAGED>
-__global__ __launch_bounds__(kThreads) void prefill_aggregate_kernel(PrefillParams p) {
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2)))
+void prefill_aggregate_kernel(PrefillParams p) {
     __shared__ __attribute__((aligned(16))) half_t sK[kAggKT * kKStride];
     __shared__ __attribute__((aligned(16))) float s_lse[128];
 

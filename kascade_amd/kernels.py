@@ -77,7 +77,17 @@ def _out_buffer(out, B, device) -> torch.Tensor:
     return out
 
 
-def decode_reuse(Q, K, V, topk_indices, head_mapping, glse, Output_partial) -> torch.Tensor:
+def _sync_arg(sync, B):
+    """Optional [B*G] int32 counter array for the fused combine (zero-initialised by the caller)."""
+    if sync is None:
+        return None
+    _req(sync, torch.int32, "sync_counters")
+    if sync.numel() < B * G:
+        raise KascadeError(f"sync_counters needs {B * G} entries")
+    return _ptr(sync)
+
+
+def decode_reuse(Q, K, V, topk_indices, head_mapping, glse, Output_partial, sync=None) -> torch.Tensor:
     """``decode_reuse_kernel(Q, K, V, topk_indices, head_mapping, glse, Output_partial) -> O``
     (out_idx=[7]; EfficientKascadeStrategy.py:30-38, 113, 122).  Contiguous cache
     K,V [B,L,G,D]; the split count is glse.shape[2]."""
@@ -95,12 +105,13 @@ def decode_reuse(Q, K, V, topk_indices, head_mapping, glse, Output_partial) -> t
     out = torch.empty(B, H, D, device=Q.device, dtype=torch.float16)
     _lib.check(lib.kascade_decode_reuse_call(
         _ptr(Q), _ptr(K), _ptr(V), _ptr(topk_indices), _ptr(head_mapping), _ptr(glse),
-        _ptr(Output_partial), _ptr(out), B, L, topk_indices.shape[-1], ns, _stream()))
+        _ptr(Output_partial), _ptr(out), B, L, topk_indices.shape[-1], ns, _sync_arg(sync, B), _stream()))
     return out
 
 
 def decode_reuse_paged(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_percent, glse,
-                       Output_partial, block_table=None, page_size: int = 16, out=None) -> torch.Tensor:
+                       Output_partial, block_table=None, page_size: int = 16, out=None,
+                       sync=None) -> torch.Tensor:
     """``reuse kvcache kernel(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_percent,
     glse, Output_partial) -> O`` (out_idx=[9]; reuse_kascade_gqa_decode_with_kvcache.py:160-173)
     with an optional block table.  Without one K,V are the padded [B,maxL,G,D] cache;
@@ -122,12 +133,13 @@ def decode_reuse_paged(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_
     _lib.check(lib.kascade_decode_reuse_paged_call(
         _ptr(Q), _ptr(K), _ptr(V), _ptr(cache_seqlens), _ptr(topk_indices), _ptr(head_mapping),
         float(topk_percent), _ptr(glse), _ptr(Output_partial), _ptr(out), B, stride_tokens,
-        topk_indices.shape[-1], ns, _ptr(block_table), max_pages, page_size, _stream()))
+        topk_indices.shape[-1], ns, _ptr(block_table), max_pages, page_size, _sync_arg(sync, B), _stream()))
     return out
 
 
 def decode_dense_paged(Q, K, V, cache_seqlens, glse, Output_partial, block_table=None,
-                       page_size: int = 16, kv_len: Optional[int] = None, out=None) -> torch.Tensor:
+                       page_size: int = 16, kv_len: Optional[int] = None, out=None,
+                       sync=None) -> torch.Tensor:
     """Dense split-K decode, the baseline of gqa_decode.py / gqa_decode_with_kvcache.py:
     ``kernel(Q, K, V, [cache_seqlens,] glse, Output_partial) -> O``."""
     lib = _lib.init()
@@ -143,13 +155,14 @@ def decode_dense_paged(Q, K, V, cache_seqlens, glse, Output_partial, block_table
     out = _out_buffer(out, B, Q.device)
     _lib.check(lib.kascade_decode_dense_paged_call(
         _ptr(Q), _ptr(K), _ptr(V), _ptr(cache_seqlens), _ptr(glse), _ptr(Output_partial), _ptr(out),
-        B, stride_tokens, ns, _ptr(block_table), max_pages, page_size, _stream()))
+        B, stride_tokens, ns, _ptr(block_table), max_pages, page_size, _sync_arg(sync, B), _stream()))
     return out
 
 
 def decode_recompute(Q, K, V, glse, Output_partial, row_sums, scores, layer: int,
                      cache_seqlens=None, block_table=None, page_size: int = 16,
-                     kv_len: Optional[int] = None, out=None) -> Tuple[Optional[torch.Tensor], torch.Tensor]:
+                     kv_len: Optional[int] = None, out=None,
+                     sync=None) -> Tuple[Optional[torch.Tensor], torch.Tensor]:
     """``decode_recomp{0,1}_kernel(Q, K, V, glse, Output_partial, row_sums, scores) -> (O, agg)``
     (out_idx=[7,8]; EfficientKascadeStrategy.py:24-28, 107-110) and its kvcache form
     (recompute_kascade_gqa_decode_with_kvcache.py:302-333).  ``scores`` is fp32 scratch
@@ -173,7 +186,7 @@ def decode_recompute(Q, K, V, glse, Output_partial, row_sums, scores, layer: int
     _lib.check(lib.kascade_decode_recompute_paged_call(
         _ptr(Q), _ptr(K), _ptr(V), _ptr(cache_seqlens), _ptr(glse), _ptr(Output_partial),
         _ptr(row_sums), _ptr(scores), _ptr(out), _ptr(agg), B, stride_tokens, stride, ns, with_out,
-        _ptr(block_table), max_pages, page_size, _stream()))
+        _ptr(block_table), max_pages, page_size, _sync_arg(sync, B), _stream()))
     return out, agg
 
 

@@ -210,8 +210,9 @@ class PagedKascadeDecoder:
     def __init__(self, k: float, head_mapping: List[List[int]], recompute_layers: Sequence[int],
                  max_batch: int, max_seqlen: int, page_size: int = 16, device="cuda",
                  num_split_dense: Optional[int] = None, num_split_reuse: Optional[int] = None,
-                 total_tokens: Optional[int] = None):
-        """total_tokens: expected sum of the sequence lengths of a batch (default
+                 total_tokens: Optional[int] = None, fused_combine: bool = True):
+        """fused_combine: merge the splits inside the split launch (one launch fewer per layer).
+        total_tokens: expected sum of the sequence lengths of a batch (default
         max_batch*max_seqlen); with ragged batches it sizes the splits so that the non-empty
         workgroups, not the grid, cover the device about twice."""
         self.k = k
@@ -237,6 +238,13 @@ class PagedKascadeDecoder:
             self._hm[l] = torch.tensor(row, device=dev, dtype=torch.int32)
         self._topk_to_reuse = None
         self._counts = None
+        # arrival counters of the fused combine: zero now, set back to zero by every launch
+        self._sync = torch.zeros(max_batch * G, device=dev, dtype=torch.int32) if fused_combine else None
+        # one workgroup merges all splits of a (sequence, KV head): a win up to about 16 splits
+        # (one trip to memory); beyond that the combine launch, which spreads the merge over
+        # 32 workgroups per sequence, is faster
+        self._sync_dense = self._sync if self.ns_dense <= 16 else None
+        self._sync_reuse = self._sync if self.ns_reuse <= 16 else None
 
     def _scratch(self, B, ns):
         return self._glse[:B * H * ns].view(B, H, ns), self._part[:B * H * ns * D].view(B, H, ns, D)
@@ -245,7 +253,7 @@ class PagedKascadeDecoder:
         B = q.shape[0]
         glse, part = self._scratch(B, self.ns_dense)
         return kernels.decode_dense_paged(q, k_pages, v_pages, seqlens, glse, part, block_table,
-                                          self.page_size, kv_len=max_len, out=out)
+                                          self.page_size, kv_len=max_len, out=out, sync=self._sync_dense)
 
     def anchor(self, layer, q, k_pages, v_pages, block_table, seqlens, max_len: int,
                ragged: bool = True, out=None):
@@ -257,7 +265,7 @@ class PagedKascadeDecoder:
         scores = self._scores[:B * H * stride].view(B, H, stride)
         o, agg = kernels.decode_recompute(q, k_pages, v_pages, glse, part, self._row_sums[:B], scores, layer,
                                           cache_seqlens=seqlens, block_table=block_table,
-                                          page_size=self.page_size, kv_len=max_len, out=out)
+                                          page_size=self.page_size, kv_len=max_len, out=out, sync=self._sync_dense)
         if ragged:
             width = budgets.decode_budget(max_len, self.k)
             lens_rows, counts = self._row_budgets(seqlens)
@@ -294,7 +302,8 @@ class PagedKascadeDecoder:
         B = q.shape[0]
         glse, part = self._scratch(B, self.ns_reuse)
         return kernels.decode_reuse_paged(q, k_pages, v_pages, seqlens, self._topk_to_reuse, hm, self._pct,
-                                          glse, part, block_table=block_table, page_size=self.page_size, out=out)
+                                          glse, part, block_table=block_table, page_size=self.page_size, out=out,
+                                          sync=self._sync_reuse)
 
     def reuse(self, layer, q, k_pages, v_pages, block_table, seqlens, out=None):
         """Reuse layer: attends to rows head_mapping[layer] of the last anchor's indices."""

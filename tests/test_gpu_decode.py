@@ -211,3 +211,53 @@ def test_kv_append_roundtrip(cuda):
             assert torch.equal(Kc[pg, tok % page], kn[b, t])
             assert torch.equal(Vc[pg, tok % page], vn[b, t])
     assert int((Kc != 0).any(dim=-1).any(dim=-1).sum()) == B * n_new
+
+
+@pytest.mark.parametrize("seqlens,ns", [([300, 1000, 515], 4), ([4500, 64], 70), ([700], 1)])
+def test_fused_combine_matches_combine_launch(cuda, seqlens, ns):
+    """Merging the splits inside the split launch (arrival counters) gives the result of the
+    separate combine launch, checked against the oracle, on repeated calls with one counter
+    array (every launch leaves it zero)."""
+    from kascade_amd import kernels
+    p = 10
+    w = _paged_case(seqlens, seed=21)
+    B, Lmax = len(seqlens), max(seqlens)
+    kc = orc.paged_to_contiguous(w.k_pages, w.block_table, seqlens)
+    vc = orc.paged_to_contiguous(w.v_pages, w.block_table, seqlens)
+    q, kp, vp = w.q.to(cuda), w.k_pages.to(cuda), w.v_pages.to(cuda)
+    lens, bt = w.seqlens.to(cuda), w.block_table.to(cuda)
+    sync = torch.zeros(B * G, dtype=torch.int32, device=cuda)
+    glse, part = _scratch(B, ns, cuda)
+    want, lse = orc.dense_decode(w.q, kc, vc, seqlens)
+    two = kernels.decode_dense_paged(q, kp, vp, lens, glse, part, bt, w.page_size)
+    for rep in range(3):
+        got = kernels.decode_dense_paged(q, kp, vp, lens, glse, part, bt, w.page_size, sync=sync)
+        torch.cuda.synchronize()
+        assert int(sync.abs().sum()) == 0, "arrival counters not back to zero"
+        assert_close(got, want, f"fused dense decode, call {rep}")
+        assert_close(got, two, "fused vs combine launch", atol=1e-3, rtol=2e-3)
+    # anchor pass: row_sums and (layer 0) the output come from the fused merge
+    row_sums = torch.empty(B, H, device=cuda, dtype=torch.float32)
+    stride = ((Lmax + 7) // 8) * 8
+    scores = torch.empty(B, H, stride, device=cuda, dtype=torch.float32)
+    for layer in (0, 1):
+        o, agg = kernels.decode_recompute(q, kp, vp, glse, part, row_sums, scores, layer, cache_seqlens=lens,
+                                          block_table=bt, page_size=w.page_size, sync=sync)
+        torch.cuda.synchronize()
+        assert int(sync.abs().sum()) == 0
+        assert_close(row_sums, lse * orc.LOG2E, "row_sums (fused)", atol=2e-3, rtol=1e-4)
+        assert_close(agg.cpu()[:, :, :Lmax], orc.pooled_decode_scores(w.q, kc, seqlens), "agg (fused)",
+                     atol=2e-6, rtol=2e-3)
+        if layer == 0:
+            assert_close(o, want, "anchor-0 output (fused)")
+    # reuse pass
+    gen = torch.Generator().manual_seed(4)
+    idx = _rand_idx(B, min(seqlens), 256 if min(seqlens) >= 256 else 64, gen)
+    hm = torch.tensor([3, 3, 0, 1, 7, 6, 5, 2], dtype=torch.int32, device=cuda)
+    r2 = kernels.decode_reuse_paged(q, kp, vp, lens, idx.to(cuda), hm, 0.0, glse, part, block_table=bt,
+                                    page_size=w.page_size)
+    r1 = kernels.decode_reuse_paged(q, kp, vp, lens, idx.to(cuda), hm, 0.0, glse, part, block_table=bt,
+                                    page_size=w.page_size, sync=sync)
+    assert_close(r1, orc.reuse_decode(w.q, kc, vc, idx, hm.tolist()), "fused reuse decode")
+    assert_close(r1, r2, "fused vs combine launch (reuse)", atol=1e-3, rtol=2e-3)
+    assert int(sync.abs().sum()) == 0
