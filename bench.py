@@ -396,7 +396,7 @@ def main():
         Lc = args.seq_len
         log(f"[bench] cpu baseline: oracle on {nthreads} threads (os.cpu_count()={os.cpu_count()})")
         wc = workloads.prefill_inputs(1, Lc, seed=0, device="cpu")
-        nblk, rows = 4, 256
+        nblk, rows = 4, 1024      # about 10-15 s of CPU work on 16 threads
         est = {"anchor0": 0.0, "anchor": 0.0, "reuse": 0.0}
         idx_full = None
         for i in range(nblk):

@@ -51,6 +51,7 @@ int check_strides(const kascade_strides& s, const char* name) {
     REQUIRE(s.b % 8 == 0 && s.l % 8 == 0 && s.h % 8 == 0,
             "%s strides must be multiples of 8 elements (16-byte rows)", name);
     REQUIRE(s.l > 0 && s.h > 0, "%s strides must be positive", name);
+    REQUIRE(s.l < (1LL << 31), "%s row stride must be below 2^31 elements", name);
     return 0;
 }
 
@@ -328,6 +329,7 @@ static int chunk_params(PrefillParams& p, const char* what, const kascade_half* 
     if (check_strides(q_strides, "Q")) return -1;
     int shift;
     if (check_paging(block_table, max_pages, page_size, &shift)) return -1;
+    REQUIRE(page_size >= 4, "prefill_chunk: page_size must be at least 4");
     REQUIRE(num_pages > 0 && (long long)num_pages * page_size < (1LL << 31),
             "prefill_chunk: num_pages out of range");
     REQUIRE((long long)max_pages * page_size >= (long long)q_start + q_len,

@@ -30,8 +30,17 @@ namespace kascade {
 
 namespace {
 
+// Wavefront priority while a block of MFMAs is being issued (0 = leave the arbiter alone).
+#ifndef KASCADE_PRIO_HI
+#define KASCADE_PRIO_HI 0
+#endif
+#define KASCADE_MFMA_PRIO(x)                                  \
+    do {                                                      \
+        if (KASCADE_PRIO_HI != 0) __builtin_amdgcn_s_setprio(x); \
+    } while (0)
+
 constexpr int kThreads = 256;
-constexpr int kKT = 64;            // keys per tile (attention kernel)
+constexpr int kKT = 64;           // keys per tile (attention kernel)
 constexpr int kKStride = 136;      // halves per K row in LDS (128 + 8 pad)
 constexpr int kVStride = 64;       // halves per V^T row in LDS (one 64-key tile)
 constexpr int kAggKT = 128;        // keys per tile (aggregate kernel)
@@ -100,7 +109,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
     }
     const int ntiles = sparse ? ng + 1 : (min(q0 + QT, L) + kKT - 1) / kKT;
 
-    const int krow = tid >> 4;   // K: key position krow + 16 i, 16-byte column kcol
+    const int krow = tid >> 4;   // tile positions 4*krow + i, 16-byte column kcol
     const int kcol = tid & 15;
     const half_t* kbase = PAGED ? p.K + (long long)g * kDim + kcol * 8
                                 : p.K + (long long)b * p.k_sb + (long long)g * p.k_sh + kcol * 8;
@@ -114,54 +123,48 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
     auto tile_key = [&](int ti, int pos) {
         return min((sparse ? q0 : ti * kKT) + pos, L - 1);
     };
-    // nk/nv: what the next tile's loads need.  Strided K/V: key ids.  PAGED: block-table
-    // entries for contiguous keys (combined with the key's slot when the loads are issued, so
-    // that nothing waits on the table load here) or physical rows for gathered tiles.
-    int nk[4], nv[4];
+    // A thread stages the same four key positions 4*krow .. 4*krow+3 of a tile for K and for V
+    // (V needs four consecutive keys per thread for its transposition; K rows can go anywhere),
+    // so one id and one address offset per position serve both tensors.
+    // ids[]: what the next tile's loads need.  Gathered tiles: key ids (physical rows when
+    // PAGED).  Consecutive keys, PAGED: ids[0] is the block-table entry of the four positions'
+    // common page, fetched a tile ahead so that the loads never wait on the table.  Consecutive
+    // keys, strided: nothing (addresses follow from the tile index).
+    int ids[4];
     int pend_ti = 0;        // tile the ids belong to
     uint4_t kr[4], vr[4];   // tile data in flight
+    const unsigned row_stride = PAGED ? (unsigned)(kGroups * kDim) : (unsigned)p.k_sl;   // host checks < 2^31
     auto fetch_ids = [&](int ti) {
         pend_ti = ti;
+        if (sparse && ti < ng) {
+            const int base = ti * kKT + 4 * krow;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int pk = krow + 16 * i;       // K position of chunk i
-            const int pv = 4 * krow + i;        // V position of chunk i
-            if (sparse && ti < ng) {
-                const int a = idx_row[min(ti * kKT + pk, n - 1)];
-                const int c = idx_row[min(ti * kKT + pv, n - 1)];
-                nk[i] = max(0, min(a, PAGED ? max_row : L - 1));
-                nv[i] = max(0, min(c, PAGED ? max_row : L - 1));
-            } else if (PAGED) {
-                nk[i] = bt_row[tile_key(ti, pk) >> p.page_shift];
-                nv[i] = bt_row[tile_key(ti, pv) >> p.page_shift];
-            } else {
-                nk[i] = tile_key(ti, pk);
-                nv[i] = tile_key(ti, pv);
+            for (int i = 0; i < 4; ++i) {
+                const int a = idx_row[min(base + i, n - 1)];
+                ids[i] = max(0, min(a, PAGED ? max_row : L - 1));
             }
+        } else if (PAGED) {
+            ids[0] = bt_row[tile_key(ti, 4 * krow) >> p.page_shift];
         }
     };
     auto issue_loads = [&]() {
-        if (PAGED) {
-            const bool gathered = sparse && pend_ti < ng;
+        long long off[4];
+        if (sparse && pend_ti < ng) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int rk = gathered ? nk[i] : (nk[i] << p.page_shift) + (tile_key(pend_ti, krow + 16 * i) & page_mask);
-                kr[i] = ld_global_16(kbase + (long long)rk * (kGroups * kDim));
-            }
-            if (WITH_V) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int rv = gathered ? nv[i] : (nv[i] << p.page_shift) + (tile_key(pend_ti, 4 * krow + i) & page_mask);
-                    vr[i] = ld_global_16(vbase + (long long)rv * (kGroups * kDim));
-                }
-            }
+            for (int i = 0; i < 4; ++i) off[i] = (long long)((unsigned long long)(unsigned)ids[i] * row_stride);
         } else {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) kr[i] = ld_global_16(kbase + (long long)nk[i] * p.k_sl);
-            if (WITH_V) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) vr[i] = ld_global_16(vbase + (long long)nv[i] * p.k_sl);
+            for (int i = 0; i < 4; ++i) {
+                const int key = tile_key(pend_ti, 4 * krow + i);
+                const int row = PAGED ? (ids[0] << p.page_shift) + (key & page_mask) : key;
+                off[i] = (long long)((unsigned long long)(unsigned)row * row_stride);
             }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) kr[i] = ld_global_16(kbase + off[i]);
+        if (WITH_V) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) vr[i] = ld_global_16(vbase + off[i]);
         }
     };
 
@@ -186,7 +189,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
         // ---- registers -> LDS ----
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int slot = swap_bits23(krow + 16 * i);
+            const int slot = swap_bits23(4 * krow + i);
             *reinterpret_cast<uint4_t*>(&sK[slot * kKStride + kcol * 8]) = kr[i];
         }
         if (WITH_V) {
@@ -208,15 +211,13 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
         }
 
         // ---- S^T = K_tile Q^T ----
+        KASCADE_MFMA_PRIO(KASCADE_PRIO_HI);
         const bool diag_tile = sparse && (ti == ng);
         const int nkb = (diag_tile && QT == 32) ? 1 : 2;
         float16_t sT[NQB][2];
+        float16_t zero16;
 #pragma unroll
-        for (int qb = 0; qb < NQB; ++qb)
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) sT[qb][kb][v] = 0.f;
+        for (int v = 0; v < 16; ++v) zero16[v] = 0.f;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
             if (kb < nkb) {
@@ -225,11 +226,18 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
                     half8_t a = *reinterpret_cast<const half8_t*>(
                         &sK[(32 * kb + li) * kKStride + ks * 16 + lg * 8]);
 #pragma unroll
-                    for (int qb = 0; qb < NQB; ++qb)
-                        sT[qb][kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[qb][ks], sT[qb][kb], 0, 0, 0);
+                    for (int qb = 0; qb < NQB; ++qb)   // the first product starts from a constant zero
+                        sT[qb][kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[qb][ks],
+                                                                            ks == 0 ? zero16 : sT[qb][kb], 0, 0, 0);
                 }
+            } else {   // second key block of a 32-key diagonal tile: nothing there
+#pragma unroll
+                for (int qb = 0; qb < NQB; ++qb)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) sT[qb][kb][v] = -INFINITY;
             }
         }
+        KASCADE_MFMA_PRIO(0);
         // ---- masks: accumulator v of key block kb is tile position 32kb + 16(v/8) + 8lg + v%8 ----
         if (!sparse || diag_tile) {
             const int kstart = diag_tile ? q0 : ti * kKT;
@@ -256,12 +264,6 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
                         const int pos = ti * kKT + 32 * kb + 16 * (v >> 3) + 8 * lg + (v & 7);
                         if (pos >= n) sT[qb][kb][v] = -INFINITY;
                     }
-        }
-        if (nkb == 1) {
-#pragma unroll
-            for (int qb = 0; qb < NQB; ++qb)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) sT[qb][1][v] = -INFINITY;
         }
         // ---- online softmax (one query column per lane) ----
         half8_t pf[NQB][4];
@@ -305,6 +307,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
         }
         // ---- O^T += V^T P^T ----
         if (WITH_V) {
+            KASCADE_MFMA_PRIO(KASCADE_PRIO_HI);
 #pragma unroll
             for (int db = 0; db < 4; ++db) {
                 const int d = 32 * db + li;
@@ -320,6 +323,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
                     }
                 }
             }
+            KASCADE_MFMA_PRIO(0);
         }
     }
 
@@ -361,9 +365,15 @@ void prefill_attn_kernel_q32(PrefillParams p) {
     prefill_attn_body<1, REUSE, WITH_V, PAGED>(p, sK, sV);
 }
 
-// 64 queries per wavefront: one wavefront per SIMD with the whole register file.
+// 64 queries per wavefront.  Without V the state fits 256 registers: two workgroups per compute
+// unit, and the MFMA results stay in ordinary registers (with the full 512-register budget the
+// compiler parks them in accumulation registers and copies each one out before the softmax).
+#ifndef KASCADE_Q64_WAVES
+#define KASCADE_Q64_WAVES 2
+#endif
 template <bool WITH_V>
-__global__ __launch_bounds__(kThreads) void prefill_attn_kernel_q64(PrefillParams p) {
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(WITH_V ? 1 : KASCADE_Q64_WAVES, WITH_V ? 1 : KASCADE_Q64_WAVES)))
+void prefill_attn_kernel_q64(PrefillParams p) {
     __shared__ __attribute__((aligned(16))) half_t sK[kKT * kKStride];
     __shared__ __attribute__((aligned(16))) half_t sV[kDim * kVStride];
     prefill_attn_body<2, false, WITH_V, false>(p, sK, sV);
@@ -458,6 +468,7 @@ void prefill_aggregate_kernel(PrefillParams p) {
             for (int rb = 0; rb < kGroupSize; ++rb)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[rb][v] = 0.f;
+            KASCADE_MFMA_PRIO(KASCADE_PRIO_HI);
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks) {
                 half8_t bf = *reinterpret_cast<const half8_t*>(
@@ -466,6 +477,7 @@ void prefill_aggregate_kernel(PrefillParams p) {
                 for (int rb = 0; rb < kGroupSize; ++rb)
                     acc[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa[rb][ks], bf, acc[rb], 0, 0, 0);
             }
+            KASCADE_MFMA_PRIO(0);
             // accumulator v of row block rb is query row 8(v/4) + 4lg + v%4, column = key li
             float sum = 0.f;
 #pragma unroll
