@@ -365,3 +365,40 @@ def test_head_mapping_fixtures():
         assert a.min() >= 0 and a.max() <= 7
         for l in anchors:
             assert a[l].tolist() == list(range(8))
+
+
+# ------------------------------------------------------------ config 0 (CPU plumbing run)
+def test_config0_cpu_plumbing_run():
+    """BASELINE config 0 in full on the strategy-semantics oracle: batch 1, 8 q-heads / 2 KV heads,
+    head_dim 64, causal prefill of 2048 tokens in fp32, tile 32, top-k 10 %, identity head map,
+    N(0,1) inputs from seed 0, reuse layer = anchor + 0.3 N(0,1).  Layer 0 must be dense attention
+    (SDPA), the reuse layer the masked softmax over (stored indices U in-tile diagonal) on
+    sampled rows, and the stored state must have the shapes the reference keeps."""
+    L, Hq, Gk, Dh, tile, p = 2048, 8, 2, 64, 32, 10
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(1, Hq, L, Dh, generator=g)
+    k = torch.randn(1, Gk, L, Dh, generator=g)
+    v = torch.randn(1, Gk, L, Dh, generator=g)
+    q1 = q + 0.3 * torch.randn(q.shape, generator=g)
+    k1 = k + 0.3 * torch.randn(k.shape, generator=g)
+    mask = orc.causal_additive_mask(L, L, torch.float32)
+    st = orc.StrategyOracle([0], [[0, 1], [0, 1]], k=p, tile_size=tile, rolling_prefill=False)
+    scaling = Dh ** -0.5
+    o0 = st.attention_forward(0, q, k, v, mask, scaling)
+    want0 = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
+    assert torch.allclose(o0, want0.transpose(1, 2), atol=2e-5)
+    kw = orc.k_strat(L, p, tile)
+    assert kw == 172 and orc.k_kern(L, p) == 256
+    assert tuple(st._topk_to_reuse.shape) == (1, Gk, L, kw)
+    o1 = st.attention_forward(1, q1, k1, v, mask, scaling)
+    assert tuple(o1.shape) == (1, L, Hq, Dh) and bool(torch.isfinite(o1).all())
+    idx = st._topk_to_reuse
+    rep = Hq // Gk
+    for i in (0, 31, 32, 500, 1023, 2047):
+        for h in (0, 3, 4, 7):
+            gk = h // rep
+            keys = {int(x) for x in idx[0, gk, i]} | set(range((i // tile) * tile, i + 1))
+            ks = sorted(j for j in keys if j <= i)
+            s = (k1[0, gk, ks] @ q1[0, h, i]) * scaling
+            want = torch.softmax(s, 0) @ v[0, gk, ks]
+            assert torch.allclose(o1[0, i, h], want, atol=2e-5), (i, h)
