@@ -15,10 +15,6 @@
 
 using namespace kascade;
 
-#ifndef KASCADE_DENSE_NQB
-#define KASCADE_DENSE_NQB 1   // 32-query blocks per wavefront in the dense prefill kernels
-#endif
-
 namespace {
 
 thread_local char g_err[1024] = "";
@@ -251,7 +247,7 @@ int kascade_prefill_dense_call(const kascade_half* Q, const kascade_half* K, con
     p.q_sb = q_strides.b; p.q_sl = q_strides.l; p.q_sh = q_strides.h;
     p.k_sb = kv_strides.b; p.k_sl = kv_strides.l; p.k_sh = kv_strides.h;
     p.B = batch; p.L = seq_len; p.Lq = seq_len; p.T = (seq_len + kTile - 1) / kTile;
-    return check_hip(launch_prefill_attn(p, false, with_output != 0, with_output ? KASCADE_DENSE_NQB : 2,
+    return check_hip(launch_prefill_attn(p, false, with_output != 0, with_output ? 1 : 2,
                                          static_cast<hipStream_t>(stream)), "prefill_dense");
 }
 

@@ -30,15 +30,6 @@ namespace kascade {
 
 namespace {
 
-// Wavefront priority while a block of MFMAs is being issued (0 = leave the arbiter alone).
-#ifndef KASCADE_PRIO_HI
-#define KASCADE_PRIO_HI 0
-#endif
-#define KASCADE_MFMA_PRIO(x)                                  \
-    do {                                                      \
-        if (KASCADE_PRIO_HI != 0) __builtin_amdgcn_s_setprio(x); \
-    } while (0)
-
 constexpr int kThreads = 256;
 constexpr int kKT = 64;           // keys per tile (attention kernel)
 constexpr int kKStride = 136;      // halves per K row in LDS (128 + 8 pad)
@@ -211,7 +202,6 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
         }
 
         // ---- S^T = K_tile Q^T ----
-        KASCADE_MFMA_PRIO(KASCADE_PRIO_HI);
         const bool diag_tile = sparse && (ti == ng);
         const int nkb = (diag_tile && QT == 32) ? 1 : 2;
         float16_t sT[NQB][2];
@@ -237,7 +227,6 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
                     for (int v = 0; v < 16; ++v) sT[qb][kb][v] = -INFINITY;
             }
         }
-        KASCADE_MFMA_PRIO(0);
         // ---- masks: accumulator v of key block kb is tile position 32kb + 16(v/8) + 8lg + v%8 ----
         if (!sparse || diag_tile) {
             const int kstart = diag_tile ? q0 : ti * kKT;
@@ -307,7 +296,6 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
         }
         // ---- O^T += V^T P^T ----
         if (WITH_V) {
-            KASCADE_MFMA_PRIO(KASCADE_PRIO_HI);
 #pragma unroll
             for (int db = 0; db < 4; ++db) {
                 const int d = 32 * db + li;
@@ -323,7 +311,6 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
                     }
                 }
             }
-            KASCADE_MFMA_PRIO(0);
         }
     }
 
@@ -351,32 +338,25 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
     }
 }
 
-#ifndef KASCADE_PREFILL_WAVES_NQB1
-#define KASCADE_PREFILL_WAVES_NQB1 2
-#endif
 
 // 32 queries per wavefront: register budget capped so that two workgroups share a
 // compute unit and hide each other's LDS staging and gather latency.
 template <bool REUSE, bool WITH_V, bool PAGED>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(KASCADE_PREFILL_WAVES_NQB1)))
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2)))
 void prefill_attn_kernel_q32(PrefillParams p) {
     __shared__ __attribute__((aligned(16))) half_t sK[kKT * kKStride];
-    __shared__ __attribute__((aligned(16))) half_t sV[kDim * kVStride];
+    __shared__ __attribute__((aligned(16))) half_t sV[WITH_V ? kDim * kVStride : 8];
     prefill_attn_body<1, REUSE, WITH_V, PAGED>(p, sK, sV);
 }
 
-// 64 queries per wavefront.  Without V the state fits 256 registers: two workgroups per compute
-// unit, and the MFMA results stay in ordinary registers (with the full 512-register budget the
-// compiler parks them in accumulation registers and copies each one out before the softmax).
-#ifndef KASCADE_Q64_WAVES
-#define KASCADE_Q64_WAVES 2
-#endif
-template <bool WITH_V>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(WITH_V ? 1 : KASCADE_Q64_WAVES, WITH_V ? 1 : KASCADE_Q64_WAVES)))
+// 64 queries per wavefront for the K-only log-sum pass, whose state fits 256 registers: two
+// workgroups per compute unit, and the MFMA results stay in ordinary registers (with the full
+// 512-register budget the compiler parks them in accumulation registers and copies each one out
+// before the softmax).
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2)))
 void prefill_attn_kernel_q64(PrefillParams p) {
     __shared__ __attribute__((aligned(16))) half_t sK[kKT * kKStride];
-    __shared__ __attribute__((aligned(16))) half_t sV[kDim * kVStride];
-    prefill_attn_body<2, false, WITH_V, false>(p, sK, sV);
+    prefill_attn_body<2, false, false, false>(p, sK, nullptr);
 }
 
 // Pooled tile scores: out[b,g,t,key] = sum over the 32 queries of tile t and the 4 q-heads of g
@@ -468,7 +448,6 @@ void prefill_aggregate_kernel(PrefillParams p) {
             for (int rb = 0; rb < kGroupSize; ++rb)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[rb][v] = 0.f;
-            KASCADE_MFMA_PRIO(KASCADE_PRIO_HI);
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks) {
                 half8_t bf = *reinterpret_cast<const half8_t*>(
@@ -477,7 +456,6 @@ void prefill_aggregate_kernel(PrefillParams p) {
                 for (int rb = 0; rb < kGroupSize; ++rb)
                     acc[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa[rb][ks], bf, acc[rb], 0, 0, 0);
             }
-            KASCADE_MFMA_PRIO(0);
             // accumulator v of row block rb is query row 8(v/4) + 4lg + v%4, column = key li
             float sum = 0.f;
 #pragma unroll
@@ -520,11 +498,8 @@ hipError_t launch_prefill_attn(const PrefillParams& p, bool reuse, bool with_v, 
             hipLaunchKernelGGL((prefill_attn_kernel_q32<false, false, true>), grid, block, 0, stream, p);
     } else if (reuse) {
         hipLaunchKernelGGL((prefill_attn_kernel_q32<true, true, false>), grid, block, 0, stream, p);
-    } else if (nqb == 2) {
-        if (with_v)
-            hipLaunchKernelGGL((prefill_attn_kernel_q64<true>), grid, block, 0, stream, p);
-        else
-            hipLaunchKernelGGL((prefill_attn_kernel_q64<false>), grid, block, 0, stream, p);
+    } else if (nqb == 2) {   // K-only log-sum pass
+        hipLaunchKernelGGL(prefill_attn_kernel_q64, grid, block, 0, stream, p);
     } else {
         if (with_v)
             hipLaunchKernelGGL((prefill_attn_kernel_q32<false, true, false>), grid, block, 0, stream, p);
