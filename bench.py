@@ -118,6 +118,7 @@ def main():
     ap.add_argument("--skip-decode", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-stack", action="store_true", help="skip the 36-layer chunked-prefill + decode stack")
+    ap.add_argument("--skip-ceilings", action="store_true", help="skip the library copy / gather / GEMM rates")
     ap.add_argument("--decode-only", action="store_true", help="skip the per-kernel prefill section")
     ap.add_argument("--kernel", choices=sorted(SINGLE_KERNELS), default=None,
                     help="profiling mode: run only this kernel --iters times on its benchmark workload")
@@ -388,6 +389,37 @@ def main():
         del qs, ks, vs, dq, dk, dv, chunks
         torch.cuda.empty_cache()
 
+    # ---------------------------------------------- what this device delivers to library kernels
+    # Context for the roofline fractions (which are priced against the published peaks): library
+    # routines on the same box in the same run -- a 1 GiB device copy, a streaming reduction, a
+    # gather of random 256-byte rows (the reuse decode access pattern) and an fp16 GEMM on random
+    # and on all-zero operands (the difference is the power limit at work).
+    ceilings = {}
+    if not args.skip_ceilings:
+        x = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        y = torch.empty_like(x)
+        t = ev_time(lambda: y.copy_(x), n=5)
+        ceilings["copy_1GiB_read_plus_write_GBps"] = round(2 * (1 << 30) / t / 1e3, 1)
+        xf = x.view(torch.float16)
+        t = ev_time(lambda: xf.sum(dtype=torch.float32), n=5)
+        ceilings["stream_read_sum_GBps"] = round((1 << 30) / t / 1e3, 1)
+        del y
+        rows = x.view(-1, 256)                                    # 4 Mi rows of 256 bytes
+        gi = torch.randint(0, rows.shape[0], (1 << 21,), device=dev)
+        t = ev_time(lambda: torch.index_select(rows, 0, gi), n=5)
+        ceilings["gather_256B_rows_read_GBps"] = round(gi.numel() * 256 / t / 1e3, 1)
+        del x, xf, rows, gi
+        n = 8192
+        a, b2 = torch.randn(n, n, device=dev, dtype=torch.float16), torch.randn(n, n, device=dev, dtype=torch.float16)
+        t = ev_time(lambda: a @ b2, n=5, warm=2)
+        ceilings["gemm_fp16_8192_randn_TFLOPs"] = round(2 * n ** 3 / t / 1e6, 1)
+        a.zero_(); b2.zero_()
+        t = ev_time(lambda: a @ b2, n=5, warm=2)
+        ceilings["gemm_fp16_8192_zeros_TFLOPs"] = round(2 * n ** 3 / t / 1e6, 1)
+        del a, b2
+        torch.cuda.empty_cache()
+        log(f"[bench] library ceilings: {ceilings}")
+
     # ------------------------------------------------------------------ CPU baseline (oracle)
     cpu = None
     if not args.skip_cpu:
@@ -441,6 +473,7 @@ def main():
                    "seq_len": L, "layers_per_step": N_LAYERS,
                    "baseline_note": "vs_baseline = value / 6.42 ms, the reference's published H100 figure"},
         "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "decode": decode, "stack": stack_res,
+        "library_ceilings": ceilings,
         "kernels": kern,
     }
     print(json.dumps(out), flush=True)
