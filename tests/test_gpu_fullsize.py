@@ -1,0 +1,207 @@
+"""The benchmark configurations at their full sizes: parity against the CPU oracle on sampled
+rows / tiles / sequences, and size-independent properties checked on every row on the device
+(selection threshold property, probability mass, permutation invariance, chunked = whole)."""
+import math
+
+import pytest
+import torch
+
+from oracle import kascade_oracle as orc
+from tests.helpers import assert_close
+
+pytestmark = pytest.mark.gpu
+
+H, G, D, TILE, P = 32, 8, 128, 32, 10
+
+
+def _check_selection_on_device(scores, idx, n_sel, valid):
+    """Every row of idx [R,K] must hold, in slots [0, n), n distinct ascending positions < valid
+    whose scores are all >= every unselected valid score (exact selection on these scores).
+    scores [R,L] fp16 (device), n_sel / valid: int64 tensors [R]."""
+    R, L = scores.shape
+    K = idx.shape[1]
+    slot = torch.arange(K, device=idx.device).view(1, -1)
+    live = slot < torch.minimum(n_sel, valid).view(-1, 1)     # rows with fewer candidates than slots hold them all
+    ii = idx.long()
+    assert bool(((ii >= 0) & (ii < valid.view(-1, 1)) | ~live).all()), "index outside the valid prefix"
+    asc = (ii[:, 1:] > ii[:, :-1]) | ~live[:, 1:]
+    assert bool(asc.all()), "selected positions are not strictly ascending (duplicates?)"
+    s = scores.float()
+    pos = torch.arange(L, device=s.device).view(1, -1)
+    s = torch.where(pos < valid.view(-1, 1), s, torch.full_like(s, float("-inf")))
+    chosen = torch.zeros(R, L + 1, dtype=torch.bool, device=s.device)
+    chosen.scatter_(1, torch.where(live, ii, torch.full_like(ii, L)), True)
+    chosen = chosen[:, :L]
+    lo = torch.where(chosen, s, torch.full_like(s, float("inf"))).amin(1)       # weakest selected
+    hi = torch.where(chosen, torch.full_like(s, float("-inf")), s).amax(1)      # strongest left out
+    full = n_sel < valid
+    assert bool((lo[full] >= hi[full]).all()), "a left-out score beats a selected one"
+    assert bool((chosen.sum(1) == torch.minimum(n_sel, valid)).all())
+
+
+def _sequence_to_host(pages, block_table_row, n):
+    """Rows of one sequence gathered on the device: [1,n,G,D] on the host."""
+    ps = pages.shape[1]
+    rows = (block_table_row.long().view(-1, 1) * ps + torch.arange(ps, device=pages.device)).view(-1)[:n]
+    return pages.view(-1, G, D)[rows].view(1, n, G, D).cpu()
+
+
+def test_config1_prefill_32k(cuda):
+    from kascade_amd import kernels, budgets, workloads
+    L = 32768
+    T = L // TILE
+    w = workloads.prefill_inputs(1, L, seed=0, device=cuda)
+    wc_q, wc_k, wc_v = w.q.cpu(), w.k.cpu(), w.v.cpu()
+    log_sum, o = kernels.prefill_recompute0(w.q, w.k, w.v)
+    ls1 = kernels.prefill_recompute1(w.q, w.k)
+    assert torch.equal(ls1, log_sum), "K-only log-sum pass differs from the dense pass"
+    for s in (0, 4096 + 32, 32768 - 64):       # sampled query rows against the oracle
+        want, lse = orc.dense_prefill(wc_q, wc_k, wc_v, rows=(s, s + 64))
+        assert_close(o[:, s:s + 64], want, f"dense prefill rows {s}..")
+        assert_close(log_sum[:, s:s + 64], lse, f"log_sum rows {s}..", atol=2e-3, rtol=1e-4)
+    scores = torch.empty(1, G, T, L, device=cuda, dtype=torch.float16)
+    kernels.prefill_aggregate(w.q, w.k, log_sum, scores, fill_invalid=True)
+    for ta in (1, 300, T - 1):                  # sampled tiles
+        want = orc.pooled_prefill_scores(wc_q, wc_k, TILE, tiles=(ta, ta + 1))
+        got = scores[:, :, ta:ta + 1].cpu()
+        fin = torch.isfinite(want)
+        assert torch.equal(torch.isfinite(got), fin)
+        assert_close(torch.where(fin, got, torch.zeros(())), torch.where(fin, want, torch.zeros(())).float(),
+                     f"pooled scores tile {ta}", atol=2e-6, rtol=2e-3)
+    # mass: a tile row holds at most the 128 unit masses of its (query, head) rows
+    mass = torch.where(torch.isfinite(scores), scores.float(), torch.zeros((), device=cuda)).sum(-1)
+    assert float(mass.max()) <= 128.5 and float(mass.min()) >= 0.0
+    K = budgets.topk_width(L, P)
+    assert K == 3328
+    valid, nsel = budgets.prefill_tile_budgets(L, TILE, P, True, K)
+    vl = torch.tensor(valid, dtype=torch.int32, device=cuda)
+    ns = torch.tensor(nsel, dtype=torch.int32, device=cuda)
+    idx = kernels.topk_indices(scores, K, valid_len=vl, n_sel=ns)
+    _check_selection_on_device(scores.view(G * T, L), idx.view(G * T, K), ns.long().repeat(G), vl.long().repeat(G))
+    hm = torch.tensor(w.head_mapping, dtype=torch.int32, device=cuda)
+    got = kernels.prefill_reuse(w.q_reuse, w.k_reuse, w.v, idx, hm, float(P), True)
+    idx_c = idx.cpu()
+    for ta in (3, 200, T - 1):
+        want = orc.reuse_prefill(w.q_reuse.cpu(), w.k_reuse.cpu(), wc_v, idx_c, w.head_mapping, TILE, True, P,
+                                 tiles=(ta, ta + 1))
+        assert_close(got[:, ta * TILE:(ta + 1) * TILE], want, f"reuse prefill tile {ta}")
+
+
+def test_config2_paged_decode_b16_65536(cuda):
+    from kascade_amd import kernels, budgets, workloads
+    from kascade_amd.strategy import PagedKascadeDecoder
+    B, L = 16, 65536
+    c = workloads.paged_decode_inputs([L] * B, seed=10, device=cuda, reuse_keys=False)
+    maps = [list(range(G)), c.head_mapping]
+    dec = PagedKascadeDecoder(P, maps, [0], B, L, page_size=c.page_size, device=cuda)
+    o0 = dec.forward(0, c.q, c.k_pages, c.v_pages, c.block_table, c.seqlens, L, ragged=False).clone()
+    idx = dec._topk_to_reuse
+    K = budgets.topk_width(L, P)
+    assert tuple(idx.shape) == (B, G, K) and K == 6656
+    o1 = dec.forward(1, c.q_reuse, c.k_pages, c.v_pages, c.block_table, c.seqlens, L).clone()
+    # oracle on two sequences (their pages gathered to the host)
+    for b in (0, B - 1):
+        kc = _sequence_to_host(c.k_pages, c.block_table[b], L)
+        vc = _sequence_to_host(c.v_pages, c.block_table[b], L)
+        want0, _ = orc.dense_decode(c.q[b:b + 1].cpu(), kc, vc)
+        assert_close(o0[b:b + 1], want0, f"dense decode, sequence {b}")
+        want1 = orc.reuse_decode(c.q_reuse[b:b + 1].cpu(), kc, vc, idx[b:b + 1].cpu(), c.head_mapping)
+        assert_close(o1[b:b + 1], want1, f"reuse decode, sequence {b}")
+        agg_want = orc.pooled_decode_scores(c.q[b:b + 1].cpu(), kc)
+        for g in (0, 5):
+            ok, _, msg = orc.topk_agreement(agg_want[0, g], idx[b, g].cpu(), K, L, ulps=1.0)
+            assert ok, f"sequence {b} group {g}: {msg}"
+    # the pooled probabilities of a (sequence, KV head) sum to its 4 heads; selection is exact on them
+    glse, part = dec._scratch(B, dec.ns_dense)
+    row_sums = torch.empty(B, H, device=cuda, dtype=torch.float32)
+    scr = torch.empty(B, H, L, device=cuda, dtype=torch.float32)
+    _, agg = kernels.decode_recompute(c.q, c.k_pages, c.v_pages, glse, part, row_sums, scr, 1, cache_seqlens=c.seqlens,
+                                      block_table=c.block_table, page_size=c.page_size, kv_len=L)
+    assert float((agg.float().sum(-1) - 4.0).abs().max()) < 5e-2
+    full = torch.full((B * G,), L, dtype=torch.int64, device=cuda)
+    own = kernels.topk_indices(agg, K, fill_value=0)
+    _check_selection_on_device(agg.view(B * G, L), own.view(B * G, K), torch.full_like(full, K), full)
+    # split-count independence and block-table permutation invariance (contiguous layout = identity table)
+    glse7 = torch.empty(B, H, 7, device=cuda, dtype=torch.float32)
+    part7 = torch.empty(B, H, 7, D, device=cuda, dtype=torch.float32)
+    o7 = kernels.decode_dense_paged(c.q, c.k_pages, c.v_pages, c.seqlens, glse7, part7, c.block_table, c.page_size, kv_len=L)
+    assert_close(o7, o0, "dense decode with 7 splits vs the default", atol=1e-3, rtol=2e-3)
+    b = 3
+    rows = (c.block_table[b].long().view(-1, 1) * c.page_size + torch.arange(c.page_size, device=cuda)).view(-1)
+    kc = c.k_pages.view(-1, G, D)[rows].view(1, L, G, D)
+    vc = c.v_pages.view(-1, G, D)[rows].view(1, L, G, D)
+    hm = torch.tensor(c.head_mapping, dtype=torch.int32, device=cuda)
+    g4, p4 = torch.empty(1, H, 4, device=cuda, dtype=torch.float32), torch.empty(1, H, 4, D, device=cuda, dtype=torch.float32)
+    lens1 = c.seqlens[b:b + 1].contiguous()
+    r_paged = kernels.decode_reuse_paged(c.q_reuse[b:b + 1], c.k_pages, c.v_pages, lens1, idx[b:b + 1].contiguous(), hm, 0.0,
+                                         g4, p4, block_table=c.block_table[b:b + 1].contiguous(), page_size=c.page_size)
+    r_contig = kernels.decode_reuse_paged(c.q_reuse[b:b + 1], kc, vc, lens1, idx[b:b + 1].contiguous(), hm, 0.0,
+                                          g4.clone(), p4.clone())
+    assert torch.equal(r_paged, r_contig), "paged and contiguous layouts differ"
+
+
+def test_config3_ragged_long_decode(cuda):
+    from kascade_amd import kernels, budgets, workloads
+    from kascade_amd.strategy import PagedKascadeDecoder
+    seqlens = [131072, 196608, 262144, 524288]
+    B, Lmax = len(seqlens), max(seqlens)
+    c = workloads.paged_decode_inputs(seqlens, seed=20, device=cuda, reuse_keys=False)
+    maps = [list(range(G)), c.head_mapping]
+    dec = PagedKascadeDecoder(P, maps, [0], B, Lmax, page_size=c.page_size, device=cuda, total_tokens=sum(seqlens))
+    o0 = dec.forward(0, c.q, c.k_pages, c.v_pages, c.block_table, c.seqlens, Lmax, ragged=True).clone()
+    idx = dec._topk_to_reuse
+    W = budgets.decode_budget(Lmax, P)
+    counts = [budgets.decode_budget(n, P) for n in seqlens]
+    assert W == 52480 and counts == [13184, 19712, 26240, 52480] and tuple(idx.shape) == (B, G, W)
+    o1 = dec.forward(1, c.q_reuse, c.k_pages, c.v_pages, c.block_table, c.seqlens, Lmax).clone()
+    # oracle on the shortest sequence
+    b, n = 0, seqlens[0]
+    kc = _sequence_to_host(c.k_pages, c.block_table[b], n)
+    vc = _sequence_to_host(c.v_pages, c.block_table[b], n)
+    want0, _ = orc.dense_decode(c.q[b:b + 1].cpu(), kc, vc)
+    assert_close(o0[b:b + 1], want0, "ragged dense decode, shortest sequence")
+    want1 = orc.reuse_decode(c.q_reuse[b:b + 1].cpu(), kc, vc, idx[b:b + 1].cpu(), c.head_mapping, [counts[b]])
+    assert_close(o1[b:b + 1], want1, "ragged reuse decode, shortest sequence")
+    # pooled probabilities: mass 4 per (sequence, KV head), zero beyond each length; the multi-workgroup
+    # selection is exact on them for every row
+    glse, part = dec._scratch(B, dec.ns_dense)
+    row_sums = torch.empty(B, H, device=cuda, dtype=torch.float32)
+    scr = torch.empty(B, H, Lmax, device=cuda, dtype=torch.float32)
+    _, agg = kernels.decode_recompute(c.q, c.k_pages, c.v_pages, glse, part, row_sums, scr, 1, cache_seqlens=c.seqlens,
+                                      block_table=c.block_table, page_size=c.page_size, kv_len=Lmax)
+    assert float((agg.float().sum(-1) - 4.0).abs().max()) < 5e-2
+    for bb, nn in enumerate(seqlens):
+        if nn < Lmax:
+            assert float(agg[bb, :, nn:].abs().max()) == 0.0
+    lens_rows = c.seqlens.repeat_interleave(G)
+    cnt_rows = torch.tensor(counts, dtype=torch.int32, device=cuda).repeat_interleave(G)
+    own = kernels.topk_indices(agg[:, :, :Lmax], W, valid_len=lens_rows, n_sel=cnt_rows, fill_value=0)
+    _check_selection_on_device(agg.view(B * G, Lmax), own.view(B * G, W), cnt_rows.long(), lens_rows.long())
+
+
+def test_config4_chunked_prefill_16384_equals_whole_prompt(cuda):
+    """One anchor and one reuse layer of the 16384-token prompt in 8 chunks of 2048 over the paged
+    cache against the whole-prompt calls: bit-equal rows."""
+    from kascade_amd import kernels, workloads
+    from kascade_amd.strategy import EfficientKascadeStrategy, PagedKascadePrefill
+    L, chunk = 16384, 2048
+    w = workloads.prefill_inputs(1, L, seed=4, device=cuda)
+    maps = [list(range(G)), w.head_mapping]
+    whole = EfficientKascadeStrategy([0], None, k=P, tile_size=TILE, rolling_prefill=True, head_mapping=maps,
+                                     register=False)
+    want0 = whole._prefill_recomp_forward(w.q, w.k, w.v, orc.k_kern(L, P), TILE, 0, P)
+    want1 = whole._prefill_reuse_forward(w.q_reuse, w.k_reuse, w.v, P, 1)
+    pre = PagedKascadePrefill(P, maps, [0], page_size=16, rolling_prefill=True, device=cuda)
+    n_pages = L // 16
+    bt = torch.randperm(n_pages, generator=torch.Generator().manual_seed(1)).to(torch.int32).view(1, -1).to(cuda)
+    caches = [(torch.zeros(n_pages, 16, G, D, device=cuda, dtype=torch.float16),
+               torch.zeros(n_pages, 16, G, D, device=cuda, dtype=torch.float16)) for _ in range(2)]
+    for s in range(0, L, chunk):
+        sl = slice(s, s + chunk)
+        start = torch.full((1,), s, dtype=torch.int32, device=cuda)
+        kernels.paged_kv_append(caches[0][0], caches[0][1], w.k[:, sl], w.v[:, sl], start, bt, 16)
+        kernels.paged_kv_append(caches[1][0], caches[1][1], w.k_reuse[:, sl], w.v[:, sl], start, bt, 16)
+        got0 = pre.forward(0, w.q[:, sl], caches[0][0], caches[0][1], bt, s)
+        got1 = pre.forward(1, w.q_reuse[:, sl], caches[1][0], caches[1][1], bt, s)
+        assert torch.equal(got0, want0[:, sl]), f"anchor layer differs in the chunk at {s}"
+        assert torch.equal(got1, want1[:, sl]), f"reuse layer differs in the chunk at {s}"
