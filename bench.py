@@ -408,7 +408,42 @@ def main():
         gi = torch.randint(0, rows.shape[0], (1 << 21,), device=dev)
         t = ev_time(lambda: torch.index_select(rows, 0, gi), n=5)
         ceilings["gather_256B_rows_read_GBps"] = round(gi.numel() * 256 / t / 1e3, 1)
-        del x, xf, rows, gi
+        # the same two patterns with this library's plain read kernels (no arithmetic, no tuning
+        # beyond 8 loads in flight per lane): 8 GiB stream; a gather shaped like the reuse decode --
+        # 128 ascending lists of distinct random 256-byte rows, 10 % of the 262144 tokens of
+        # "their" sequence, row pitch 2 KiB (8 KV heads), K alone and K+V
+        lib = _lib.init()
+        sink = torch.zeros(16, dtype=torch.uint8, device=dev)
+        big = torch.empty(8 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        big2 = torch.empty_like(big).fill_(2)
+        st = torch.cuda.current_stream().cuda_stream
+        flush = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+
+        def cold_time(fn, n=5):
+            """Median duration (us) with the caches flushed (1 GiB fill) before every timed call."""
+            ts = []
+            for _ in range(n + 1):
+                flush.fill_(3)
+                s0, e0 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                s0.record(); fn(); e0.record(); e0.synchronize()
+                ts.append(s0.elapsed_time(e0) * 1e3)
+            ts = sorted(ts[1:])
+            return ts[len(ts) // 2]
+
+        t = cold_time(lambda: _lib.check(lib.kascade_diag_stream_read_call(big.data_ptr(), big.numel(), sink.data_ptr(), st)))
+        ceilings["plain_stream_read_GBps"] = round(big.numel() / t / 1e3, 1)
+        ntok = big.numel() // 2048                      # 16 sequences of 262144 tokens
+        per_seq, n_sel = ntok // 16, (ntok // 16) // 10 // 128 * 128
+        gen = torch.Generator(device=dev); gen.manual_seed(1)
+        ids = torch.rand(16, 8, per_seq, device=dev, generator=gen).argsort(-1)[..., :n_sel].to(torch.int32)   # distinct
+        ids = (ids.sort(-1).values + (torch.arange(16, device=dev, dtype=torch.int32) * per_seq).view(16, 1, 1)).contiguous()
+        for name, second in (("plain_gather_256B_K_GBps", None), ("plain_gather_256B_K_and_V_GBps", big2)):
+            t = cold_time(lambda: _lib.check(lib.kascade_diag_gather_rows_call(
+                big.data_ptr(), None if second is None else second.data_ptr(), ids.data_ptr(), ids.numel(), 2048,
+                sink.data_ptr(), st)))
+            ceilings[name] = round(ids.numel() * 256 * (1 if second is None else 2) / t / 1e3, 1)
+        del flush
+        del x, xf, rows, gi, big, big2, ids
         n = 8192
         a, b2 = torch.randn(n, n, device=dev, dtype=torch.float16), torch.randn(n, n, device=dev, dtype=torch.float16)
         t = ev_time(lambda: a @ b2, n=5, warm=2)

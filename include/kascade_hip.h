@@ -251,6 +251,19 @@ int kascade_translate_indices_call(const int32_t* token_idx, int32_t* physical_r
                                    const int32_t* block_table, int batch, int64_t per_sequence,
                                    int max_pages, int page_size, int kv_len, void* stream);
 
+/* ------------------------------------------------------------- diagnostics */
+
+/* Read-only kernels with no arithmetic, for measuring what the device delivers to the two access
+ * patterns of the decode path (no counterpart in the reference; used by the benchmark only).
+ * Nothing is written except, never in practice, 16 bytes at `sink`.
+ *   stream_read: reads `bytes` bytes of src, 16 bytes per lane, four loads in flight per lane.
+ *   gather_rows: for each of the n_rows entries of row_ids reads the 256 bytes at
+ *                rows_a + row_ids[i]*row_stride_bytes (and the same row of rows_b when non-NULL),
+ *                16 lanes per row; every id must address a row inside the arrays. */
+int kascade_diag_stream_read_call(const void* src, int64_t bytes, void* sink, void* stream);
+int kascade_diag_gather_rows_call(const void* rows_a, const void* rows_b, const int32_t* row_ids,
+                                  int64_t n_rows, int64_t row_stride_bytes, void* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -57,6 +57,8 @@ SIGNATURES = {
     "kascade_prefill_chunk_reuse_call": (_I, [_P, _P, _P, _P, _P, _F, _P, _I, _I, _I, _I, _I, Strides,
                                               _P, _I, _I, _I, _P]),
     "kascade_translate_indices_call": (_I, [_P, _P, _P, _I, C.c_int64, _I, _I, _I, _P]),
+    "kascade_diag_stream_read_call": (_I, [_P, _L, _P, _P]),
+    "kascade_diag_gather_rows_call": (_I, [_P, _P, _P, _L, _L, _P, _P]),
 }
 
 _lib = None

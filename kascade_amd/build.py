@@ -16,7 +16,7 @@ from pathlib import Path
 PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "libkascade_hip.so"
-SOURCES = ["capi.hip", "decode.hip", "topk.hip", "prefill.hip", "paged.hip"]
+SOURCES = ["capi.hip", "decode.hip", "topk.hip", "prefill.hip", "paged.hip", "diag.hip"]
 ARCH = "gfx950"
 
 # -packed-fp32-ops is switched off for device code: hipcc otherwise forms

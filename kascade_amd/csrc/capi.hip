@@ -9,6 +9,7 @@
 #include <string.h>
 
 #include "decode.h"
+#include "diag.h"
 #include "paged.h"
 #include "prefill.h"
 #include "topk.h"
@@ -418,6 +419,27 @@ int kascade_translate_indices_call(const int32_t* token_idx, int32_t* physical_r
                                               per_sequence, max_pages, shift, kv_len,
                                               static_cast<hipStream_t>(stream)),
                      "translate_indices");
+}
+
+// ---- diagnostics ----
+
+int kascade_diag_stream_read_call(const void* src, int64_t bytes, void* sink, void* stream) {
+    REQUIRE(src && sink, "diag_stream_read: null pointer argument");
+    REQUIRE(bytes >= 16 && aligned16(src) && aligned16(sink), "diag_stream_read: need >= 16 bytes, 16-byte aligned");
+    const int cus = g_cu_count > 0 ? g_cu_count : 256;
+    return check_hip(launch_diag_stream_read(src, bytes, sink, cus * 32, static_cast<hipStream_t>(stream)),
+                     "diag_stream_read");
+}
+
+int kascade_diag_gather_rows_call(const void* rows_a, const void* rows_b, const int32_t* row_ids,
+                                  int64_t n_rows, int64_t row_stride_bytes, void* sink, void* stream) {
+    REQUIRE(rows_a && row_ids && sink, "diag_gather_rows: null pointer argument");
+    REQUIRE(n_rows > 0 && row_stride_bytes >= 256 && row_stride_bytes % 16 == 0,
+            "diag_gather_rows: n_rows > 0 and a row stride of at least 256 bytes, multiple of 16, required");
+    REQUIRE(aligned16(rows_a) && (!rows_b || aligned16(rows_b)) && aligned16(sink),
+            "diag_gather_rows: arrays must be 16-byte aligned");
+    return check_hip(launch_diag_gather_rows(rows_a, rows_b, row_ids, n_rows, 128, row_stride_bytes, sink,
+                                             static_cast<hipStream_t>(stream)), "diag_gather_rows");
 }
 
 }  // extern "C"
