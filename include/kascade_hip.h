@@ -38,6 +38,13 @@ extern "C" {
 
 typedef uint16_t kascade_half; /* IEEE binary16 bit pattern */
 
+/* Strides are in elements; the innermost (D) dimension is contiguous.  A tensor
+ * laid out [B,L,H,D] has (s_b, s_l, s_h) = (L*H*D, H*D, D); HF's [B,H,L,D]
+ * seen as [B,L,H,D] has (H*L*D, D, L*D). */
+typedef struct {
+    int64_t b, l, h;
+} kascade_strides;
+
 /* Replaces `init()` of every reference kernel object (e.g. decode reuse .cu:253-258):
  * one-time device query and kernel attribute set-up for the current device. */
 int kascade_init(void);
@@ -84,15 +91,20 @@ int kascade_decode_reuse_call(const kascade_half* Q, const kascade_half* K, cons
  *   n(b) = 128*ceil(floor(topk_percent*cache_seqlens[b]/100)/128)  if topk_percent > 0
  *   n(b) = topk                                                   otherwise,
  * clamped to `topk` (the row width of topk_indices).
- *   block_table [B,max_pages] i32 or NULL (then K,V are [B,kv_stride_tokens,G,D]). */
+ *   block_table [B,max_pages] i32 or NULL (then K,V are [B,kv_stride_tokens,G,D]).
+ *   kv_strides  NULL, or (only without a block table) the element strides (b, l, h) of K and V
+ *               seen as [B,tokens,G,D]: multiples of 8, D contiguous.  Lets the kernels read a
+ *               head-major [B,G,tokens,D] cache (Hugging Face's layout) in place, where the
+ *               reference copies the whole cache to [B,tokens,G,D] on every decode step
+ *               (EfficientKascadeStrategy.py:149-150). */
 int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K,
                                     const kascade_half* V, const int32_t* cache_seqlens,
                                     const int32_t* topk_indices, const int32_t* head_mapping,
                                     float topk_percent, float* glse, float* Output_partial,
                                     kascade_half* Output, int batch, int kv_stride_tokens,
                                     int topk, int num_split, const int32_t* block_table,
-                                    int max_pages, int page_size, int32_t* sync_counters,
-                                    void* stream);
+                                    int max_pages, int page_size, const kascade_strides* kv_strides,
+                                    int32_t* sync_counters, void* stream);
 
 /* Dense split-K decode (the reference's TileLang dense baseline, gqa_decode.py:117-254 and
  * gqa_decode_with_kvcache.py:118-257), same cache conventions as above.
@@ -104,7 +116,8 @@ int kascade_decode_dense_paged_call(const kascade_half* Q, const kascade_half* K
                                     float* glse, float* Output_partial, kascade_half* Output,
                                     int batch, int kv_stride_tokens, int num_split,
                                     const int32_t* block_table, int max_pages, int page_size,
-                                    int32_t* sync_counters, void* stream);
+                                    const kascade_strides* kv_strides, int32_t* sync_counters,
+                                    void* stream);
 
 /* Anchor-layer decode: split QK^T (+PV when with_output != 0), log-sum merge and
  * pooled post-softmax scores.  Replaces the three launches of the reference's
@@ -123,8 +136,9 @@ int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_hal
                                         kascade_half* aggregated_scores, int batch,
                                         int kv_stride_tokens, int scores_stride, int num_split,
                                         int with_output, const int32_t* block_table,
-                                        int max_pages, int page_size, int32_t* sync_counters,
-                                        void* stream);
+                                        int max_pages, int page_size,
+                                        const kascade_strides* kv_strides,
+                                        int32_t* sync_counters, void* stream);
 
 /* ------------------------------------------------------------------- top-k */
 
@@ -149,13 +163,6 @@ int kascade_topk_call(const kascade_half* scores, int32_t* out_idx, int rows, in
                       int k, int fill_value, void* workspace, void* stream);
 
 /* ----------------------------------------------------------------- prefill */
-
-/* Strides are in elements; the innermost (D) dimension is contiguous.  A tensor
- * laid out [B,L,H,D] has (s_b, s_l, s_h) = (L*H*D, H*D, D); HF's [B,H,L,D]
- * seen as [B,L,H,D] has (H*L*D, D, L*D). */
-typedef struct {
-    int64_t b, l, h;
-} kascade_strides;
 
 /* Anchor layer 0: dense causal GQA flash attention that also emits the log2
  * log-sum per (token, head).  Replaces `prefill`

@@ -29,6 +29,7 @@ _P = C.c_void_p
 _I = C.c_int
 _F = C.c_float
 _L = C.c_int64
+_SP = C.POINTER(Strides)   # optional kascade_strides*
 
 # name -> (restype, argtypes); must list every symbol of include/kascade_hip.h
 SIGNATURES = {
@@ -38,11 +39,11 @@ SIGNATURES = {
     "kascade_device_cu_count": (_I, []),
     "kascade_decode_reuse_call": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _P]),
     "kascade_decode_reuse_paged_call": (_I, [_P, _P, _P, _P, _P, _P, _F, _P, _P, _P, _I, _I, _I, _I,
-                                             _P, _I, _I, _P, _P]),
-    "kascade_decode_dense_paged_call": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _I, _I, _P,
-                                             _P]),
+                                             _P, _I, _I, _SP, _P, _P]),
+    "kascade_decode_dense_paged_call": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _I, _I, _SP,
+                                             _P, _P]),
     "kascade_decode_recompute_paged_call": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I,
-                                                 _I, _I, _P, _I, _I, _P, _P]),
+                                                 _I, _I, _P, _I, _I, _SP, _P, _P]),
     "kascade_topk_workspace_bytes": (_L, [_I, _L]),
     "kascade_topk_call": (_I, [_P, _P, _I, _L, _I, _P, _P, _I, _I, _I, _P, _P]),
     "kascade_prefill_dense_call": (_I, [_P, _P, _P, _P, _P, _I, _I, Strides, Strides, _I, _P]),

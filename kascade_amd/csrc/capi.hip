@@ -69,11 +69,30 @@ int check_paging(const int32_t* block_table, int max_pages, int page_size, int* 
     return 0;
 }
 
+// K/V addressing of the decode calls without a block table: `strides` (elements, may be NULL
+// for the contiguous [B,kv_stride_tokens,G,D] cache).
+int set_kv_strides(DecodeParams& p, const kascade_strides* strides, const int32_t* block_table,
+                   int kv_stride_tokens) {
+    if (!strides) {
+        p.kv_stride_b = (long long)kv_stride_tokens * kGroups * kDim;
+        p.kv_stride_l = kGroups * kDim;
+        p.kv_stride_h = kDim;
+        return 0;
+    }
+    REQUIRE(!block_table, "kv_strides and block_table exclude each other");
+    if (check_strides(*strides, "decode K/V")) return -1;
+    REQUIRE(strides->b >= 0, "decode K/V batch stride must not be negative");
+    p.kv_stride_b = strides->b;
+    p.kv_stride_l = (unsigned)strides->l;
+    p.kv_stride_h = strides->h;
+    return 0;
+}
+
 }  // namespace
 
 extern "C" {
 
-int kascade_abi_version(void) { return 2; }
+int kascade_abi_version(void) { return 3; }
 
 const char* kascade_get_last_error(void) { return g_err; }
 
@@ -97,7 +116,7 @@ int kascade_decode_reuse_call(const kascade_half* Q, const kascade_half* K, cons
                               void* stream) {
     return kascade_decode_reuse_paged_call(Q, K, V, nullptr, topk_indices, head_mapping, 0.f, glse,
                                            Output_partial, Output, batch, kv_seqlen, topk,
-                                           num_split, nullptr, 0, 1, sync_counters, stream);
+                                           num_split, nullptr, 0, 1, nullptr, sync_counters, stream);
 }
 
 int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K,
@@ -106,8 +125,8 @@ int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K
                                     float topk_percent, float* glse, float* Output_partial,
                                     kascade_half* Output, int batch, int kv_stride_tokens,
                                     int topk, int num_split, const int32_t* block_table,
-                                    int max_pages, int page_size, int32_t* sync_counters,
-                                    void* stream) {
+                                    int max_pages, int page_size, const kascade_strides* kv_strides,
+                                    int32_t* sync_counters, void* stream) {
     REQUIRE(Q && K && V && topk_indices && head_mapping && glse && Output_partial && Output,
             "decode_reuse: null pointer argument");
     REQUIRE(batch > 0 && topk > 0 && num_split > 0, "decode_reuse: batch, topk, num_split must be > 0");
@@ -122,6 +141,7 @@ int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K
     p.seqlens = cache_seqlens; p.idx = topk_indices; p.head_map = head_mapping;
     p.block_table = block_table; p.glse = glse; p.opart = Output_partial; p.scores = nullptr;
     p.max_pages = max_pages; p.page_shift = shift; p.kv_stride_tokens = kv_stride_tokens;
+    if (set_kv_strides(p, kv_strides, block_table, kv_stride_tokens)) return -1;
     p.topk = topk; p.topk_percent = topk_percent; p.scores_stride = 0; p.num_split = num_split;
     p.rows_per_split = rows_per_split(topk, num_split);
     p.B = batch;
@@ -138,7 +158,8 @@ int kascade_decode_dense_paged_call(const kascade_half* Q, const kascade_half* K
                                     float* glse, float* Output_partial, kascade_half* Output,
                                     int batch, int kv_stride_tokens, int num_split,
                                     const int32_t* block_table, int max_pages, int page_size,
-                                    int32_t* sync_counters, void* stream) {
+                                    const kascade_strides* kv_strides, int32_t* sync_counters,
+                                    void* stream) {
     REQUIRE(Q && K && V && glse && Output_partial && Output, "decode_dense: null pointer argument");
     REQUIRE(batch > 0 && num_split > 0, "decode_dense: batch, num_split must be > 0");
     REQUIRE(batch <= 65535, "decode_dense: batch exceeds grid limit");
@@ -151,6 +172,7 @@ int kascade_decode_dense_paged_call(const kascade_half* Q, const kascade_half* K
     p.Q = H(Q); p.K = H(K); p.V = H(V);
     p.seqlens = cache_seqlens; p.block_table = block_table; p.glse = glse; p.opart = Output_partial;
     p.max_pages = max_pages; p.page_shift = shift; p.kv_stride_tokens = kv_stride_tokens;
+    if (set_kv_strides(p, kv_strides, block_table, kv_stride_tokens)) return -1;
     p.num_split = num_split; p.B = batch;
     const long long max_rows = kv_stride_tokens > 0 ? kv_stride_tokens : (long long)max_pages * page_size;
     p.rows_per_split = rows_per_split(max_rows, num_split);
@@ -169,8 +191,9 @@ int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_hal
                                         kascade_half* aggregated_scores, int batch,
                                         int kv_stride_tokens, int scores_stride, int num_split,
                                         int with_output, const int32_t* block_table,
-                                        int max_pages, int page_size, int32_t* sync_counters,
-                                        void* stream) {
+                                        int max_pages, int page_size,
+                                        const kascade_strides* kv_strides,
+                                        int32_t* sync_counters, void* stream) {
     REQUIRE(Q && K && glse && row_sums && scores && aggregated_scores,
             "decode_recompute: null pointer argument");
     REQUIRE(!with_output || (V && Output && Output_partial),
@@ -193,6 +216,7 @@ int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_hal
     p.seqlens = cache_seqlens; p.block_table = block_table; p.glse = glse; p.opart = Output_partial;
     p.scores = scores; p.scores_stride = scores_stride;
     p.max_pages = max_pages; p.page_shift = shift; p.kv_stride_tokens = kv_stride_tokens;
+    if (set_kv_strides(p, kv_strides, block_table, kv_stride_tokens)) return -1;
     p.num_split = num_split; p.B = batch;
     long long max_rows = kv_stride_tokens > 0 ? kv_stride_tokens : (long long)max_pages * page_size;
     if (max_rows > scores_stride) max_rows = scores_stride;

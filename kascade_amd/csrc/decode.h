@@ -6,7 +6,7 @@ namespace kascade {
 
 struct DecodeParams {
     const half_t* Q;        // [B,H,D]
-    const half_t* K;        // pages [P,page,G,D] or contiguous [B,stride,G,D]
+    const half_t* K;        // pages [P,page,G,D], or a strided [B,tokens,G,D] view
     const half_t* V;
     const int* seqlens;     // [B] or null
     const int* idx;         // [B,G,topk] logical token ids (gather mode)
@@ -23,7 +23,12 @@ struct DecodeParams {
     float* row_sums;
     int max_pages;
     int page_shift;
-    int kv_stride_tokens;
+    int kv_stride_tokens;   // without seqlens: tokens per sequence; with: an upper bound
+    // Without a block table, element (b, token, g, 0) of K and V sits at
+    // b*kv_stride_b + token*kv_stride_l + g*kv_stride_h (multiples of 8 elements).
+    long long kv_stride_b;
+    long long kv_stride_h;
+    unsigned kv_stride_l;
     int topk;
     float topk_percent;
     int scores_stride;

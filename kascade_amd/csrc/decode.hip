@@ -114,7 +114,12 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
     const int* idx_row = nullptr;
     if (GATHER) idx_row = p.idx + ((size_t)b * kGroups + p.head_map[g]) * p.topk;
     const int page_mask = (1 << p.page_shift) - 1;
+    // Element offset of (token row r, this head, this lane's slice): paged rows are physical rows
+    // of [P*page,G,D]; without a table rows are token numbers of sequence b behind the caller's
+    // (batch, token, head) strides, so a head-major cache is read in place.
     const size_t head_off = (size_t)g * kDim + dl * 8;
+    const size_t strided_off = (size_t)b * p.kv_stride_b + (size_t)g * p.kv_stride_h + dl * 8;
+    const unsigned stride_l = p.kv_stride_l;
 
     struct Batch {
         Pack16 k[kUnroll];
@@ -122,10 +127,12 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
     };
     // A wavefront covers 4*kUnroll consecutive rows of an iteration: row = it + wave*4U + u*4 + rg.
     // `rows` are physical row numbers (page*page_size + slot, or b*stride + token).
-    auto issue_loads = [&](const int (&rows)[kUnroll], Batch& bt) {
+    auto issue_loads = [&](auto paged_tag, const int (&rows)[kUnroll], Batch& bt) {
+        constexpr bool PAGED = decltype(paged_tag)::value;
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-            const size_t off = (size_t)rows[u] * (kGroups * kDim) + head_off;
+            const size_t off = PAGED ? (size_t)rows[u] * (kGroups * kDim) + head_off
+                                     : (size_t)(unsigned)rows[u] * stride_l + strided_off;
             bt.k[u].u = ld_global_16(p.K + off);
             if (WITH_V) bt.v[u].u = ld_global_16(p.V + off);
         }
@@ -194,6 +201,7 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
 
     if (GATHER) {
         // Index list -> block table -> physical row, staged in LDS one sub-chunk at a time.
+        auto run = [&](auto paged_tag) {
         for (int c0 = r0; c0 < r1; c0 += kSubChunk) {
             const int cn = min(kSubChunk, r1 - c0);
             __syncthreads();
@@ -205,7 +213,7 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
                     int pg = p.block_table[(size_t)b * p.max_pages + (tok >> p.page_shift)];
                     row = (pg << p.page_shift) + (tok & page_mask);
                 } else {
-                    row = b * p.kv_stride_tokens + tok;
+                    row = tok;
                 }
                 s_row[i] = row;
             }
@@ -219,20 +227,22 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
             Batch ba, bb;
             int rows[kUnroll];
             staged_rows(0, rows);
-            issue_loads(rows, ba);
+            issue_loads(paged_tag, rows, ba);
             for (int it = 0; it < cn; it += 2 * kRowsPerIter) {
                 staged_rows(it + kRowsPerIter, rows);      // rows past the end are clamped and masked
-                issue_loads(rows, bb);
+                issue_loads(paged_tag, rows, bb);
                 KASCADE_SCHED_FENCE();
                 compute_batch(it + wave * (4 * kUnroll) + rg, cn, c0, 0, 0, ba);
                 KASCADE_SCHED_FENCE();
                 staged_rows(it + 2 * kRowsPerIter, rows);
-                issue_loads(rows, ba);
+                issue_loads(paged_tag, rows, ba);
                 KASCADE_SCHED_FENCE();
                 compute_batch(it + kRowsPerIter + wave * (4 * kUnroll) + rg, cn, c0, 0, 0, bb);
                 KASCADE_SCHED_FENCE();
             }
         }
+        };
+        if (p.block_table) run(std::true_type{}); else run(std::false_type{});
     } else {
         // Dense range [r0, r1): no staging and no barriers.  Three-stage pipeline: block-table
         // entries two iterations ahead, K/V rows one iteration ahead, arithmetic on the current.
@@ -280,7 +290,7 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u) {
                 const int tok = tok_of(it, u);
-                rows[u] = PAGED ? (pg[u] << p.page_shift) + (tok & page_mask) : b * p.kv_stride_tokens + tok;
+                rows[u] = PAGED ? (pg[u] << p.page_shift) + (tok & page_mask) : tok;
             }
         };
         if (cn > 0) {
@@ -291,7 +301,7 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
             int pga[kUnroll], pgb[kUnroll], rows[kUnroll];
             fetch_pages(0, pga);
             rows_of(0, pga, rows);
-            issue_loads(rows, ba);
+            issue_loads(paged_tag, rows, ba);
             fetch_pages(kRowsPerIter, pgb);
             // every wavefront runs the same number of batches: enough for the longest strip
             const int full = cn / (4 * kStripRows), rem = cn - full * (4 * kStripRows);
@@ -309,13 +319,13 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
                 const int q = it / kRowsPerIter;
                 fetch_pages(it + 2 * kRowsPerIter, pga);   // tokens past the end are clamped and masked
                 rows_of(it + kRowsPerIter, pgb, rows);
-                issue_loads(rows, bb);
+                issue_loads(paged_tag, rows, bb);
                 KASCADE_SCHED_FENCE();
                 compute_batch(rbase_of(it), cn, r0, q % kScoreBatches, (q / kScoreBatches) & 1, ba);
                 KASCADE_SCHED_FENCE();
                 fetch_pages(it + 3 * kRowsPerIter, pgb);
                 rows_of(it + 2 * kRowsPerIter, pga, rows);
-                issue_loads(rows, ba);
+                issue_loads(paged_tag, rows, ba);
                 KASCADE_SCHED_FENCE();
                 compute_batch(rbase_of(it + kRowsPerIter), cn, r0, (q + 1) % kScoreBatches, (q / kScoreBatches) & 1, bb);
                 KASCADE_SCHED_FENCE();

@@ -77,6 +77,22 @@ def _out_buffer(out, B, device) -> torch.Tensor:
     return out
 
 
+def _decode_kv(K, V, block_table):
+    """dtype / layout check of the decode K and V operands; returns the optional strides argument.
+    Pages must be contiguous.  Without a block table any [B,L,G,D] view with a contiguous last
+    dimension is read in place (e.g. a head-major [B,G,L,D] cache transposed), and the strides
+    are passed only when the view is not the plain contiguous layout."""
+    import ctypes
+    for t, name in ((K, "K"), (V, "V")):
+        _req(t, torch.float16, name, contiguous=block_table is not None)
+    if block_table is not None or (K.is_contiguous() and V.is_contiguous()):
+        return None
+    ks, vs = _blhd_strides(K, "K"), _blhd_strides(V, "V")
+    if (ks.b, ks.l, ks.h) != (vs.b, vs.l, vs.h) or K.shape != V.shape or K.shape[2] != G:
+        raise KascadeError("K and V must share one [B,L,8,128] shape and one set of strides")
+    return ctypes.byref(ks)
+
+
 def _sync_arg(sync, B):
     """Optional [B*G] int32 counter array for the fused combine (zero-initialised by the caller)."""
     if sync is None:
@@ -94,7 +110,8 @@ def decode_reuse(Q, K, V, topk_indices, head_mapping, glse, Output_partial, sync
     lib = _lib.init()
     B, Hq, Dq = Q.shape
     L = K.shape[1]
-    _req(Q, torch.float16, "Q"); _req(K, torch.float16, "K"); _req(V, torch.float16, "V")
+    _req(Q, torch.float16, "Q")
+    kv_strides = _decode_kv(K, V, None)
     _req(topk_indices, torch.int32, "topk_indices"); _req(head_mapping, torch.int32, "head_mapping")
     _req(glse, torch.float32, "glse"); _req(Output_partial, torch.float32, "Output_partial")
     if (Hq, Dq, K.shape[2]) != (H, D, G):
@@ -103,9 +120,15 @@ def decode_reuse(Q, K, V, topk_indices, head_mapping, glse, Output_partial, sync
     if tuple(glse.shape) != (B, H, ns) or tuple(Output_partial.shape) != (B, H, ns, D):
         raise KascadeError("glse must be [B,H,S] and Output_partial [B,H,S,D]")
     out = torch.empty(B, H, D, device=Q.device, dtype=torch.float16)
-    _lib.check(lib.kascade_decode_reuse_call(
-        _ptr(Q), _ptr(K), _ptr(V), _ptr(topk_indices), _ptr(head_mapping), _ptr(glse),
-        _ptr(Output_partial), _ptr(out), B, L, topk_indices.shape[-1], ns, _sync_arg(sync, B), _stream()))
+    if kv_strides is None:
+        _lib.check(lib.kascade_decode_reuse_call(
+            _ptr(Q), _ptr(K), _ptr(V), _ptr(topk_indices), _ptr(head_mapping), _ptr(glse),
+            _ptr(Output_partial), _ptr(out), B, L, topk_indices.shape[-1], ns, _sync_arg(sync, B), _stream()))
+    else:
+        _lib.check(lib.kascade_decode_reuse_paged_call(
+            _ptr(Q), _ptr(K), _ptr(V), None, _ptr(topk_indices), _ptr(head_mapping), 0.0, _ptr(glse),
+            _ptr(Output_partial), _ptr(out), B, L, topk_indices.shape[-1], ns, None, 0, 1, kv_strides,
+            _sync_arg(sync, B), _stream()))
     return out
 
 
@@ -118,7 +141,8 @@ def decode_reuse_paged(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_
     with one they are pages [P,page_size,G,D]."""
     lib = _lib.init()
     B = Q.shape[0]
-    _req(Q, torch.float16, "Q"); _req(K, torch.float16, "K"); _req(V, torch.float16, "V")
+    _req(Q, torch.float16, "Q")
+    kv_strides = _decode_kv(K, V, block_table)
     _req(topk_indices, torch.int32, "topk_indices"); _req(head_mapping, torch.int32, "head_mapping")
     _req(glse, torch.float32, "glse"); _req(Output_partial, torch.float32, "Output_partial")
     if cache_seqlens is not None:
@@ -133,7 +157,8 @@ def decode_reuse_paged(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_
     _lib.check(lib.kascade_decode_reuse_paged_call(
         _ptr(Q), _ptr(K), _ptr(V), _ptr(cache_seqlens), _ptr(topk_indices), _ptr(head_mapping),
         float(topk_percent), _ptr(glse), _ptr(Output_partial), _ptr(out), B, stride_tokens,
-        topk_indices.shape[-1], ns, _ptr(block_table), max_pages, page_size, _sync_arg(sync, B), _stream()))
+        topk_indices.shape[-1], ns, _ptr(block_table), max_pages, page_size, kv_strides,
+        _sync_arg(sync, B), _stream()))
     return out
 
 
@@ -144,7 +169,8 @@ def decode_dense_paged(Q, K, V, cache_seqlens, glse, Output_partial, block_table
     ``kernel(Q, K, V, [cache_seqlens,] glse, Output_partial) -> O``."""
     lib = _lib.init()
     B = Q.shape[0]
-    _req(Q, torch.float16, "Q"); _req(K, torch.float16, "K"); _req(V, torch.float16, "V")
+    _req(Q, torch.float16, "Q")
+    kv_strides = _decode_kv(K, V, block_table)
     _req(glse, torch.float32, "glse"); _req(Output_partial, torch.float32, "Output_partial")
     ns = glse.shape[2]
     if block_table is not None:
@@ -155,7 +181,8 @@ def decode_dense_paged(Q, K, V, cache_seqlens, glse, Output_partial, block_table
     out = _out_buffer(out, B, Q.device)
     _lib.check(lib.kascade_decode_dense_paged_call(
         _ptr(Q), _ptr(K), _ptr(V), _ptr(cache_seqlens), _ptr(glse), _ptr(Output_partial), _ptr(out),
-        B, stride_tokens, ns, _ptr(block_table), max_pages, page_size, _sync_arg(sync, B), _stream()))
+        B, stride_tokens, ns, _ptr(block_table), max_pages, page_size, kv_strides, _sync_arg(sync, B),
+        _stream()))
     return out
 
 
@@ -170,7 +197,8 @@ def decode_recompute(Q, K, V, glse, Output_partial, row_sums, scores, layer: int
     otherwise O is None."""
     lib = _lib.init()
     B = Q.shape[0]
-    _req(Q, torch.float16, "Q"); _req(K, torch.float16, "K")
+    _req(Q, torch.float16, "Q")
+    kv_strides = _decode_kv(K, V, block_table)
     _req(glse, torch.float32, "glse"); _req(row_sums, torch.float32, "row_sums")
     _req(scores, torch.float32, "scores")
     with_out = 1 if layer == 0 else 0
@@ -186,7 +214,7 @@ def decode_recompute(Q, K, V, glse, Output_partial, row_sums, scores, layer: int
     _lib.check(lib.kascade_decode_recompute_paged_call(
         _ptr(Q), _ptr(K), _ptr(V), _ptr(cache_seqlens), _ptr(glse), _ptr(Output_partial),
         _ptr(row_sums), _ptr(scores), _ptr(out), _ptr(agg), B, stride_tokens, stride, ns, with_out,
-        _ptr(block_table), max_pages, page_size, _sync_arg(sync, B), _stream()))
+        _ptr(block_table), max_pages, page_size, kv_strides, _sync_arg(sync, B), _stream()))
     return out, agg
 
 

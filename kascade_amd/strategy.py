@@ -169,8 +169,11 @@ class EfficientKascadeStrategy:
         layer = module.layer_idx
         if is_decode:
             query = query.squeeze(1).contiguous()
-            key = key.contiguous()
-            value = value.contiguous()
+            # The reference copies the whole cache to [B,L,G,D] here on every step
+            # (EfficientKascadeStrategy.py:149-150); the decode kernels take the strided view of
+            # HF's head-major cache instead and read it in place.
+            if key.stride(-1) != 1 or value.stride() != key.stride():
+                key, value = key.contiguous(), value.contiguous()
             if layer in self.recompute_layers:
                 o = self._decode_recomp_forward(query, key, value, rounded_k, layer)
             else:

@@ -261,3 +261,48 @@ def test_fused_combine_matches_combine_launch(cuda, seqlens, ns):
     assert_close(r1, orc.reuse_decode(w.q, kc, vc, idx, hm.tolist()), "fused reuse decode")
     assert_close(r1, r2, "fused vs combine launch (reuse)", atol=1e-3, rtol=2e-3)
     assert int(sync.abs().sum()) == 0
+
+
+@pytest.mark.parametrize("seqlens", [[900, 333], [2100]])
+def test_head_major_cache_is_read_in_place(cuda, seqlens):
+    """A head-major [B,G,L,D] cache (Hugging Face's layout) handed over as the strided [B,L,G,D]
+    view gives bit-identical results to its [B,L,G,D] copy, for every decode kernel, and without
+    the kernels touching anything outside the view (a slice of a larger buffer is used)."""
+    from kascade_amd import kernels
+    w = _paged_case(seqlens, seed=13)
+    B, Lmax = len(seqlens), max(seqlens)
+    kc = orc.paged_to_contiguous(w.k_pages, w.block_table, seqlens).to(cuda)   # [B,Lmax,G,D]
+    vc = orc.paged_to_contiguous(w.v_pages, w.block_table, seqlens).to(cuda)
+    # head-major storage with room for more tokens, as a preallocated HF cache would have
+    k_store = torch.full((B, G, Lmax + 40, D), float("nan"), dtype=torch.float16, device=cuda)
+    v_store = torch.full_like(k_store, float("nan"))
+    k_store[:, :, :Lmax] = kc.permute(0, 2, 1, 3)
+    v_store[:, :, :Lmax] = vc.permute(0, 2, 1, 3)
+    kh = k_store[:, :, :Lmax].transpose(1, 2)     # [B,Lmax,G,D] view, strides (G*(Lmax+40)*D, D, (Lmax+40)*D)
+    vh = v_store[:, :, :Lmax].transpose(1, 2)
+    assert not kh.is_contiguous()
+    q, lens = w.q.to(cuda), w.seqlens.to(cuda)
+    glse, part = _scratch(B, 3, cuda)
+    a = kernels.decode_dense_paged(q, kc, vc, lens, glse, part)
+    b = kernels.decode_dense_paged(q, kh, vh, lens, glse.clone(), part.clone())
+    assert torch.isfinite(b).all() and torch.equal(a, b), "dense decode"
+    row_sums = torch.empty(B, H, device=cuda, dtype=torch.float32)
+    stride = ((Lmax + 7) // 8) * 8
+    scores = torch.empty(B, H, stride, device=cuda, dtype=torch.float32)
+    for layer in (0, 1):
+        o1, agg1 = kernels.decode_recompute(q, kc, vc, glse, part, row_sums, scores, layer, cache_seqlens=lens)
+        o2, agg2 = kernels.decode_recompute(q, kh, vh, glse, part, row_sums, scores, layer, cache_seqlens=lens)
+        assert torch.equal(agg1[:, :, :Lmax], agg2[:, :, :Lmax]), f"agg, layer {layer}"
+        if layer == 0:
+            assert torch.equal(o1, o2), "anchor-0 output"
+    gen = torch.Generator().manual_seed(6)
+    idx = _rand_idx(B, min(seqlens), 256, gen).to(cuda)
+    hm = torch.tensor([3, 3, 0, 1, 7, 6, 5, 2], dtype=torch.int32, device=cuda)
+    c = kernels.decode_reuse_paged(q, kc, vc, lens, idx, hm, 0.0, glse, part)
+    d = kernels.decode_reuse_paged(q, kh, vh, lens, idx, hm, 0.0, glse, part)
+    assert torch.isfinite(d).all() and torch.equal(c, d), "reuse decode (kvcache form)"
+    if len(set(seqlens)) == 1:
+        e = kernels.decode_reuse(q, kc, vc, idx, hm, glse, part)
+        f = kernels.decode_reuse(q, kh, vh, idx, hm, glse, part)
+        assert torch.equal(e, f), "reuse decode"
+        assert_close(f, orc.reuse_decode(w.q, kc.cpu(), vc.cpu(), idx.cpu(), hm.tolist()), "reuse decode vs oracle")
