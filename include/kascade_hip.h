@@ -96,7 +96,11 @@ int kascade_decode_reuse_call(const kascade_half* Q, const kascade_half* K, cons
  *               seen as [B,tokens,G,D]: multiples of 8, D contiguous.  Lets the kernels read a
  *               head-major [B,G,tokens,D] cache (Hugging Face's layout) in place, where the
  *               reference copies the whole cache to [B,tokens,G,D] on every decode step
- *               (EfficientKascadeStrategy.py:149-150). */
+ *               (EfficientKascadeStrategy.py:149-150).
+ *   k_new,v_new NULL, or [B,G,D] f16: the K and V rows of each sequence's newest token, i.e. of
+ *               position cache_seqlens[b]-1 (kv_stride_tokens-1 without cache_seqlens).  The
+ *               launch writes them into that slot of the cache (through K and V) and attends
+ *               to them, so a decode step needs no separate kascade_paged_kv_append_call. */
 int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K,
                                     const kascade_half* V, const int32_t* cache_seqlens,
                                     const int32_t* topk_indices, const int32_t* head_mapping,
@@ -104,6 +108,7 @@ int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K
                                     kascade_half* Output, int batch, int kv_stride_tokens,
                                     int topk, int num_split, const int32_t* block_table,
                                     int max_pages, int page_size, const kascade_strides* kv_strides,
+                                    const kascade_half* k_new, const kascade_half* v_new,
                                     int32_t* sync_counters, void* stream);
 
 /* Dense split-K decode (the reference's TileLang dense baseline, gqa_decode.py:117-254 and
@@ -116,7 +121,8 @@ int kascade_decode_dense_paged_call(const kascade_half* Q, const kascade_half* K
                                     float* glse, float* Output_partial, kascade_half* Output,
                                     int batch, int kv_stride_tokens, int num_split,
                                     const int32_t* block_table, int max_pages, int page_size,
-                                    const kascade_strides* kv_strides, int32_t* sync_counters,
+                                    const kascade_strides* kv_strides, const kascade_half* k_new,
+                                    const kascade_half* v_new, int32_t* sync_counters,
                                     void* stream);
 
 /* Anchor-layer decode: split QK^T (+PV when with_output != 0), log-sum merge and
@@ -138,6 +144,7 @@ int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_hal
                                         int with_output, const int32_t* block_table,
                                         int max_pages, int page_size,
                                         const kascade_strides* kv_strides,
+                                        const kascade_half* k_new, const kascade_half* v_new,
                                         int32_t* sync_counters, void* stream);
 
 /* ------------------------------------------------------------------- top-k */
@@ -211,6 +218,17 @@ int kascade_paged_kv_append_call(kascade_half* K_pages, kascade_half* V_pages,
                                  const int32_t* start_pos, const int32_t* block_table, int batch,
                                  int n_new, int max_pages, int page_size,
                                  kascade_strides new_strides, void* stream);
+
+/* Bookkeeping of a ragged decode step in one small launch (no reference counterpart; the
+ * reference's benchmark computes these on the host, recompute_kascade_gqa_decode_with_kvcache.py:
+ * 368-377).  Adds `advance` to every cache_seqlens[b] in place (1 when the step's new token is
+ * appended by the decode calls themselves, 0 to leave the lengths alone) and writes, per
+ * (sequence, KV head) row r = b*8+g of the pooled scores, what kascade_topk_call takes as
+ * valid_len / n_sel:  valid_len_rows[r] = len_b,
+ *                     n_sel_rows[r]     = 128*ceil(floor(topk_percent*len_b/100)/128),
+ * with len_b the length after the advance.  Either output may be NULL. */
+int kascade_decode_budgets_call(int32_t* cache_seqlens, int advance, float topk_percent, int batch,
+                                int32_t* valid_len_rows, int32_t* n_sel_rows, void* stream);
 
 /* ------------------------------------------- chunked prefill over the paged cache */
 

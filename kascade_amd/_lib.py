@@ -39,11 +39,11 @@ SIGNATURES = {
     "kascade_device_cu_count": (_I, []),
     "kascade_decode_reuse_call": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _P]),
     "kascade_decode_reuse_paged_call": (_I, [_P, _P, _P, _P, _P, _P, _F, _P, _P, _P, _I, _I, _I, _I,
-                                             _P, _I, _I, _SP, _P, _P]),
+                                             _P, _I, _I, _SP, _P, _P, _P, _P]),
     "kascade_decode_dense_paged_call": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _I, _I, _SP,
-                                             _P, _P]),
+                                             _P, _P, _P, _P]),
     "kascade_decode_recompute_paged_call": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I,
-                                                 _I, _I, _P, _I, _I, _SP, _P, _P]),
+                                                 _I, _I, _P, _I, _I, _SP, _P, _P, _P, _P]),
     "kascade_topk_workspace_bytes": (_L, [_I, _L]),
     "kascade_topk_call": (_I, [_P, _P, _I, _L, _I, _P, _P, _I, _I, _I, _P, _P]),
     "kascade_prefill_dense_call": (_I, [_P, _P, _P, _P, _P, _I, _I, Strides, Strides, _I, _P]),
@@ -51,6 +51,7 @@ SIGNATURES = {
     "kascade_prefill_reuse_call": (_I, [_P, _P, _P, _P, _P, _F, _P, _I, _I, _I, _I, Strides, Strides,
                                         _P]),
     "kascade_paged_kv_append_call": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, Strides, _P]),
+    "kascade_decode_budgets_call": (_I, [_P, _I, _F, _I, _P, _P, _P]),
     "kascade_prefill_chunk_dense_call": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, Strides, _P, _I, _I, _I,
                                               _I, _P]),
     "kascade_prefill_chunk_aggregate_call": (_I, [_P, _P, _P, _P, _I, _I, _I, Strides, _P, _I, _I, _I,

@@ -88,11 +88,23 @@ int set_kv_strides(DecodeParams& p, const kascade_strides* strides, const int32_
     return 0;
 }
 
+// Fused append of the decode calls: both rows or neither; the caches are written through the
+// K / V arguments.
+int set_append(DecodeParams& p, const kascade_half* k_new, const kascade_half* v_new,
+               const kascade_half* K, const kascade_half* V) {
+    if (!k_new && !v_new) return 0;
+    REQUIRE(k_new && v_new && K && V, "k_new and v_new come together, with both caches");
+    REQUIRE(aligned16(k_new) && aligned16(v_new), "k_new/v_new must be 16-byte aligned");
+    p.k_new = H(k_new); p.v_new = H(v_new);
+    p.k_cache = const_cast<half_t*>(H(K)); p.v_cache = const_cast<half_t*>(H(V));
+    return 0;
+}
+
 }  // namespace
 
 extern "C" {
 
-int kascade_abi_version(void) { return 3; }
+int kascade_abi_version(void) { return 4; }
 
 const char* kascade_get_last_error(void) { return g_err; }
 
@@ -116,7 +128,8 @@ int kascade_decode_reuse_call(const kascade_half* Q, const kascade_half* K, cons
                               void* stream) {
     return kascade_decode_reuse_paged_call(Q, K, V, nullptr, topk_indices, head_mapping, 0.f, glse,
                                            Output_partial, Output, batch, kv_seqlen, topk,
-                                           num_split, nullptr, 0, 1, nullptr, sync_counters, stream);
+                                           num_split, nullptr, 0, 1, nullptr, nullptr, nullptr, sync_counters,
+                                           stream);
 }
 
 int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K,
@@ -126,6 +139,7 @@ int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K
                                     kascade_half* Output, int batch, int kv_stride_tokens,
                                     int topk, int num_split, const int32_t* block_table,
                                     int max_pages, int page_size, const kascade_strides* kv_strides,
+                                    const kascade_half* k_new, const kascade_half* v_new,
                                     int32_t* sync_counters, void* stream) {
     REQUIRE(Q && K && V && topk_indices && head_mapping && glse && Output_partial && Output,
             "decode_reuse: null pointer argument");
@@ -142,6 +156,7 @@ int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K
     p.block_table = block_table; p.glse = glse; p.opart = Output_partial; p.scores = nullptr;
     p.max_pages = max_pages; p.page_shift = shift; p.kv_stride_tokens = kv_stride_tokens;
     if (set_kv_strides(p, kv_strides, block_table, kv_stride_tokens)) return -1;
+    if (set_append(p, k_new, v_new, K, V)) return -1;
     p.topk = topk; p.topk_percent = topk_percent; p.scores_stride = 0; p.num_split = num_split;
     p.rows_per_split = rows_per_split(topk, num_split);
     p.B = batch;
@@ -158,7 +173,8 @@ int kascade_decode_dense_paged_call(const kascade_half* Q, const kascade_half* K
                                     float* glse, float* Output_partial, kascade_half* Output,
                                     int batch, int kv_stride_tokens, int num_split,
                                     const int32_t* block_table, int max_pages, int page_size,
-                                    const kascade_strides* kv_strides, int32_t* sync_counters,
+                                    const kascade_strides* kv_strides, const kascade_half* k_new,
+                                    const kascade_half* v_new, int32_t* sync_counters,
                                     void* stream) {
     REQUIRE(Q && K && V && glse && Output_partial && Output, "decode_dense: null pointer argument");
     REQUIRE(batch > 0 && num_split > 0, "decode_dense: batch, num_split must be > 0");
@@ -173,6 +189,7 @@ int kascade_decode_dense_paged_call(const kascade_half* Q, const kascade_half* K
     p.seqlens = cache_seqlens; p.block_table = block_table; p.glse = glse; p.opart = Output_partial;
     p.max_pages = max_pages; p.page_shift = shift; p.kv_stride_tokens = kv_stride_tokens;
     if (set_kv_strides(p, kv_strides, block_table, kv_stride_tokens)) return -1;
+    if (set_append(p, k_new, v_new, K, V)) return -1;
     p.num_split = num_split; p.B = batch;
     const long long max_rows = kv_stride_tokens > 0 ? kv_stride_tokens : (long long)max_pages * page_size;
     p.rows_per_split = rows_per_split(max_rows, num_split);
@@ -193,6 +210,7 @@ int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_hal
                                         int with_output, const int32_t* block_table,
                                         int max_pages, int page_size,
                                         const kascade_strides* kv_strides,
+                                        const kascade_half* k_new, const kascade_half* v_new,
                                         int32_t* sync_counters, void* stream) {
     REQUIRE(Q && K && glse && row_sums && scores && aggregated_scores,
             "decode_recompute: null pointer argument");
@@ -217,6 +235,7 @@ int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_hal
     p.scores = scores; p.scores_stride = scores_stride;
     p.max_pages = max_pages; p.page_shift = shift; p.kv_stride_tokens = kv_stride_tokens;
     if (set_kv_strides(p, kv_strides, block_table, kv_stride_tokens)) return -1;
+    if (set_append(p, k_new, v_new, K, V)) return -1;
     p.num_split = num_split; p.B = batch;
     long long max_rows = kv_stride_tokens > 0 ? kv_stride_tokens : (long long)max_pages * page_size;
     if (max_rows > scores_stride) max_rows = scores_stride;
@@ -336,6 +355,16 @@ int kascade_paged_kv_append_call(kascade_half* K_pages, kascade_half* V_pages,
                                             new_strides.b, new_strides.l, new_strides.h,
                                             static_cast<hipStream_t>(stream)),
                      "paged_kv_append");
+}
+
+int kascade_decode_budgets_call(int32_t* cache_seqlens, int advance, float topk_percent, int batch,
+                                int32_t* valid_len_rows, int32_t* n_sel_rows, void* stream) {
+    REQUIRE(cache_seqlens, "decode_budgets: null pointer argument");
+    REQUIRE(batch > 0 && batch <= 65535, "decode_budgets: bad batch");
+    REQUIRE(topk_percent >= 0.f && topk_percent <= 100.f, "decode_budgets: topk_percent out of range");
+    return check_hip(launch_decode_budgets(cache_seqlens, advance, topk_percent, batch, valid_len_rows,
+                                           n_sel_rows, static_cast<hipStream_t>(stream)),
+                     "decode_budgets");
 }
 
 // ---- chunked prefill over the paged cache ----

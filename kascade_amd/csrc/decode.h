@@ -18,6 +18,12 @@ struct DecodeParams {
     // Fused combine: with counters != null ([B*G] ints, zero before the first launch and zero
     // again after every launch) the last split workgroup of each (b, g) merges the splits into
     // out [B,H,D] and row_sums [B,H] (either may be null), and no combine launch is needed.
+    // Fused append: with k_new != null the rows k_new/v_new [B,G,D] of each sequence's newest
+    // token (position seqlen-1) are written into k_cache / v_cache by the launch itself.
+    const half_t* k_new;
+    const half_t* v_new;
+    half_t* k_cache;
+    half_t* v_cache;
     int* counters;
     half_t* out;
     float* row_sums;

@@ -64,6 +64,7 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
     __shared__ int s_row[GATHER ? kSubChunk : 1];
     __shared__ MergeState s_merge[4];
     __shared__ int s_last;
+    __shared__ int s_found;   // gather mode: sub-chunk whose index list names the newest token
     // anchor mode: two buffers of four wavefront strips (4 heads x kStripRows raw scores)
     __shared__ __attribute__((aligned(16))) float s_sc[WRITE_SCORES ? 2 : 1][WRITE_SCORES ? 4 : 1][kGroupSize][WRITE_SCORES ? kStripRows : 4];
 
@@ -95,6 +96,39 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
     const long long r0l = (long long)split * p.rows_per_split;
     const int r0 = (int)min((long long)n, r0l);
     const int r1 = (int)min((long long)n, r0l + p.rows_per_split);
+
+    // Fused append.  With k_new/v_new the K/V rows of the newest token (position seqlen-1)
+    // arrive beside the cache and have to end up in it.  A workgroup that is going to read that
+    // row writes it first and waits for its own stores at a barrier; what other workgroups write
+    // there is the same bytes.  `write_newest` is uniform over the workgroup.
+    const int newest = seqlen - 1;
+    auto write_newest = [&]() {
+        if (tid < 32) {
+            const int part = tid >> 4, c = tid & 15;
+            size_t off;
+            if (p.block_table) {
+                const int pg = p.block_table[(size_t)b * p.max_pages + (newest >> p.page_shift)];
+                const int row = (pg << p.page_shift) + (newest & ((1 << p.page_shift) - 1));
+                off = (size_t)row * (kGroups * kDim) + (size_t)g * kDim + c * 8;
+            } else {
+                off = (size_t)b * p.kv_stride_b + (size_t)g * p.kv_stride_h + (size_t)newest * p.kv_stride_l + c * 8;
+            }
+            const half_t* src = (part ? p.v_new : p.k_new) + ((size_t)b * kGroups + g) * kDim + c * 8;
+            half_t* dst = (part ? p.v_cache : p.k_cache) + off;
+            *reinterpret_cast<uint4_t*>(dst) = ld_global_16(src);
+        }
+    };
+    if (p.k_new != nullptr && newest >= 0) {
+        if (!GATHER) {
+            if (newest >= r0 && newest < r1) {   // the split that streams the newest row
+                write_newest();
+                __syncthreads();
+            }
+        } else if (split == 0) {
+            write_newest();   // lists that do not name the newest token still leave it cached
+        }
+    }
+    if (GATHER && tid == 0) s_found = -1;
 
     // q fragments: 4 heads x 8 halves of this lane's d-slice
     Pack16 qf[kGroupSize];
@@ -208,6 +242,7 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
             for (int i = tid; i < cn; i += kThreads) {
                 int tok = idx_row[c0 + i];
                 tok = max(0, min(tok, seqlen - 1));   // a corrupt index must not leave the sequence
+                if (tok == newest) s_found = c0;
                 int row;
                 if (p.block_table) {
                     int pg = p.block_table[(size_t)b * p.max_pages + (tok >> p.page_shift)];
@@ -218,6 +253,10 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
                 s_row[i] = row;
             }
             __syncthreads();
+            if (p.k_new != nullptr && s_found == c0) {   // c0 differs per sub-chunk: no reset needed
+                write_newest();
+                __syncthreads();
+            }
             auto staged_rows = [&](int it, int (&rows)[kUnroll]) {
                 const int rbase = it + wave * (4 * kUnroll) + rg;
 #pragma unroll

@@ -28,7 +28,33 @@ __global__ __launch_bounds__(256) void paged_kv_append_kernel(
     *reinterpret_cast<uint4_t*>(Vp + dst) = ld_global_16(v_new + src);
 }
 
+// Per (sequence, KV head) row of a ragged decode step: how many pooled scores are valid and how
+// many of them the selection keeps, n(b) = 128*ceil(floor(percent*len_b/100)/128), optionally
+// after adding `advance` to every length in place (the step's new token).
+__global__ __launch_bounds__(256) void decode_budgets_kernel(int* __restrict__ seqlens, int advance,
+                                                             float percent, int batch,
+                                                             int* __restrict__ valid_rows,
+                                                             int* __restrict__ n_sel_rows) {
+    // a single workgroup: the barrier puts the in-place update after every read of a length
+    for (int i = threadIdx.x; i < batch * kGroups; i += blockDim.x) {
+        const int len = seqlens[i / kGroups] + advance;
+        const long long fl = (long long)floor((double)percent * (double)len / 100.0);
+        if (valid_rows) valid_rows[i] = len;
+        if (n_sel_rows) n_sel_rows[i] = (int)(((fl + 127) / 128) * 128);
+    }
+    __syncthreads();
+    if (advance != 0)
+        for (int b = threadIdx.x; b < batch; b += blockDim.x) seqlens[b] += advance;
+}
+
 }  // namespace
+
+hipError_t launch_decode_budgets(int* seqlens, int advance, float percent, int batch, int* valid_rows,
+                                 int* n_sel_rows, hipStream_t stream) {
+    hipLaunchKernelGGL(decode_budgets_kernel, dim3(1), dim3(256), 0, stream, seqlens, advance, percent,
+                       batch, valid_rows, n_sel_rows);
+    return hipGetLastError();
+}
 
 hipError_t launch_paged_kv_append(half_t* Kp, half_t* Vp, const half_t* k_new, const half_t* v_new,
                                   const int* start_pos, const int* block_table, int batch,

@@ -93,6 +93,40 @@ def _decode_kv(K, V, block_table):
     return ctypes.byref(ks)
 
 
+def _new_rows(k_new, v_new, B):
+    """Optional [B,G,D] rows of the newest token for the fused append (both or neither)."""
+    if k_new is None and v_new is None:
+        return None, None
+    if k_new is None or v_new is None:
+        raise KascadeError("k_new and v_new come together")
+    for t, name in ((k_new, "k_new"), (v_new, "v_new")):
+        _req(t, torch.float16, name)
+        if tuple(t.shape) != (B, G, D):
+            raise KascadeError(f"{name} must be [{B},{G},{D}]")
+    return _ptr(k_new), _ptr(v_new)
+
+
+def decode_budgets(cache_seqlens, topk_percent: float, advance: int = 0, valid_out=None, n_sel_out=None):
+    """One small launch for the bookkeeping of a ragged decode step: adds ``advance`` to the
+    lengths in place and returns (valid_len, n_sel) per (sequence, KV head) row as the selection
+    takes them.  The reference's benchmark glue does this on the host
+    (recompute_kascade_gqa_decode_with_kvcache.py:368-377)."""
+    lib = _lib.init()
+    _req(cache_seqlens, torch.int32, "cache_seqlens")
+    B = cache_seqlens.numel()
+    if valid_out is None:
+        valid_out = torch.empty(B * G, device=cache_seqlens.device, dtype=torch.int32)
+    if n_sel_out is None:
+        n_sel_out = torch.empty(B * G, device=cache_seqlens.device, dtype=torch.int32)
+    for t, name in ((valid_out, "valid_out"), (n_sel_out, "n_sel_out")):
+        _req(t, torch.int32, name)
+        if t.numel() < B * G:
+            raise KascadeError(f"{name} needs {B * G} entries")
+    _lib.check(lib.kascade_decode_budgets_call(_ptr(cache_seqlens), int(advance), float(topk_percent), B,
+                                               _ptr(valid_out), _ptr(n_sel_out), _stream()))
+    return valid_out[:B * G], n_sel_out[:B * G]
+
+
 def _sync_arg(sync, B):
     """Optional [B*G] int32 counter array for the fused combine (zero-initialised by the caller)."""
     if sync is None:
@@ -128,13 +162,13 @@ def decode_reuse(Q, K, V, topk_indices, head_mapping, glse, Output_partial, sync
         _lib.check(lib.kascade_decode_reuse_paged_call(
             _ptr(Q), _ptr(K), _ptr(V), None, _ptr(topk_indices), _ptr(head_mapping), 0.0, _ptr(glse),
             _ptr(Output_partial), _ptr(out), B, L, topk_indices.shape[-1], ns, None, 0, 1, kv_strides,
-            _sync_arg(sync, B), _stream()))
+            None, None, _sync_arg(sync, B), _stream()))
     return out
 
 
 def decode_reuse_paged(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_percent, glse,
                        Output_partial, block_table=None, page_size: int = 16, out=None,
-                       sync=None) -> torch.Tensor:
+                       sync=None, k_new=None, v_new=None) -> torch.Tensor:
     """``reuse kvcache kernel(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_percent,
     glse, Output_partial) -> O`` (out_idx=[9]; reuse_kascade_gqa_decode_with_kvcache.py:160-173)
     with an optional block table.  Without one K,V are the padded [B,maxL,G,D] cache;
@@ -158,13 +192,13 @@ def decode_reuse_paged(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_
         _ptr(Q), _ptr(K), _ptr(V), _ptr(cache_seqlens), _ptr(topk_indices), _ptr(head_mapping),
         float(topk_percent), _ptr(glse), _ptr(Output_partial), _ptr(out), B, stride_tokens,
         topk_indices.shape[-1], ns, _ptr(block_table), max_pages, page_size, kv_strides,
-        _sync_arg(sync, B), _stream()))
+        *_new_rows(k_new, v_new, B), _sync_arg(sync, B), _stream()))
     return out
 
 
 def decode_dense_paged(Q, K, V, cache_seqlens, glse, Output_partial, block_table=None,
                        page_size: int = 16, kv_len: Optional[int] = None, out=None,
-                       sync=None) -> torch.Tensor:
+                       sync=None, k_new=None, v_new=None) -> torch.Tensor:
     """Dense split-K decode, the baseline of gqa_decode.py / gqa_decode_with_kvcache.py:
     ``kernel(Q, K, V, [cache_seqlens,] glse, Output_partial) -> O``."""
     lib = _lib.init()
@@ -181,15 +215,15 @@ def decode_dense_paged(Q, K, V, cache_seqlens, glse, Output_partial, block_table
     out = _out_buffer(out, B, Q.device)
     _lib.check(lib.kascade_decode_dense_paged_call(
         _ptr(Q), _ptr(K), _ptr(V), _ptr(cache_seqlens), _ptr(glse), _ptr(Output_partial), _ptr(out),
-        B, stride_tokens, ns, _ptr(block_table), max_pages, page_size, kv_strides, _sync_arg(sync, B),
-        _stream()))
+        B, stride_tokens, ns, _ptr(block_table), max_pages, page_size, kv_strides,
+        *_new_rows(k_new, v_new, B), _sync_arg(sync, B), _stream()))
     return out
 
 
 def decode_recompute(Q, K, V, glse, Output_partial, row_sums, scores, layer: int,
                      cache_seqlens=None, block_table=None, page_size: int = 16,
                      kv_len: Optional[int] = None, out=None,
-                     sync=None) -> Tuple[Optional[torch.Tensor], torch.Tensor]:
+                     sync=None, k_new=None, v_new=None) -> Tuple[Optional[torch.Tensor], torch.Tensor]:
     """``decode_recomp{0,1}_kernel(Q, K, V, glse, Output_partial, row_sums, scores) -> (O, agg)``
     (out_idx=[7,8]; EfficientKascadeStrategy.py:24-28, 107-110) and its kvcache form
     (recompute_kascade_gqa_decode_with_kvcache.py:302-333).  ``scores`` is fp32 scratch
@@ -214,7 +248,8 @@ def decode_recompute(Q, K, V, glse, Output_partial, row_sums, scores, layer: int
     _lib.check(lib.kascade_decode_recompute_paged_call(
         _ptr(Q), _ptr(K), _ptr(V), _ptr(cache_seqlens), _ptr(glse), _ptr(Output_partial),
         _ptr(row_sums), _ptr(scores), _ptr(out), _ptr(agg), B, stride_tokens, stride, ns, with_out,
-        _ptr(block_table), max_pages, page_size, kv_strides, _sync_arg(sync, B), _stream()))
+        _ptr(block_table), max_pages, page_size, kv_strides, *_new_rows(k_new, v_new, B),
+        _sync_arg(sync, B), _stream()))
     return out, agg
 
 

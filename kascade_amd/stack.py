@@ -49,7 +49,6 @@ class KascadeAttentionStack:
         self.v_pages = [torch.zeros_like(p) for p in self.k_pages]
         self.length = 0                                                 # host copy of the common length
         self.seqlens = torch.zeros(batch, device=self.device, dtype=torch.int32)
-        self._next = torch.zeros_like(self.seqlens)                     # lengths after the append
         self.prefill = PagedKascadePrefill(k, head_mapping, recompute_layers, page_size, rolling_prefill,
                                            self.device)
         self.decoder = PagedKascadeDecoder(k, head_mapping, recompute_layers, batch, max_seqlen, page_size,
@@ -88,17 +87,18 @@ class KascadeAttentionStack:
     # ------------------------------------------------------------------- decode
     def _decode_layers(self, q, k_new, v_new, out):
         """The launch sequence of one decode step; lengths are read from device memory."""
-        torch.add(self.seqlens, 1, out=self._next)
+        # one bookkeeping launch (lengths + 1, anchor budgets), then one attention launch sequence
+        # per layer; the first launch of a layer also writes the new token's K/V into the cache
+        self.decoder.begin_step(self.seqlens, 1)
         for l in range(self.num_layers):
-            kernels.paged_kv_append(self.k_pages[l], self.v_pages[l], k_new[l], v_new[l], self.seqlens,
-                                    self.block_table, self.page_size)
+            kn, vn = k_new[l][:, 0], v_new[l][:, 0]
             if self.dense_only:
-                self.decoder.dense(q[l], self.k_pages[l], self.v_pages[l], self.block_table, self._next,
-                                   self.max_seqlen, out=out[l])
+                self.decoder.dense(q[l], self.k_pages[l], self.v_pages[l], self.block_table, self.seqlens,
+                                   self.max_seqlen, out=out[l], k_new=kn, v_new=vn)
             else:
                 self.decoder.forward(l, q[l], self.k_pages[l], self.v_pages[l], self.block_table,
-                                     self._next, self.max_seqlen, ragged=True, out=out[l])
-        self.seqlens.copy_(self._next)
+                                     self.seqlens, self.max_seqlen, ragged=True, out=out[l],
+                                     k_new=kn, v_new=vn)
 
     def decode_step(self, q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor,
                     out: Optional[torch.Tensor] = None) -> torch.Tensor:

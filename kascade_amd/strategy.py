@@ -241,6 +241,8 @@ class PagedKascadeDecoder:
             self._hm[l] = torch.tensor(row, device=dev, dtype=torch.int32)
         self._topk_to_reuse = None
         self._counts = None
+        self._valid_rows = torch.empty(max_batch * G, device=dev, dtype=torch.int32)
+        self._nsel_rows = torch.empty(max_batch * G, device=dev, dtype=torch.int32)
         # arrival counters of the fused combine: zero now, set back to zero by every launch
         self._sync = torch.zeros(max_batch * G, device=dev, dtype=torch.int32) if fused_combine else None
         # one workgroup merges all splits of a (sequence, KV head): a win up to about 16 splits
@@ -252,23 +254,38 @@ class PagedKascadeDecoder:
     def _scratch(self, B, ns):
         return self._glse[:B * H * ns].view(B, H, ns), self._part[:B * H * ns * D].view(B, H, ns, D)
 
-    def dense(self, q, k_pages, v_pages, block_table, seqlens, max_len: int, out=None):
+    def dense(self, q, k_pages, v_pages, block_table, seqlens, max_len: int, out=None,
+              k_new=None, v_new=None):
         B = q.shape[0]
         glse, part = self._scratch(B, self.ns_dense)
         return kernels.decode_dense_paged(q, k_pages, v_pages, seqlens, glse, part, block_table,
-                                          self.page_size, kv_len=max_len, out=out, sync=self._sync_dense)
+                                          self.page_size, kv_len=max_len, out=out, sync=self._sync_dense,
+                                          k_new=k_new, v_new=v_new)
+
+    def begin_step(self, seqlens: torch.Tensor, advance: int = 1):
+        """One launch at the start of a decode step: the lengths grow by ``advance`` in place
+        (the new token, which the layer calls append themselves when handed ``k_new``/``v_new``)
+        and the per-row budgets of the step's anchor layers are computed from the new lengths."""
+        self._counts = (self._budget_key(seqlens),
+                        *kernels.decode_budgets(seqlens, float(self.k), advance, self._valid_rows, self._nsel_rows))
+
+    @staticmethod
+    def _budget_key(seqlens):
+        return (seqlens.data_ptr(), seqlens._version, seqlens.numel())
 
     def anchor(self, layer, q, k_pages, v_pages, block_table, seqlens, max_len: int,
-               ragged: bool = True, out=None):
+               ragged: bool = True, out=None, k_new=None, v_new=None):
         """Anchor layer: returns the attention output [B,H,D] (written to ``out`` when given);
-        keeps indices for reuse layers."""
+        keeps indices for reuse layers.  ``k_new``/``v_new`` [B,G,D]: rows of the newest token
+        (position seqlens-1), appended to the cache by the anchor launch itself."""
         B = q.shape[0]
         stride = ((max_len + 7) // 8) * 8
         glse, part = self._scratch(B, self.ns_dense)
         scores = self._scores[:B * H * stride].view(B, H, stride)
         o, agg = kernels.decode_recompute(q, k_pages, v_pages, glse, part, self._row_sums[:B], scores, layer,
                                           cache_seqlens=seqlens, block_table=block_table,
-                                          page_size=self.page_size, kv_len=max_len, out=out, sync=self._sync_dense)
+                                          page_size=self.page_size, kv_len=max_len, out=out, sync=self._sync_dense,
+                                          k_new=k_new, v_new=v_new)
         if ragged:
             width = budgets.decode_budget(max_len, self.k)
             lens_rows, counts = self._row_budgets(seqlens)
@@ -287,38 +304,31 @@ class PagedKascadeDecoder:
         """Per (sequence, KV head) row: valid length and selection count.  The anchors of one
         decode step see the same lengths, so the tensors are kept until seqlens is written again
         (a dozen tiny launches otherwise, as long as an anchor pass at short contexts)."""
-        key = (seqlens.data_ptr(), seqlens._version, seqlens.numel())
+        key = self._budget_key(seqlens)
         if self._counts is None or self._counts[0] != key:
-            self._counts = (key, seqlens.repeat_interleave(G),
-                            self._decode_counts(seqlens).repeat_interleave(G))
+            self._counts = (key, *kernels.decode_budgets(seqlens, float(self.k), 0, self._valid_rows,
+                                                         self._nsel_rows))
         return self._counts[1], self._counts[2]
 
-    def _decode_counts(self, seqlens: torch.Tensor) -> torch.Tensor:
-        # 128*ceil(floor(k*len/100)/128) on the device, exact integer arithmetic for integer k
-        if float(self.k).is_integer():
-            fl = (seqlens.to(torch.int64) * int(self.k)) // 100
-        else:
-            fl = torch.floor(seqlens.to(torch.float64) * float(self.k) / 100.0).to(torch.int64)
-        return (((fl + 127) // 128) * 128).to(torch.int32)
-
-    def _reuse(self, q, k_pages, v_pages, block_table, seqlens, hm, out=None):
+    def _reuse(self, q, k_pages, v_pages, block_table, seqlens, hm, out=None, k_new=None, v_new=None):
         B = q.shape[0]
         glse, part = self._scratch(B, self.ns_reuse)
         return kernels.decode_reuse_paged(q, k_pages, v_pages, seqlens, self._topk_to_reuse, hm, self._pct,
                                           glse, part, block_table=block_table, page_size=self.page_size, out=out,
-                                          sync=self._sync_reuse)
+                                          sync=self._sync_reuse, k_new=k_new, v_new=v_new)
 
-    def reuse(self, layer, q, k_pages, v_pages, block_table, seqlens, out=None):
+    def reuse(self, layer, q, k_pages, v_pages, block_table, seqlens, out=None, k_new=None, v_new=None):
         """Reuse layer: attends to rows head_mapping[layer] of the last anchor's indices."""
         if self._topk_to_reuse is None:
             raise KascadeError("reuse layer called before any anchor layer")
-        return self._reuse(q, k_pages, v_pages, block_table, seqlens, self._hm[layer], out)
+        return self._reuse(q, k_pages, v_pages, block_table, seqlens, self._hm[layer], out, k_new, v_new)
 
     def forward(self, layer, q, k_pages, v_pages, block_table, seqlens, max_len: int, ragged: bool = True,
-                out=None):
+                out=None, k_new=None, v_new=None):
         if layer in self.recompute_layers:
-            return self.anchor(layer, q, k_pages, v_pages, block_table, seqlens, max_len, ragged, out)
-        return self.reuse(layer, q, k_pages, v_pages, block_table, seqlens, out)
+            return self.anchor(layer, q, k_pages, v_pages, block_table, seqlens, max_len, ragged, out,
+                               k_new, v_new)
+        return self.reuse(layer, q, k_pages, v_pages, block_table, seqlens, out, k_new, v_new)
 
 
 class PagedKascadePrefill:

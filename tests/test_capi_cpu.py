@@ -56,10 +56,10 @@ def test_null_pointers_are_rejected(lib):
     s = Strides(8, 8, 8)
     assert lib.kascade_decode_reuse_call(None, None, None, None, None, None, None, None, 1, 128, 128, 8, None, None) == -1
     assert "null pointer" in _err(lib)
-    assert lib.kascade_decode_dense_paged_call(None, None, None, None, None, None, None, 1, 128, 8, None, 0, 16, None, None, None) == -1
+    assert lib.kascade_decode_dense_paged_call(None, None, None, None, None, None, None, 1, 128, 8, None, 0, 16, None, None, None, None, None) == -1
     assert "null pointer" in _err(lib)
     assert lib.kascade_decode_recompute_paged_call(None, None, None, None, None, None, None, None, None, None,
-                                                   1, 128, 128, 8, 1, None, 0, 16, None, None, None) == -1
+                                                   1, 128, 128, 8, 1, None, 0, 16, None, None, None, None, None) == -1
     assert lib.kascade_topk_call(None, None, 1, 10, 10, None, None, 1, 4, 0, None, None) == -1
     assert lib.kascade_prefill_dense_call(None, None, None, None, None, 1, 64, s, s, 1, None) == -1
     assert lib.kascade_prefill_aggregate_call(None, None, None, None, 1, 64, s, s, 0, None) == -1
@@ -72,20 +72,25 @@ def test_bad_sizes_are_rejected(lib):
     buf = (C.c_char * 4096)()
     p = C.addressof(buf) & ~15          # fake, 16-byte aligned, never dereferenced: validation fails first
     p += 16
-    assert lib.kascade_decode_reuse_paged_call(p, p, p, None, p, p, 0.0, p, p, p, 0, 128, 128, 8, None, 0, 16, None, None, None) == -1
+    assert lib.kascade_decode_reuse_paged_call(p, p, p, None, p, p, 0.0, p, p, p, 0, 128, 128, 8, None, 0, 16, None, None, None, None, None) == -1
     assert "batch" in _err(lib)
-    assert lib.kascade_decode_reuse_paged_call(p, p, p, None, p, p, 10.0, p, p, p, 1, 128, 128, 8, None, 0, 16, None, None, None) == -1
+    assert lib.kascade_decode_reuse_paged_call(p, p, p, None, p, p, 10.0, p, p, p, 1, 128, 128, 8, None, 0, 16, None, None, None, None, None) == -1
     assert "cache_seqlens" in _err(lib)
-    assert lib.kascade_decode_dense_paged_call(p, p, p, None, p, p, p, 1, 128, 8, p, 4, 12, None, None, None) == -1
+    assert lib.kascade_decode_dense_paged_call(p, p, p, None, p, p, p, 1, 128, 8, p, 4, 12, None, None, None, None, None) == -1
     assert "power of two" in _err(lib)
-    assert lib.kascade_decode_dense_paged_call(p + 2, p, p, None, p, p, p, 1, 128, 8, None, 0, 16, None, None, None) == -1
+    assert lib.kascade_decode_dense_paged_call(p + 2, p, p, None, p, p, p, 1, 128, 8, None, 0, 16, None, None, None, None, None) == -1
     assert "aligned" in _err(lib)
     hf = Strides(8 * 128 * 128, 128, 128 * 128)      # a head-major [B,G,L,D] cache seen as [B,L,G,D]
-    assert lib.kascade_decode_dense_paged_call(p, p, p, None, p, p, p, 1, 128, 8, p, 4, 16, C.byref(hf), None, None) == -1
+    assert lib.kascade_decode_dense_paged_call(p, p, p, None, p, p, p, 1, 128, 8, p, 4, 16, C.byref(hf), None, None, None, None) == -1
     assert "exclude each other" in _err(lib)
     assert lib.kascade_decode_dense_paged_call(p, p, p, None, p, p, p, 1, 128, 8, None, 0, 16,
-                                               C.byref(Strides(1024, 4, 128)), None, None) == -1
+                                               C.byref(Strides(1024, 4, 128)), None, None, None, None) == -1
     assert "strides" in _err(lib)
+    assert lib.kascade_decode_dense_paged_call(p, p, p, None, p, p, p, 1, 128, 8, None, 0, 16, None, p, None, None, None) == -1
+    assert "come together" in _err(lib)
+    assert lib.kascade_decode_budgets_call(None, 1, 10.0, 1, None, None, None) == -1
+    assert lib.kascade_decode_budgets_call(p, 1, 101.0, 1, None, None, None) == -1
+    assert "topk_percent" in _err(lib)
     assert lib.kascade_topk_call(p, p, 4, 100, 200, None, None, 1, 8, 0, None, None) == -1
     assert "uniform_len" in _err(lib)
     bad = Strides(100, 4, 128)          # not multiples of 8 elements

@@ -306,3 +306,93 @@ def test_head_major_cache_is_read_in_place(cuda, seqlens):
         f = kernels.decode_reuse(q, kh, vh, idx, hm, glse, part)
         assert torch.equal(e, f), "reuse decode"
         assert_close(f, orc.reuse_decode(w.q, kc.cpu(), vc.cpu(), idx.cpu(), hm.tolist()), "reuse decode vs oracle")
+
+
+@pytest.mark.parametrize("seqlens,ns", [([1500, 333], 4), ([2600], 3), ([2600], 1), ([1, 70], 2)])
+def test_fused_append_of_the_newest_token(cuda, seqlens, ns):
+    """Handing the newest token's K/V rows to a decode call (k_new / v_new) gives bit-identical
+    results to appending them first, leaves them in the cache slot, and changes nothing else."""
+    from kascade_amd import kernels
+    w = _paged_case(seqlens, seed=31)
+    B, Lmax = len(seqlens), max(seqlens)
+    q, lens, bt = w.q.to(cuda), w.seqlens.to(cuda), w.block_table.to(cuda)
+    k_full, v_full = w.k_pages.to(cuda), w.v_pages.to(cuda)
+    # the newest rows, and caches whose newest slot still holds rubbish
+    k_new = torch.empty(B, G, D, dtype=torch.float16, device=cuda)
+    v_new = torch.empty_like(k_new)
+    k_hole, v_hole = k_full.clone(), v_full.clone()
+    for b, n in enumerate(seqlens):
+        pg, slot = int(w.block_table[b, (n - 1) // w.page_size]), (n - 1) % w.page_size
+        k_new[b], v_new[b] = k_full[pg, slot], v_full[pg, slot]
+        k_hole[pg, slot] = float("nan")
+        v_hole[pg, slot] = float("nan")
+    glse, part = _scratch(B, ns, cuda)
+    sync = torch.zeros(B * G, dtype=torch.int32, device=cuda)
+
+    def check_cache(kc, vc, what):
+        torch.cuda.synchronize()
+        assert torch.equal(kc, k_full) and torch.equal(vc, v_full), f"{what}: cache after the fused append"
+
+    # dense
+    want = kernels.decode_dense_paged(q, k_full, v_full, lens, glse, part, bt, w.page_size)
+    for s in (None, sync):
+        kc, vc = k_hole.clone(), v_hole.clone()
+        got = kernels.decode_dense_paged(q, kc, vc, lens, glse, part, bt, w.page_size, sync=s,
+                                         k_new=k_new, v_new=v_new)
+        if s is None:
+            assert torch.equal(got, want), "dense decode with fused append"
+        else:
+            assert_close(got, want, "dense decode with fused append (fused merge)", atol=1e-3, rtol=2e-3)
+        check_cache(kc, vc, "dense")
+    # anchor passes (layer 0 with output, layer > 0 scores only: V is appended all the same)
+    row_sums = torch.empty(B, H, device=cuda, dtype=torch.float32)
+    stride = ((Lmax + 7) // 8) * 8
+    scores = torch.empty(B, H, stride, device=cuda, dtype=torch.float32)
+    for layer in (0, 1):
+        o1, agg1 = kernels.decode_recompute(q, k_full, v_full, glse, part, row_sums, scores, layer,
+                                            cache_seqlens=lens, block_table=bt, page_size=w.page_size)
+        kc, vc = k_hole.clone(), v_hole.clone()
+        o2, agg2 = kernels.decode_recompute(q, kc, vc, glse, part, row_sums, scores, layer, cache_seqlens=lens,
+                                            block_table=bt, page_size=w.page_size, k_new=k_new, v_new=v_new)
+        for b, n in enumerate(seqlens):
+            assert torch.equal(agg1[b, :, :n], agg2[b, :, :n]), f"agg, layer {layer}"
+        if layer == 0:
+            assert torch.equal(o1, o2), "anchor-0 output with fused append"
+        check_cache(kc, vc, f"anchor layer {layer}")
+    # reuse: lists with the newest token at the front, deep in the list, and absent
+    gen = torch.Generator().manual_seed(8)
+    kk = max(1, min(min(seqlens) - 1, 1300))
+    hm = torch.tensor([3, 3, 0, 1, 7, 6, 5, 2], dtype=torch.int32, device=cuda)
+    for where in ("front", "deep", "absent"):
+        idx = torch.empty(B, G, kk, dtype=torch.int32)
+        for b, n in enumerate(seqlens):
+            for g in range(G):
+                others = torch.randperm(n - 1, generator=gen)[:kk] if n > 1 else torch.zeros(kk, dtype=torch.long)
+                row = others.clone()
+                if where != "absent" and kk >= 1:
+                    row[0 if where == "front" else kk - 1 - (g % min(kk, 7))] = n - 1
+                idx[b, g] = row
+        if min(seqlens) == 1 and where == "absent":
+            continue   # a one-token sequence has nothing else to list
+        idx = idx.to(cuda)
+        want = kernels.decode_reuse_paged(q, k_full, v_full, lens, idx, hm, 0.0, glse, part, block_table=bt,
+                                          page_size=w.page_size)
+        kc, vc = k_hole.clone(), v_hole.clone()
+        got = kernels.decode_reuse_paged(q, kc, vc, lens, idx, hm, 0.0, glse, part, block_table=bt,
+                                         page_size=w.page_size, k_new=k_new, v_new=v_new)
+        assert torch.isfinite(got).all() and torch.equal(got, want), f"reuse decode, newest token {where}"
+        check_cache(kc, vc, f"reuse ({where})")
+
+
+def test_decode_budgets_launch(cuda):
+    from kascade_amd import kernels
+    lens = [1, 99, 1280, 1281, 65536, 131071, 524288]
+    for p in (10, 2.5, 100):
+        t = torch.tensor(lens, dtype=torch.int32, device=cuda)
+        valid, nsel = kernels.decode_budgets(t, p, advance=0)
+        assert valid.cpu().tolist() == [n for n in lens for _ in range(G)]
+        assert nsel.cpu().tolist() == [orc.n_kvcache(n, p) for n in lens for _ in range(G)]
+        valid, nsel = kernels.decode_budgets(t, p, advance=1)
+        assert t.cpu().tolist() == [n + 1 for n in lens]
+        assert valid.cpu().tolist() == [n + 1 for n in lens for _ in range(G)]
+        assert nsel.cpu().tolist() == [orc.n_kvcache(n + 1, p) for n in lens for _ in range(G)]

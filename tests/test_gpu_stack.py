@@ -111,6 +111,11 @@ def test_stack_decode_eager_graph_oracle(cuda):
         for g in range(G):
             ok, recall, msg = orc.topk_agreement(agg[0, g], idx[0, g], count, t + 1, ulps=1.0)
             assert ok, f"step {step} anchor 2 group {g}: {msg}"
+    # every decode launch sequence appended its layer's new token itself
+    for l in range(N_LAYERS):
+        kc = orc.paged_to_contiguous(eager.k_pages[l].cpu(), eager.block_table.cpu(), [n])
+        vc = orc.paged_to_contiguous(eager.v_pages[l].cpu(), eager.block_table.cpu(), [n])
+        assert torch.equal(kc[0], ks[l][0, :n]) and torch.equal(vc[0], vs[l][0, :n]), f"layer {l} cache"
     # dense stack decode
     dense = _stack(cuda, dense=True)
     _prefill(dense, pre(qs), pre(ks), pre(vs), cuda)
