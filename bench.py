@@ -490,10 +490,35 @@ def main():
             log(f"[bench] cpu block {i}: rows {s}..{e}: dense {t_dense_blk:.2f}s pool+topk {t_pool_blk:.2f}s "
                 f"reuse {t_reuse_blk:.2f}s")
         cpu_ms = (est["anchor0"] + 4 * est["anchor"] + 27 * est["reuse"]) / N_LAYERS * 1e3
+        # decode (config 2 shape): one step of the three layer kinds on 2 of the 16 sequences
+        cpu_decode = None
+        if not args.skip_decode:
+            Bs, Ld = 2, 65536
+            dk = torch.stack([workloads.peaked_keys(Ld, seed=70 + b, device="cpu") for b in range(Bs)])
+            dv = workloads.gaussian((Bs, Ld, G, D), seed=80, device="cpu")
+            dq = workloads.gaussian((Bs, H, D), seed=81, device="cpu")
+            t0 = time.perf_counter()
+            orc.dense_decode(dq, dk, dv)
+            t_dd = time.perf_counter() - t0
+            t0 = time.perf_counter()
+            idx_d = orc.topk_rows(orc.pooled_decode_scores(dq, dk), budgets.topk_width(Ld, PCT))
+            t_da = time.perf_counter() - t0
+            t0 = time.perf_counter()
+            orc.reuse_decode(dq, dk, dv, idx_d, list(head_map[1]))
+            t_dr = time.perf_counter() - t0
+            scale = 16 / Bs * 1e6
+            per = {"dense_us": t_dd * scale, "anchor0_us": (t_dd + t_da) * scale,
+                   "anchor_us": (t_da + t_dr) * scale, "reuse_us": t_dr * scale}
+            per["kascade_us_per_layer"] = (per["anchor0_us"] + 4 * per["anchor_us"] + 27 * per["reuse_us"]) / N_LAYERS
+            cpu_decode = {k: round(v, 0) for k, v in per.items()}
+            cpu_decode["sample"] = (f"oracle on {Bs} of the 16 sequences of configs[2] (65536-token contexts, "
+                                    f"contiguous cache), one decode step per layer kind, scaled by 16/{Bs}")
+            log(f"[bench] cpu decode: {cpu_decode}")
         cpu = {"value": round(cpu_ms, 1), "unit": "ms", "cores": nthreads, "kind": "port",
                "sample": f"oracle (dense-matrix PyTorch, fp32) on {nblk} blocks of {rows} query rows centred in "
                          f"each quarter of the {Lc}-token prompt, extrapolated by rows; layer mix 1/4/27",
-               "per_layer_ms": {k: round(v * 1e3, 1) for k, v in est.items()}}
+               "per_layer_ms": {k: round(v * 1e3, 1) for k, v in est.items()},
+               "decode_cfg2": cpu_decode}
 
     out = {
         "metric": "kascade prefill attn ms/layer @32K (value) & decode attn us/layer @64K/128K/ragged (decode), "
