@@ -112,3 +112,31 @@ def test_python_wrappers_fail_loudly_without_gpu():
     q = torch.zeros(1, 32, 128, dtype=torch.float16)
     with pytest.raises((KascadeError, RuntimeError)):
         kernels.decode_reuse(q, q, q, q, q, q, q)
+
+
+def test_header_is_plain_c_and_links_from_c(lib, tmp_path):
+    """The boundary is a C ABI: the header compiles as C99 (no C++ needed) and a C program
+    linked against the library reads the ABI version and gets the error convention
+    (-1 + message) without a GPU."""
+    import shutil
+    import subprocess
+    from kascade_amd import _lib
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "abi.c"
+    src.write_text(
+        '#include <stdio.h>\n#include <string.h>\n#include "kascade_hip.h"\n'
+        "int main(void) {\n"
+        "    if (kascade_abi_version() < 1) return 2;\n"
+        "    if (kascade_topk_call(0, 0, 1, 10, 10, 0, 0, 1, 4, 0, 0, 0) != -1) return 3;\n"
+        "    if (strlen(kascade_get_last_error()) == 0) return 4;\n"
+        '    printf("%d\\n", kascade_abi_version());\n'
+        "    return 0;\n}\n")
+    exe = tmp_path / "abi"
+    libdir = str(_lib.LIB_PATH.parent)
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"),
+                    str(src), "-o", str(exe), "-L", libdir, "-l:" + _lib.LIB_PATH.name,
+                    "-Wl,-rpath," + libdir], check=True, capture_output=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True)
+    assert int(out.stdout.strip()) == lib.kascade_abi_version()
