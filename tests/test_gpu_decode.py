@@ -396,3 +396,51 @@ def test_decode_budgets_launch(cuda):
         assert t.cpu().tolist() == [n + 1 for n in lens]
         assert valid.cpu().tolist() == [n + 1 for n in lens for _ in range(G)]
         assert nsel.cpu().tolist() == [orc.n_kvcache(n + 1, p) for n in lens for _ in range(G)]
+
+
+def test_fused_append_contiguous_and_head_major(cuda):
+    """The fused append also serves caches without a block table: the contiguous [B,L,G,D] layout
+    with a uniform length (no cache_seqlens) and a head-major [B,G,L,D] cache behind strides."""
+    from kascade_amd import kernels
+    gen = torch.Generator().manual_seed(17)
+    B, L = 2, 777
+    q = torch.randn(B, H, D, generator=gen).half().to(cuda)
+    k_full = torch.randn(B, L, G, D, generator=gen).half().to(cuda)
+    v_full = torch.randn(B, L, G, D, generator=gen).half().to(cuda)
+    k_new, v_new = k_full[:, L - 1].contiguous(), v_full[:, L - 1].contiguous()
+    glse, part = _scratch(B, 3, cuda)
+    want = kernels.decode_dense_paged(q, k_full, v_full, None, glse, part)
+    # contiguous, uniform length
+    kc, vc = k_full.clone(), v_full.clone()
+    kc[:, L - 1] = float("nan"); vc[:, L - 1] = float("nan")
+    got = kernels.decode_dense_paged(q, kc, vc, None, glse, part, k_new=k_new, v_new=v_new)
+    assert torch.equal(got, want) and torch.equal(kc, k_full) and torch.equal(vc, v_full)
+    # head-major storage with spare room, per-sequence lengths
+    lens = torch.tensor([L, L - 100], dtype=torch.int32, device=cuda)
+    ks = torch.zeros(B, G, L + 8, D, dtype=torch.float16, device=cuda)
+    vs = torch.zeros_like(ks)
+    ks[:, :, :L] = k_full.permute(0, 2, 1, 3); vs[:, :, :L] = v_full.permute(0, 2, 1, 3)
+    kn = torch.stack([k_full[b, int(lens[b]) - 1] for b in range(B)])
+    vn = torch.stack([v_full[b, int(lens[b]) - 1] for b in range(B)])
+    want = kernels.decode_dense_paged(q, ks[:, :, :L].transpose(1, 2), vs[:, :, :L].transpose(1, 2), lens, glse, part)
+    kh, vh = ks.clone(), vs.clone()
+    for b in range(B):
+        kh[b, :, int(lens[b]) - 1] = float("nan"); vh[b, :, int(lens[b]) - 1] = float("nan")
+    got = kernels.decode_dense_paged(q, kh[:, :, :L].transpose(1, 2), vh[:, :, :L].transpose(1, 2), lens, glse, part,
+                                     k_new=kn, v_new=vn)
+    assert torch.equal(got, want) and torch.equal(kh, ks) and torch.equal(vh, vs)
+    # reuse decode over the same head-major cache, list naming the newest token
+    idx = torch.stack([torch.stack([torch.randperm(L - 100, generator=gen)[:256] for _ in range(G)])
+                       for _ in range(B)]).to(torch.int32)
+    for b in range(B):
+        idx[b, :, 5] = int(lens[b]) - 1
+    idx = idx.to(cuda)
+    hm = torch.arange(G, dtype=torch.int32, device=cuda)
+    want = kernels.decode_reuse_paged(q, ks[:, :, :L].transpose(1, 2), vs[:, :, :L].transpose(1, 2), lens, idx, hm,
+                                      0.0, glse, part)
+    kh, vh = ks.clone(), vs.clone()
+    for b in range(B):
+        kh[b, :, int(lens[b]) - 1] = float("nan"); vh[b, :, int(lens[b]) - 1] = float("nan")
+    got = kernels.decode_reuse_paged(q, kh[:, :, :L].transpose(1, 2), vh[:, :, :L].transpose(1, 2), lens, idx, hm,
+                                     0.0, glse, part, k_new=kn, v_new=vn)
+    assert torch.isfinite(got).all() and torch.equal(got, want) and torch.equal(kh, ks) and torch.equal(vh, vs)
