@@ -137,8 +137,10 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
-    def ev_time(fn, n=5, warm=1):
-        """Median duration (us) of fn() measured with events on the stream the kernels launch on."""
+    def ev_time(fn, n=5, warm=1, reps=1):
+        """Median duration (us) of fn() measured with events on the stream the kernels launch on.
+        reps > 1: that many calls back to back between the two events (for calls so short that
+        the host's launch path would otherwise be part of what is timed), divided by reps."""
         for _ in range(warm):
             fn()
         ts = []
@@ -146,10 +148,11 @@ def main():
             s = torch.cuda.Event(enable_timing=True)
             e = torch.cuda.Event(enable_timing=True)
             s.record()
-            fn()
+            for _ in range(reps):
+                fn()
             e.record()
             e.synchronize()
-            ts.append(s.elapsed_time(e) * 1e3)
+            ts.append(s.elapsed_time(e) * 1e3 / reps)
         ts.sort()
         return ts[len(ts) // 2]
 
@@ -211,10 +214,10 @@ def main():
         scores = torch.empty(1, G, T, L, device=dev, dtype=torch.float16)
         t_agg = ev_time(lambda: kernels.prefill_aggregate(w.q, w.k, log_sum, scores), n=3)
         valid, nsel = strat._tile_budgets(L, width, dev)
-        t_topk = ev_time(lambda: kernels.topk_indices(scores, width, valid_len=valid, n_sel=nsel), n=3)
+        t_topk = ev_time(lambda: kernels.topk_indices(scores, width, valid_len=valid, n_sel=nsel), n=3, reps=3)
         idx = kernels.topk_indices(scores, width, valid_len=valid, n_sel=nsel)
         hm = strat._hm(1, dev)
-        t_reuse = ev_time(lambda: kernels.prefill_reuse(w.q_reuse, w.k_reuse, w.v, idx, hm, float(PCT), True), n=5)
+        t_reuse = ev_time(lambda: kernels.prefill_reuse(w.q_reuse, w.k_reuse, w.v, idx, hm, float(PCT), True), n=5, reps=3)
         del scores, idx, log_sum
 
         def mfma(flop, us):
@@ -292,10 +295,10 @@ def main():
 
             t_dense = ev_time(dense_step, n=3) / N_LAYERS
             t_kas = ev_time(kascade_step, n=3) / N_LAYERS
-            t_a0 = ev_time(lambda: kascade_layer(0), n=5)
-            t_a = ev_time(lambda: kascade_layer(2), n=5)
+            t_a0 = ev_time(lambda: kascade_layer(0), n=5, reps=3)
+            t_a = ev_time(lambda: kascade_layer(2), n=5, reps=3)
             kascade_layer(0)
-            t_r = ev_time(lambda: kascade_layer(1), n=9)
+            t_r = ev_time(lambda: kascade_layer(1), n=7, reps=6)
             counts = [budgets.decode_budget(n, PCT) if ragged else budgets.topk_width(n, PCT) for n in seqlens]
             reuse_bytes = sum(G * n * D * 2 * 2 + G * n * 4 for n in counts) + 2 * B * H * D * 2
             dense_bytes = sum(n * G * D * 2 * 2 for n in seqlens)

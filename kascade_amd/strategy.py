@@ -138,7 +138,7 @@ class EfficientKascadeStrategy:
         o, agg = kernels.decode_recompute(Q, K, V, glse, part, row_sums, scores, layer)
         self._topk_to_reuse = kernels.topk_indices(agg[:, :, :L], topk, fill_value=0)
         if layer != 0:
-            ns = kernels.default_num_split(B * G * topk, topk)
+            ns = kernels.default_num_split(B * G * topk, topk, cap_rows=kernels.GATHER_ROWS_PER_SPLIT)
             glse, part = self._decode_scratch(B, ns, Q.device)
             o = kernels.decode_reuse(Q, K, V, self._topk_to_reuse, self._hm(None, Q.device), glse, part)
         return o
@@ -147,7 +147,7 @@ class EfficientKascadeStrategy:
         """Reuse decode (EfficientKascadeStrategy.py:117-123)."""
         B = Q.shape[0]
         topk = self._topk_to_reuse.shape[-1]
-        ns = kernels.default_num_split(B * G * topk, topk)
+        ns = kernels.default_num_split(B * G * topk, topk, cap_rows=kernels.GATHER_ROWS_PER_SPLIT)
         glse, part = self._decode_scratch(B, ns, Q.device)
         return kernels.decode_reuse(Q, K, V, self._topk_to_reuse, self._hm(layer, Q.device), glse, part)
 
@@ -229,7 +229,7 @@ class PagedKascadeDecoder:
         total = total_tokens if total_tokens is not None else max_batch * max_seqlen
         self.ns_dense = num_split_dense or kernels.default_num_split(G * total, max_seqlen)
         self.ns_reuse = num_split_reuse or kernels.default_num_split(
-            G * budgets.decode_budget(total, k), self.max_topk)
+            G * budgets.decode_budget(total, k), self.max_topk, cap_rows=kernels.GATHER_ROWS_PER_SPLIT)
         ns = max(self.ns_dense, self.ns_reuse)
         dev = self.device
         self._glse = torch.empty(max_batch * H * ns, device=dev, dtype=torch.float32)

@@ -97,6 +97,10 @@ def test_default_num_split_heuristic(monkeypatch):
     assert kernels.default_num_split(8 * 300, 300) == 2
     assert kernels.default_num_split(8 * 1664, 1664) == 13
     assert kernels.default_num_split(8 * 100, 100) == 1
+    # gather launches: about 1664 rows per workgroup however large the total
+    assert kernels.default_num_split(128 * 13184, 13184) == 4
+    assert kernels.default_num_split(128 * 13184, 13184, cap_rows=kernels.GATHER_ROWS_PER_SPLIT) == 8
+    assert kernels.default_num_split(128 * 6656, 6656, cap_rows=kernels.GATHER_ROWS_PER_SPLIT) == 4
 
 
 def test_workloads_are_seeded_and_shaped():
