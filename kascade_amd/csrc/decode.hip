@@ -31,7 +31,7 @@ constexpr int kUnroll = KASCADE_DECODE_UNROLL;  // rows per row-group per iterat
 constexpr int kRowsPerIter = 16 * kUnroll;    // rows per workgroup iteration (128)
 constexpr int kScoreBatches = 16;             // batches between two score flushes (anchor mode)
 constexpr int kStripRows = 16 * kScoreBatches;  // rows a wavefront owns per super-iteration
-constexpr int kSubChunk = 1024;               // rows whose physical ids are staged in LDS at once
+constexpr int kSubChunk = 2048;               // rows whose physical ids are staged in LDS at once
 
 // Device-coherent accesses (relaxed atomics at agent scope) for data that one workgroup writes
 // and another workgroup of the same launch reads.
