@@ -175,7 +175,16 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
     issue_loads();
     if (ntiles > 1) fetch_ids(1);
 
-    for (int ti = 0; ti < ntiles; ++ti) {
+    // The diagonal tile of a sparse unit (32 keys, half the products) runs as a second phase of
+    // the tile loop; the phase loop is unrolled, so each phase is compiled with its key-block
+    // count as a constant and the tiles before the diagonal run straight-line code (with a
+    // run-time count every matrix instruction of the second half sits behind a branch).
+#pragma unroll
+    for (int phase = 0; phase < (REUSE ? 2 : 1); ++phase) {
+    const bool diag_phase = (phase == 1);
+    const int t_begin = diag_phase ? ng : 0;
+    const int t_end = diag_phase ? (sparse ? ng + 1 : ng) : (REUSE && sparse ? ng : ntiles);
+    for (int ti = t_begin; ti < t_end; ++ti) {
         __syncthreads();
         // ---- registers -> LDS ----
 #pragma unroll
@@ -202,7 +211,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
         }
 
         // ---- S^T = K_tile Q^T ----
-        const bool diag_tile = sparse && (ti == ng);
+        const bool diag_tile = diag_phase;
         const int nkb = (diag_tile && QT == 32) ? 1 : 2;
         float16_t sT[NQB][2];
         float16_t zero16;
@@ -312,6 +321,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
                 }
             }
         }
+    }
     }
 
     // ---- epilogue (rows are local to this call) ----
