@@ -17,7 +17,7 @@ constexpr int kWaves = kThreads / 64;
 constexpr int kChunk = kThreads * 8;
 constexpr int kBins1 = 2048;
 }  // namespace
-constexpr int kSplitMinLen = 32768;   // rows at least this long take the multi-workgroup path
+constexpr int kSplitMinLen = 65537;   // longer than a workgroup's registers hold: multi-workgroup path
 constexpr int kSplitMaxRows = 4096;   // workspace is 8 KB per row for the coarse histogram
 namespace {
 
@@ -183,6 +183,233 @@ __global__ __launch_bounds__(kThreads) void topk_select_kernel(
         eq_base += total >> 16;
     }
     for (int i = n + tid; i < k; i += kThreads) dst[i] = fill;
+}
+
+
+// The same selection with the row held in registers: every thread loads its share of the row
+// once (MAXC 16-byte loads in flight, instead of one per pass and chunk with its latency
+// exposed) and the three passes run on registers.
+//  * The coarse histogram is kept in kCopies copies selected by the lane number, which spreads
+//    the same-address conflicts of the LDS atomics (pooled softmax scores crowd into a few
+//    exponent bins).
+//  * The compaction computes every (chunk, thread) offset with two barriers in all (per-chunk
+//    wavefront scans, then one scan over the chunk x wavefront totals), and stages the selected
+//    indices in LDS in their final order, so that the row's list leaves as full-width stores.
+// Rows must be 16-byte aligned and at most MAXC*8192 entries long.
+template <int MAXC>
+__global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
+    const uint16_t* __restrict__ scores, int* __restrict__ out, long long row_stride,
+    int uniform_len, const int* __restrict__ valid_len, const int* __restrict__ n_sel, int period,
+    int k, int fill) {
+    constexpr int kCopies = 4;
+    constexpr int kStage = kBins1 * kCopies;       // selected indices staged in the histogram's LDS
+    __shared__ uint32_t s_hist[kBins1 * kCopies];
+    __shared__ uint32_t s_hist2[32];
+    __shared__ uint32_t s_wave[kWaves];
+    __shared__ uint32_t s_tot[MAXC * kWaves];      // pass 3: totals, then exclusive prefixes
+    __shared__ uint32_t s_sel[4];  // b1, cum_above, T, r
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const long long row = blockIdx.x;
+    const int pr = (int)(row % period);
+    const int len = valid_len ? min(valid_len[pr], uniform_len) : uniform_len;
+    int n = n_sel ? n_sel[pr] : k;
+    n = max(0, min(n, k));
+    const uint16_t* src = scores + row * row_stride;
+    int* dst = out + row * (long long)k;
+
+    if (len <= n || n == 0) {
+        for (int i = tid; i < k; i += kThreads) dst[i] = (i < n) ? i : fill;
+        return;
+    }
+    const int nchunks = (len + kChunk - 1) / kChunk;   // <= MAXC (host)
+
+    // ---- the row: chunk c, entries [c*8192 + 8*tid, +8), as packed fp16 bit patterns ----
+    uint4_t data[MAXC];
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+        const int base = c * kChunk + tid * 8;
+        if (c < nchunks && base + 8 <= len) {
+            data[c] = *reinterpret_cast<const uint4_t*>(src + base);
+        } else {
+            // ragged end (or nothing): entries past the end are never counted
+            uint32_t w[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t lo = (c < nchunks && base + 2 * e < len) ? src[base + 2 * e] : 0xFC00u;
+                const uint32_t hi = (c < nchunks && base + 2 * e + 1 < len) ? src[base + 2 * e + 1] : 0xFC00u;
+                w[e] = lo | (hi << 16);
+            }
+            data[c] = uint4_t{w[0], w[1], w[2], w[3]};
+        }
+    }
+    auto key_of = [&](int c, int e) {
+        const uint32_t w = data[c][e >> 1];
+        return order_key((uint16_t)((e & 1) ? (w >> 16) : (w & 0xFFFFu)));
+    };
+    auto valid = [&](int c, int e) { return c * kChunk + tid * 8 + e < len; };
+
+    // ---- pass 1: coarse histogram ----
+    for (int i = tid; i < kBins1 * kCopies; i += kThreads) s_hist[i] = 0;
+    if (tid < 32) s_hist2[tid] = 0;
+    __syncthreads();
+    const int copy = tid & (kCopies - 1);
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+        if (c < nchunks) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (valid(c, e)) atomicAdd(&s_hist[(key_of(c, e) >> 5) * kCopies + copy], 1u);
+        }
+    }
+    __syncthreads();
+    {
+        // thread t owns bins 2047-2t and 2046-2t (descending order)
+        const int rb0 = kBins1 - 1 - 2 * tid;
+        uint32_t c0 = 0, c1 = 0;
+#pragma unroll
+        for (int j = 0; j < kCopies; ++j) {
+            c0 += s_hist[rb0 * kCopies + j];
+            c1 += s_hist[(rb0 - 1) * kCopies + j];
+        }
+        uint32_t total;
+        const uint32_t above0 = block_excl_scan(c0 + c1, s_wave, &total);
+        const uint32_t above1 = above0 + c0;
+        const uint32_t un = (uint32_t)n;
+        if (above0 < un && un <= above0 + c0) {
+            s_sel[0] = rb0;
+            s_sel[1] = above0;
+        } else if (above1 < un && un <= above1 + c1) {
+            s_sel[0] = rb0 - 1;
+            s_sel[1] = above1;
+        }
+    }
+    __syncthreads();
+    const uint32_t b1 = s_sel[0];
+    const uint32_t cum_above = s_sel[1];
+
+    // ---- pass 2: fine histogram inside the threshold bin ----
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+        if (c < nchunks) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t key = key_of(c, e);
+                if (valid(c, e) && (key >> 5) == b1) atomicAdd(&s_hist2[key & 31u], 1u);
+            }
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {
+        uint32_t above = cum_above;
+        int b2 = 31;
+        for (; b2 > 0; --b2) {
+            uint32_t c = s_hist2[b2];
+            if (above + c >= (uint32_t)n) break;
+            above += c;
+        }
+        s_sel[2] = (b1 << 5) | (uint32_t)b2;
+        s_sel[3] = (uint32_t)n - above;  // entries equal to T to take
+    }
+    __syncthreads();
+    const uint32_t T = s_sel[2];
+    const uint32_t r = s_sel[3];
+
+    // ---- pass 3: ordered compaction (index order = chunk, then thread, then element) ----
+    // counts of one (chunk, thread): entries above T in the low half, equal to T in the high half
+    uint32_t inc[MAXC];   // inclusive scan of the counts over the wavefront
+    uint32_t own[MAXC];
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+        uint32_t gt = 0, eq = 0;
+        if (c < nchunks) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                if (valid(c, e)) {
+                    const uint32_t key = key_of(c, e);
+                    gt += (key > T);
+                    eq += (key == T);
+                }
+            }
+        }
+        own[c] = gt | (eq << 16);
+        uint32_t v = own[c];
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const uint32_t t = __shfl_up(v, o);
+            if (lane >= o) v += t;
+        }
+        inc[c] = v;
+        if (lane == 63) s_tot[c * kWaves + wave] = v;
+    }
+    __syncthreads();
+    if (wave == 0) {
+        // exclusive prefix over the MAXC*16 (chunk, wavefront) totals, chunk-major, 64 per step;
+        // both halves stay below 65536 (a row has at most 65536 entries)
+        uint32_t carry = 0;
+#pragma unroll
+        for (int i0 = 0; i0 < MAXC * kWaves; i0 += 64) {
+            const uint32_t x = s_tot[i0 + lane];
+            uint32_t v = x;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const uint32_t t = __shfl_up(v, o);
+                if (lane >= o) v += t;
+            }
+            s_tot[i0 + lane] = carry + v - x;
+            carry += __shfl(v, 63);
+        }
+    }
+    __syncthreads();
+    const bool staged = n <= kStage;   // uniform
+    int* stage = reinterpret_cast<int*>(s_hist);
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+        if (c < nchunks) {
+            const uint32_t ex = s_tot[c * kWaves + wave] + inc[c] - own[c];
+            uint32_t my_gt = ex & 0xFFFFu;
+            uint32_t my_eq = ex >> 16;
+            const int base = c * kChunk + tid * 8;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                if (valid(c, e)) {
+                    const uint32_t key = key_of(c, e);
+                    int pos = -1;
+                    if (key > T) {
+                        pos = (int)(my_gt + min(my_eq, r));
+                        ++my_gt;
+                    } else if (key == T) {
+                        if (my_eq < r) pos = (int)(my_gt + my_eq);
+                        ++my_eq;
+                    }
+                    if (pos >= 0) {
+                        if (staged) stage[pos] = base + e;
+                        else dst[pos] = base + e;
+                    }
+                }
+            }
+        }
+    }
+    if (staged) {
+        __syncthreads();
+        // k is a multiple of 4 for every budget the library produces; otherwise element stores
+        if ((k & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+            for (int i = tid * 4; i < k; i += kThreads * 4) {
+                int4 v;
+                v.x = (i + 0 < n) ? stage[i + 0] : fill;
+                v.y = (i + 1 < n) ? stage[i + 1] : fill;
+                v.z = (i + 2 < n) ? stage[i + 2] : fill;
+                v.w = (i + 3 < n) ? stage[i + 3] : fill;
+                *reinterpret_cast<int4*>(dst + i) = v;
+            }
+        } else {
+            for (int i = tid; i < k; i += kThreads) dst[i] = (i < n) ? stage[i] : fill;
+        }
+    } else {
+        for (int i = n + tid; i < k; i += kThreads) dst[i] = fill;
+    }
 }
 
 
@@ -458,9 +685,19 @@ hipError_t launch_topk(const half_t* scores, int* out_idx, int rows, long long r
                        int uniform_len, const int* valid_len, const int* n_sel, int period, int k,
                        int fill, hipStream_t stream) {
     if (rows == 0) return hipSuccess;
-    hipLaunchKernelGGL(topk_select_kernel, dim3(rows), dim3(kThreads), 0, stream,
-                       reinterpret_cast<const uint16_t*>(scores), out_idx, row_stride, uniform_len,
-                       valid_len, n_sel, period, k, fill);
+    const uint16_t* src = reinterpret_cast<const uint16_t*>(scores);
+    // rows that start 16-byte aligned and fit the register file of a workgroup are selected
+    // from registers; anything else streams the row three times
+    const bool aligned_rows = (reinterpret_cast<uintptr_t>(scores) & 15) == 0 && row_stride % 8 == 0;
+    if (aligned_rows && uniform_len <= 4 * kChunk)
+        hipLaunchKernelGGL(topk_select_reg_kernel<4>, dim3(rows), dim3(kThreads), 0, stream, src, out_idx,
+                           row_stride, uniform_len, valid_len, n_sel, period, k, fill);
+    else if (aligned_rows && uniform_len <= 8 * kChunk)
+        hipLaunchKernelGGL(topk_select_reg_kernel<8>, dim3(rows), dim3(kThreads), 0, stream, src, out_idx,
+                           row_stride, uniform_len, valid_len, n_sel, period, k, fill);
+    else
+        hipLaunchKernelGGL(topk_select_kernel, dim3(rows), dim3(kThreads), 0, stream, src, out_idx,
+                           row_stride, uniform_len, valid_len, n_sel, period, k, fill);
     return hipGetLastError();
 }
 

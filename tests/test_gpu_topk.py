@@ -82,3 +82,31 @@ def test_topk_matches_torch_topk_sets_when_no_ties(cuda):
     idx = kernels.topk_indices(sc.to(cuda), K)
     want = torch.topk(sc.float(), K, dim=-1).indices.sort(dim=-1).values.int()
     assert torch.equal(idx.cpu(), want)
+
+
+@pytest.mark.parametrize("L", [60000, 65536, 20000])
+def test_topk_register_kernel_equals_streaming_kernel(cuda, L):
+    """Aligned rows of up to 65536 entries are selected from registers; the same values behind an
+    unaligned row pointer take the streaming kernel.  Both must agree bit for bit, on ragged
+    lengths around the 8192-entry chunk boundaries, ties, -inf runs and degenerate budgets."""
+    from kascade_amd import kernels
+    rows, K = 8, 6016
+    sc = _scores(rows, L, seed=L + 1)
+    sc[1, 500:900] = float("-inf")
+    sc[2] = 0.25                                     # one value everywhere: pure tie-breaking
+    sc[3, : L // 2] = 0.0
+    valid = torch.tensor([L, min(L, 33000), 8192, 8193, 5000, L - 1, 16384, 100], dtype=torch.int32)
+    nsel = torch.tensor([6016, 3328, 1024, 1024, 512, 0, 6016, 128], dtype=torch.int32)
+    assert L % 8 == 0
+    aligned = sc.to(cuda)
+    store = torch.zeros(rows * (L + 1) + 1, dtype=torch.float16, device=cuda)
+    unaligned = store.as_strided((rows, L), (L + 1, 1), storage_offset=1)
+    unaligned.copy_(aligned)
+    assert unaligned.data_ptr() % 16 != 0
+    dvalid, dnsel = valid.to(cuda), nsel.to(cuda)
+    a = kernels.topk_indices(aligned, K, valid_len=dvalid, n_sel=dnsel, fill_value=-1)
+    b = kernels.topk_indices(unaligned, K, valid_len=dvalid, n_sel=dnsel, fill_value=-1)
+    torch.cuda.synchronize()
+    assert torch.equal(a.cpu(), b.cpu())
+    _check(sc, a.cpu(), lambda r: nsel[r], lambda r: valid[r], K, -1)
+    assert torch.equal(a[2, :1024].cpu(), torch.arange(1024, dtype=torch.int32))
