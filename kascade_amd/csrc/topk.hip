@@ -188,10 +188,15 @@ __global__ __launch_bounds__(kThreads) void topk_select_kernel(
 
 // The same selection with the row held in registers: every thread loads its share of the row
 // once (MAXC 16-byte loads in flight, instead of one per pass and chunk with its latency
-// exposed) and the three passes run on registers.
+// exposed), turns it into packed order keys once, and the three passes run on registers.  With
+// 16 to 64 entries per thread and eight wavefronts per SIMD the kernel is bound by the
+// instructions spent per entry, so the per-entry work is branch-free and works on the packed
+// pairs where it can.
 //  * The coarse histogram is kept in kCopies copies selected by the lane number, which spreads
 //    the same-address conflicts of the LDS atomics (pooled softmax scores crowd into a few
 //    exponent bins).
+//  * Entries past the end of the row carry key 0 (below every real key but a negative NaN) and
+//    a separate validity count per chunk keeps them out of every count.
 //  * The compaction computes every (chunk, thread) offset with two barriers in all (per-chunk
 //    wavefront scans, then one scan over the chunk x wavefront totals), and stages the selected
 //    indices in LDS in their final order, so that the row's list leaves as full-width stores.
@@ -207,6 +212,7 @@ __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
     __shared__ uint32_t s_hist2[32];
     __shared__ uint32_t s_wave[kWaves];
     __shared__ uint32_t s_tot[MAXC * kWaves];      // pass 3: totals, then exclusive prefixes
+    __shared__ uint32_t s_zero[64];                // pass 1: where the zeros' idle atomics go
     __shared__ uint32_t s_sel[4];  // b1, cum_above, T, r
 
     const int tid = threadIdx.x;
@@ -226,44 +232,64 @@ __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
     }
     const int nchunks = (len + kChunk - 1) / kChunk;   // <= MAXC (host)
 
-    // ---- the row: chunk c, entries [c*8192 + 8*tid, +8), as packed fp16 bit patterns ----
+    // ---- the row: chunk c, entries [c*8192 + 8*tid, +8) as packed order keys; nv[c] of them
+    //      are inside the row ----
     uint4_t data[MAXC];
+    int nv[MAXC];
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
         const int base = c * kChunk + tid * 8;
-        if (c < nchunks && base + 8 <= len) {
-            data[c] = *reinterpret_cast<const uint4_t*>(src + base);
+        nv[c] = (c < nchunks) ? max(0, min(8, len - base)) : 0;
+        uint4_t raw;
+        if (nv[c] == 8) {
+            raw = *reinterpret_cast<const uint4_t*>(src + base);
         } else {
-            // ragged end (or nothing): entries past the end are never counted
             uint32_t w[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const uint32_t lo = (c < nchunks && base + 2 * e < len) ? src[base + 2 * e] : 0xFC00u;
-                const uint32_t hi = (c < nchunks && base + 2 * e + 1 < len) ? src[base + 2 * e + 1] : 0xFC00u;
+                const uint32_t lo = (2 * e < nv[c]) ? src[base + 2 * e] : 0xFFFFu;       // key 0
+                const uint32_t hi = (2 * e + 1 < nv[c]) ? src[base + 2 * e + 1] : 0xFFFFu;
                 w[e] = lo | (hi << 16);
             }
-            data[c] = uint4_t{w[0], w[1], w[2], w[3]};
+            raw = uint4_t{w[0], w[1], w[2], w[3]};
         }
+        // order_key on both halves at once: negative values flip every bit, others the sign bit
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t neg = ((raw[j] >> 15) & 0x00010001u) * 0xFFFFu;
+            raw[j] ^= (neg | 0x80008000u);
+        }
+        data[c] = raw;
     }
-    auto key_of = [&](int c, int e) {
+    auto key_of = [&](int c, int e) {   // e is a compile-time constant at every use
         const uint32_t w = data[c][e >> 1];
-        return order_key((uint16_t)((e & 1) ? (w >> 16) : (w & 0xFFFFu)));
+        return (e & 1) ? (w >> 16) : (w & 0xFFFFu);
     };
-    auto valid = [&](int c, int e) { return c * kChunk + tid * 8 + e < len; };
 
     // ---- pass 1: coarse histogram ----
     for (int i = tid; i < kBins1 * kCopies; i += kThreads) s_hist[i] = 0;
     if (tid < 32) s_hist2[tid] = 0;
     __syncthreads();
-    const int copy = tid & (kCopies - 1);
+    // Zeros are counted apart: pooled probabilities underflow to +0 by the thousand, and that
+    // many atomics on one address serialise.  Each wavefront counts its zeros with a ballot and
+    // sends those lanes' atomics (adding nothing) to a slot of their own.
+    const uint32_t copy = tid & (kCopies - 1);
+    constexpr uint32_t kZeroKey = 0x8000u;         // order key of +0
+    uint32_t zeros = 0;                            // wavefront-uniform
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
         if (c < nchunks) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e)
-                if (valid(c, e)) atomicAdd(&s_hist[(key_of(c, e) >> 5) * kCopies + copy], 1u);
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t key = key_of(c, e);
+                const bool in = e < nv[c];
+                const bool zero = key == kZeroKey;
+                zeros += (uint32_t)__popcll(__ballot(in && zero));
+                atomicAdd(zero ? &s_zero[lane] : &s_hist[(key >> 5) * kCopies + copy], (in && !zero) ? 1u : 0u);
+            }
         }
     }
+    if (lane == 0 && zeros) atomicAdd(&s_hist[(kZeroKey >> 5) * kCopies], zeros);
     __syncthreads();
     {
         // thread t owns bins 2047-2t and 2046-2t (descending order)
@@ -290,28 +316,39 @@ __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
     const uint32_t b1 = s_sel[0];
     const uint32_t cum_above = s_sel[1];
 
-    // ---- pass 2: fine histogram inside the threshold bin ----
+    // ---- pass 2: fine histogram inside the threshold bin (few entries: a branch is fine) ----
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
         if (c < nchunks) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const uint32_t key = key_of(c, e);
-                if (valid(c, e) && (key >> 5) == b1) atomicAdd(&s_hist2[key & 31u], 1u);
+                if ((key >> 5) == b1 && e < nv[c] && key != kZeroKey) atomicAdd(&s_hist2[key & 31u], 1u);
             }
         }
     }
+    if (b1 == (kZeroKey >> 5) && lane == 0 && zeros) atomicAdd(&s_hist2[kZeroKey & 31u], zeros);
     __syncthreads();
-    if (tid == 0) {
-        uint32_t above = cum_above;
-        int b2 = 31;
-        for (; b2 > 0; --b2) {
-            uint32_t c = s_hist2[b2];
-            if (above + c >= (uint32_t)n) break;
-            above += c;
+    if (tid < 64) {
+        // suffix sums of the 32 fine bins, top bin first; the threshold is the first bin whose
+        // running count reaches n
+        const uint32_t c = (lane < 32) ? s_hist2[31 - lane] : 0u;
+        uint32_t v = c;
+#pragma unroll
+        for (int o = 1; o < 32; o <<= 1) {
+            const uint32_t t = __shfl_up(v, o);
+            if (lane >= o) v += t;
         }
-        s_sel[2] = (b1 << 5) | (uint32_t)b2;
-        s_sel[3] = (uint32_t)n - above;  // entries equal to T to take
+        const uint32_t above = cum_above + v - c;             // entries in finer bins above this one
+        const bool hit = lane < 32 && above < (uint32_t)n && (uint32_t)n <= above + c;
+        // bin 0 takes what is left when no finer bin reaches n (cannot happen for a consistent
+        // histogram; kept so that s_sel is always written)
+        const unsigned long long m = __ballot(hit);
+        const int first = m ? __ffsll((long long)m) - 1 : 31;
+        if (lane == first) {
+            s_sel[2] = (b1 << 5) | (uint32_t)(31 - first);
+            s_sel[3] = (uint32_t)n - above;  // entries equal to T to take
+        }
     }
     __syncthreads();
     const uint32_t T = s_sel[2];
@@ -323,19 +360,17 @@ __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
     uint32_t own[MAXC];
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
-        uint32_t gt = 0, eq = 0;
+        uint32_t cnt = 0;
         if (c < nchunks) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                if (valid(c, e)) {
-                    const uint32_t key = key_of(c, e);
-                    gt += (key > T);
-                    eq += (key == T);
-                }
+                const uint32_t key = key_of(c, e);
+                const uint32_t in = (e < nv[c]) ? 1u : 0u;
+                cnt += ((key > T) ? in : 0u) + ((key == T) ? (in << 16) : 0u);
             }
         }
-        own[c] = gt | (eq << 16);
-        uint32_t v = own[c];
+        own[c] = cnt;
+        uint32_t v = cnt;
 #pragma unroll
         for (int o = 1; o < 64; o <<= 1) {
             const uint32_t t = __shfl_up(v, o);
@@ -347,7 +382,7 @@ __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
     __syncthreads();
     if (wave == 0) {
         // exclusive prefix over the MAXC*16 (chunk, wavefront) totals, chunk-major, 64 per step;
-        // both halves stay below 65536 (a row has at most 65536 entries)
+        // an exclusive prefix of either half stays below 65536 (a row has at most 65536 entries)
         uint32_t carry = 0;
 #pragma unroll
         for (int i0 = 0; i0 < MAXC * kWaves; i0 += 64) {
@@ -374,21 +409,19 @@ __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
             const int base = c * kChunk + tid * 8;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                if (valid(c, e)) {
-                    const uint32_t key = key_of(c, e);
-                    int pos = -1;
-                    if (key > T) {
-                        pos = (int)(my_gt + min(my_eq, r));
-                        ++my_gt;
-                    } else if (key == T) {
-                        if (my_eq < r) pos = (int)(my_gt + my_eq);
-                        ++my_eq;
-                    }
-                    if (pos >= 0) {
-                        if (staged) stage[pos] = base + e;
-                        else dst[pos] = base + e;
-                    }
+                const uint32_t key = key_of(c, e);
+                const bool in = e < nv[c];
+                const bool is_gt = in && key > T;
+                const bool is_eq = in && key == T;
+                // an entry above T sits after the earlier ones above T and the earlier ties taken;
+                // a tie that is taken (my_eq < r) has min(my_eq, r) = my_eq: one formula for both
+                const int pos = (int)(my_gt + min(my_eq, r));
+                if (is_gt || (is_eq && my_eq < r)) {
+                    if (staged) stage[pos] = base + e;
+                    else dst[pos] = base + e;
                 }
+                my_gt += is_gt ? 1u : 0u;
+                my_eq += is_eq ? 1u : 0u;
             }
         }
     }
@@ -463,13 +496,23 @@ __global__ __launch_bounds__(kThreads) void topk_split_hist1_kernel(
     const bool aligned = ((reinterpret_cast<uintptr_t>(src) & 15) == 0);
     for (int i = tid; i < kBins1; i += kThreads) s_hist[i] = 0;
     __syncthreads();
-    for (int base = c0 + tid * 8; base < c1; base += kChunk) {
+    // zeros (pooled probabilities underflow to +0 by the thousand) are counted with a ballot
+    // per wavefront instead of that many atomics on one address; the loop bounds are uniform
+    // over a wavefront's lanes up to the ragged end, where absent lanes contribute nothing
+    uint32_t zeros = 0;
+    for (int base0 = c0; base0 < c1; base0 += kChunk) {
+        const int base = base0 + tid * 8;
         uint32_t keys[8];
-        int nv = load_keys(src, aligned, base, c1, keys);
+        const int nv = (base < c1) ? load_keys(src, aligned, base, c1, keys) : 0;
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-            if (e < nv) atomicAdd(&s_hist[keys[e] >> 5], 1u);
+        for (int e = 0; e < 8; ++e) {
+            const bool in = e < nv;
+            const bool zero = in && keys[e] == 0x8000u;
+            zeros += (uint32_t)__popcll(__ballot(zero));
+            if (in && !zero) atomicAdd(&s_hist[keys[e] >> 5], 1u);
+        }
     }
+    if ((tid & 63) == 0 && zeros) atomicAdd(&s_hist[0x8000u >> 5], zeros);
     __syncthreads();
     uint32_t* gh = ws.hist1 + row * kBins1;
     for (int i = tid; i < kBins1; i += kThreads) {
