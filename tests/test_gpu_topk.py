@@ -84,19 +84,19 @@ def test_topk_matches_torch_topk_sets_when_no_ties(cuda):
     assert torch.equal(idx.cpu(), want)
 
 
-@pytest.mark.parametrize("L", [60000, 65536, 20000])
-def test_topk_register_kernel_equals_streaming_kernel(cuda, L):
+@pytest.mark.parametrize("L,K", [(60000, 6016), (65536, 6016), (20000, 6016), (40000, 20096), (65536, 6018)])
+def test_topk_register_kernel_equals_streaming_kernel(cuda, L, K):
     """Aligned rows of up to 65536 entries are selected from registers; the same values behind an
     unaligned row pointer take the streaming kernel.  Both must agree bit for bit, on ragged
     lengths around the 8192-entry chunk boundaries, ties, -inf runs and degenerate budgets."""
     from kascade_amd import kernels
-    rows, K = 8, 6016
+    rows = 8      # K above 8192: lists too long to stage in LDS; K % 4 != 0: element stores
     sc = _scores(rows, L, seed=L + 1)
     sc[1, 500:900] = float("-inf")
     sc[2] = 0.25                                     # one value everywhere: pure tie-breaking
     sc[3, : L // 2] = 0.0
     valid = torch.tensor([L, min(L, 33000), 8192, 8193, 5000, L - 1, 16384, 100], dtype=torch.int32)
-    nsel = torch.tensor([6016, 3328, 1024, 1024, 512, 0, 6016, 128], dtype=torch.int32)
+    nsel = torch.tensor([K, 3328, 1024, 1024, 512, 0, K, 128], dtype=torch.int32)
     assert L % 8 == 0
     aligned = sc.to(cuda)
     store = torch.zeros(rows * (L + 1) + 1, dtype=torch.float16, device=cuda)
