@@ -37,7 +37,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 MFMA_PEAK_TFLOPS = 2500.0      # MI355X published dense fp16 MFMA rate
 H100_PREFILL_32K_MS = 6.42     # reference's published Kascade prefill ms @32768 (H100)
 # rocprofv3 FETCH_SIZE*2.0 + WRITE_SIZE*1.0 per launch at config 1 (profiles/prefill_reuse.md)
-MEASURED_TRAFFIC_BYTES = {"prefill_attn_reuse": 1.191e9}
+MEASURED_TRAFFIC_BYTES = {"prefill_attn_reuse": 1.199e9}
 
 
 def log(msg):
