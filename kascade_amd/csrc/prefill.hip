@@ -376,7 +376,6 @@ void prefill_attn_kernel_q64(PrefillParams p) {
 template <bool PAGED>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2)))
 void prefill_aggregate_kernel(PrefillParams p) {
-    __shared__ __attribute__((aligned(16))) half_t sK[kAggKT * kKStride];
     __shared__ __attribute__((aligned(16))) float s_lse[128];
 
     const int L = p.L;
@@ -417,54 +416,67 @@ void prefill_aggregate_kernel(PrefillParams p) {
             s_lse[tid] = (q < Lq) ? p.log_sum_in[((long long)b * Lq + q) * kHeads + g * kGroupSize + (tid >> 5)]
                                   : INFINITY;
         }
-        const int krow = tid >> 4, kcol = tid & 15;
-        const half_t* kbase = PAGED ? p.K + (long long)g * kDim + kcol * 8
-                                    : p.K + (long long)b * p.k_sb + (long long)g * p.k_sh + kcol * 8;
+        // A wavefront takes 32 keys of every 128-key tile and nobody else reads them, so its B
+        // operands (lane li = key, 8 halves at d = 16 ks + 8 lg) come straight from global
+        // memory in the layout the matrix instruction wants: no LDS staging, no barriers in the
+        // tile loop.  The registers of operand ks are refilled with the next tile's data as soon
+        // as the products that read them have been issued, which leaves the rest of the tile
+        // (remaining products, exponentials) to cover the load latency.
+        const half_t* kbase = PAGED ? p.K + (long long)g * kDim + lg * 8
+                                    : p.K + (long long)b * p.k_sb + (long long)g * p.k_sh + lg * 8;
         const int* bt_row = PAGED ? p.block_table + (long long)b * p.max_pages : nullptr;
         const int page_mask = (1 << p.page_shift) - 1;
-        uint4_t kr[8];
-        int pg[8];   // block-table entries of the tile after the one in flight (paged)
-        auto fetch_pages = [&](int ti) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                pg[i] = bt_row[min(ti * kAggKT + krow + 16 * i, L - 1) >> p.page_shift];
+        auto key_of = [&](int ti) { return min(ti * kAggKT + 32 * wave + li, L - 1); };
+        auto row_ptr = [&](int ti, int pgv) {
+            const int key = key_of(ti);
+            return PAGED ? kbase + (long long)((pgv << p.page_shift) + (key & page_mask)) * (kGroups * kDim)
+                         : kbase + (long long)key * p.k_sl;
         };
-        auto issue_loads = [&](int ti) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int key = min(ti * kAggKT + krow + 16 * i, L - 1);
-                if (PAGED)
-                    kr[i] = ld_global_16(kbase + (long long)((pg[i] << p.page_shift) + (key & page_mask)) * (kGroups * kDim));
-                else
-                    kr[i] = ld_global_16(kbase + (long long)key * p.k_sl);
-            }
-        };
-        if (PAGED) fetch_pages(0);
-        issue_loads(0);
-        if (PAGED && ntiles > 1) fetch_pages(1);
-        for (int ti = 0; ti < ntiles; ++ti) {
-            __syncthreads();
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                *reinterpret_cast<uint4_t*>(&sK[(krow + 16 * i) * kKStride + kcol * 8]) = kr[i];
-            __syncthreads();
-            if (ti + 1 < ntiles) {
-                issue_loads(ti + 1);
-                if (PAGED && ti + 2 < ntiles) fetch_pages(ti + 2);
-            }
-
-            float16_t acc[kGroupSize];
-#pragma unroll
-            for (int rb = 0; rb < kGroupSize; ++rb)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc[rb][v] = 0.f;
+        int pg_next = 0;    // block-table entry of this lane's key in the tile after the current one
+        int pg_after = 0;   // ... and in the one after that (fetched a tile ahead of its use)
+        if (PAGED) {
+            pg_next = bt_row[key_of(0) >> p.page_shift];
+            if (ntiles > 1) pg_after = bt_row[key_of(1) >> p.page_shift];
+        }
+        half8_t kb[8];
+        {
+            const half_t* rp = row_ptr(0, pg_next);
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks) {
-                half8_t bf = *reinterpret_cast<const half8_t*>(
-                    &sK[(32 * wave + li) * kKStride + ks * 16 + lg * 8]);
+                Pack16 x;
+                x.u = ld_global_16(rp + ks * 16);
+                kb[ks] = x.h8;
+            }
+        }
+        __syncthreads();   // s_lse
+        for (int ti = 0; ti < ntiles; ++ti) {
+            const bool more = ti + 1 < ntiles;
+            if (PAGED) {
+                pg_next = pg_after;
+                if (ti + 2 < ntiles) pg_after = bt_row[key_of(ti + 2) >> p.page_shift];
+            }
+            const half_t* rp = row_ptr(more ? ti + 1 : ti, pg_next);
+
+            float16_t acc[kGroupSize];
+            float16_t zero16;   // the first product of a tile starts from a constant zero
+#pragma unroll
+            for (int v = 0; v < 16; ++v) zero16[v] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) {
 #pragma unroll
                 for (int rb = 0; rb < kGroupSize; ++rb)
-                    acc[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa[rb][ks], bf, acc[rb], 0, 0, 0);
+                    acc[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa[rb][ks], kb[ks],
+                                                                     ks == 0 ? zero16 : acc[rb], 0, 0, 0);
+                if (more) {
+                    // the refill must stay behind the products that read the old contents, or
+                    // the compiler hoists all eight loads and needs a second set of registers:
+                    // its address is made to depend on the last product of this step
+                    long long off = ks * 16;
+                    asm volatile("" : "+v"(off) : "v"(acc[kGroupSize - 1][0]));
+                    Pack16 x;
+                    x.u = ld_global_16(rp + off);
+                    kb[ks] = x.h8;
+                }
             }
             // accumulator v of row block rb is query row 8(v/4) + 4lg + v%4, column = key li
             float sum = 0.f;
