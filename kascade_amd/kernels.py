@@ -13,7 +13,7 @@ raises ``KascadeError`` when libkascade_hip.so is missing or a call fails.
 from __future__ import annotations
 
 import math
-from typing import Optional, Sequence, Tuple
+from typing import Optional, Tuple
 
 import torch
 

@@ -12,7 +12,7 @@ fp32 by the given generator and cast to fp16 once.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import List, Optional, Sequence
+from typing import List, Sequence
 
 import torch
 

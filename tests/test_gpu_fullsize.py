@@ -1,7 +1,6 @@
 """The benchmark configurations at their full sizes: parity against the CPU oracle on sampled
 rows / tiles / sequences, and size-independent properties checked on every row on the device
 (selection threshold property, probability mass, permutation invariance, chunked = whole)."""
-import math
 
 import pytest
 import torch
