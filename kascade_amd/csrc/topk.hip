@@ -232,23 +232,24 @@ __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
     }
     const int nchunks = (len + kChunk - 1) / kChunk;   // <= MAXC (host)
 
-    // ---- the row: chunk c, entries [c*8192 + 8*tid, +8) as packed order keys; nv[c] of them
-    //      are inside the row ----
+    // ---- the row: chunk c, entries [c*8192 + 8*tid, +8) as packed order keys ----
     uint4_t data[MAXC];
-    int nv[MAXC];
+    // entries of chunk c that lie inside the row (recomputed where needed: an array of them
+    // would cost MAXC registers)
+    auto nv_of = [&](int c) { return max(0, min(8, len - (c * kChunk + tid * 8))); };
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
         const int base = c * kChunk + tid * 8;
-        nv[c] = (c < nchunks) ? max(0, min(8, len - base)) : 0;
+        const int nvc = nv_of(c);
         uint4_t raw;
-        if (nv[c] == 8) {
+        if (nvc == 8) {
             raw = *reinterpret_cast<const uint4_t*>(src + base);
         } else {
             uint32_t w[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const uint32_t lo = (2 * e < nv[c]) ? src[base + 2 * e] : 0xFFFFu;       // key 0
-                const uint32_t hi = (2 * e + 1 < nv[c]) ? src[base + 2 * e + 1] : 0xFFFFu;
+                const uint32_t lo = (2 * e < nvc) ? src[base + 2 * e] : 0xFFFFu;       // key 0
+                const uint32_t hi = (2 * e + 1 < nvc) ? src[base + 2 * e + 1] : 0xFFFFu;
                 w[e] = lo | (hi << 16);
             }
             raw = uint4_t{w[0], w[1], w[2], w[3]};
@@ -279,10 +280,11 @@ __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
         if (c < nchunks) {
+            const int nvc = nv_of(c);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const uint32_t key = key_of(c, e);
-                const bool in = e < nv[c];
+                const bool in = e < nvc;
                 const bool zero = key == kZeroKey;
                 zeros += (uint32_t)__popcll(__ballot(in && zero));
                 atomicAdd(zero ? &s_zero[lane] : &s_hist[(key >> 5) * kCopies + copy], (in && !zero) ? 1u : 0u);
@@ -320,10 +322,11 @@ __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
         if (c < nchunks) {
+            const int nvc = nv_of(c);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const uint32_t key = key_of(c, e);
-                if ((key >> 5) == b1 && e < nv[c] && key != kZeroKey) atomicAdd(&s_hist2[key & 31u], 1u);
+                if ((key >> 5) == b1 && e < nvc && key != kZeroKey) atomicAdd(&s_hist2[key & 31u], 1u);
             }
         }
     }
@@ -356,27 +359,26 @@ __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
 
     // ---- pass 3: ordered compaction (index order = chunk, then thread, then element) ----
     // counts of one (chunk, thread): entries above T in the low half, equal to T in the high half
-    uint32_t inc[MAXC];   // inclusive scan of the counts over the wavefront
-    uint32_t own[MAXC];
+    uint32_t exw[MAXC];   // exclusive scan of the counts over the wavefront
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
         uint32_t cnt = 0;
         if (c < nchunks) {
+            const int nvc = nv_of(c);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const uint32_t key = key_of(c, e);
-                const uint32_t in = (e < nv[c]) ? 1u : 0u;
+                const uint32_t in = (e < nvc) ? 1u : 0u;
                 cnt += ((key > T) ? in : 0u) + ((key == T) ? (in << 16) : 0u);
             }
         }
-        own[c] = cnt;
         uint32_t v = cnt;
 #pragma unroll
         for (int o = 1; o < 64; o <<= 1) {
             const uint32_t t = __shfl_up(v, o);
             if (lane >= o) v += t;
         }
-        inc[c] = v;
+        exw[c] = v - cnt;
         if (lane == 63) s_tot[c * kWaves + wave] = v;
     }
     __syncthreads();
@@ -403,14 +405,15 @@ __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
         if (c < nchunks) {
-            const uint32_t ex = s_tot[c * kWaves + wave] + inc[c] - own[c];
+            const uint32_t ex = s_tot[c * kWaves + wave] + exw[c];
+            const int nvc = nv_of(c);
             uint32_t my_gt = ex & 0xFFFFu;
             uint32_t my_eq = ex >> 16;
             const int base = c * kChunk + tid * 8;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const uint32_t key = key_of(c, e);
-                const bool in = e < nv[c];
+                const bool in = e < nvc;
                 const bool is_gt = in && key > T;
                 const bool is_eq = in && key == T;
                 // an entry above T sits after the earlier ones above T and the earlier ties taken;
