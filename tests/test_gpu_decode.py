@@ -444,3 +444,38 @@ def test_fused_append_contiguous_and_head_major(cuda):
     got = kernels.decode_reuse_paged(q, kh[:, :, :L].transpose(1, 2), vh[:, :, :L].transpose(1, 2), lens, idx, hm,
                                      0.0, glse, part, k_new=kn, v_new=vn)
     assert torch.isfinite(got).all() and torch.equal(got, want) and torch.equal(kh, ks) and torch.equal(vh, vs)
+
+
+@pytest.mark.parametrize("page_size", [1, 4, 64, 256])
+def test_page_sizes(cuda, page_size):
+    """Any power-of-two page size: dense, anchor and reuse decode over a paged cache equal the
+    oracle on the gathered contiguous cache (page 16 is what every other test uses)."""
+    from kascade_amd import kernels, workloads
+    p = 10
+    seqlens = [1300, 700]
+    w = workloads.paged_decode_inputs(seqlens, seed=41, device="cpu", page_size=page_size)
+    assert w.page_size == page_size
+    B, Lmax = len(seqlens), max(seqlens)
+    kc = orc.paged_to_contiguous(w.k_pages, w.block_table, seqlens)
+    vc = orc.paged_to_contiguous(w.v_pages, w.block_table, seqlens)
+    q, kp, vp = w.q.to(cuda), w.k_pages.to(cuda), w.v_pages.to(cuda)
+    lens, bt = w.seqlens.to(cuda), w.block_table.to(cuda)
+    glse, part = _scratch(B, 3, cuda)
+    want, _ = orc.dense_decode(w.q, kc, vc, seqlens)
+    got = kernels.decode_dense_paged(q, kp, vp, lens, glse, part, bt, page_size, kv_len=Lmax)
+    assert_close(got, want, f"dense decode, page {page_size}")
+    row_sums = torch.empty(B, H, device=cuda, dtype=torch.float32)
+    stride = ((Lmax + 7) // 8) * 8
+    scores = torch.empty(B, H, stride, device=cuda, dtype=torch.float32)
+    o, agg = kernels.decode_recompute(q, kp, vp, glse, part, row_sums, scores, 0, cache_seqlens=lens,
+                                      block_table=bt, page_size=page_size, kv_len=Lmax)
+    assert_close(o, want, f"anchor-0 output, page {page_size}")
+    assert_close(agg.cpu()[:, :, :Lmax], orc.pooled_decode_scores(w.q, kc, seqlens), "agg", atol=2e-6, rtol=2e-3)
+    counts = [orc.n_kvcache(n, p) for n in seqlens]
+    K = max(counts)
+    valid, nsel = kernels.decode_budgets(lens, p)
+    idx = kernels.topk_indices(agg[:, :, :Lmax], K, valid_len=valid, n_sel=nsel, fill_value=0)
+    hm = torch.tensor(w.head_mapping, dtype=torch.int32, device=cuda)
+    got = kernels.decode_reuse_paged(q, kp, vp, lens, idx, hm, float(p), glse, part, block_table=bt,
+                                     page_size=page_size)
+    assert_close(got, orc.reuse_decode(w.q, kc, vc, idx.cpu(), w.head_mapping, counts), f"reuse decode, page {page_size}")
