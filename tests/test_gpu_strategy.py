@@ -119,3 +119,37 @@ def test_full_kernel_observables(cuda):
     assert_close(agg.cpu(), agg_w, "agg", atol=2e-6, rtol=2e-3)
     counts = [orc.n_kvcache(n, 10) for n in seqlens]
     assert_close(o, orc.reuse_decode(pw.q, kc, vc, idx.cpu(), list(range(G)), counts), "kvcache full_kernel O")
+
+
+def test_results_are_deterministic(cuda):
+    """Every path gives bit-identical results on repeated calls: split merges run in split order
+    whichever workgroup arrives last, selections break ties by index, and nothing accumulates
+    through floating-point atomics."""
+    from kascade_amd import workloads
+    from kascade_amd.strategy import EfficientKascadeStrategy, PagedKascadeDecoder
+    L, p = 1500, 10
+    w = workloads.prefill_inputs(1, L, seed=12, device=cuda)
+    hm = [list(range(G)), w.head_mapping, list(range(G))]
+    runs = []
+    for _ in range(2):
+        s = EfficientKascadeStrategy([0, 2], None, k=p, tile_size=TILE, rolling_prefill=True, head_mapping=hm,
+                                     register=False)
+        o0, _ = s.attention_forward(_Module(0), _hf(w.q), _hf(w.k), _hf(w.v), None, D ** -0.5)
+        i0 = s._topk_to_reuse.clone()
+        o1, _ = s.attention_forward(_Module(1), _hf(w.q_reuse), _hf(w.k_reuse), _hf(w.v), None, D ** -0.5)
+        o2, _ = s.attention_forward(_Module(2), _hf(w.q_reuse), _hf(w.k_reuse), _hf(w.v), None, D ** -0.5)
+        runs.append((o0.clone(), i0, o1.clone(), o2.clone(), s._topk_to_reuse.clone()))
+    for a, b in zip(*runs):
+        assert torch.equal(a, b)
+    seqlens = [3000, 1111, 2048]
+    c = workloads.paged_decode_inputs(seqlens, seed=13, device=cuda)
+    maps = [list(range(G)), c.head_mapping]
+    outs = []
+    for _ in range(2):
+        dec = PagedKascadeDecoder(p, maps, [0], len(seqlens), max(seqlens), page_size=c.page_size, device=cuda)
+        a = dec.forward(0, c.q, c.k_pages, c.v_pages, c.block_table, c.seqlens, max(seqlens)).clone()
+        idx = dec._topk_to_reuse.clone()
+        r = dec.forward(1, c.q_reuse, c.k_pages_reuse, c.v_pages, c.block_table, c.seqlens, max(seqlens)).clone()
+        outs.append((a, idx, r))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
