@@ -244,12 +244,17 @@ int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_hal
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (check_hip(launch_decode_split(p, false, with_output != 0, true, s), "decode_recompute split"))
         return -1;
-    if (!sync_counters &&
+    // Without an output the only thing left to merge is the log-sums, which the aggregate
+    // launch does for itself: no combine launch.
+    const bool merge_in_aggregate = !sync_counters && !with_output;
+    if (!sync_counters && with_output &&
         check_hip(launch_decode_combine(glse, Output_partial, H(Output), row_sums, batch, num_split,
-                                        with_output != 0, s), "decode_recompute combine"))
+                                        true, s), "decode_recompute combine"))
         return -1;
-    return check_hip(launch_decode_aggregate(scores, row_sums, cache_seqlens, H(aggregated_scores),
-                                             batch, scores_stride, kv_stride_tokens, s),
+    return check_hip(launch_decode_aggregate(scores, merge_in_aggregate ? nullptr : row_sums,
+                                             merge_in_aggregate ? glse : nullptr, num_split, row_sums,
+                                             cache_seqlens, H(aggregated_scores), batch, scores_stride,
+                                             kv_stride_tokens, s),
                      "decode_recompute aggregate");
 }
 

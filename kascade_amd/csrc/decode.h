@@ -48,7 +48,10 @@ hipError_t launch_decode_split(const DecodeParams& p, bool gather, bool with_v, 
 hipError_t launch_decode_combine(const float* glse, const float* opart, half_t* out,
                                  float* row_sums, int batch, int num_split, bool with_v,
                                  hipStream_t stream);
-hipError_t launch_decode_aggregate(const float* scores, const float* row_sums, const int* seqlens,
+// Log-sums per head: merged (row_sums_in), or glse [B,H,num_split] to be merged by the kernel,
+// which then also writes them to row_sums_out.
+hipError_t launch_decode_aggregate(const float* scores, const float* row_sums_in, const float* glse,
+                                   int num_split, float* row_sums_out, const int* seqlens,
                                    half_t* agg, int batch, int scores_stride, int uniform_len,
                                    hipStream_t stream);
 

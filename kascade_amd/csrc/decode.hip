@@ -584,19 +584,48 @@ __global__ __launch_bounds__(128) void decode_combine_kernel(const float* __rest
 
 // agg[b,g,j] = fp16( sum_h exp2(s[b,4g+h,j]*scale - lse[b,4g+h]) ), 0 beyond the sequence.
 // grid (ceil(stride/2048), G, B), 256 threads x 8 tokens.
+// The per-head log-sums come either merged (row_sums_in) or as the splits' partial log-sums
+// (glse [B,H,num_split]): then every workgroup merges them itself -- one wavefront per head --
+// and the first workgroup of a (sequence, KV head) also writes them to row_sums_out, which saves
+// the combine launch of an anchor pass that produces no output.
 __global__ __launch_bounds__(256) void decode_aggregate_kernel(const float* __restrict__ scores,
-                                                              const float* __restrict__ row_sums,
+                                                              const float* __restrict__ row_sums_in,
+                                                              const float* __restrict__ glse, int num_split,
+                                                              float* __restrict__ row_sums_out,
                                                               const int* __restrict__ seqlens,
                                                               half_t* __restrict__ agg,
                                                               int scores_stride, int uniform_len) {
+    __shared__ float s_lse[kGroupSize];
     const int g = blockIdx.y;
     const int b = blockIdx.z;
     const int len = seqlens ? seqlens[b] : uniform_len;
     const int j0 = (blockIdx.x * 256 + threadIdx.x) * 8;
-    if (j0 >= scores_stride) return;
     float lse[kGroupSize];
+    if (glse != nullptr) {   // uniform over the launch
+        const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+        const float* gl = glse + ((size_t)b * kHeads + g * kGroupSize + wave) * num_split;
+        float mx = -INFINITY;
+        for (int sidx = lane; sidx < num_split; sidx += 64) mx = fmaxf(mx, gl[sidx]);
 #pragma unroll
-    for (int h = 0; h < kGroupSize; ++h) lse[h] = row_sums[(size_t)b * kHeads + g * kGroupSize + h];
+        for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+        const float mref = (mx == -INFINITY) ? 0.f : mx;
+        float sum = 0.f;
+        for (int sidx = lane; sidx < num_split; sidx += 64) sum += fast_exp2(gl[sidx] - mref);
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
+        const float v = (sum > 0.f) ? fast_log2(sum) + mref : -INFINITY;
+        if (lane == 0) {
+            s_lse[wave] = v;
+            if (blockIdx.x == 0 && row_sums_out) row_sums_out[(size_t)b * kHeads + g * kGroupSize + wave] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int h = 0; h < kGroupSize; ++h) lse[h] = s_lse[h];
+    } else {
+#pragma unroll
+        for (int h = 0; h < kGroupSize; ++h) lse[h] = row_sums_in[(size_t)b * kHeads + g * kGroupSize + h];
+    }
+    if (j0 >= scores_stride) return;
     float sum[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) sum[e] = 0.f;
@@ -661,12 +690,13 @@ hipError_t launch_decode_combine(const float* glse, const float* opart, half_t* 
     return hipGetLastError();
 }
 
-hipError_t launch_decode_aggregate(const float* scores, const float* row_sums, const int* seqlens,
+hipError_t launch_decode_aggregate(const float* scores, const float* row_sums_in, const float* glse,
+                                   int num_split, float* row_sums_out, const int* seqlens,
                                    half_t* agg, int batch, int scores_stride, int uniform_len,
                                    hipStream_t stream) {
     dim3 grid((scores_stride + 2047) / 2048, kGroups, batch), block(256);
-    hipLaunchKernelGGL(decode_aggregate_kernel, grid, block, 0, stream, scores, row_sums, seqlens,
-                       agg, scores_stride, uniform_len);
+    hipLaunchKernelGGL(decode_aggregate_kernel, grid, block, 0, stream, scores, row_sums_in, glse,
+                       num_split, row_sums_out, seqlens, agg, scores_stride, uniform_len);
     return hipGetLastError();
 }
 
