@@ -77,7 +77,10 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
     const int rg = lane >> 4;   // row group within the wavefront
     const int dl = lane & 15;   // 16-byte slice of the 256-byte row
 
-    const int seqlen = p.seqlens ? p.seqlens[b] : p.kv_stride_tokens;
+    int seqlen = p.seqlens ? p.seqlens[b] : p.kv_stride_tokens;
+    // a length beyond what the block table covers must not index past the table
+    if (p.block_table) seqlen = min(seqlen, p.max_pages << p.page_shift);
+    seqlen = max(seqlen, 0);
     int n;  // rows this (b, g) pair attends to
     if (GATHER) {
         if (p.topk_percent > 0.f) {

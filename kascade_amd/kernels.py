@@ -267,8 +267,9 @@ _TOPK_WS = {}
 
 
 def _topk_workspace(nbytes: int, device) -> torch.Tensor:
-    """Scratch for the multi-workgroup selection, grown on demand and kept per device."""
-    key = str(device)
+    """Scratch for the multi-workgroup selection, grown on demand and kept per (device, stream):
+    selections that run concurrently on different streams must not share it."""
+    key = (str(device), torch.cuda.current_stream(device).cuda_stream)
     ws = _TOPK_WS.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(nbytes, device=device, dtype=torch.uint8)
