@@ -219,6 +219,32 @@ int kascade_paged_kv_append_call(kascade_half* K_pages, kascade_half* V_pages,
                                  int n_new, int max_pages, int page_size,
                                  kascade_strides new_strides, void* stream);
 
+/* The hand-off from a decoder layer's projections to the attention path in one launch: RMS
+ * normalisation of every query and key head (optional), rotary position embedding of queries
+ * and keys, queries written as [B,n_new,H,D], keys and values written into their page slots.
+ * No kernel of the reference does this: its transformers dependency runs these steps as
+ * separate tensor operations inside the attention module before the registered attention
+ * function is called, and the strategy then transposes (and, when decoding, copies) the
+ * results (EfficientKascadeStrategy.py:144-150).
+ *   q_in [B,n_new,H,D], k_in / v_in [B,n_new,G,D] through element strides (b, l, h), multiples
+ *        of 8 with D contiguous (e.g. views of one packed projection output); NULL strides =
+ *        contiguous.
+ *   cos_sin [max_pos, D] f32: row p holds cos(p*f_i), i < D/2, then sin(p*f_i); element i of a
+ *        head pairs with element i + D/2 ("rotate half").
+ *   q_norm_weight, k_norm_weight [D] f16 or NULL (no normalisation); the normalised value is
+ *        rounded to f16 before and after the weight, as the library's module does.
+ *   Token t of sequence b sits at position start_pos[b] + pos_offset + t; negative positions
+ *   and positions beyond the block table are skipped, angles beyond max_pos use the last row. */
+int kascade_rope_append_paged_call(const kascade_half* q_in, const kascade_strides* q_strides,
+                                   const kascade_half* k_in, const kascade_half* v_in,
+                                   const kascade_strides* kv_strides, const float* cos_sin,
+                                   int max_pos, const kascade_half* q_norm_weight,
+                                   const kascade_half* k_norm_weight, float norm_eps,
+                                   const int32_t* start_pos, int pos_offset, kascade_half* q_out,
+                                   kascade_half* K_pages, kascade_half* V_pages,
+                                   const int32_t* block_table, int max_pages, int page_size,
+                                   int batch, int n_new, void* stream);
+
 /* Bookkeeping of a ragged decode step in one small launch (no reference counterpart; the
  * reference's benchmark computes these on the host, recompute_kascade_gqa_decode_with_kvcache.py:
  * 368-377).  Adds `advance` to every cache_seqlens[b] in place (1 when the step's new token is

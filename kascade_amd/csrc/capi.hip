@@ -104,7 +104,7 @@ int set_append(DecodeParams& p, const kascade_half* k_new, const kascade_half* v
 
 extern "C" {
 
-int kascade_abi_version(void) { return 4; }
+int kascade_abi_version(void) { return 5; }
 
 const char* kascade_get_last_error(void) { return g_err; }
 
@@ -360,6 +360,44 @@ int kascade_paged_kv_append_call(kascade_half* K_pages, kascade_half* V_pages,
                                             new_strides.b, new_strides.l, new_strides.h,
                                             static_cast<hipStream_t>(stream)),
                      "paged_kv_append");
+}
+
+int kascade_rope_append_paged_call(const kascade_half* q_in, const kascade_strides* q_strides,
+                                   const kascade_half* k_in, const kascade_half* v_in,
+                                   const kascade_strides* kv_strides, const float* cos_sin,
+                                   int max_pos, const kascade_half* q_norm_weight,
+                                   const kascade_half* k_norm_weight, float norm_eps,
+                                   const int32_t* start_pos, int pos_offset, kascade_half* q_out,
+                                   kascade_half* K_pages, kascade_half* V_pages,
+                                   const int32_t* block_table, int max_pages, int page_size,
+                                   int batch, int n_new, void* stream) {
+    REQUIRE(q_in && k_in && v_in && cos_sin && start_pos && q_out && K_pages && V_pages && block_table,
+            "rope_append: null pointer argument");
+    REQUIRE(batch > 0 && n_new >= 0 && max_pos > 0, "rope_append: bad batch/n_new/max_pos");
+    REQUIRE((long long)batch * n_new * (kHeads + 2 * kGroups) / 16 < (1LL << 31),
+            "rope_append: too many rows for one launch");
+    REQUIRE(norm_eps >= 0.f, "rope_append: norm_eps must not be negative");
+    int shift;
+    if (check_paging(block_table, max_pages, page_size, &shift)) return -1;
+    RopeAppendParams p{};
+    const kascade_strides qs = q_strides ? *q_strides
+        : kascade_strides{(long long)n_new * kHeads * kDim, (long long)kHeads * kDim, kDim};
+    const kascade_strides ks = kv_strides ? *kv_strides
+        : kascade_strides{(long long)n_new * kGroups * kDim, (long long)kGroups * kDim, kDim};
+    if (check_strides(qs, "q_in") || check_strides(ks, "k_in/v_in")) return -1;
+    REQUIRE(aligned16(q_in) && aligned16(k_in) && aligned16(v_in) && aligned16(q_out) &&
+                aligned16(K_pages) && aligned16(V_pages) && aligned16(cos_sin) &&
+                aligned16(q_norm_weight) && aligned16(k_norm_weight),
+            "rope_append: tensors must be 16-byte aligned");
+    p.q_in = H(q_in); p.k_in = H(k_in); p.v_in = H(v_in);
+    p.cos_sin = cos_sin; p.q_weight = H(q_norm_weight); p.k_weight = H(k_norm_weight);
+    p.start_pos = start_pos; p.q_out = H(q_out); p.Kp = H(K_pages); p.Vp = H(V_pages);
+    p.block_table = block_table;
+    p.q_sb = qs.b; p.q_sl = qs.l; p.q_sh = qs.h;
+    p.kv_sb = ks.b; p.kv_sl = ks.l; p.kv_sh = ks.h;
+    p.eps = norm_eps; p.pos_offset = pos_offset; p.batch = batch; p.n_new = n_new;
+    p.max_pages = max_pages; p.page_shift = shift; p.max_pos = max_pos;
+    return check_hip(launch_rope_append(p, static_cast<hipStream_t>(stream)), "rope_append");
 }
 
 int kascade_decode_budgets_call(int32_t* cache_seqlens, int advance, float topk_percent, int batch,

@@ -12,6 +12,7 @@ raises ``KascadeError`` when libkascade_hip.so is missing or a call fails.
 """
 from __future__ import annotations
 
+import ctypes
 import math
 from typing import Optional, Tuple
 
@@ -91,7 +92,6 @@ def _decode_kv(K, V, block_table):
     Pages must be contiguous.  Without a block table any [B,L,G,D] view with a contiguous last
     dimension is read in place (e.g. a head-major [B,G,L,D] cache transposed), and the strides
     are passed only when the view is not the plain contiguous layout."""
-    import ctypes
     for t, name in ((K, "K"), (V, "V")):
         _req(t, torch.float16, name, contiguous=block_table is not None)
     if block_table is not None or (K.is_contiguous() and V.is_contiguous()):
@@ -416,6 +416,64 @@ def paged_kv_append(K_pages, V_pages, k_new, v_new, start_pos, block_table, page
     _lib.check(lib.kascade_paged_kv_append_call(
         _ptr(K_pages), _ptr(V_pages), _ptr(k_new), _ptr(v_new), _ptr(start_pos), _ptr(block_table),
         B, n_new, block_table.shape[1], page_size, st, _stream()))
+
+
+def rope_table(max_pos: int, theta: float = 1e6, device="cuda", round_to=torch.float16) -> torch.Tensor:
+    """[max_pos, D] fp32: cos of position * theta^(-2i/D) for the D/2 pairs, then the sines.  The
+    angles are formed in fp32 and the values rounded to ``round_to`` (what the transformers
+    rotary module hands an fp16 model; None keeps fp32)."""
+    inv = (1.0 / (theta ** (torch.arange(0, D, 2, dtype=torch.int64).float() / D))).to(device)
+    ang = torch.arange(max_pos, device=device, dtype=torch.float32)[:, None] * inv
+    table = torch.cat((ang.cos(), ang.sin()), dim=1)
+    if round_to is not None:
+        table = table.to(round_to).float()
+    return table.contiguous()
+
+
+def rope_append_paged(q_in, k_in, v_in, cos_sin, start_pos, K_pages, V_pages, block_table,
+                      page_size: int = 16, pos_offset: int = 0, q_norm_weight=None, k_norm_weight=None,
+                      norm_eps: float = 1e-6, out=None) -> torch.Tensor:
+    """What a decoder's attention module does between its projections and the attention call
+    (normalise q/k heads, rotate by position, extend the cache), in one launch.  q_in [B,n,H,D],
+    k_in/v_in [B,n,G,D] may be views of one packed projection output.  Returns the rotated
+    queries [B,n,H,D]; the rotated keys and the values land in their page slots, token t of
+    sequence b at position start_pos[b] + pos_offset + t."""
+    lib = _lib.init()
+    for t, name in ((q_in, "q_in"), (k_in, "k_in"), (v_in, "v_in")):
+        _req(t, torch.float16, name, False)
+    _req(cos_sin, torch.float32, "cos_sin"); _req(start_pos, torch.int32, "start_pos")
+    _req(K_pages, torch.float16, "K_pages"); _req(V_pages, torch.float16, "V_pages")
+    _req(block_table, torch.int32, "block_table")
+    B, n = q_in.shape[0], q_in.shape[1]
+    if tuple(q_in.shape) != (B, n, H, D) or tuple(k_in.shape) != (B, n, G, D) or k_in.shape != v_in.shape:
+        raise KascadeError(f"q_in must be [B,n,{H},{D}] and k_in/v_in [B,n,{G},{D}]")
+    if tuple(k_in.stride()) != tuple(v_in.stride()):
+        raise KascadeError("k_in and v_in must share strides")
+    if cos_sin.dim() != 2 or cos_sin.shape[1] != D:
+        raise KascadeError(f"cos_sin must be [max_pos,{D}]")
+    if start_pos.numel() != B or block_table.shape[0] != B:
+        raise KascadeError("start_pos and block_table must have one row per sequence")
+    if K_pages.dim() != 4 or K_pages.shape[1] != page_size or tuple(K_pages.shape[2:]) != (G, D) \
+            or K_pages.shape != V_pages.shape:
+        raise KascadeError(f"pages must be [num_pages,{page_size},{G},{D}]")
+    for w, name in ((q_norm_weight, "q_norm_weight"), (k_norm_weight, "k_norm_weight")):
+        if w is not None:
+            _req(w, torch.float16, name)
+            if w.numel() != D:
+                raise KascadeError(f"{name} must have {D} elements")
+    if out is None:
+        out = torch.empty(B, n, H, D, device=q_in.device, dtype=torch.float16)
+    else:
+        _req(out, torch.float16, "out")
+        if tuple(out.shape) != (B, n, H, D):
+            raise KascadeError("out must be [B,n,H,D]")
+    qs, ks = _blhd_strides(q_in, "q_in"), _blhd_strides(k_in, "k_in")
+    _lib.check(lib.kascade_rope_append_paged_call(
+        _ptr(q_in), ctypes.byref(qs), _ptr(k_in), _ptr(v_in), ctypes.byref(ks), _ptr(cos_sin), cos_sin.shape[0],
+        _ptr(q_norm_weight), _ptr(k_norm_weight), float(norm_eps), _ptr(start_pos), int(pos_offset),
+        _ptr(out), _ptr(K_pages), _ptr(V_pages), _ptr(block_table), block_table.shape[1], page_size,
+        B, n, _stream()))
+    return out
 
 
 # ------------------------------------------- chunked prefill over the paged cache

@@ -23,7 +23,10 @@ independent mathematics in tests/test_oracle_*.py (SDPA for dense attention,
 brute-force loops for pooling/masks/top-k, closed-form budgets, invariants,
 equivalence of the gather and scatter formulations).  Implementation-defined
 behaviour of ``torch.topk`` among tied / -inf candidates is not pinned and is
-handled by the tie-aware comparison in ``topk_agreement``.
+handled by the tie-aware comparison in ``topk_agreement``.  The steps that
+precede the strategy call (head normalisation, rotary embedding; last section)
+belong to the reference's transformers dependency and are pinned against the
+installed library's own functions.
 
 Softmax is always taken with a per-row maximum (the reference's
 kernel_utils.softmax_ subtracts the global maximum, kernel_utils.py:259-277,
@@ -561,3 +564,53 @@ class StrategyOracle:
                 w = w / w.sum(dim=-1, keepdim=True)
         out = torch.matmul(w, vs)
         return out.transpose(1, 2).contiguous()
+
+
+# --------------------------------------------------------------------------
+# what the attention module does before it calls the strategy
+# --------------------------------------------------------------------------
+# The reference leaves these steps to its pinned third-party dependency
+# (transformers==4.53.0, pyproject.toml:34): the decoder's attention module
+# normalises the projected heads, rotates q and k, appends k/v to the cache and
+# only then calls the registered attention function
+# (EfficientKascadeStrategy.py:126-161 receives the results and, at :144-150,
+# transposes and copies them).  Restated here from the published algorithms
+# (RoFormer's rotary embedding in the "rotate half" form; RMS normalisation),
+# in float64, and pinned against the installed transformers' own functions in
+# tests/test_oracle_pins.py.
+def rope_angles(positions: torch.Tensor, dim: int, theta: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """cos, sin [..., dim/2] of position * theta^(-2i/dim), the angles formed in fp32 as the
+    library does (an fp32 product of an fp32 inverse frequency and an fp32 position)."""
+    inv = 1.0 / (theta ** (torch.arange(0, dim, 2, dtype=torch.int64).to(torch.float32) / dim))
+    ang = positions.to(torch.float32)[..., None] * inv
+    return ang.cos(), ang.sin()
+
+
+def rope_rotate_half(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """x [..., dim] rotated: pairs are (i, i + dim/2); cos/sin [..., dim/2] broadcast over x's
+    leading axes.  out[i] = x[i] cos_i - x[i+dim/2] sin_i; out[i+dim/2] = x[i+dim/2] cos_i + x[i] sin_i."""
+    h = x.shape[-1] // 2
+    x = x.double()
+    c, s = cos.double(), sin.double()
+    x1, x2 = x[..., :h], x[..., h:]
+    return torch.cat((x1 * c - x2 * s, x2 * c + x1 * s), dim=-1)
+
+
+def rms_head_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """x / sqrt(mean(x^2) + eps) * weight over the last axis, in float64."""
+    x = x.double()
+    return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * weight.double()
+
+
+def rope_append(q: torch.Tensor, k: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor,
+                sin: torch.Tensor, q_weight: Optional[torch.Tensor] = None,
+                k_weight: Optional[torch.Tensor] = None, eps: float = 1e-6
+                ) -> Tuple[torch.Tensor, torch.Tensor]:
+    """q [B,n,H,D], k [B,n,G,D] -> (normalised and) rotated q, k in float64.  cos/sin are tables
+    [max_pos, D/2]; positions [B,n] index them."""
+    if q_weight is not None:
+        q = rms_head_norm(q, q_weight, eps)
+    if k_weight is not None:
+        k = rms_head_norm(k, k_weight, eps)
+    c, s = cos[positions.long()][:, :, None], sin[positions.long()][:, :, None]
+    return rope_rotate_half(q, c, s), rope_rotate_half(k, c, s)

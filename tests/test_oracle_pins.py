@@ -402,3 +402,57 @@ def test_config0_cpu_plumbing_run():
             s = (k1[0, gk, ks] @ q1[0, h, i]) * scaling
             want = torch.softmax(s, 0) @ v[0, gk, ks]
             assert torch.allclose(o1[0, i, h], want, atol=2e-5), (i, h)
+
+
+# ---------------------------------------------------------------- module steps before the strategy
+def test_rope_and_head_norm_vs_library():
+    """The oracle's rotary embedding and head normalisation equal the transformers library's
+    Qwen3 functions (fp32), and the rotation has the properties that define it."""
+    qwen3 = pytest.importorskip("transformers.models.qwen3.modeling_qwen3")
+    from transformers import Qwen3Config
+    D, Hh, Gg, B, n = 128, 4, 2, 2, 9
+    cfg = Qwen3Config(hidden_size=256, num_attention_heads=Hh, num_key_value_heads=Gg, head_dim=D,
+                      rope_theta=1e6, max_position_embeddings=4096, num_hidden_layers=1,
+                      intermediate_size=64, vocab_size=32)
+    theta = cfg.rope_parameters["rope_theta"] if getattr(cfg, "rope_parameters", None) else cfg.rope_theta
+    gen = torch.Generator().manual_seed(5)
+    q = torch.randn(B, n, Hh, D, generator=gen)
+    k = torch.randn(B, n, Gg, D, generator=gen)
+    pos = torch.stack([torch.arange(n) + 3000, torch.arange(n) + 17])
+    rot = qwen3.Qwen3RotaryEmbedding(cfg)
+    cos_l, sin_l = rot(q, pos)                                           # [B,n,D], halves repeated
+    q_l, k_l = qwen3.apply_rotary_pos_emb(q, k, cos_l, sin_l, unsqueeze_dim=2)
+    table_pos = torch.arange(4096)
+    cos_t, sin_t = orc.rope_angles(table_pos, D, theta)
+    assert torch.equal(cos_t[pos], cos_l[..., :D // 2]) and torch.equal(sin_t[pos], sin_l[..., D // 2:])
+    q_o, k_o = orc.rope_append(q, k, pos, cos_t, sin_t)
+    assert torch.allclose(q_o.float(), q_l, atol=2e-6, rtol=1e-6)
+    assert torch.allclose(k_o.float(), k_l, atol=2e-6, rtol=1e-6)
+    # head normalisation
+    norm = qwen3.Qwen3RMSNorm(D, eps=1e-6)
+    with torch.no_grad():
+        norm.weight.copy_(1 + 0.1 * torch.randn(D, generator=gen))
+        want = norm(q)
+    got = orc.rms_head_norm(q, norm.weight.detach(), 1e-6)
+    assert torch.allclose(got.float(), want, atol=2e-6, rtol=1e-6)
+    # with weights, norm comes before the rotation
+    q_o2, _ = orc.rope_append(q, k, pos, cos_t, sin_t, norm.weight.detach(), norm.weight.detach())
+    with torch.no_grad():
+        q_l2, _ = qwen3.apply_rotary_pos_emb(norm(q), norm(k), cos_l, sin_l, unsqueeze_dim=2)
+    assert torch.allclose(q_o2.float(), q_l2, atol=4e-6, rtol=1e-6)
+    # defining properties: position 0 is the identity, pair norms are kept, and q.k depends on
+    # the distance between the two positions only
+    z = torch.zeros(B, n, dtype=torch.long)
+    q0, _ = orc.rope_append(q, k, z, cos_t, sin_t)
+    assert torch.allclose(q0, q.double(), atol=0, rtol=0)
+    h = D // 2
+    assert torch.allclose(q_o[..., :h] ** 2 + q_o[..., h:] ** 2,
+                          q.double()[..., :h] ** 2 + q.double()[..., h:] ** 2, atol=1e-9)
+    qa = q[:1, :1, :1]; ka = k[:1, :1, :1]
+    dots = []
+    for shift in (0, 100, 2500):
+        pq = torch.tensor([[40 + shift]]); pk = torch.tensor([[33 + shift]])
+        a, _ = orc.rope_append(qa, ka, pq, cos_t, sin_t)
+        _, b = orc.rope_append(qa, ka, pk, cos_t, sin_t)
+        dots.append(float((a * b).sum()))
+    assert abs(dots[0] - dots[1]) < 2e-3 and abs(dots[0] - dots[2]) < 2e-3   # fp32 angles
