@@ -45,7 +45,7 @@ def log(msg):
 
 
 SINGLE_KERNELS = ("membw_copy", "prefill_dense", "prefill_scores", "prefill_aggregate", "prefill_topk", "prefill_reuse",
-                  "decode_dense", "decode_anchor0", "decode_anchor", "decode_topk", "decode_reuse")
+                  "decode_dense", "decode_anchor0", "decode_anchor", "decode_topk", "decode_reuse", "rope_append")
 
 
 def run_single_kernel(name, iters, seq_len, dev, head_map):
@@ -63,6 +63,26 @@ def run_single_kernel(name, iters, seq_len, dev, head_map):
             y.copy_(x)
         torch.cuda.synchronize()
         print(json.dumps({"kernel": name, "iters": iters, "bytes_per_copy": 1 << 30}), flush=True)
+        return
+    if name == "rope_append":
+        # the projection -> attention hand-off on one 2048-token chunk of config 4 (page 16), three
+        # rotating projection outputs and caches
+        n, n_pages = 2048, 2048 // 16
+        qkvs = [workloads.gaussian((1, n, (H + 2 * G) * D), seed=20 + i, device=dev) for i in range(3)]
+        pages = [(torch.zeros(n_pages, 16, G, D, device=dev, dtype=torch.float16),
+                  torch.zeros(n_pages, 16, G, D, device=dev, dtype=torch.float16)) for _ in range(3)]
+        table = torch.randperm(n_pages).to(torch.int32).view(1, n_pages).to(dev)
+        cs = kernels.rope_table(n, device=dev)
+        wq = torch.ones(D, device=dev, dtype=torch.float16)
+        start = torch.zeros(1, device=dev, dtype=torch.int32)
+        out = torch.empty(1, n, H, D, device=dev, dtype=torch.float16)
+        for i in range(iters):
+            x = qkvs[i % 3]
+            kernels.rope_append_paged(x[..., :H * D].view(1, n, H, D), x[..., H * D:(H + G) * D].view(1, n, G, D),
+                                      x[..., (H + G) * D:].view(1, n, G, D), cs, start, *pages[i % 3], table, 16, 0,
+                                      wq, wq, 1e-6, out=out)
+        torch.cuda.synchronize()
+        print(json.dumps({"kernel": name, "iters": iters}), flush=True)
         return
     if name.startswith("prefill"):
         L = seq_len
@@ -390,6 +410,59 @@ def main():
                                  "chunks over a paged cache (page 16), then 256 decode steps replayed as one HIP graph "
                                  "per step; attention only, per-layer Q/K/V synthetic")
         del qs, ks, vs, dq, dk, dv, chunks
+        torch.cuda.empty_cache()
+
+        # the same stack as decoder attention blocks: hidden states in, the projections as library
+        # GEMMs, one hand-off launch (head norm + rotary embedding + paged append) per layer
+        from kascade_amd.blocks import KascadeBlockStack
+        hidden = 4096
+        xs = workloads.gaussian((1, n_tok, hidden), seed=900, device=dev)
+        blocks = {}
+        for name, dense in (("kascade", False), ("dense", True)):
+            st = KascadeBlockStack(n_layers, anchors, maps, PCT, n_tok, hidden=hidden, batch=1, page_size=16,
+                                   rolling_prefill=True, device=dev, table_seed=2, dense=dense)
+
+            def run_prefill():
+                st.reset()
+                for s0 in range(0, prompt, chunk):
+                    st.prefill_chunk_hidden(xs[:, s0:s0 + chunk])
+
+            def run_decode_graph():
+                st.reset(prompt)
+                for s0 in range(steps):
+                    st.graph_x.copy_(xs[:, prompt + s0:prompt + s0 + 1])
+                    st.replay_decode_hidden()
+
+            run_prefill()
+            t_pre = min(wall(run_prefill) for _ in range(3))
+            st.reset(prompt)
+            st.capture_decode_hidden()
+            run_decode_graph()
+            t_graph = min(wall(run_decode_graph) for _ in range(2))
+            blocks[name] = {"prefill_ms": round(t_pre, 2), "decode_ms_graph": round(t_graph, 2),
+                            "us_per_token": round((t_pre + t_graph) * 1e3 / n_tok, 2)}
+            if not dense:   # the hand-off launch alone, on one chunk and on one decode token
+                qkv = torch.nn.functional.linear(xs[:, :chunk], st.w_qkv[0])
+                views = (qkv[..., :H * D].view(1, chunk, H, D), qkv[..., H * D:(H + G) * D].view(1, chunk, G, D),
+                         qkv[..., (H + G) * D:].view(1, chunk, G, D))
+                st.reset(0)
+                q_buf = torch.empty(1, chunk, H, D, device=dev, dtype=torch.float16)
+                t_hand = ev_time(lambda: kernels.rope_append_paged(
+                    *views, st.cos_sin, st.seqlens, st.k_pages[0], st.v_pages[0], st.block_table, 16, 0,
+                    st.q_norm_w[0], st.k_norm_w[0], st.norm_eps, out=q_buf), n=5, warm=2, reps=20)
+                hand_bytes = chunk * ((H + 2 * G) * D * 2 * 2 + D * 4)      # rows in and out, one angle row per token
+                blocks["handoff_us_chunk"] = round(t_hand, 2)
+                blocks["handoff_hbm_frac"] = round(hand_bytes / t_hand / 1e3 / HBM_PEAK_GBS, 4)
+                del qkv, views, q_buf
+            log(f"[bench] stack blocks {name}: {blocks[name]}")
+            del st
+            torch.cuda.empty_cache()
+        blocks["speedup_per_token"] = round(blocks["dense"]["us_per_token"] / blocks["kascade"]["us_per_token"], 3)
+        blocks["workload"] = ("the same 36 layers as decoder attention blocks on random weights: rms norm, q/k/v "
+                              "projection (hidden 4096), head norm + rotary embedding + paged append in one "
+                              "launch, attention, output projection, residual; no MLP")
+        stack_res["blocks"] = blocks
+        del xs
         torch.cuda.empty_cache()
 
     # ---------------------------------------------- what this device delivers to library kernels

@@ -374,8 +374,7 @@ int kascade_rope_append_paged_call(const kascade_half* q_in, const kascade_strid
     REQUIRE(q_in && k_in && v_in && cos_sin && start_pos && q_out && K_pages && V_pages && block_table,
             "rope_append: null pointer argument");
     REQUIRE(batch > 0 && n_new >= 0 && max_pos > 0, "rope_append: bad batch/n_new/max_pos");
-    REQUIRE((long long)batch * n_new * (kHeads + 2 * kGroups) / 16 < (1LL << 31),
-            "rope_append: too many rows for one launch");
+    REQUIRE((long long)batch * n_new < (1LL << 31), "rope_append: too many tokens for one launch");
     REQUIRE(norm_eps >= 0.f, "rope_append: norm_eps must not be negative");
     int shift;
     if (check_paging(block_table, max_pages, page_size, &shift)) return -1;

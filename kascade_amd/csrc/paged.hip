@@ -48,73 +48,77 @@ __global__ __launch_bounds__(256) void decode_budgets_kernel(int* __restrict__ s
 }
 
 
-// One 16-lane row per (token, head): 32 query heads, 8 key heads, 8 value heads = 48 rows per
-// token, 16 rows per workgroup, so a workgroup stays within one token.  Query and key heads are
-// (optionally) RMS-normalised over the head dimension, then rotated by the token's position in
-// the "rotate half" pairing (i, i + 64): the partner element sits 8 lanes away in the row.
-// Queries go to a dense [B,n,H,D] tensor; keys and values go straight to their page slots.
+// One workgroup per token, one 16-lane row per head: 32 query heads, 8 key heads, 8 value heads
+// = 48 rows, three per 16-lane group (two query heads; a key head or a value head).  Query and
+// key heads are (optionally) RMS-normalised over the head dimension, then rotated by the token's
+// position in the "rotate half" pairing (i, i + 64): the partner element sits 8 lanes away in the
+// row.  Queries go to a dense [B,n,H,D] tensor; keys and values go straight to their page slots.
+// The position, the page and the angles are the same for the whole workgroup.
 __global__ __launch_bounds__(256) void rope_append_kernel(RopeAppendParams p) {
     const int lane = threadIdx.x & 15;
-    const long long r = (long long)blockIdx.x * 16 + (threadIdx.x >> 4);
-    const int hh = (int)(r % (kHeads + 2 * kGroups));
-    const long long bt = r / (kHeads + 2 * kGroups);
-    const int t = (int)(bt % p.n_new);
-    const int b = (int)(bt / p.n_new);
+    const int grp = threadIdx.x >> 4;                       // 0..15
+    const int t = blockIdx.x % p.n_new;
+    const int b = blockIdx.x / p.n_new;
     const int pos = p.start_pos[b] + p.pos_offset + t;
     if (pos < 0) return;
-    const bool is_q = hh < kHeads;
-    const bool is_v = hh >= kHeads + kGroups;
-    const int g = is_q ? hh : (hh - kHeads) & (kGroups - 1);
+    const bool cache_ok = (pos >> p.page_shift) < p.max_pages;
+    const bool is_v = grp >= kGroups;                       // third row of this group: key or value head
+    const int g_kv = grp & (kGroups - 1);
 
-    const half_t* src = is_q ? p.q_in + b * p.q_sb + t * p.q_sl + g * p.q_sh
-                             : (is_v ? p.v_in : p.k_in) + b * p.kv_sb + t * p.kv_sl + g * p.kv_sh;
-    Pack16 x;
-    x.u = ld_global_16(src + lane * 8);
-
-    half_t* dst;
-    if (is_q) {
-        dst = p.q_out + ((bt * kHeads) + g) * kDim;
-    } else {
-        if ((pos >> p.page_shift) >= p.max_pages) return;
+    // all loads first
+    Pack16 x[3], wq, wk;
+    const half_t* qrow = p.q_in + b * p.q_sb + t * p.q_sl;
+    x[0].u = ld_global_16(qrow + grp * p.q_sh + lane * 8);
+    x[1].u = ld_global_16(qrow + (grp + 16) * p.q_sh + lane * 8);
+    x[2].u = ld_global_16((is_v ? p.v_in : p.k_in) + b * p.kv_sb + t * p.kv_sl + g_kv * p.kv_sh + lane * 8);
+    if (p.q_weight) wq.u = ld_global_16(p.q_weight + lane * 8);
+    if (p.k_weight) wk.u = ld_global_16(p.k_weight + lane * 8);
+    const int pc = pos < p.max_pos ? pos : p.max_pos - 1;
+    const float* cs = p.cos_sin + (long long)pc * kDim + (lane & 7) * 8;
+    float c[8], sn[8];
+    *reinterpret_cast<float4_t*>(c) = *reinterpret_cast<const float4_t*>(cs);
+    *reinterpret_cast<float4_t*>(c + 4) = *reinterpret_cast<const float4_t*>(cs + 4);
+    *reinterpret_cast<float4_t*>(sn) = *reinterpret_cast<const float4_t*>(cs + kDim / 2);
+    *reinterpret_cast<float4_t*>(sn + 4) = *reinterpret_cast<const float4_t*>(cs + kDim / 2 + 4);
+    long long cache_row = 0;
+    if (cache_ok) {
         const int pg = p.block_table[(long long)b * p.max_pages + (pos >> p.page_shift)];
-        const long long row = ((long long)pg << p.page_shift) + (pos & ((1 << p.page_shift) - 1));
-        dst = (is_v ? p.Vp : p.Kp) + (row * kGroups + g) * kDim;
+        cache_row = ((long long)pg << p.page_shift) + (pos & ((1 << p.page_shift) - 1));
     }
-    if (!is_v) {
-        const half_t* w = is_q ? p.q_weight : p.k_weight;
+    const float sign = lane < 8 ? -1.f : 1.f;
+
+    auto rotate = [&](Pack16 v, const half_t* w, const Pack16& wv) {
         if (w) {
             float ss = 0.f;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) ss += (float)x.h[e] * (float)x.h[e];
+            for (int e = 0; e < 8; ++e) ss += (float)v.h[e] * (float)v.h[e];
             ss = row16_sum(ss);
             const float inv = 1.0f / sqrtf(ss * (1.0f / kDim) + p.eps);
-            Pack16 wv;
-            wv.u = ld_global_16(w + lane * 8);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const half_t n = (half_t)((float)x.h[e] * inv);      // normalised, in storage type
-                x.h[e] = (half_t)((float)n * (float)wv.h[e]);        // times the weight, rounded once
+                const half_t n = (half_t)((float)v.h[e] * inv);          // normalised, in storage type
+                v.h[e] = (half_t)((float)n * (float)wv.h[e]);            // times the weight, rounded once
             }
         }
         Pack16 y;   // the partner half of the head: lanes 8 apart within the row of 16
 #pragma unroll
         for (int d = 0; d < 4; ++d)
-            y.u[d] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x.u[d], 0x128, 0xF, 0xF, false);  // row_ror:8
-        const int pc = pos < p.max_pos ? pos : p.max_pos - 1;
-        const float* cs = p.cos_sin + (long long)pc * kDim + (lane & 7) * 8;
-        const float4_t c0 = *reinterpret_cast<const float4_t*>(cs);
-        const float4_t c1 = *reinterpret_cast<const float4_t*>(cs + 4);
-        const float4_t s0 = *reinterpret_cast<const float4_t*>(cs + kDim / 2);
-        const float4_t s1 = *reinterpret_cast<const float4_t*>(cs + kDim / 2 + 4);
-        const float sign = lane < 8 ? -1.f : 1.f;
+            y.u[d] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v.u[d], 0x128, 0xF, 0xF, false);  // row_ror:8
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const float c = e < 4 ? c0[e] : c1[e - 4];
-            const float s = e < 4 ? s0[e] : s1[e - 4];
-            x.h[e] = (half_t)((float)x.h[e] * c + sign * ((float)y.h[e] * s));
-        }
+        for (int e = 0; e < 8; ++e) v.h[e] = (half_t)((float)v.h[e] * c[e] + sign * ((float)y.h[e] * sn[e]));
+        return v;
+    };
+
+    half_t* qdst = p.q_out + (long long)blockIdx.x * kHeads * kDim + lane * 8;
+    *reinterpret_cast<uint4_t*>(qdst + grp * kDim) = rotate(x[0], p.q_weight, wq).u;
+    *reinterpret_cast<uint4_t*>(qdst + (grp + 16) * kDim) = rotate(x[1], p.q_weight, wq).u;
+    if (cache_ok) {
+        const long long off = (cache_row * kGroups + g_kv) * kDim + lane * 8;
+        if (is_v)      // uniform over the 16 lanes of a row, so the row-wide exchanges above stay whole
+            *reinterpret_cast<uint4_t*>(p.Vp + off) = x[2].u;
+        else
+            *reinterpret_cast<uint4_t*>(p.Kp + off) = rotate(x[2], p.k_weight, wk).u;
     }
-    *reinterpret_cast<uint4_t*>(dst + lane * 8) = x.u;
 }
 
 }  // namespace
@@ -141,7 +145,7 @@ hipError_t launch_paged_kv_append(half_t* Kp, half_t* Vp, const half_t* k_new, c
 hipError_t launch_rope_append(const RopeAppendParams& p, hipStream_t stream) {
     const long long rows = (long long)p.batch * p.n_new * (kHeads + 2 * kGroups);
     if (rows == 0) return hipSuccess;
-    hipLaunchKernelGGL(rope_append_kernel, dim3((unsigned)(rows / 16)), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL(rope_append_kernel, dim3((unsigned)(p.batch * p.n_new)), dim3(256), 0, stream, p);
     return hipGetLastError();
 }
 

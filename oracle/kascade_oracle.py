@@ -614,3 +614,28 @@ def rope_append(q: torch.Tensor, k: torch.Tensor, positions: torch.Tensor, cos: 
         k = rms_head_norm(k, k_weight, eps)
     c, s = cos[positions.long()][:, :, None], sin[positions.long()][:, :, None]
     return rope_rotate_half(q, c, s), rope_rotate_half(k, c, s)
+
+
+def attention_blocks_dense(x: torch.Tensor, w_qkv: Sequence[torch.Tensor], w_o: Sequence[torch.Tensor],
+                           ln_w: Sequence[torch.Tensor], q_norm_w: Sequence[Optional[torch.Tensor]],
+                           k_norm_w: Sequence[Optional[torch.Tensor]], cos: torch.Tensor, sin: torch.Tensor,
+                           n_heads: int, n_kv: int, eps: float = 1e-6) -> torch.Tensor:
+    """The attention halves of a stack of decoder layers with dense causal attention, whole
+    sequence at once, fp32:  x <- x + o_proj(attn(rope(norm(q)), rope(norm(k)), v)) with
+    q,k,v = split(qkv_proj(rms_norm(x))).  x [B,L,hidden]; rows of w_qkv are the query heads,
+    then the key heads, then the value heads.  Causality makes this equal to feeding the same
+    tokens in chunks and then one at a time."""
+    B, L, hidden = x.shape
+    x = x.float()
+    pos = torch.arange(L)[None].expand(B, L)
+    for l in range(len(w_qkv)):
+        h = rms_head_norm(x, ln_w[l].float(), eps).float()
+        qkv = h @ w_qkv[l].float().t()
+        d = qkv.shape[-1] // (n_heads + 2 * n_kv)
+        q = qkv[..., :n_heads * d].reshape(B, L, n_heads, d)
+        k = qkv[..., n_heads * d:(n_heads + n_kv) * d].reshape(B, L, n_kv, d)
+        v = qkv[..., (n_heads + n_kv) * d:].reshape(B, L, n_kv, d)
+        q, k = rope_append(q, k, pos, cos, sin, q_norm_w[l], k_norm_w[l], eps)
+        o, _ = dense_prefill(q.float(), k.float(), v)
+        x = x + o.reshape(B, L, n_heads * d).float() @ w_o[l].float().t()
+    return x

@@ -65,6 +65,9 @@ def test_null_pointers_are_rejected(lib):
     assert lib.kascade_prefill_aggregate_call(None, None, None, None, 1, 64, s, s, 0, None) == -1
     assert lib.kascade_prefill_reuse_call(None, None, None, None, None, 10.0, None, 1, 64, 128, 1, s, s, None) == -1
     assert lib.kascade_paged_kv_append_call(None, None, None, None, None, None, 1, 1, 1, 16, s, None) == -1
+    assert lib.kascade_rope_append_paged_call(None, None, None, None, None, None, 64, None, None, 1e-6, None, 0,
+                                              None, None, None, None, 4, 16, 1, 1, None) == -1
+    assert "null pointer" in _err(lib)
 
 
 def test_bad_sizes_are_rejected(lib):
@@ -93,6 +96,15 @@ def test_bad_sizes_are_rejected(lib):
     assert "topk_percent" in _err(lib)
     assert lib.kascade_topk_call(p, p, 4, 100, 200, None, None, 1, 8, 0, None, None) == -1
     assert "uniform_len" in _err(lib)
+    assert lib.kascade_rope_append_paged_call(p, None, p, p, None, p, 64, None, None, 1e-6, p, 0, p, p, p, p,
+                                              4, 12, 1, 1, None) == -1
+    assert "power of two" in _err(lib)
+    assert lib.kascade_rope_append_paged_call(p, C.byref(Strides(6144, 6140, 128)), p, p, None, p, 64, None, None,
+                                              1e-6, p, 0, p, p, p, p, 4, 16, 1, 1, None) == -1
+    assert "strides" in _err(lib)
+    assert lib.kascade_rope_append_paged_call(p, None, p, p, None, p, 0, None, None, 1e-6, p, 0, p, p, p, p,
+                                              4, 16, 1, 1, None) == -1
+    assert "max_pos" in _err(lib)
     bad = Strides(100, 4, 128)          # not multiples of 8 elements
     ok = Strides(4096 * 128, 4096, 128)
     assert lib.kascade_prefill_dense_call(p, p, p, p, p, 1, 64, bad, ok, 1, None) == -1
