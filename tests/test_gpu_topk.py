@@ -110,3 +110,43 @@ def test_topk_register_kernel_equals_streaming_kernel(cuda, L, K):
     assert torch.equal(a.cpu(), b.cpu())
     _check(sc, a.cpu(), lambda r: nsel[r], lambda r: valid[r], K, -1)
     assert torch.equal(a[2, :1024].cpu(), torch.arange(1024, dtype=torch.int32))
+
+
+def _check_exact_sets(sc: torch.Tensor, idx: torch.Tensor, K: int, what: str):
+    """No tolerance: every returned index is distinct and in range, the values taken are exactly
+    the K largest as a multiset (which of several equal values is taken is free)."""
+    R, L = sc.shape
+    idx = idx.cpu().long()
+    for r in range(R):
+        got = idx[r]
+        assert int(got.min()) >= 0 and int(got.max()) < L, f"{what}: row {r} index out of range"
+        assert got.unique().numel() == K, f"{what}: row {r} repeats an index"
+        took = sc[r, got].float().sort(descending=True).values
+        want = sc[r].float().topk(K).values
+        assert torch.equal(took, want), f"{what}: row {r} did not take the {K} largest values"
+
+
+@pytest.mark.parametrize("L,K", [(4096, 512), (20000, 2048), (70016, 7040)])
+def test_topk_crowded_thresholds_and_special_values(cuda, L, K):
+    """Rows built to crowd the bin that holds the threshold: all entries equal, two levels with the
+    cut inside the lower one, a few distinct values among thousands of copies, signed zeros,
+    subnormals and -inf.  Covers the one-workgroup kernels and (70016) the multi-workgroup path."""
+    from kascade_amd import kernels
+    gen = torch.Generator().manual_seed(L)
+    rows = []
+    rows.append(torch.full((L,), 0.37))                                            # one value
+    two = torch.full((L,), 0.25); two[torch.randperm(L, generator=gen)[:K // 3]] = 0.75
+    rows.append(two)                                                               # cut inside the copies
+    few = torch.full((L,), 1e-3); few[torch.randperm(L, generator=gen)[:K + 5]] = torch.rand(K + 5, generator=gen) + 1
+    rows.append(few)                                                               # cut among distinct values
+    z = torch.zeros(L); z[::2] = -0.0; z[torch.randperm(L, generator=gen)[:K // 2]] = 6e-8   # subnormal halves
+    rows.append(z)
+    ninf = torch.full((L,), float("-inf")); ninf[torch.randperm(L, generator=gen)[:K + 1]] = torch.rand(K + 1, generator=gen)
+    rows.append(ninf)                                                              # exactly K+1 finite entries
+    steps = (torch.arange(L) % 7).float() / 8                                      # seven levels, equal shares
+    rows.append(steps)
+    sc = torch.stack(rows).half()
+    idx = kernels.topk_indices(sc.to(cuda), K)
+    torch.cuda.synchronize()
+    # signed zeros compare equal as values; the multiset check works on values, so it holds either way
+    _check_exact_sets(sc, idx, K, f"L={L} K={K}")
