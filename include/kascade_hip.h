@@ -129,8 +129,12 @@ int kascade_decode_dense_paged_call(const kascade_half* Q, const kascade_half* K
  * pooled post-softmax scores.  Replaces the three launches of the reference's
  * flashattn_gqa_decode_split_{0,1} (recompute_kascade_gqa_decode.py:318-348;
  * kvcache form recompute_kascade_gqa_decode_with_kvcache.py:302-333).
- *   scores            [B,H,scores_stride] f32 scratch, scores_stride a multiple of 8 (raw q.k; the reference
- *                     stores fp16 here, fp32 avoids that extra rounding)
+ *   scores            B*H*scores_stride floats of scratch, scores_stride a multiple of 8, that
+ *                     carry the raw q.k from the streaming launch to the pooling launch; the
+ *                     contents are private to the library (per head 16-bit codes in steps of
+ *                     2^-11 of the exponent below a per-64-token fp32 reference: a third of an
+ *                     fp16 step on the pooled value, where the reference's fp16 raw scores
+ *                     (recompute_kascade_gqa_decode.py:102) lose up to two)
  *   row_sums          [B,H] f32: global log2-domain log-sum per head
  *   aggregated_scores [B,G,scores_stride] f16: sum over the 4 heads of a KV head
  *                     of softmax probabilities; 0 at positions >= cache_seqlens[b]

@@ -14,7 +14,7 @@ struct DecodeParams {
     const int* block_table; // [B,max_pages] or null
     float* glse;            // [B,H,num_split]
     float* opart;           // [B,H,num_split,D]
-    float* scores;          // [B,H,scores_stride] raw q.k (anchor mode)
+    float* scores;          // [B,H,scores_stride] floats of scratch: compact raw scores (anchor mode)
     // Fused combine: with counters != null ([B*G] ints, zero before the first launch and zero
     // again after every launch) the last split workgroup of each (b, g) merges the splits into
     // out [B,H,D] and row_sums [B,H] (either may be null), and no combine launch is needed.

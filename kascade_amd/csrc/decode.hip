@@ -32,6 +32,17 @@ constexpr int kRowsPerIter = 16 * kUnroll;    // rows per workgroup iteration (1
 constexpr int kScoreBatches = 16;             // batches between two score flushes (anchor mode)
 constexpr int kStripRows = 16 * kScoreBatches;  // rows a wavefront owns per super-iteration
 constexpr int kSubChunk = 2048;               // rows whose physical ids are staged in LDS at once
+// Raw scores travel from the anchor pass to the pooling kernel in a compact form: per head a row of
+// scores_stride floats holds, in its first half, one 16-bit code per token and, behind them, one
+// fp32 reference per granule of 64 tokens (the granule's largest scaled score, log2 domain).
+// code = round((reference - score*scale) * 2048), i.e. steps of 2^-11 in the exponent: the
+// probability recovered from it is within 1.7e-4 (a third of an fp16 step) of the exact one, and
+// a code of 65534 steps (2^-32 of the granule's maximum, itself at most the row's log-sum) is far
+// below what survives the pooled sum's fp16 rounding.  65535 marks a masked position.  Splits
+// start at multiples of 64 tokens, so a granule belongs to one workgroup.  Half the bytes of fp32
+// scores: their write-back to HBM, interleaved with the K stream, costs several times its size.
+constexpr float kScoreSteps = 2048.f;
+constexpr uint32_t kScoreNone = 65535u;
 
 // Device-coherent accesses (relaxed atomics at agent scope) for data that one workgroup writes
 // and another workgroup of the same launch reads.
@@ -67,7 +78,11 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
     __shared__ int s_found;   // gather mode: sub-chunk whose index list names the newest token
     // anchor mode: two buffers of four wavefront strips (4 heads x kStripRows raw scores)
     __shared__ __attribute__((aligned(16))) float s_sc[WRITE_SCORES ? 2 : 1][WRITE_SCORES ? 4 : 1][kGroupSize][WRITE_SCORES ? kStripRows : 4];
+    // anchor pass without output: per wavefront one tile of 16 K rows on its way into the matrix layout
+    constexpr int kKtStride = 136;   // halves per row (128 + 8): rows 272 bytes apart
+    __shared__ __attribute__((aligned(16))) half_t s_kt[(!GATHER && !WITH_V && WRITE_SCORES) ? 4 : 1][(!GATHER && !WITH_V && WRITE_SCORES) ? 16 * kKtStride : 8];
 
+    constexpr bool kMfmaScores = !GATHER && !WITH_V && WRITE_SCORES;
     const int g = blockIdx.x;       // the 8 KV heads of one token range are adjacent in dispatch order
     const int split = blockIdx.y;
     const int b = blockIdx.z;
@@ -240,6 +255,44 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
         }
     };
 
+    // Writer wavefront of the anchor passes: stores the four strips of super-iteration `sup`
+    // (buffer sup & 1) in the compact score format (see kScoreSteps): per instruction one
+    // (strip, head) row of 256 tokens, 16 lanes per granule of 64 tokens, four tokens per lane;
+    // 128 contiguous bytes per granule plus its reference value.
+    auto flush_scores = [&](int sup) {
+        const int cn = r1 - r0;
+        constexpr int kVecPerStrip = kGroupSize * kStripRows / 4;   // float4 per strip
+#pragma unroll 4
+        for (int i = 0; i < 4 * kVecPerStrip / 64; ++i) {
+            const int idx = i * 64 + lane;
+            const int w = idx / kVecPerStrip, rem = idx % kVecPerStrip;
+            const int h = rem / (kStripRows / 4), t4 = (rem % (kStripRows / 4)) * 4;
+            float4_t v = *reinterpret_cast<const float4_t*>(&s_sc[sup & 1][w][h][t4]);
+            const int r = sup * (4 * kStripRows) + w * kStripRows + t4;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)      // strip positions past the range were never filled
+                v[e] = (r + e < cn) ? v[e] : -INFINITY;
+            const float mx = row16_max(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])));
+            const float base = (mx == -INFINITY) ? 0.f : mx;
+            uint32_t q[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float d = (base - v[e]) * (kScaleLog2 * kScoreSteps);      // >= 0, +inf if masked
+                q[e] = (v[e] == -INFINITY) ? kScoreNone : (uint32_t)fminf(rintf(d), (float)(kScoreNone - 1));
+            }
+            float* row = p.scores + ((size_t)b * kHeads + g * kGroupSize + h) * p.scores_stride;
+            uint16_t* dst = reinterpret_cast<uint16_t*>(row) + r0 + r;
+            if (r + 3 < cn) {
+                *reinterpret_cast<uint2*>(dst) = make_uint2(q[0] | (q[1] << 16), q[2] | (q[3] << 16));
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (r + e < cn) dst[e] = (uint16_t)q[e];
+            }
+            if ((lane & 15) == 0 && r < cn) row[p.scores_stride / 2 + ((r0 + r) >> 6)] = base * kScaleLog2;
+        }
+    };
+
     if (GATHER) {
         // Index list -> block table -> physical row, staged in LDS one sub-chunk at a time.
         auto run = [&](auto paged_tag) {
@@ -289,6 +342,123 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
         }
         };
         if (p.block_table) run(std::true_type{}); else run(std::false_type{});
+    } else if constexpr (kMfmaScores) {
+        // Anchor pass without output: raw scores and log-sums only, so all a row needs is its dot
+        // product with the four queries.  That runs on the matrix unit (v_mfma_f32_16x16x32_f16,
+        // S^T = K Q^T with 16 keys as rows, the four heads as columns 0-3 of 16, d as the
+        // contraction index): no cross-lane reduction and ~6 vector instructions per key instead
+        // of ~80, which is what bounded the rate before.  Rows are loaded as before, 16 lanes per
+        // 256-byte row (four rows per instruction), and pass through a wavefront-private LDS tile
+        // (16 rows of 272 bytes: conflict-free both ways, no barrier) into the A-operand layout,
+        // where lane key + 16*dq holds d [32*step + 8*dq, +8) of its key for step 0..3.  Loading
+        // that layout directly makes every quarter-wavefront touch 16 rows and runs 20 % slower.
+        const int cn = r1 - r0;
+        const int* bt_row = p.block_table ? p.block_table + (size_t)b * p.max_pages : nullptr;
+        const int col = lane & 15, dq = lane >> 4;
+        half8_t qb[4];
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+            Pack16 t;
+            t.u = ld_global_16(p.Q + ((size_t)b * kHeads + g * kGroupSize + (col & 3)) * kDim + 32 * st + 8 * dq);
+            if (col >= kGroupSize) t.u = uint4_t{0, 0, 0, 0};
+            qb[st] = t.h8;
+        }
+        float mcol = -INFINITY, lcol = 0.f;   // running max / sum of this lane's keys of its column
+        auto run = [&](auto paged_tag) {
+        constexpr bool PAGED = decltype(paged_tag)::value;
+        constexpr int kTilesPerStrip = kStripRows / 16;
+        // tile k of this wavefront: 16 keys from row (k / 16) * 1024 + wave * 256 + (k % 16) * 16
+        auto tile_row = [&](int k) { return (k / kTilesPerStrip) * (4 * kStripRows) + wave * kStripRows + (k % kTilesPerStrip) * 16; };
+        // loads: lane (dq, col) takes chunk col of rows 4i + dq of the tile; past the end: clamped, masked later
+        auto tok_of = [&](int k, int i) { return min(r0 + tile_row(k) + 4 * i + dq, r1 - 1); };
+        auto fetch_pages = [&](int k, int (&pg)[4]) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) pg[i] = PAGED ? bt_row[tok_of(k, i) >> p.page_shift] : 0;
+        };
+        auto issue = [&](int k, const int (&pg)[4], uint4_t (&buf)[4]) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int tok = tok_of(k, i);
+                const size_t off = PAGED ? ((size_t)((pg[i] << p.page_shift) + (tok & page_mask)) * kGroups + g) * kDim
+                                         : (size_t)b * p.kv_stride_b + (size_t)g * p.kv_stride_h + (size_t)(unsigned)tok * stride_l;
+                buf[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.K + off + 8 * col));
+            }
+        };
+        half_t* kt = &s_kt[wave < 4 ? wave : 0][0];
+        auto compute = [&](int k, const uint4_t (&buf)[4]) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                *reinterpret_cast<uint4_t*>(&kt[(4 * i + dq) * kKtStride + 8 * col]) = buf[i];
+            __builtin_amdgcn_wave_barrier();   // the reads below are other lanes' writes (same wavefront: in order)
+            float4_t sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int st = 0; st < 4; ++st) {
+                const half8_t a = *reinterpret_cast<const half8_t*>(&kt[col * kKtStride + 32 * st + 8 * dq]);
+                sc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qb[st], sc, 0, 0, 0);
+            }
+            __builtin_amdgcn_wave_barrier();
+            // sc[e] = q_col . k of key tile_row(k) + 4*dq + e
+            const int key0 = tile_row(k) + 4 * dq;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (key0 + e >= cn) sc[e] = -INFINITY;
+            if (col < kGroupSize)
+                *reinterpret_cast<float4_t*>(&s_sc[(k / kTilesPerStrip) & 1][wave][col][(k % kTilesPerStrip) * 16 + 4 * dq]) = sc;
+            const float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), mcol);
+            const float mref = (mx == -INFINITY) ? 0.f : mx * kScaleLog2;
+            float sum = lcol * fast_exp2(mcol * kScaleLog2 - mref);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sum += fast_exp2(sc[e] * kScaleLog2 - mref);
+            lcol = sum;
+            mcol = mx;
+        };
+        if (cn > 0) {
+            const int nsup = (cn + 4 * kStripRows - 1) / (4 * kStripRows);
+            if (wave == 4) {
+                for (int sup = 0; sup < nsup; ++sup) {
+                    __syncthreads();
+                    flush_scores(sup);
+                }
+            } else {
+                // four tiles in flight per wavefront (16 KB); page numbers one round further ahead
+                const int ntile = nsup * kTilesPerStrip;
+                uint4_t buf[4][4];
+                int pgn[4][4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    fetch_pages(j, pgn[j]);
+                    issue(j, pgn[j], buf[j]);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) fetch_pages(4 + j, pgn[j]);
+                for (int k = 0; k < ntile; k += 4) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        compute(k + j, buf[j]);
+                        KASCADE_SCHED_FENCE();
+                        issue(k + 4 + j, pgn[j], buf[j]);      // past the last tile: clamped rows, never used
+                        fetch_pages(k + 8 + j, pgn[j]);
+                        KASCADE_SCHED_FENCE();
+                    }
+                    if ((k + 4) % kTilesPerStrip == 0) __syncthreads();   // a strip is complete: hand it to the writer
+                }
+            }
+        }
+        };
+        if (bt_row) run(std::true_type{}); else run(std::false_type{});
+        // the four key subsets of a column sit in lanes col, col+16, col+32, col+48
+#pragma unroll
+        for (int sh = 16; sh <= 32; sh <<= 1) {
+            const float mo = __shfl_xor(mcol, sh), lo = __shfl_xor(lcol, sh);
+            const float mx = fmaxf(mcol, mo);
+            const float mref = (mx == -INFINITY) ? 0.f : mx * kScaleLog2;
+            lcol = lcol * fast_exp2(mcol * kScaleLog2 - mref) + lo * fast_exp2(mo * kScaleLog2 - mref);
+            mcol = mx;
+        }
+        if (wave < 4 && lane < kGroupSize) {
+            s_merge[wave].m[lane] = mcol;
+            s_merge[wave].l[lane] = lcol;
+        }
     } else {
         // Dense range [r0, r1): no staging and no barriers.  Three-stage pipeline: block-table
         // entries two iterations ahead, K/V rows one iteration ahead, arithmetic on the current.
@@ -300,27 +470,6 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
         auto rbase_of = [&](int it) {
             const int q = it / kRowsPerIter;
             return (q / kScoreBatches) * (4 * kStripRows) + wave * kStripRows + (q % kScoreBatches) * 16 + rg;
-        };
-        // Writer wavefront: stores the four strips of super-iteration `sup` (buffer sup & 1), one
-        // 16-byte store per lane per instruction, 1 KB contiguous per (strip, head).
-        auto flush_scores = [&](int sup) {
-            constexpr int kVecPerStrip = kGroupSize * kStripRows / 4;   // float4 per strip
-#pragma unroll 4
-            for (int i = 0; i < 4 * kVecPerStrip / 64; ++i) {
-                const int idx = i * 64 + lane;
-                const int w = idx / kVecPerStrip, rem = idx % kVecPerStrip;
-                const int h = rem / (kStripRows / 4), t4 = (rem % (kStripRows / 4)) * 4;
-                const float4_t v = *reinterpret_cast<const float4_t*>(&s_sc[sup & 1][w][h][t4]);
-                const int r = sup * (4 * kStripRows) + w * kStripRows + t4;
-                float* dst = p.scores + ((size_t)b * kHeads + g * kGroupSize + h) * p.scores_stride + r0 + r;
-                if (r + 3 < cn) {
-                    *reinterpret_cast<float4_t*>(dst) = v;
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (r + e < cn) dst[e] = v[e];
-                }
-            }
         };
         auto tok_of = [&](int it, int u) { return min(r0 + rbase_of(it) + u * 4, r1 - 1); };
         // The paged / contiguous choice is hoisted out of the loop as a compile-time tag: a
@@ -385,6 +534,7 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
     }
 
     // ---- merge the four row-groups of the wavefront (lanes l, l^16, l^32) ----
+    if constexpr (!kMfmaScores) {
 #pragma unroll
     for (int h = 0; h < kGroupSize; ++h) {
 #pragma unroll
@@ -418,6 +568,7 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
                 for (int d = 0; d < 8; ++d) s_merge[wave].acc[h][dl * 8 + d] = acc[h][d];
             }
         }
+    }
     }
     __syncthreads();
     // ---- merge the four wavefronts; thread -> (head, two d's) ----
@@ -632,22 +783,28 @@ __global__ __launch_bounds__(256) void decode_aggregate_kernel(const float* __re
     float sum[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) sum[e] = 0.f;
-    const bool full = (j0 + 8 <= scores_stride) && ((scores_stride & 3) == 0);
+    const bool full = (j0 + 8 <= scores_stride) && ((scores_stride & 7) == 0);
+    if (j0 < len) {   // codes and references beyond the sequence were never written
 #pragma unroll
-    for (int h = 0; h < kGroupSize; ++h) {
-        const float* sp = scores + ((size_t)b * kHeads + g * kGroupSize + h) * scores_stride + j0;
-        float v[8];
-        if (full && j0 + 8 <= len) {
-            float4 a = *reinterpret_cast<const float4*>(sp);
-            float4 c = *reinterpret_cast<const float4*>(sp + 4);
-            v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
-            v[4] = c.x; v[5] = c.y; v[6] = c.z; v[7] = c.w;
-        } else {
+        for (int h = 0; h < kGroupSize; ++h) {
+            const float* row = scores + ((size_t)b * kHeads + g * kGroupSize + h) * scores_stride;
+            const uint16_t* sp = reinterpret_cast<const uint16_t*>(row) + j0;
+            const float ref = row[scores_stride / 2 + (j0 >> 6)] - lse[h];
+            uint32_t q[8];
+            if (full) {
+                const uint4_t raw = ld_global_16(sp);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) v[e] = (j0 + e < len) ? sp[e] : -INFINITY;
+                for (int e = 0; e < 8; ++e) q[e] = (raw[e >> 1] >> (16 * (e & 1))) & 0xFFFFu;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) q[e] = (j0 + e < len) ? sp[e] : kScoreNone;
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float pr = fast_exp2(ref - (float)q[e] * (1.f / kScoreSteps));
+                sum[e] += (q[e] == kScoreNone) ? 0.f : pr;
+            }
         }
-#pragma unroll
-        for (int e = 0; e < 8; ++e) sum[e] += fast_exp2(v[e] * kScaleLog2 - lse[h]);
     }
     half_t* ap = agg + ((size_t)b * kGroups + g) * scores_stride + j0;
     if (full && ((scores_stride & 7) == 0)) {
