@@ -27,6 +27,12 @@ constexpr int kThreads = 256;
 #ifndef KASCADE_DECODE_UNROLL
 #define KASCADE_DECODE_UNROLL 4
 #endif
+#ifndef KASCADE_GATHER_MFMA
+#define KASCADE_GATHER_MFMA 1
+#endif
+#ifndef KASCADE_DENSE_MFMA
+#define KASCADE_DENSE_MFMA 1
+#endif
 constexpr int kUnroll = KASCADE_DECODE_UNROLL;  // rows per row-group per iteration
 constexpr int kRowsPerIter = 16 * kUnroll;    // rows per workgroup iteration (128)
 constexpr int kScoreBatches = 16;             // batches between two score flushes (anchor mode)
@@ -64,14 +70,15 @@ __device__ __forceinline__ float2 load_device2(const float* p) {
     return make_float2(x.f[0], x.f[1]);
 }
 
-struct MergeState {  // one per wavefront after the in-wave merge
+struct alignas(16) MergeState {  // one per wavefront after the in-wave merge
     float m[kGroupSize];
     float l[kGroupSize];
     float acc[kGroupSize][kDim];
 };
 
 template <bool GATHER, bool WITH_V, bool WRITE_SCORES>
-__global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decode_split_kernel(DecodeParams p) {
+__global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) __attribute__((amdgpu_waves_per_eu(3)))
+void decode_split_kernel(DecodeParams p) {
     __shared__ int s_row[GATHER ? kSubChunk : 1];
     __shared__ MergeState s_merge[4];
     __shared__ int s_last;
@@ -79,10 +86,15 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
     // anchor mode: two buffers of four wavefront strips (4 heads x kStripRows raw scores)
     __shared__ __attribute__((aligned(16))) float s_sc[WRITE_SCORES ? 2 : 1][WRITE_SCORES ? 4 : 1][kGroupSize][WRITE_SCORES ? kStripRows : 4];
     // anchor pass without output: per wavefront one tile of 16 K rows on its way into the matrix layout
-    constexpr int kKtStride = 136;   // halves per row (128 + 8): rows 272 bytes apart
-    __shared__ __attribute__((aligned(16))) half_t s_kt[(!GATHER && !WITH_V && WRITE_SCORES) ? 4 : 1][(!GATHER && !WITH_V && WRITE_SCORES) ? 16 * kKtStride : 8];
+    constexpr int kKtStride = 136;   // halves per K row (128 + 8): rows 272 bytes apart
+    constexpr int kVtStride = 144;   // halves per V row: 288 bytes, conflict-free for the transposing reads
+    constexpr bool kGatherMfma = GATHER && (KASCADE_GATHER_MFMA != 0);
+    constexpr bool kDenseMfma = !GATHER && ((!WITH_V && WRITE_SCORES) || (KASCADE_DENSE_MFMA != 0));
+    constexpr bool kTiles = kDenseMfma || kGatherMfma;
+    constexpr bool kTilesV = kTiles && WITH_V;
+    __shared__ __attribute__((aligned(16))) half_t s_kt[kTiles ? 4 : 1][kTiles ? 16 * kKtStride : 8];
+    __shared__ __attribute__((aligned(16))) half_t s_vt[kTilesV ? 4 : 1][kTilesV ? 16 * kVtStride : 8];
 
-    constexpr bool kMfmaScores = !GATHER && !WITH_V && WRITE_SCORES;
     const int g = blockIdx.x;       // the 8 KV heads of one token range are adjacent in dispatch order
     const int split = blockIdx.y;
     const int b = blockIdx.z;
@@ -293,7 +305,146 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
         }
     };
 
-    if (GATHER) {
+    if constexpr (kGatherMfma) {
+        // Gathered rows on the matrix unit.  Tiles of 16 rows per wavefront: rows are loaded as
+        // 16 lanes x 16 bytes each (four rows per instruction, K and V), pass through
+        // wavefront-private LDS tiles, and S^T = K Q^T (16 keys x 4 of 16 columns, contraction
+        // over d, v_mfma_f32_16x16x32_f16) leaves every lane with four keys of one column: the
+        // B-operand layout of O^T += V^T P^T (v_mfma_f32_16x16x16_f16, contraction over the 16
+        // keys), whose A operand comes out of the row-major V tile through the transposing LDS
+        // read.  One running maximum per column (two cross-lane exchanges per tile); ~10 vector
+        // instructions per row instead of ~110.
+        const int col = lane & 15, dq = lane >> 4;
+        half8_t qb[4];
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+            Pack16 t;
+            t.u = ld_global_16(p.Q + ((size_t)b * kHeads + g * kGroupSize + (col & 3)) * kDim + 32 * st + 8 * dq);
+            if (col >= kGroupSize) t.u = uint4_t{0, 0, 0, 0};
+            qb[st] = t.h8;
+        }
+        float mcol = -INFINITY, lcol = 0.f;
+        float4_t oacc[8];
+#pragma unroll
+        for (int blk = 0; blk < 8; ++blk) oacc[blk] = float4_t{0.f, 0.f, 0.f, 0.f};
+        half_t* kt = &s_kt[wave][0];
+        half_t* vt = &s_vt[wave][0];
+        struct Tile {
+            uint4_t k[4], v[4];
+        };
+        auto run = [&](auto paged_tag) {
+        constexpr bool PAGED = decltype(paged_tag)::value;
+        for (int c0 = r0; c0 < r1; c0 += kSubChunk) {
+            const int cn = min(kSubChunk, r1 - c0);
+            __syncthreads();
+            for (int i = tid; i < cn; i += kThreads) {
+                int tok = idx_row[c0 + i];
+                tok = max(0, min(tok, seqlen - 1));   // a corrupt index must not leave the sequence
+                if (tok == newest) s_found = c0;
+                int row;
+                if (p.block_table) {
+                    int pg = p.block_table[(size_t)b * p.max_pages + (tok >> p.page_shift)];
+                    row = (pg << p.page_shift) + (tok & page_mask);
+                } else {
+                    row = tok;
+                }
+                s_row[i] = row;
+            }
+            __syncthreads();
+            if (p.k_new != nullptr && s_found == c0) {   // c0 differs per sub-chunk: no reset needed
+                write_newest();
+                __syncthreads();
+            }
+            // tile t: rows [16t, 16t+16) of the sub-chunk; lane (dq, col) loads chunk col of rows 4i + dq
+            auto issue = [&](int t, Tile& tb) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int row = s_row[min(16 * t + 4 * i + dq, cn - 1)];   // past the end: clamped, masked later
+                    const size_t off = PAGED ? ((size_t)row * kGroups + g) * kDim + 8 * col
+                                             : (size_t)b * p.kv_stride_b + (size_t)g * p.kv_stride_h +
+                                                   (size_t)(unsigned)row * stride_l + 8 * col;
+                    tb.k[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.K + off));
+                    tb.v[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.V + off));
+                }
+            };
+            auto compute = [&](int t, const Tile& tb) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    *reinterpret_cast<uint4_t*>(&kt[(4 * i + dq) * kKtStride + 8 * col]) = tb.k[i];
+                    *reinterpret_cast<uint4_t*>(&vt[(4 * i + dq) * kVtStride + 8 * col]) = tb.v[i];
+                }
+                __builtin_amdgcn_wave_barrier();   // the reads below are other lanes' writes (same wavefront: in order)
+                float4_t sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int st = 0; st < 4; ++st) {
+                    const half8_t a = *reinterpret_cast<const half8_t*>(&kt[col * kKtStride + 32 * st + 8 * dq]);
+                    sc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qb[st], sc, 0, 0, 0);
+                }
+                // sc[e] = q_col . k of row 16t + 4*dq + e
+                const int key0 = 16 * t + 4 * dq;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (key0 + e >= cn) sc[e] = -INFINITY;
+                float mx = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+                mx = fmaxf(mx, __shfl_xor(mx, 16));
+                mx = fmaxf(mx, __shfl_xor(mx, 32));
+                mx = fmaxf(mx, mcol);
+                const float mref = (mx == -INFINITY) ? 0.f : mx * kScaleLog2;
+                const float corr = fast_exp2(mcol * kScaleLog2 - mref);
+                mcol = mx;
+                float pe[4];
+                float sum = 0.f;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    pe[e] = fast_exp2(sc[e] * kScaleLog2 - mref);
+                    sum += pe[e];
+                }
+                lcol = lcol * corr + sum;
+                if (__any(corr != 1.f)) {
+#pragma unroll
+                    for (int blk = 0; blk < 8; ++blk) oacc[blk] *= corr;
+                }
+                const half4_t pb = {(half_t)pe[0], (half_t)pe[1], (half_t)pe[2], (half_t)pe[3]};
+                typedef short short4_t __attribute__((ext_vector_type(4)));
+                // lane (dq, col) points at V[row 4dq + col/4][16blk + 4(col%4), +4) and receives
+                // V[rows 4dq .. 4dq+3][16blk + col]
+                const half_t* vp = &vt[(4 * dq + (col >> 2)) * kVtStride + 4 * (col & 3)];
+#pragma unroll
+                for (int blk = 0; blk < 8; ++blk) {
+                    const short4_t raw = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (__attribute__((address_space(3))) short4_t*)(vp + 16 * blk));
+                    oacc[blk] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4_t, raw), pb, oacc[blk], 0, 0, 0);
+                }
+                __builtin_amdgcn_wave_barrier();
+            };
+            const int ntiles = (cn + 15) / 16;
+            Tile ta, tb;
+            issue(wave, ta);
+            for (int t = wave; t < ntiles; t += 8) {
+                issue(t + 4, tb);
+                KASCADE_SCHED_FENCE();
+                compute(t, ta);
+                KASCADE_SCHED_FENCE();
+                issue(t + 8, ta);
+                KASCADE_SCHED_FENCE();
+                compute(t + 4, tb);
+                KASCADE_SCHED_FENCE();
+            }
+        }
+        };
+        if (p.block_table) run(std::true_type{}); else run(std::false_type{});
+        lcol += __shfl_xor(lcol, 16);
+        lcol += __shfl_xor(lcol, 32);
+        if (col < kGroupSize) {
+            if (dq == 0) {
+                s_merge[wave].m[col] = mcol;
+                s_merge[wave].l[col] = lcol;
+            }
+#pragma unroll
+            for (int blk = 0; blk < 8; ++blk)
+                *reinterpret_cast<float4_t*>(&s_merge[wave].acc[col][16 * blk + 4 * dq]) = oacc[blk];
+        }
+    } else if constexpr (GATHER) {
         // Index list -> block table -> physical row, staged in LDS one sub-chunk at a time.
         auto run = [&](auto paged_tag) {
         for (int c0 = r0; c0 < r1; c0 += kSubChunk) {
@@ -342,16 +493,13 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
         }
         };
         if (p.block_table) run(std::true_type{}); else run(std::false_type{});
-    } else if constexpr (kMfmaScores) {
-        // Anchor pass without output: raw scores and log-sums only, so all a row needs is its dot
-        // product with the four queries.  That runs on the matrix unit (v_mfma_f32_16x16x32_f16,
-        // S^T = K Q^T with 16 keys as rows, the four heads as columns 0-3 of 16, d as the
-        // contraction index): no cross-lane reduction and ~6 vector instructions per key instead
-        // of ~80, which is what bounded the rate before.  Rows are loaded as before, 16 lanes per
-        // 256-byte row (four rows per instruction), and pass through a wavefront-private LDS tile
-        // (16 rows of 272 bytes: conflict-free both ways, no barrier) into the A-operand layout,
-        // where lane key + 16*dq holds d [32*step + 8*dq, +8) of its key for step 0..3.  Loading
-        // that layout directly makes every quarter-wavefront touch 16 rows and runs 20 % slower.
+    } else if constexpr (kDenseMfma) {
+        // Token ranges (dense baseline, anchor passes) on the matrix unit, tile for tile like the
+        // gathered rows above.  A wavefront owns 256 consecutive tokens of every 1024 (the strips
+        // whose raw scores the anchor passes park in LDS for the writer wavefront) and walks them
+        // in tiles of 16.  Without V (anchor pass that produces no output) a lane only needs the
+        // log-sum of its own keys, four tiles are in flight and nothing crosses lanes until the
+        // end; with V two tiles (K and V) are in flight.
         const int cn = r1 - r0;
         const int* bt_row = p.block_table ? p.block_table + (size_t)b * p.max_pages : nullptr;
         const int col = lane & 15, dq = lane >> 4;
@@ -363,7 +511,15 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
             if (col >= kGroupSize) t.u = uint4_t{0, 0, 0, 0};
             qb[st] = t.h8;
         }
-        float mcol = -INFINITY, lcol = 0.f;   // running max / sum of this lane's keys of its column
+        float mcol = -INFINITY, lcol = 0.f;   // running max / sum (with V: one max per column)
+        float4_t oacc[WITH_V ? 8 : 1];
+#pragma unroll
+        for (int blk = 0; blk < (WITH_V ? 8 : 1); ++blk) oacc[blk] = float4_t{0.f, 0.f, 0.f, 0.f};
+        struct Tile {
+            uint4_t k[4];
+            uint4_t v[WITH_V ? 4 : 1];
+        };
+        constexpr int kDepth = WITH_V ? 2 : 4;
         auto run = [&](auto paged_tag) {
         constexpr bool PAGED = decltype(paged_tag)::value;
         constexpr int kTilesPerStrip = kStripRows / 16;
@@ -375,20 +531,25 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
 #pragma unroll
             for (int i = 0; i < 4; ++i) pg[i] = PAGED ? bt_row[tok_of(k, i) >> p.page_shift] : 0;
         };
-        auto issue = [&](int k, const int (&pg)[4], uint4_t (&buf)[4]) {
+        auto issue = [&](int k, const int (&pg)[4], Tile& tb) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int tok = tok_of(k, i);
-                const size_t off = PAGED ? ((size_t)((pg[i] << p.page_shift) + (tok & page_mask)) * kGroups + g) * kDim
-                                         : (size_t)b * p.kv_stride_b + (size_t)g * p.kv_stride_h + (size_t)(unsigned)tok * stride_l;
-                buf[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.K + off + 8 * col));
+                const size_t off = PAGED ? ((size_t)((pg[i] << p.page_shift) + (tok & page_mask)) * kGroups + g) * kDim + 8 * col
+                                         : (size_t)b * p.kv_stride_b + (size_t)g * p.kv_stride_h +
+                                               (size_t)(unsigned)tok * stride_l + 8 * col;
+                tb.k[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.K + off));
+                if (WITH_V) tb.v[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.V + off));
             }
         };
         half_t* kt = &s_kt[wave < 4 ? wave : 0][0];
-        auto compute = [&](int k, const uint4_t (&buf)[4]) {
+        half_t* vt = &s_vt[wave < 4 ? wave : 0][0];
+        auto compute = [&](int k, const Tile& tb) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                *reinterpret_cast<uint4_t*>(&kt[(4 * i + dq) * kKtStride + 8 * col]) = buf[i];
+            for (int i = 0; i < 4; ++i) {
+                *reinterpret_cast<uint4_t*>(&kt[(4 * i + dq) * kKtStride + 8 * col]) = tb.k[i];
+                if (WITH_V) *reinterpret_cast<uint4_t*>(&vt[(4 * i + dq) * kVtStride + 8 * col]) = tb.v[i];
+            }
             __builtin_amdgcn_wave_barrier();   // the reads below are other lanes' writes (same wavefront: in order)
             float4_t sc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -396,68 +557,109 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
                 const half8_t a = *reinterpret_cast<const half8_t*>(&kt[col * kKtStride + 32 * st + 8 * dq]);
                 sc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qb[st], sc, 0, 0, 0);
             }
-            __builtin_amdgcn_wave_barrier();
             // sc[e] = q_col . k of key tile_row(k) + 4*dq + e
             const int key0 = tile_row(k) + 4 * dq;
 #pragma unroll
             for (int e = 0; e < 4; ++e)
                 if (key0 + e >= cn) sc[e] = -INFINITY;
-            if (col < kGroupSize)
-                *reinterpret_cast<float4_t*>(&s_sc[(k / kTilesPerStrip) & 1][wave][col][(k % kTilesPerStrip) * 16 + 4 * dq]) = sc;
-            const float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), mcol);
+            if (WRITE_SCORES) {
+                if (col < kGroupSize)
+                    *reinterpret_cast<float4_t*>(&s_sc[(k / kTilesPerStrip) & 1][wave][col][(k % kTilesPerStrip) * 16 + 4 * dq]) = sc;
+            }
+            float mx = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+            if (WITH_V) {   // the second product needs one reference per column
+                mx = fmaxf(mx, __shfl_xor(mx, 16));
+                mx = fmaxf(mx, __shfl_xor(mx, 32));
+            }
+            mx = fmaxf(mx, mcol);
             const float mref = (mx == -INFINITY) ? 0.f : mx * kScaleLog2;
-            float sum = lcol * fast_exp2(mcol * kScaleLog2 - mref);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) sum += fast_exp2(sc[e] * kScaleLog2 - mref);
-            lcol = sum;
+            const float corr = fast_exp2(mcol * kScaleLog2 - mref);
             mcol = mx;
+            float pe[4];
+            float sum = 0.f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                pe[e] = fast_exp2(sc[e] * kScaleLog2 - mref);
+                sum += pe[e];
+            }
+            lcol = lcol * corr + sum;
+            if (WITH_V) {
+                if (__any(corr != 1.f)) {
+#pragma unroll
+                    for (int blk = 0; blk < 8; ++blk) oacc[blk] *= corr;
+                }
+                const half4_t pb = {(half_t)pe[0], (half_t)pe[1], (half_t)pe[2], (half_t)pe[3]};
+                typedef short short4_t __attribute__((ext_vector_type(4)));
+                // lane (dq, col) points at V[row 4dq + col/4][16blk + 4(col%4), +4) and receives
+                // V[rows 4dq .. 4dq+3][16blk + col]
+                const half_t* vp = &vt[(4 * dq + (col >> 2)) * kVtStride + 4 * (col & 3)];
+#pragma unroll
+                for (int blk = 0; blk < 8; ++blk) {
+                    const short4_t raw = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (__attribute__((address_space(3))) short4_t*)(vp + 16 * blk));
+                    oacc[blk] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4_t, raw), pb, oacc[blk], 0, 0, 0);
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
         };
         if (cn > 0) {
             const int nsup = (cn + 4 * kStripRows - 1) / (4 * kStripRows);
-            if (wave == 4) {
+            if (WRITE_SCORES && wave == 4) {
                 for (int sup = 0; sup < nsup; ++sup) {
                     __syncthreads();
                     flush_scores(sup);
                 }
             } else {
-                // four tiles in flight per wavefront (16 KB); page numbers one round further ahead
+                // kDepth tiles in flight per wavefront (16 KB); page numbers one round further ahead
                 const int ntile = nsup * kTilesPerStrip;
-                uint4_t buf[4][4];
-                int pgn[4][4];
+                Tile buf[kDepth];
+                int pgn[kDepth][4];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
+                for (int j = 0; j < kDepth; ++j) {
                     fetch_pages(j, pgn[j]);
                     issue(j, pgn[j], buf[j]);
                 }
 #pragma unroll
-                for (int j = 0; j < 4; ++j) fetch_pages(4 + j, pgn[j]);
-                for (int k = 0; k < ntile; k += 4) {
+                for (int j = 0; j < kDepth; ++j) fetch_pages(kDepth + j, pgn[j]);
+                for (int k = 0; k < ntile; k += kDepth) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
+                    for (int j = 0; j < kDepth; ++j) {
                         compute(k + j, buf[j]);
                         KASCADE_SCHED_FENCE();
-                        issue(k + 4 + j, pgn[j], buf[j]);      // past the last tile: clamped rows, never used
-                        fetch_pages(k + 8 + j, pgn[j]);
+                        issue(k + kDepth + j, pgn[j], buf[j]);      // past the last tile: clamped rows, never used
+                        fetch_pages(k + 2 * kDepth + j, pgn[j]);
                         KASCADE_SCHED_FENCE();
                     }
-                    if ((k + 4) % kTilesPerStrip == 0) __syncthreads();   // a strip is complete: hand it to the writer
+                    if (WRITE_SCORES && (k + kDepth) % kTilesPerStrip == 0)
+                        __syncthreads();   // a strip is complete: hand it to the writer
                 }
             }
         }
         };
         if (bt_row) run(std::true_type{}); else run(std::false_type{});
-        // the four key subsets of a column sit in lanes col, col+16, col+32, col+48
+        if (WITH_V) {   // one reference per column: the partial sums just add
+            lcol += __shfl_xor(lcol, 16);
+            lcol += __shfl_xor(lcol, 32);
+        } else {        // the four key subsets of a column (lanes col, col+16, col+32, col+48) have their own
 #pragma unroll
-        for (int sh = 16; sh <= 32; sh <<= 1) {
-            const float mo = __shfl_xor(mcol, sh), lo = __shfl_xor(lcol, sh);
-            const float mx = fmaxf(mcol, mo);
-            const float mref = (mx == -INFINITY) ? 0.f : mx * kScaleLog2;
-            lcol = lcol * fast_exp2(mcol * kScaleLog2 - mref) + lo * fast_exp2(mo * kScaleLog2 - mref);
-            mcol = mx;
+            for (int sh = 16; sh <= 32; sh <<= 1) {
+                const float mo = __shfl_xor(mcol, sh), lo = __shfl_xor(lcol, sh);
+                const float mx = fmaxf(mcol, mo);
+                const float mref = (mx == -INFINITY) ? 0.f : mx * kScaleLog2;
+                lcol = lcol * fast_exp2(mcol * kScaleLog2 - mref) + lo * fast_exp2(mo * kScaleLog2 - mref);
+                mcol = mx;
+            }
         }
-        if (wave < 4 && lane < kGroupSize) {
-            s_merge[wave].m[lane] = mcol;
-            s_merge[wave].l[lane] = lcol;
+        if (wave < 4 && col < kGroupSize) {
+            if (dq == 0) {
+                s_merge[wave].m[col] = mcol;
+                s_merge[wave].l[col] = lcol;
+            }
+            if (WITH_V) {
+#pragma unroll
+                for (int blk = 0; blk < 8; ++blk)
+                    *reinterpret_cast<float4_t*>(&s_merge[wave].acc[col][16 * blk + 4 * dq]) = oacc[blk];
+            }
         }
     } else {
         // Dense range [r0, r1): no staging and no barriers.  Three-stage pipeline: block-table
@@ -534,7 +736,7 @@ __global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) void decod
     }
 
     // ---- merge the four row-groups of the wavefront (lanes l, l^16, l^32) ----
-    if constexpr (!kMfmaScores) {
+    if constexpr (!kDenseMfma && !kGatherMfma) {
 #pragma unroll
     for (int h = 0; h < kGroupSize; ++h) {
 #pragma unroll
