@@ -3,15 +3,18 @@
 // pooled post-softmax scores for anchor layers.
 //
 // Work decomposition (one launch = all sequences, KV heads and splits):
-//   grid  (num_split, G, B), 256 threads = 4 wavefronts.
-//   A wavefront is four row-groups of 16 lanes; lane d-slice dl = lane%16 owns
-//   halves [8*dl, 8*dl+8) of every row it touches, so one 16-byte load per lane
-//   fetches four complete 256-byte K (or V) rows per wavefront instruction.
-//   Each row-group keeps an independent online-softmax state (max, sum, 4x8
-//   output accumulators per lane); the 16 states of a workgroup are merged once
-//   at the end, the splits by the combine kernel.
-//   q.k dot products run on v_dot2_f32_f16 + a 4-step DPP row reduction; p.v on
-//   fp32 FMAs.  2 flop/byte is far below the machine balance, so no MFMA here.
+//   grid  (G, num_split, B), 256 threads = 4 streaming wavefronts (+ 1 writer
+//   wavefront in the anchor variants).  A wavefront works on tiles of 16 rows:
+//   16 lanes fetch one 256-byte row with one 16-byte load each (four rows per
+//   instruction), the tile crosses a wavefront-private piece of LDS into the
+//   operand layouts of the matrix unit, and both products of the step run there
+//   (q.k as 16 keys x 4-of-16 columns, p.v with the tile's keys contracted).
+//   The arithmetic is 2 flop/byte, far below the machine balance; the matrix
+//   unit is used because it does the dot products without cross-lane reductions,
+//   which on the vector unit cost ~110 instructions per row and capped every
+//   variant below what HBM delivers.  Every wavefront keeps one online-softmax
+//   state per query head; the four states of a workgroup are merged once at the
+//   end, the splits by the last workgroup to arrive (or the combine kernel).
 #include "decode.h"
 
 #include <type_traits>
@@ -24,19 +27,7 @@ constexpr int kThreads = 256;
 // The instruction scheduler otherwise sinks every prefetch load down to its first use (to save
 // registers), which serialises load -> wait -> use and removes all memory-level parallelism.
 #define KASCADE_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
-#ifndef KASCADE_DECODE_UNROLL
-#define KASCADE_DECODE_UNROLL 4
-#endif
-#ifndef KASCADE_GATHER_MFMA
-#define KASCADE_GATHER_MFMA 1
-#endif
-#ifndef KASCADE_DENSE_MFMA
-#define KASCADE_DENSE_MFMA 1
-#endif
-constexpr int kUnroll = KASCADE_DECODE_UNROLL;  // rows per row-group per iteration
-constexpr int kRowsPerIter = 16 * kUnroll;    // rows per workgroup iteration (128)
-constexpr int kScoreBatches = 16;             // batches between two score flushes (anchor mode)
-constexpr int kStripRows = 16 * kScoreBatches;  // rows a wavefront owns per super-iteration
+constexpr int kStripRows = 256;               // consecutive tokens a wavefront owns per 1024 (anchor strips)
 constexpr int kSubChunk = 2048;               // rows whose physical ids are staged in LDS at once
 // Raw scores travel from the anchor pass to the pooling kernel in a compact form: per head a row of
 // scores_stride floats holds, in its first half, one 16-bit code per token and, behind them, one
@@ -85,15 +76,11 @@ void decode_split_kernel(DecodeParams p) {
     __shared__ int s_found;   // gather mode: sub-chunk whose index list names the newest token
     // anchor mode: two buffers of four wavefront strips (4 heads x kStripRows raw scores)
     __shared__ __attribute__((aligned(16))) float s_sc[WRITE_SCORES ? 2 : 1][WRITE_SCORES ? 4 : 1][kGroupSize][WRITE_SCORES ? kStripRows : 4];
-    // anchor pass without output: per wavefront one tile of 16 K rows on its way into the matrix layout
-    constexpr int kKtStride = 136;   // halves per K row (128 + 8): rows 272 bytes apart
+    // per wavefront one tile of 16 K rows (and V rows) on its way into the matrix layouts
+    constexpr int kKtStride = 136;   // halves per K row (128 + 8): rows 272 bytes apart, conflict-free both ways
     constexpr int kVtStride = 144;   // halves per V row: 288 bytes, conflict-free for the transposing reads
-    constexpr bool kGatherMfma = GATHER && (KASCADE_GATHER_MFMA != 0);
-    constexpr bool kDenseMfma = !GATHER && ((!WITH_V && WRITE_SCORES) || (KASCADE_DENSE_MFMA != 0));
-    constexpr bool kTiles = kDenseMfma || kGatherMfma;
-    constexpr bool kTilesV = kTiles && WITH_V;
-    __shared__ __attribute__((aligned(16))) half_t s_kt[kTiles ? 4 : 1][kTiles ? 16 * kKtStride : 8];
-    __shared__ __attribute__((aligned(16))) half_t s_vt[kTilesV ? 4 : 1][kTilesV ? 16 * kVtStride : 8];
+    __shared__ __attribute__((aligned(16))) half_t s_kt[4][16 * kKtStride];
+    __shared__ __attribute__((aligned(16))) half_t s_vt[WITH_V ? 4 : 1][WITH_V ? 16 * kVtStride : 8];
 
     const int g = blockIdx.x;       // the 8 KV heads of one token range are adjacent in dispatch order
     const int split = blockIdx.y;
@@ -101,8 +88,6 @@ void decode_split_kernel(DecodeParams p) {
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
     const int lane = tid & 63;
-    const int rg = lane >> 4;   // row group within the wavefront
-    const int dl = lane & 15;   // 16-byte slice of the 256-byte row
 
     int seqlen = p.seqlens ? p.seqlens[b] : p.kv_stride_tokens;
     // a length beyond what the block table covers must not index past the table
@@ -160,117 +145,125 @@ void decode_split_kernel(DecodeParams p) {
     }
     if (GATHER && tid == 0) s_found = -1;
 
-    // q fragments: 4 heads x 8 halves of this lane's d-slice
-    Pack16 qf[kGroupSize];
+    // ---- tiles of 16 rows on the matrix unit ----
+    // Lane roles.  Loading: lane (dq, col) = (lane / 16, lane % 16) takes the 16-byte chunk `col`
+    // of rows 4i + dq of a tile, i = 0..3, so 16 lanes fetch one 256-byte row and an instruction
+    // four rows.  Computing: the same lane is key `col` / part dq of the A operand of
+    // S^T = K Q^T (v_mfma_f32_16x16x32_f16: 16 keys x 16 columns, d contracted 32 at a time; the
+    // four query heads are columns 0-3, the rest zero) and ends up with S^T[4dq .. 4dq+3][col]:
+    // exactly the B-operand layout of O^T += V^T P^T (v_mfma_f32_16x16x16_f16, the tile's 16 keys
+    // contracted), whose A operand V^T is read out of the row-major V tile by the transposing LDS
+    // read.  The tiles pass through wavefront-private LDS (no workgroup barrier).  Nothing here is
+    // a cross-lane reduction: ~10 vector instructions per row, where dot products on the vector
+    // unit needed ~110 and bounded every variant of this kernel.
+    const int col = lane & 15, dq = lane >> 4;
+    half8_t qb[4];   // B operand of the first product: Q[col][32*st + 8*dq, +8)
 #pragma unroll
-    for (int h = 0; h < kGroupSize; ++h)
-        qf[h].u = ld_global_16(p.Q + ((size_t)b * kHeads + g * kGroupSize + h) * kDim + dl * 8);
-
-    float m[kGroupSize], l[kGroupSize], acc[kGroupSize][8];
-#pragma unroll
-    for (int h = 0; h < kGroupSize; ++h) {
-        m[h] = -INFINITY;
-        l[h] = 0.f;
-#pragma unroll
-        for (int d = 0; d < 8; ++d) acc[h][d] = 0.f;
+    for (int st = 0; st < 4; ++st) {
+        Pack16 t;
+        t.u = ld_global_16(p.Q + ((size_t)b * kHeads + g * kGroupSize + (col & 3)) * kDim + 32 * st + 8 * dq);
+        if (col >= kGroupSize) t.u = uint4_t{0, 0, 0, 0};
+        qb[st] = t.h8;
     }
+    // Online softmax state of this lane's column.  With V one running maximum per column (the
+    // second product needs a common reference: two cross-lane exchanges per tile); without V
+    // every lane keeps the maximum and sum of its own keys and the four parts meet at the end.
+    float mcol = -INFINITY, lcol = 0.f;
+    float4_t oacc[WITH_V ? 8 : 1];   // O^T[16*blk + 4*dq + r][col]
+#pragma unroll
+    for (int blk = 0; blk < (WITH_V ? 8 : 1); ++blk) oacc[blk] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     const int* idx_row = nullptr;
     if (GATHER) idx_row = p.idx + ((size_t)b * kGroups + p.head_map[g]) * p.topk;
     const int page_mask = (1 << p.page_shift) - 1;
-    // Element offset of (token row r, this head, this lane's slice): paged rows are physical rows
-    // of [P*page,G,D]; without a table rows are token numbers of sequence b behind the caller's
-    // (batch, token, head) strides, so a head-major cache is read in place.
-    const size_t head_off = (size_t)g * kDim + dl * 8;
-    const size_t strided_off = (size_t)b * p.kv_stride_b + (size_t)g * p.kv_stride_h + dl * 8;
     const unsigned stride_l = p.kv_stride_l;
+    half_t* kt = &s_kt[wave & 3][0];
+    half_t* vt = &s_vt[wave & 3][0];
 
-    struct Batch {
-        Pack16 k[kUnroll];
-        Pack16 v[kUnroll];
+    struct Tile {
+        uint4_t k[4];
+        uint4_t v[WITH_V ? 4 : 1];
     };
-    // A wavefront covers 4*kUnroll consecutive rows of an iteration: row = it + wave*4U + u*4 + rg.
-    // `rows` are physical row numbers (page*page_size + slot, or b*stride + token).
-    auto issue_loads = [&](auto paged_tag, const int (&rows)[kUnroll], Batch& bt) {
+    // `row`: physical row (page * page_size + slot) behind a block table; otherwise the token
+    // number of sequence b behind the caller's (batch, token, head) strides, so that a head-major
+    // cache is read in place.  Every K/V row is read once per launch: non-temporal loads keep
+    // the stream from displacing what the launch does want cached (index lists, block table,
+    // the raw scores of an anchor pass).
+    auto load_row = [&](auto paged_tag, int row, Tile& tb, int i) {
         constexpr bool PAGED = decltype(paged_tag)::value;
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            const size_t off = PAGED ? (size_t)rows[u] * (kGroups * kDim) + head_off
-                                     : (size_t)(unsigned)rows[u] * stride_l + strided_off;
-            // every K/V row is read once per launch: non-temporal loads keep the stream from
-            // displacing what the launch does want cached (index lists, block table, the raw
-            // scores an anchor pass writes for the kernels that follow) -- measured -12 % on the
-            // gather, -7 % on the anchor passes
-            bt.k[u].u = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.K + off));
-            if (WITH_V) bt.v[u].u = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.V + off));
-        }
+        const size_t off = PAGED ? ((size_t)row * kGroups + g) * kDim + 8 * col
+                                 : (size_t)b * p.kv_stride_b + (size_t)g * p.kv_stride_h +
+                                       (size_t)(unsigned)row * stride_l + 8 * col;
+        tb.k[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.K + off));
+        if (WITH_V) tb.v[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.V + off));
     };
-    // Straight-line on purpose (no early exit, loads never skipped): a branch between issuing
-    // a batch and consuming it makes the compiler wait for every outstanding load.
-    // rbase: first row (relative to c0) of this lane's row-group in the batch, rows rbase + 4u.
-    auto compute_batch = [&](int rbase, int cn, int c0, int phase, int buf, const Batch& bt) {
-        float s[kUnroll][kGroupSize];
+    // One tile: `key0` is the position of this lane's first key within the range, `cn` the number
+    // of rows of the range (keys at or beyond it are masked); anchor passes park the raw scores of
+    // the four heads at `stage` (this lane's four keys).
+    // Straight-line on purpose (no early exit): a branch between issuing a tile's loads and
+    // consuming them makes the compiler wait for every load in flight.
+    auto compute_tile = [&](const Tile& tb, int key0, int cn, float* stage) {
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            const bool valid = (rbase + u * 4) < cn;
-#pragma unroll
-            for (int h = 0; h < kGroupSize; ++h) {
-                float d = dot8(bt.k[u], qf[h], 0.f);
-                d = row16_sum(d);
-                s[u][h] = valid ? d : -INFINITY;
-            }
+        for (int i = 0; i < 4; ++i) {
+            *reinterpret_cast<uint4_t*>(&kt[(4 * i + dq) * kKtStride + 8 * col]) = tb.k[i];
+            if (WITH_V) *reinterpret_cast<uint4_t*>(&vt[(4 * i + dq) * kVtStride + 8 * col]) = tb.v[i];
         }
+        __builtin_amdgcn_wave_barrier();   // the reads below are other lanes' writes (same wavefront: in order)
+        float4_t sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+            const half8_t a = *reinterpret_cast<const half8_t*>(&kt[col * kKtStride + 32 * st + 8 * dq]);
+            sc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qb[st], sc, 0, 0, 0);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (key0 + e >= cn) sc[e] = -INFINITY;
         if (WRITE_SCORES) {
-            // Raw scores are parked in LDS strips (per wavefront: 4 heads x kStripRows tokens)
-            // and written to HBM by a fifth wavefront that streams nothing.  A store issued by
-            // a streaming wavefront costs it dearly: loads and stores complete in order on one
-            // counter, so every younger K/V load is held back until the store is acknowledged.
-            static_assert(!WRITE_SCORES || kUnroll == 4, "score staging assumes 4 rows per row-group");
-            const int usel = dl & 3, hsel = dl >> 2;
-            float w[kGroupSize];
-#pragma unroll
-            for (int h = 0; h < kGroupSize; ++h) {
-                w[h] = s[0][h];
-#pragma unroll
-                for (int u = 1; u < kUnroll; ++u) w[h] = (usel == u) ? s[u][h] : w[h];
-            }
-            float val = w[0];
-#pragma unroll
-            for (int h = 1; h < kGroupSize; ++h) val = (hsel == h) ? w[h] : val;
-            s_sc[buf][wave][hsel][phase * 16 + usel * 4 + rg] = val;
+            if (col < kGroupSize) *reinterpret_cast<float4_t*>(stage) = sc;
         }
+        float mx = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+        if (WITH_V) {
+            mx = fmaxf(mx, __shfl_xor(mx, 16));
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+        }
+        mx = fmaxf(mx, mcol);
+        const float mref = (mx == -INFINITY) ? 0.f : mx * kScaleLog2;
+        const float corr = fast_exp2(mcol * kScaleLog2 - mref);   // mcol = -inf -> 0
+        mcol = mx;
+        float pe[4];
+        float sum = 0.f;
 #pragma unroll
-        for (int h = 0; h < kGroupSize; ++h) {
-            float mx = m[h];
+        for (int e = 0; e < 4; ++e) {
+            pe[e] = fast_exp2(sc[e] * kScaleLog2 - mref);
+            sum += pe[e];
+        }
+        lcol = lcol * corr + sum;
+        if (WITH_V) {
+            if (__any(corr != 1.f)) {   // wavefront-uniform: skip when no maximum moved
 #pragma unroll
-            for (int u = 0; u < kUnroll; ++u) mx = fmaxf(mx, s[u][h]);
-            const float mref = (mx == -INFINITY) ? 0.f : mx * kScaleLog2;
-            const float corr = fast_exp2(m[h] * kScaleLog2 - mref);  // m=-inf -> 0
-            m[h] = mx;
-            float ps[kUnroll];
-            float sum = 0.f;
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
-                ps[u] = fast_exp2(s[u][h] * kScaleLog2 - mref);
-                sum += ps[u];
+                for (int blk = 0; blk < 8; ++blk) oacc[blk] *= corr;
             }
-            l[h] = l[h] * corr + sum;
-            if (WITH_V) {
+            const half4_t pb = {(half_t)pe[0], (half_t)pe[1], (half_t)pe[2], (half_t)pe[3]};
+            typedef short short4_t __attribute__((ext_vector_type(4)));
+            // ds_read_b64_tr_b16: lane (dq, col) points at V[row 4dq + col/4][16blk + 4(col%4), +4)
+            // and receives V[rows 4dq .. 4dq+3][16blk + col]
+            const half_t* vp = &vt[(4 * dq + (col >> 2)) * kVtStride + 4 * (col & 3)];
 #pragma unroll
-                for (int d = 0; d < 8; ++d) {
-                    float a = acc[h][d] * corr;
-#pragma unroll
-                    for (int u = 0; u < kUnroll; ++u) a = fmaf(ps[u], (float)bt.v[u].h[d], a);
-                    acc[h][d] = a;
-                }
+            for (int blk = 0; blk < 8; ++blk) {
+                const short4_t raw = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (__attribute__((address_space(3))) short4_t*)(vp + 16 * blk));
+                oacc[blk] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4_t, raw), pb, oacc[blk], 0, 0, 0);
             }
         }
+        __builtin_amdgcn_wave_barrier();
     };
 
     // Writer wavefront of the anchor passes: stores the four strips of super-iteration `sup`
     // (buffer sup & 1) in the compact score format (see kScoreSteps): per instruction one
     // (strip, head) row of 256 tokens, 16 lanes per granule of 64 tokens, four tokens per lane;
-    // 128 contiguous bytes per granule plus its reference value.
+    // 128 contiguous bytes per granule plus its reference value.  A store issued by a streaming
+    // wavefront would cost it dearly: loads and stores complete in order on one counter, so
+    // every younger K/V load would be held back until the store is acknowledged.
     auto flush_scores = [&](int sup) {
         const int cn = r1 - r0;
         constexpr int kVecPerStrip = kGroupSize * kStripRows / 4;   // float4 per strip
@@ -305,35 +298,10 @@ void decode_split_kernel(DecodeParams p) {
         }
     };
 
-    if constexpr (kGatherMfma) {
-        // Gathered rows on the matrix unit.  Tiles of 16 rows per wavefront: rows are loaded as
-        // 16 lanes x 16 bytes each (four rows per instruction, K and V), pass through
-        // wavefront-private LDS tiles, and S^T = K Q^T (16 keys x 4 of 16 columns, contraction
-        // over d, v_mfma_f32_16x16x32_f16) leaves every lane with four keys of one column: the
-        // B-operand layout of O^T += V^T P^T (v_mfma_f32_16x16x16_f16, contraction over the 16
-        // keys), whose A operand comes out of the row-major V tile through the transposing LDS
-        // read.  One running maximum per column (two cross-lane exchanges per tile); ~10 vector
-        // instructions per row instead of ~110.
-        const int col = lane & 15, dq = lane >> 4;
-        half8_t qb[4];
-#pragma unroll
-        for (int st = 0; st < 4; ++st) {
-            Pack16 t;
-            t.u = ld_global_16(p.Q + ((size_t)b * kHeads + g * kGroupSize + (col & 3)) * kDim + 32 * st + 8 * dq);
-            if (col >= kGroupSize) t.u = uint4_t{0, 0, 0, 0};
-            qb[st] = t.h8;
-        }
-        float mcol = -INFINITY, lcol = 0.f;
-        float4_t oacc[8];
-#pragma unroll
-        for (int blk = 0; blk < 8; ++blk) oacc[blk] = float4_t{0.f, 0.f, 0.f, 0.f};
-        half_t* kt = &s_kt[wave][0];
-        half_t* vt = &s_vt[wave][0];
-        struct Tile {
-            uint4_t k[4], v[4];
-        };
+    if constexpr (GATHER) {
+        // Index list -> block table -> physical row, staged in LDS one sub-chunk at a time; the
+        // wavefronts take the sub-chunk's tiles in turn, two tiles (16 KB) in flight each.
         auto run = [&](auto paged_tag) {
-        constexpr bool PAGED = decltype(paged_tag)::value;
         for (int c0 = r0; c0 < r1; c0 += kSubChunk) {
             const int cn = min(kSubChunk, r1 - c0);
             __syncthreads();
@@ -355,178 +323,42 @@ void decode_split_kernel(DecodeParams p) {
                 write_newest();
                 __syncthreads();
             }
-            // tile t: rows [16t, 16t+16) of the sub-chunk; lane (dq, col) loads chunk col of rows 4i + dq
-            auto issue = [&](int t, Tile& tb) {
+            auto issue = [&](int t, Tile& tb) {   // tile t: rows [16t, 16t+16) of the sub-chunk
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int row = s_row[min(16 * t + 4 * i + dq, cn - 1)];   // past the end: clamped, masked later
-                    const size_t off = PAGED ? ((size_t)row * kGroups + g) * kDim + 8 * col
-                                             : (size_t)b * p.kv_stride_b + (size_t)g * p.kv_stride_h +
-                                                   (size_t)(unsigned)row * stride_l + 8 * col;
-                    tb.k[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.K + off));
-                    tb.v[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.V + off));
-                }
+                for (int i = 0; i < 4; ++i)      // past the end: clamped, masked later
+                    load_row(paged_tag, s_row[min(16 * t + 4 * i + dq, cn - 1)], tb, i);
             };
-            auto compute = [&](int t, const Tile& tb) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    *reinterpret_cast<uint4_t*>(&kt[(4 * i + dq) * kKtStride + 8 * col]) = tb.k[i];
-                    *reinterpret_cast<uint4_t*>(&vt[(4 * i + dq) * kVtStride + 8 * col]) = tb.v[i];
-                }
-                __builtin_amdgcn_wave_barrier();   // the reads below are other lanes' writes (same wavefront: in order)
-                float4_t sc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int st = 0; st < 4; ++st) {
-                    const half8_t a = *reinterpret_cast<const half8_t*>(&kt[col * kKtStride + 32 * st + 8 * dq]);
-                    sc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qb[st], sc, 0, 0, 0);
-                }
-                // sc[e] = q_col . k of row 16t + 4*dq + e
-                const int key0 = 16 * t + 4 * dq;
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (key0 + e >= cn) sc[e] = -INFINITY;
-                float mx = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
-                mx = fmaxf(mx, __shfl_xor(mx, 16));
-                mx = fmaxf(mx, __shfl_xor(mx, 32));
-                mx = fmaxf(mx, mcol);
-                const float mref = (mx == -INFINITY) ? 0.f : mx * kScaleLog2;
-                const float corr = fast_exp2(mcol * kScaleLog2 - mref);
-                mcol = mx;
-                float pe[4];
-                float sum = 0.f;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    pe[e] = fast_exp2(sc[e] * kScaleLog2 - mref);
-                    sum += pe[e];
-                }
-                lcol = lcol * corr + sum;
-                if (__any(corr != 1.f)) {
-#pragma unroll
-                    for (int blk = 0; blk < 8; ++blk) oacc[blk] *= corr;
-                }
-                const half4_t pb = {(half_t)pe[0], (half_t)pe[1], (half_t)pe[2], (half_t)pe[3]};
-                typedef short short4_t __attribute__((ext_vector_type(4)));
-                // lane (dq, col) points at V[row 4dq + col/4][16blk + 4(col%4), +4) and receives
-                // V[rows 4dq .. 4dq+3][16blk + col]
-                const half_t* vp = &vt[(4 * dq + (col >> 2)) * kVtStride + 4 * (col & 3)];
-#pragma unroll
-                for (int blk = 0; blk < 8; ++blk) {
-                    const short4_t raw = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (__attribute__((address_space(3))) short4_t*)(vp + 16 * blk));
-                    oacc[blk] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4_t, raw), pb, oacc[blk], 0, 0, 0);
-                }
-                __builtin_amdgcn_wave_barrier();
-            };
-            const int ntiles = (cn + 15) / 16;
             Tile ta, tb;
             issue(wave, ta);
+            const int ntiles = (cn + 15) / 16;
             for (int t = wave; t < ntiles; t += 8) {
                 issue(t + 4, tb);
-                KASCADE_SCHED_FENCE();
-                compute(t, ta);
+                KASCADE_SCHED_FENCE();   // the scheduler otherwise sinks the loads down to their first use
+                compute_tile(ta, 16 * t + 4 * dq, cn, nullptr);
                 KASCADE_SCHED_FENCE();
                 issue(t + 8, ta);
                 KASCADE_SCHED_FENCE();
-                compute(t + 4, tb);
+                compute_tile(tb, 16 * (t + 4) + 4 * dq, cn, nullptr);
                 KASCADE_SCHED_FENCE();
             }
         }
         };
         if (p.block_table) run(std::true_type{}); else run(std::false_type{});
-        lcol += __shfl_xor(lcol, 16);
-        lcol += __shfl_xor(lcol, 32);
-        if (col < kGroupSize) {
-            if (dq == 0) {
-                s_merge[wave].m[col] = mcol;
-                s_merge[wave].l[col] = lcol;
-            }
-#pragma unroll
-            for (int blk = 0; blk < 8; ++blk)
-                *reinterpret_cast<float4_t*>(&s_merge[wave].acc[col][16 * blk + 4 * dq]) = oacc[blk];
-        }
-    } else if constexpr (GATHER) {
-        // Index list -> block table -> physical row, staged in LDS one sub-chunk at a time.
-        auto run = [&](auto paged_tag) {
-        for (int c0 = r0; c0 < r1; c0 += kSubChunk) {
-            const int cn = min(kSubChunk, r1 - c0);
-            __syncthreads();
-            for (int i = tid; i < cn; i += kThreads) {
-                int tok = idx_row[c0 + i];
-                tok = max(0, min(tok, seqlen - 1));   // a corrupt index must not leave the sequence
-                if (tok == newest) s_found = c0;
-                int row;
-                if (p.block_table) {
-                    int pg = p.block_table[(size_t)b * p.max_pages + (tok >> p.page_shift)];
-                    row = (pg << p.page_shift) + (tok & page_mask);
-                } else {
-                    row = tok;
-                }
-                s_row[i] = row;
-            }
-            __syncthreads();
-            if (p.k_new != nullptr && s_found == c0) {   // c0 differs per sub-chunk: no reset needed
-                write_newest();
-                __syncthreads();
-            }
-            auto staged_rows = [&](int it, int (&rows)[kUnroll]) {
-                const int rbase = it + wave * (4 * kUnroll) + rg;
-#pragma unroll
-                for (int u = 0; u < kUnroll; ++u) rows[u] = s_row[min(rbase + u * 4, cn - 1)];
-            };
-            // software pipeline: the loads of iteration i+1 are in flight while iteration i computes
-            Batch ba, bb;
-            int rows[kUnroll];
-            staged_rows(0, rows);
-            issue_loads(paged_tag, rows, ba);
-            for (int it = 0; it < cn; it += 2 * kRowsPerIter) {
-                staged_rows(it + kRowsPerIter, rows);      // rows past the end are clamped and masked
-                issue_loads(paged_tag, rows, bb);
-                KASCADE_SCHED_FENCE();
-                compute_batch(it + wave * (4 * kUnroll) + rg, cn, c0, 0, 0, ba);
-                KASCADE_SCHED_FENCE();
-                staged_rows(it + 2 * kRowsPerIter, rows);
-                issue_loads(paged_tag, rows, ba);
-                KASCADE_SCHED_FENCE();
-                compute_batch(it + kRowsPerIter + wave * (4 * kUnroll) + rg, cn, c0, 0, 0, bb);
-                KASCADE_SCHED_FENCE();
-            }
-        }
-        };
-        if (p.block_table) run(std::true_type{}); else run(std::false_type{});
-    } else if constexpr (kDenseMfma) {
-        // Token ranges (dense baseline, anchor passes) on the matrix unit, tile for tile like the
-        // gathered rows above.  A wavefront owns 256 consecutive tokens of every 1024 (the strips
-        // whose raw scores the anchor passes park in LDS for the writer wavefront) and walks them
-        // in tiles of 16.  Without V (anchor pass that produces no output) a lane only needs the
-        // log-sum of its own keys, four tiles are in flight and nothing crosses lanes until the
-        // end; with V two tiles (K and V) are in flight.
+    } else {
+        // Token range [r0, r1) (dense baseline, anchor passes): no staging.  A wavefront owns 256
+        // consecutive tokens of every 1024 -- the strips whose raw scores the anchor passes park
+        // in LDS for the writer wavefront, one barrier per 1024 tokens -- and walks them in tiles
+        // of 16: 16 KB in flight per wavefront (two tiles of K and V, or four of K alone), block
+        // table entries one round further ahead so that no row address waits for its page number.
         const int cn = r1 - r0;
         const int* bt_row = p.block_table ? p.block_table + (size_t)b * p.max_pages : nullptr;
-        const int col = lane & 15, dq = lane >> 4;
-        half8_t qb[4];
-#pragma unroll
-        for (int st = 0; st < 4; ++st) {
-            Pack16 t;
-            t.u = ld_global_16(p.Q + ((size_t)b * kHeads + g * kGroupSize + (col & 3)) * kDim + 32 * st + 8 * dq);
-            if (col >= kGroupSize) t.u = uint4_t{0, 0, 0, 0};
-            qb[st] = t.h8;
-        }
-        float mcol = -INFINITY, lcol = 0.f;   // running max / sum (with V: one max per column)
-        float4_t oacc[WITH_V ? 8 : 1];
-#pragma unroll
-        for (int blk = 0; blk < (WITH_V ? 8 : 1); ++blk) oacc[blk] = float4_t{0.f, 0.f, 0.f, 0.f};
-        struct Tile {
-            uint4_t k[4];
-            uint4_t v[WITH_V ? 4 : 1];
-        };
         constexpr int kDepth = WITH_V ? 2 : 4;
+        constexpr int kTilesPerStrip = kStripRows / 16;
         auto run = [&](auto paged_tag) {
         constexpr bool PAGED = decltype(paged_tag)::value;
-        constexpr int kTilesPerStrip = kStripRows / 16;
         // tile k of this wavefront: 16 keys from row (k / 16) * 1024 + wave * 256 + (k % 16) * 16
         auto tile_row = [&](int k) { return (k / kTilesPerStrip) * (4 * kStripRows) + wave * kStripRows + (k % kTilesPerStrip) * 16; };
-        // loads: lane (dq, col) takes chunk col of rows 4i + dq of the tile; past the end: clamped, masked later
-        auto tok_of = [&](int k, int i) { return min(r0 + tile_row(k) + 4 * i + dq, r1 - 1); };
+        auto tok_of = [&](int k, int i) { return min(r0 + tile_row(k) + 4 * i + dq, r1 - 1); };   // past the end: clamped, masked later
         auto fetch_pages = [&](int k, int (&pg)[4]) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) pg[i] = PAGED ? bt_row[tok_of(k, i) >> p.page_shift] : 0;
@@ -535,83 +367,18 @@ void decode_split_kernel(DecodeParams p) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int tok = tok_of(k, i);
-                const size_t off = PAGED ? ((size_t)((pg[i] << p.page_shift) + (tok & page_mask)) * kGroups + g) * kDim + 8 * col
-                                         : (size_t)b * p.kv_stride_b + (size_t)g * p.kv_stride_h +
-                                               (size_t)(unsigned)tok * stride_l + 8 * col;
-                tb.k[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.K + off));
-                if (WITH_V) tb.v[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.V + off));
+                load_row(paged_tag, PAGED ? (pg[i] << p.page_shift) + (tok & page_mask) : tok, tb, i);
             }
-        };
-        half_t* kt = &s_kt[wave < 4 ? wave : 0][0];
-        half_t* vt = &s_vt[wave < 4 ? wave : 0][0];
-        auto compute = [&](int k, const Tile& tb) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                *reinterpret_cast<uint4_t*>(&kt[(4 * i + dq) * kKtStride + 8 * col]) = tb.k[i];
-                if (WITH_V) *reinterpret_cast<uint4_t*>(&vt[(4 * i + dq) * kVtStride + 8 * col]) = tb.v[i];
-            }
-            __builtin_amdgcn_wave_barrier();   // the reads below are other lanes' writes (same wavefront: in order)
-            float4_t sc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int st = 0; st < 4; ++st) {
-                const half8_t a = *reinterpret_cast<const half8_t*>(&kt[col * kKtStride + 32 * st + 8 * dq]);
-                sc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qb[st], sc, 0, 0, 0);
-            }
-            // sc[e] = q_col . k of key tile_row(k) + 4*dq + e
-            const int key0 = tile_row(k) + 4 * dq;
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (key0 + e >= cn) sc[e] = -INFINITY;
-            if (WRITE_SCORES) {
-                if (col < kGroupSize)
-                    *reinterpret_cast<float4_t*>(&s_sc[(k / kTilesPerStrip) & 1][wave][col][(k % kTilesPerStrip) * 16 + 4 * dq]) = sc;
-            }
-            float mx = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
-            if (WITH_V) {   // the second product needs one reference per column
-                mx = fmaxf(mx, __shfl_xor(mx, 16));
-                mx = fmaxf(mx, __shfl_xor(mx, 32));
-            }
-            mx = fmaxf(mx, mcol);
-            const float mref = (mx == -INFINITY) ? 0.f : mx * kScaleLog2;
-            const float corr = fast_exp2(mcol * kScaleLog2 - mref);
-            mcol = mx;
-            float pe[4];
-            float sum = 0.f;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                pe[e] = fast_exp2(sc[e] * kScaleLog2 - mref);
-                sum += pe[e];
-            }
-            lcol = lcol * corr + sum;
-            if (WITH_V) {
-                if (__any(corr != 1.f)) {
-#pragma unroll
-                    for (int blk = 0; blk < 8; ++blk) oacc[blk] *= corr;
-                }
-                const half4_t pb = {(half_t)pe[0], (half_t)pe[1], (half_t)pe[2], (half_t)pe[3]};
-                typedef short short4_t __attribute__((ext_vector_type(4)));
-                // lane (dq, col) points at V[row 4dq + col/4][16blk + 4(col%4), +4) and receives
-                // V[rows 4dq .. 4dq+3][16blk + col]
-                const half_t* vp = &vt[(4 * dq + (col >> 2)) * kVtStride + 4 * (col & 3)];
-#pragma unroll
-                for (int blk = 0; blk < 8; ++blk) {
-                    const short4_t raw = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (__attribute__((address_space(3))) short4_t*)(vp + 16 * blk));
-                    oacc[blk] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4_t, raw), pb, oacc[blk], 0, 0, 0);
-                }
-            }
-            __builtin_amdgcn_wave_barrier();
         };
         if (cn > 0) {
             const int nsup = (cn + 4 * kStripRows - 1) / (4 * kStripRows);
             if (WRITE_SCORES && wave == 4) {
-                for (int sup = 0; sup < nsup; ++sup) {
+                for (int sup = 0; sup < nsup; ++sup) {   // one barrier per strip, matched below
                     __syncthreads();
                     flush_scores(sup);
                 }
             } else {
-                // kDepth tiles in flight per wavefront (16 KB); page numbers one round further ahead
-                const int ntile = nsup * kTilesPerStrip;
+                const int ntile = nsup * kTilesPerStrip;   // the same for every wavefront
                 Tile buf[kDepth];
                 int pgn[kDepth][4];
 #pragma unroll
@@ -624,7 +391,10 @@ void decode_split_kernel(DecodeParams p) {
                 for (int k = 0; k < ntile; k += kDepth) {
 #pragma unroll
                     for (int j = 0; j < kDepth; ++j) {
-                        compute(k + j, buf[j]);
+                        compute_tile(buf[j], tile_row(k + j) + 4 * dq, cn,
+                                     WRITE_SCORES ? &s_sc[((k + j) / kTilesPerStrip) & 1][wave & 3][col & 3]
+                                                         [((k + j) % kTilesPerStrip) * 16 + 4 * dq]
+                                                  : nullptr);
                         KASCADE_SCHED_FENCE();
                         issue(k + kDepth + j, pgn[j], buf[j]);      // past the last tile: clamped rows, never used
                         fetch_pages(k + 2 * kDepth + j, pgn[j]);
@@ -637,140 +407,32 @@ void decode_split_kernel(DecodeParams p) {
         }
         };
         if (bt_row) run(std::true_type{}); else run(std::false_type{});
-        if (WITH_V) {   // one reference per column: the partial sums just add
-            lcol += __shfl_xor(lcol, 16);
-            lcol += __shfl_xor(lcol, 32);
-        } else {        // the four key subsets of a column (lanes col, col+16, col+32, col+48) have their own
-#pragma unroll
-            for (int sh = 16; sh <= 32; sh <<= 1) {
-                const float mo = __shfl_xor(mcol, sh), lo = __shfl_xor(lcol, sh);
-                const float mx = fmaxf(mcol, mo);
-                const float mref = (mx == -INFINITY) ? 0.f : mx * kScaleLog2;
-                lcol = lcol * fast_exp2(mcol * kScaleLog2 - mref) + lo * fast_exp2(mo * kScaleLog2 - mref);
-                mcol = mx;
-            }
-        }
-        if (wave < 4 && col < kGroupSize) {
-            if (dq == 0) {
-                s_merge[wave].m[col] = mcol;
-                s_merge[wave].l[col] = lcol;
-            }
-            if (WITH_V) {
-#pragma unroll
-                for (int blk = 0; blk < 8; ++blk)
-                    *reinterpret_cast<float4_t*>(&s_merge[wave].acc[col][16 * blk + 4 * dq]) = oacc[blk];
-            }
-        }
-    } else {
-        // Dense range [r0, r1): no staging and no barriers.  Three-stage pipeline: block-table
-        // entries two iterations ahead, K/V rows one iteration ahead, arithmetic on the current.
-        const int cn = r1 - r0;
-        const int* bt_row = p.block_table ? p.block_table + (size_t)b * p.max_pages : nullptr;
-        // A wavefront owns kStripRows consecutive rows of every super-iteration of
-        // 4*kStripRows rows and walks them in kScoreBatches batches of 16 (batch number
-        // q = it / kRowsPerIter, phase q % kScoreBatches).
-        auto rbase_of = [&](int it) {
-            const int q = it / kRowsPerIter;
-            return (q / kScoreBatches) * (4 * kStripRows) + wave * kStripRows + (q % kScoreBatches) * 16 + rg;
-        };
-        auto tok_of = [&](int it, int u) { return min(r0 + rbase_of(it) + u * 4, r1 - 1); };
-        // The paged / contiguous choice is hoisted out of the loop as a compile-time tag: a
-        // per-load "table ? table[i] : 0" turns into a branch whose join waits for every load
-        // in flight.
-        auto run = [&](auto paged_tag) {
-        constexpr bool PAGED = decltype(paged_tag)::value;
-        auto fetch_pages = [&](int it, int (&pg)[kUnroll]) {
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u) pg[u] = PAGED ? bt_row[tok_of(it, u) >> p.page_shift] : 0;
-        };
-        auto rows_of = [&](int it, const int (&pg)[kUnroll], int (&rows)[kUnroll]) {
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
-                const int tok = tok_of(it, u);
-                rows[u] = PAGED ? (pg[u] << p.page_shift) + (tok & page_mask) : tok;
-            }
-        };
-        if (cn > 0) {
-            // Block-table entries are fetched *before* the K/V loads of the preceding batch in
-            // program order: loads complete in order, so waiting for a younger table entry would
-            // otherwise drain the K/V loads in flight.
-            Batch ba, bb;
-            int pga[kUnroll], pgb[kUnroll], rows[kUnroll];
-            fetch_pages(0, pga);
-            rows_of(0, pga, rows);
-            issue_loads(paged_tag, rows, ba);
-            fetch_pages(kRowsPerIter, pgb);
-            // every wavefront runs the same number of batches: enough for the longest strip
-            const int full = cn / (4 * kStripRows), rem = cn - full * (4 * kStripRows);
-            const int nbatch = full * kScoreBatches + min(kScoreBatches, (rem + 15) / 16);
-            const int it_end = ((nbatch + 1) & ~1) * kRowsPerIter;   // the loop body handles two batches
-            if (WRITE_SCORES && wave == 4) {
-                // one barrier per super-iteration, matched by the streaming wavefronts below
-                const int nsup = (it_end / kRowsPerIter + kScoreBatches - 1) / kScoreBatches;
-                for (int sup = 0; sup < nsup; ++sup) {
-                    __syncthreads();
-                    flush_scores(sup);
-                }
-            } else {
-            for (int it = 0; it < it_end; it += 2 * kRowsPerIter) {
-                const int q = it / kRowsPerIter;
-                fetch_pages(it + 2 * kRowsPerIter, pga);   // tokens past the end are clamped and masked
-                rows_of(it + kRowsPerIter, pgb, rows);
-                issue_loads(paged_tag, rows, bb);
-                KASCADE_SCHED_FENCE();
-                compute_batch(rbase_of(it), cn, r0, q % kScoreBatches, (q / kScoreBatches) & 1, ba);
-                KASCADE_SCHED_FENCE();
-                fetch_pages(it + 3 * kRowsPerIter, pgb);
-                rows_of(it + 2 * kRowsPerIter, pga, rows);
-                issue_loads(paged_tag, rows, ba);
-                KASCADE_SCHED_FENCE();
-                compute_batch(rbase_of(it + kRowsPerIter), cn, r0, (q + 1) % kScoreBatches, (q / kScoreBatches) & 1, bb);
-                KASCADE_SCHED_FENCE();
-                if (WRITE_SCORES && ((q + 2) % kScoreBatches == 0 || it + 2 * kRowsPerIter >= it_end))
-                    __syncthreads();   // strips of this super-iteration are complete: hand them to the writer
-            }
-            }
-        }
-        };
-        if (bt_row) run(std::true_type{}); else run(std::false_type{});
     }
 
-    // ---- merge the four row-groups of the wavefront (lanes l, l^16, l^32) ----
-    if constexpr (!kDenseMfma && !kGatherMfma) {
-#pragma unroll
-    for (int h = 0; h < kGroupSize; ++h) {
+    // ---- the wavefront's state: columns 0-3, the four parts of a column in lanes col + 16*dq ----
+    if (WITH_V) {   // one reference per column: the partial sums just add
+        lcol += __shfl_xor(lcol, 16);
+        lcol += __shfl_xor(lcol, 32);
+    } else {
 #pragma unroll
         for (int sh = 16; sh <= 32; sh <<= 1) {
-            float mo = __shfl_xor(m[h], sh);
-            float lo = __shfl_xor(l[h], sh);
-            float mx = fmaxf(m[h], mo);
-            float mref = (mx == -INFINITY) ? 0.f : mx * kScaleLog2;
-            float ca = fast_exp2(m[h] * kScaleLog2 - mref);
-            float cb = fast_exp2(mo * kScaleLog2 - mref);
-            l[h] = l[h] * ca + lo * cb;
-            if (WITH_V) {
-#pragma unroll
-                for (int d = 0; d < 8; ++d) {
-                    float ao = __shfl_xor(acc[h][d], sh);
-                    acc[h][d] = acc[h][d] * ca + ao * cb;
-                }
-            }
-            m[h] = mx;
+            const float mo = __shfl_xor(mcol, sh), lo = __shfl_xor(lcol, sh);
+            const float mx = fmaxf(mcol, mo);
+            const float mref = (mx == -INFINITY) ? 0.f : mx * kScaleLog2;
+            lcol = lcol * fast_exp2(mcol * kScaleLog2 - mref) + lo * fast_exp2(mo * kScaleLog2 - mref);
+            mcol = mx;
         }
     }
-    if (rg == 0 && wave < 4) {   // the writer wavefront of the anchor variants holds no state
-#pragma unroll
-        for (int h = 0; h < kGroupSize; ++h) {
-            if (dl == 0) {
-                s_merge[wave].m[h] = m[h];
-                s_merge[wave].l[h] = l[h];
-            }
-            if (WITH_V) {
-#pragma unroll
-                for (int d = 0; d < 8; ++d) s_merge[wave].acc[h][dl * 8 + d] = acc[h][d];
-            }
+    if (wave < 4 && col < kGroupSize) {   // the writer wavefront of the anchor variants holds no state
+        if (dq == 0) {
+            s_merge[wave].m[col] = mcol;
+            s_merge[wave].l[col] = lcol;
         }
-    }
+        if (WITH_V) {
+#pragma unroll
+            for (int blk = 0; blk < 8; ++blk)
+                *reinterpret_cast<float4_t*>(&s_merge[wave].acc[col][16 * blk + 4 * dq]) = oacc[blk];
+        }
     }
     __syncthreads();
     // ---- merge the four wavefronts; thread -> (head, two d's) ----
