@@ -235,8 +235,9 @@ def decode_recompute(Q, K, V, glse, Output_partial, row_sums, scores, layer: int
                      sync=None, k_new=None, v_new=None) -> Tuple[Optional[torch.Tensor], torch.Tensor]:
     """``decode_recomp{0,1}_kernel(Q, K, V, glse, Output_partial, row_sums, scores) -> (O, agg)``
     (out_idx=[7,8]; EfficientKascadeStrategy.py:24-28, 107-110) and its kvcache form
-    (recompute_kascade_gqa_decode_with_kvcache.py:302-333).  ``scores`` is fp32 scratch
-    [B,H,stride]; agg is [B,G,stride] fp16.  layer == 0 also computes the dense output;
+    (recompute_kascade_gqa_decode_with_kvcache.py:302-333).  ``scores`` is scratch of
+    [B,H,stride] fp32 elements whose contents are private to the library (the raw scores travel
+    in a compact form); agg is [B,G,stride] fp16.  layer == 0 also computes the dense output;
     otherwise O is None."""
     lib = _lib.init()
     B = Q.shape[0]
