@@ -68,14 +68,27 @@ struct alignas(16) MergeState {  // one per wavefront after the in-wave merge
 };
 
 template <bool GATHER, bool WITH_V, bool WRITE_SCORES>
-__global__ __launch_bounds__(WRITE_SCORES ? kThreads + 64 : kThreads) __attribute__((amdgpu_waves_per_eu(3)))
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2)))
 void decode_split_kernel(DecodeParams p) {
     __shared__ int s_row[GATHER ? kSubChunk : 1];
-    __shared__ MergeState s_merge[4];
     __shared__ int s_last;
     __shared__ int s_found;   // gather mode: sub-chunk whose index list names the newest token
-    // anchor mode: two buffers of four wavefront strips (4 heads x kStripRows raw scores)
-    __shared__ __attribute__((aligned(16))) float s_sc[WRITE_SCORES ? 2 : 1][WRITE_SCORES ? 4 : 1][kGroupSize][WRITE_SCORES ? kStripRows : 4];
+    // anchor mode: the compact raw scores of kCodePhase * 1024 tokens (see kScoreSteps), written to
+    // HBM in one burst per phase; they share their LDS with the merge state, which is only needed
+    // after the last burst
+    constexpr int kCodePhase = WITH_V ? 5 : 7;             // what fits beside two workgroups' tiles
+    constexpr int kPhaseRows = WRITE_SCORES ? kCodePhase * 4 * kStripRows : 64;
+    union Shared {
+        MergeState merge[4];
+        struct {
+            uint16_t code[kGroupSize][kPhaseRows];
+            float ref[kGroupSize][kPhaseRows / 64];
+        } sc;
+    };
+    __shared__ __attribute__((aligned(16))) Shared s_u;
+    MergeState* s_merge = s_u.merge;
+    auto& s_code = s_u.sc.code;
+    auto& s_ref = s_u.sc.ref;
     // per wavefront one tile of 16 K rows (and V rows) on its way into the matrix layouts
     constexpr int kKtStride = 136;   // halves per K row (128 + 8): rows 272 bytes apart, conflict-free both ways
     constexpr int kVtStride = 144;   // halves per V row: 288 bytes, conflict-free for the transposing reads
@@ -177,8 +190,8 @@ void decode_split_kernel(DecodeParams p) {
     if (GATHER) idx_row = p.idx + ((size_t)b * kGroups + p.head_map[g]) * p.topk;
     const int page_mask = (1 << p.page_shift) - 1;
     const unsigned stride_l = p.kv_stride_l;
-    half_t* kt = &s_kt[wave & 3][0];
-    half_t* vt = &s_vt[wave & 3][0];
+    half_t* kt = &s_kt[wave][0];
+    half_t* vt = &s_vt[wave][0];
 
     struct Tile {
         uint4_t k[4];
@@ -198,11 +211,10 @@ void decode_split_kernel(DecodeParams p) {
         if (WITH_V) tb.v[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.V + off));
     };
     // One tile: `key0` is the position of this lane's first key within the range, `cn` the number
-    // of rows of the range (keys at or beyond it are masked); anchor passes park the raw scores of
-    // the four heads at `stage` (this lane's four keys).
+    // of rows of the range (keys at or beyond it are masked).  Returns this lane's four raw scores.
     // Straight-line on purpose (no early exit): a branch between issuing a tile's loads and
     // consuming them makes the compiler wait for every load in flight.
-    auto compute_tile = [&](const Tile& tb, int key0, int cn, float* stage) {
+    auto compute_tile = [&](const Tile& tb, int key0, int cn) -> float4_t {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             *reinterpret_cast<uint4_t*>(&kt[(4 * i + dq) * kKtStride + 8 * col]) = tb.k[i];
@@ -218,9 +230,6 @@ void decode_split_kernel(DecodeParams p) {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
             if (key0 + e >= cn) sc[e] = -INFINITY;
-        if (WRITE_SCORES) {
-            if (col < kGroupSize) *reinterpret_cast<float4_t*>(stage) = sc;
-        }
         float mx = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
         if (WITH_V) {
             mx = fmaxf(mx, __shfl_xor(mx, 16));
@@ -256,46 +265,61 @@ void decode_split_kernel(DecodeParams p) {
             }
         }
         __builtin_amdgcn_wave_barrier();
+        return sc;
     };
 
-    // Writer wavefront of the anchor passes: stores the four strips of super-iteration `sup`
-    // (buffer sup & 1) in the compact score format (see kScoreSteps): per instruction one
-    // (strip, head) row of 256 tokens, 16 lanes per granule of 64 tokens, four tokens per lane;
-    // 128 contiguous bytes per granule plus its reference value.  A store issued by a streaming
-    // wavefront would cost it dearly: loads and stores complete in order on one counter, so
-    // every younger K/V load would be held back until the store is acknowledged.
-    auto flush_scores = [&](int sup) {
-        const int cn = r1 - r0;
-        constexpr int kVecPerStrip = kGroupSize * kStripRows / 4;   // float4 per strip
-#pragma unroll 4
-        for (int i = 0; i < 4 * kVecPerStrip / 64; ++i) {
-            const int idx = i * 64 + lane;
-            const int w = idx / kVecPerStrip, rem = idx % kVecPerStrip;
-            const int h = rem / (kStripRows / 4), t4 = (rem % (kStripRows / 4)) * 4;
-            float4_t v = *reinterpret_cast<const float4_t*>(&s_sc[sup & 1][w][h][t4]);
-            const int r = sup * (4 * kStripRows) + w * kStripRows + t4;
+    // Anchor passes: a granule's raw scores (four consecutive tiles of this wavefront, 64 tokens at
+    // position `prow` of the phase buffer) become 16-bit codes below the granule's maximum.
+    auto encode_granule = [&](const float4_t (&sc)[4], int prow) {
+        float mx = -INFINITY;
 #pragma unroll
-            for (int e = 0; e < 4; ++e)      // strip positions past the range were never filled
-                v[e] = (r + e < cn) ? v[e] : -INFINITY;
-            const float mx = row16_max(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])));
-            const float base = (mx == -INFINITY) ? 0.f : mx;
-            uint32_t q[4];
+        for (int j = 0; j < 4; ++j) mx = fmaxf(mx, fmaxf(fmaxf(sc[j][0], sc[j][1]), fmaxf(sc[j][2], sc[j][3])));
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float base = (mx == -INFINITY) ? 0.f : mx;
+        if (col < kGroupSize) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float d = (base - v[e]) * (kScaleLog2 * kScoreSteps);      // >= 0, +inf if masked
-                q[e] = (v[e] == -INFINITY) ? kScoreNone : (uint32_t)fminf(rintf(d), (float)(kScoreNone - 1));
+            for (int j = 0; j < 4; ++j) {
+                uint32_t q[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float d = (base - sc[j][e]) * (kScaleLog2 * kScoreSteps);      // >= 0, +inf if masked
+                    q[e] = (sc[j][e] == -INFINITY) ? kScoreNone : (uint32_t)fminf(rintf(d), (float)(kScoreNone - 1));
+                }
+                *reinterpret_cast<uint2*>(&s_code[col][prow + 16 * j + 4 * dq]) =
+                    make_uint2(q[0] | (q[1] << 16), q[2] | (q[3] << 16));
             }
-            float* row = p.scores + ((size_t)b * kHeads + g * kGroupSize + h) * p.scores_stride;
-            uint16_t* dst = reinterpret_cast<uint16_t*>(row) + r0 + r;
-            if (r + 3 < cn) {
-                *reinterpret_cast<uint2*>(dst) = make_uint2(q[0] | (q[1] << 16), q[2] | (q[3] << 16));
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (r + e < cn) dst[e] = (uint16_t)q[e];
-            }
-            if ((lane & 15) == 0 && r < cn) row[p.scores_stride / 2 + ((r0 + r) >> 6)] = base * kScaleLog2;
+            if (dq == 0) s_ref[col][prow >> 6] = base * kScaleLog2;
         }
+    };
+    // The codes of phase `ph` (tokens [ph * kPhaseRows, +kPhaseRows) of the range) leave in one
+    // burst from all threads.  Score stores trickling out while K streams cost the stream far
+    // more than their bytes (HBM turning between reads and writes); workgroups of one launch run
+    // in step, so their bursts coincide and the device alternates between long read and short
+    // write phases.  The streaming wavefronts issue these stores themselves -- loads and stores
+    // retire in order on one counter, so the next tiles wait for them -- once per phase.
+    auto flush_phase = [&](int ph) {
+        const int cn = r1 - r0;
+        const int lo = ph * kPhaseRows;
+        const int nrows = min(kPhaseRows, cn - lo);
+        __syncthreads();
+        if (nrows > 0) {
+#pragma unroll
+            for (int h = 0; h < kGroupSize; ++h) {
+                float* row = p.scores + ((size_t)b * kHeads + g * kGroupSize + h) * p.scores_stride;
+                uint16_t* dst = reinterpret_cast<uint16_t*>(row) + r0 + lo;
+                for (int i = tid * 8; i < nrows; i += kThreads * 8) {
+                    if (i + 8 <= nrows) {
+                        *reinterpret_cast<uint4_t*>(dst + i) = *reinterpret_cast<const uint4_t*>(&s_code[h][i]);
+                    } else {
+                        for (int e = 0; i + e < nrows; ++e) dst[i + e] = s_code[h][i + e];
+                    }
+                }
+                for (int i = tid; i < (nrows + 63) / 64; i += kThreads)
+                    row[p.scores_stride / 2 + ((r0 + lo) >> 6) + i] = s_ref[h][i];
+            }
+        }
+        __syncthreads();
     };
 
     if constexpr (GATHER) {
@@ -334,11 +358,11 @@ void decode_split_kernel(DecodeParams p) {
             for (int t = wave; t < ntiles; t += 8) {
                 issue(t + 4, tb);
                 KASCADE_SCHED_FENCE();   // the scheduler otherwise sinks the loads down to their first use
-                compute_tile(ta, 16 * t + 4 * dq, cn, nullptr);
+                compute_tile(ta, 16 * t + 4 * dq, cn);
                 KASCADE_SCHED_FENCE();
                 issue(t + 8, ta);
                 KASCADE_SCHED_FENCE();
-                compute_tile(tb, 16 * (t + 4) + 4 * dq, cn, nullptr);
+                compute_tile(tb, 16 * (t + 4) + 4 * dq, cn);
                 KASCADE_SCHED_FENCE();
             }
         }
@@ -372,38 +396,34 @@ void decode_split_kernel(DecodeParams p) {
         };
         if (cn > 0) {
             const int nsup = (cn + 4 * kStripRows - 1) / (4 * kStripRows);
-            if (WRITE_SCORES && wave == 4) {
-                for (int sup = 0; sup < nsup; ++sup) {   // one barrier per strip, matched below
-                    __syncthreads();
-                    flush_scores(sup);
+            const int ntile = nsup * kTilesPerStrip;   // the same for every wavefront
+            Tile buf[kDepth];
+            int pgn[kDepth][4];
+#pragma unroll
+            for (int j = 0; j < kDepth; ++j) {
+                fetch_pages(j, pgn[j]);
+                issue(j, pgn[j], buf[j]);
+            }
+#pragma unroll
+            for (int j = 0; j < kDepth; ++j) fetch_pages(kDepth + j, pgn[j]);
+            for (int k = 0; k < ntile; k += 4) {   // four consecutive tiles: one granule of 64 tokens
+                float4_t sc[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int jb = j % kDepth;
+                    sc[j] = compute_tile(buf[jb], tile_row(k + j) + 4 * dq, cn);
+                    KASCADE_SCHED_FENCE();
+                    issue(k + kDepth + j, pgn[jb], buf[jb]);      // past the last tile: clamped rows, never used
+                    fetch_pages(k + 2 * kDepth + j, pgn[jb]);
+                    KASCADE_SCHED_FENCE();
                 }
-            } else {
-                const int ntile = nsup * kTilesPerStrip;   // the same for every wavefront
-                Tile buf[kDepth];
-                int pgn[kDepth][4];
-#pragma unroll
-                for (int j = 0; j < kDepth; ++j) {
-                    fetch_pages(j, pgn[j]);
-                    issue(j, pgn[j], buf[j]);
-                }
-#pragma unroll
-                for (int j = 0; j < kDepth; ++j) fetch_pages(kDepth + j, pgn[j]);
-                for (int k = 0; k < ntile; k += kDepth) {
-#pragma unroll
-                    for (int j = 0; j < kDepth; ++j) {
-                        compute_tile(buf[j], tile_row(k + j) + 4 * dq, cn,
-                                     WRITE_SCORES ? &s_sc[((k + j) / kTilesPerStrip) & 1][wave & 3][col & 3]
-                                                         [((k + j) % kTilesPerStrip) * 16 + 4 * dq]
-                                                  : nullptr);
-                        KASCADE_SCHED_FENCE();
-                        issue(k + kDepth + j, pgn[j], buf[j]);      // past the last tile: clamped rows, never used
-                        fetch_pages(k + 2 * kDepth + j, pgn[j]);
-                        KASCADE_SCHED_FENCE();
-                    }
-                    if (WRITE_SCORES && (k + kDepth) % kTilesPerStrip == 0)
-                        __syncthreads();   // a strip is complete: hand it to the writer
+                if (WRITE_SCORES) {
+                    const int sup = k / kTilesPerStrip;
+                    encode_granule(sc, (sup % kCodePhase) * (4 * kStripRows) + wave * kStripRows + (k % kTilesPerStrip) * 16);
+                    if ((k + 4) % (kTilesPerStrip * kCodePhase) == 0) flush_phase(sup / kCodePhase);
                 }
             }
+            if (WRITE_SCORES && nsup % kCodePhase != 0) flush_phase(nsup / kCodePhase);
         }
         };
         if (bt_row) run(std::true_type{}); else run(std::false_type{});
@@ -423,7 +443,7 @@ void decode_split_kernel(DecodeParams p) {
             mcol = mx;
         }
     }
-    if (wave < 4 && col < kGroupSize) {   // the writer wavefront of the anchor variants holds no state
+    if (col < kGroupSize) {
         if (dq == 0) {
             s_merge[wave].m[col] = mcol;
             s_merge[wave].l[col] = lcol;
@@ -687,7 +707,7 @@ __global__ __launch_bounds__(256) void decode_aggregate_kernel(const float* __re
 
 hipError_t launch_decode_split(const DecodeParams& p, bool gather, bool with_v, bool write_scores,
                                hipStream_t stream) {
-    dim3 grid(kGroups, p.num_split, p.B), block(write_scores ? kThreads + 64 : kThreads);
+    dim3 grid(kGroups, p.num_split, p.B), block(kThreads);
     if (gather) {
         hipLaunchKernelGGL((decode_split_kernel<true, true, false>), grid, block, 0, stream, p);
     } else if (write_scores) {
