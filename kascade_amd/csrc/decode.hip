@@ -3,8 +3,8 @@
 // pooled post-softmax scores for anchor layers.
 //
 // Work decomposition (one launch = all sequences, KV heads and splits):
-//   grid  (G, num_split, B), 256 threads = 4 streaming wavefronts (+ 1 writer
-//   wavefront in the anchor variants).  A wavefront works on tiles of 16 rows:
+//   grid  (G, num_split, B), 256 threads = 4 wavefronts.  A wavefront works on
+//   tiles of 16 rows:
 //   16 lanes fetch one 256-byte row with one 16-byte load each (four rows per
 //   instruction), the tile crosses a wavefront-private piece of LDS into the
 //   operand layouts of the matrix unit, and both products of the step run there
@@ -27,7 +27,7 @@ constexpr int kThreads = 256;
 // The instruction scheduler otherwise sinks every prefetch load down to its first use (to save
 // registers), which serialises load -> wait -> use and removes all memory-level parallelism.
 #define KASCADE_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
-constexpr int kStripRows = 256;               // consecutive tokens a wavefront owns per 1024 (anchor strips)
+constexpr int kStripRows = 256;               // consecutive tokens a wavefront owns per 1024
 constexpr int kSubChunk = 2048;               // rows whose physical ids are staged in LDS at once
 // Raw scores travel from the anchor pass to the pooling kernel in a compact form: per head a row of
 // scores_stride floats holds, in its first half, one 16-bit code per token and, behind them, one
@@ -370,10 +370,10 @@ void decode_split_kernel(DecodeParams p) {
         if (p.block_table) run(std::true_type{}); else run(std::false_type{});
     } else {
         // Token range [r0, r1) (dense baseline, anchor passes): no staging.  A wavefront owns 256
-        // consecutive tokens of every 1024 -- the strips whose raw scores the anchor passes park
-        // in LDS for the writer wavefront, one barrier per 1024 tokens -- and walks them in tiles
-        // of 16: 16 KB in flight per wavefront (two tiles of K and V, or four of K alone), block
-        // table entries one round further ahead so that no row address waits for its page number.
+        // consecutive tokens of every 1024 and walks them in tiles of 16, four consecutive tiles
+        // (one 64-token granule of the score codes) per loop iteration: 16 KB in flight per
+        // wavefront (two tiles of K and V, or four of K alone), block table entries one round
+        // further ahead so that no row address waits for its page number.
         const int cn = r1 - r0;
         const int* bt_row = p.block_table ? p.block_table + (size_t)b * p.max_pages : nullptr;
         constexpr int kDepth = WITH_V ? 2 : 4;
