@@ -59,9 +59,10 @@ def default_num_split(total_rows: int, max_rows: int, wgs_per_cu: int = 2, min_r
     total_rows / rows_per_split; aim at wgs_per_cu of them per compute unit without
     dropping below min_rows rows per workgroup (per-workgroup set-up is not free).
     total_rows = sum over (sequence, KV head) of the rows visited; max_rows = longest list.
-    cap_rows: upper limit on the rows of a split.  The gather kernel is fastest at about
-    GATHER_ROWS_PER_SPLIT rows per workgroup whatever the total (batch 16 x 13184 rows: 159 us at
-    1648 rows per workgroup against 179 us at 3296); the streaming kernels do not care."""
+    cap_rows: upper limit on the rows of a split.  Gather launches keep a split at about
+    GATHER_ROWS_PER_SPLIT rows: twice that is 1-3 % faster on uniform batches (batch 16 x 26240
+    rows: 307 us against 316 us) but 6 % slower on the ragged batch of four long sequences
+    (109 us against 103 us); the streaming kernels do not care."""
     cus = _lib.init().kascade_device_cu_count() or 256
     target_wgs = wgs_per_cu * cus
     rows_per_split = max(min_rows, total_rows / target_wgs)
