@@ -134,6 +134,36 @@ def test_decode_recompute_paged(cuda, seqlens, layer):
         assert_close(o2, want2, "anchor decode sparse output (own indices)")
 
 
+@pytest.mark.parametrize("layer", [0, 1])
+@pytest.mark.parametrize("seqlens,ns", [([23011], 1), ([9000, 17500], 2)])
+def test_decode_recompute_long_ranges(cuda, seqlens, ns, layer):
+    """One workgroup streams more tokens than its score buffer holds (several store bursts per
+    workgroup, the last one partial), ranges end inside a tile and inside a 64-token granule."""
+    from kascade_amd import kernels
+    w = _paged_case(seqlens, seed=31 + layer)
+    B, Lmax = len(seqlens), max(seqlens)
+    kc = orc.paged_to_contiguous(w.k_pages, w.block_table, seqlens)
+    vc = orc.paged_to_contiguous(w.v_pages, w.block_table, seqlens)
+    o_want, _, agg_want = orc.anchor_decode(w.q, kc, vc, 10, layer == 0, seqlens)
+    glse, part = _scratch(B, ns, cuda)
+    row_sums = torch.empty(B, H, device=cuda, dtype=torch.float32)
+    stride = ((Lmax + 7) // 8) * 8
+    scores = torch.full((B, H, stride), float("nan"), device=cuda, dtype=torch.float32)
+    o, agg = kernels.decode_recompute(w.q.to(cuda), w.k_pages.to(cuda), w.v_pages.to(cuda), glse, part,
+                                      row_sums, scores, layer, cache_seqlens=w.seqlens.to(cuda),
+                                      block_table=w.block_table.to(cuda), page_size=w.page_size)
+    torch.cuda.synchronize()
+    agg_c = agg.cpu()[:, :, :Lmax]
+    assert torch.isfinite(agg_c).all()
+    assert_close(agg_c, agg_want, "agg", atol=2e-6, rtol=2e-3)
+    for b, n in enumerate(seqlens):
+        assert float(agg_c[b, :, n:].abs().max()) == 0.0 if n < Lmax else True
+    _, lse = orc.dense_decode(w.q, kc, vc, seqlens)
+    assert_close(row_sums, lse * orc.LOG2E, "row_sums", atol=2e-3, rtol=1e-4)
+    if layer == 0:
+        assert_close(o, o_want, "anchor-0 decode output")
+
+
 def test_decode_reuse_paged_ragged_head_mapping(cuda):
     """Reuse layer on a ragged paged batch through a random head map, indices from the oracle anchor."""
     from kascade_amd import kernels
