@@ -326,22 +326,36 @@ void decode_split_kernel(DecodeParams p) {
         // Index list -> block table -> physical row, staged in LDS one sub-chunk at a time; the
         // wavefronts take the sub-chunk's tiles in turn, two tiles (16 KB) in flight each.
         auto run = [&](auto paged_tag) {
+        constexpr bool PAGED = decltype(paged_tag)::value;
         for (int c0 = r0; c0 < r1; c0 += kSubChunk) {
             const int cn = min(kSubChunk, r1 - c0);
             __syncthreads();
-            for (int i = tid; i < cn; i += kThreads) {
-                int tok = idx_row[c0 + i];
-                tok = max(0, min(tok, seqlen - 1));   // a corrupt index must not leave the sequence
-                if (tok == newest) s_found = c0;
-                int row;
-                if (p.block_table) {
-                    int pg = p.block_table[(size_t)b * p.max_pages + (tok >> p.page_shift)];
-                    row = (pg << p.page_shift) + (tok & page_mask);
-                } else {
-                    row = tok;
+            // all of a thread's index loads first, then all of its block-table loads: two trips to
+            // memory per sub-chunk instead of two per entry (the count per thread is a compile-time
+            // constant per case, so that short lists do not pay for eight loads)
+            auto stage = [&](auto per_tag) {
+                constexpr int kPer = decltype(per_tag)::value;
+                int toks[kPer], rows[kPer];
+#pragma unroll
+                for (int j = 0; j < kPer; ++j) toks[j] = idx_row[c0 + min(tid + j * kThreads, cn - 1)];
+#pragma unroll
+                for (int j = 0; j < kPer; ++j) {
+                    toks[j] = max(0, min(toks[j], seqlen - 1));   // a corrupt index must not leave the sequence
+                    rows[j] = PAGED ? p.block_table[(size_t)b * p.max_pages + (toks[j] >> p.page_shift)] : toks[j];
                 }
-                s_row[i] = row;
-            }
+#pragma unroll
+                for (int j = 0; j < kPer; ++j) {
+                    const int i = tid + j * kThreads;
+                    if (i < cn) {
+                        if (toks[j] == newest) s_found = c0;
+                        s_row[i] = PAGED ? (rows[j] << p.page_shift) + (toks[j] & page_mask) : rows[j];
+                    }
+                }
+            };
+            if (cn <= kThreads) stage(std::integral_constant<int, 1>{});
+            else if (cn <= 2 * kThreads) stage(std::integral_constant<int, 2>{});
+            else if (cn <= 4 * kThreads) stage(std::integral_constant<int, 4>{});
+            else stage(std::integral_constant<int, kSubChunk / kThreads>{});
             __syncthreads();
             if (p.k_new != nullptr && s_found == c0) {   // c0 differs per sub-chunk: no reset needed
                 write_newest();
