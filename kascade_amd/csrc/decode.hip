@@ -72,6 +72,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2)))
 void decode_split_kernel(DecodeParams p) {
     __shared__ int s_row[GATHER ? kSubChunk : 1];
     __shared__ int s_last;
+    __shared__ int s_map[3];
     __shared__ int s_found;   // gather mode: sub-chunk whose index list names the newest token
     // anchor mode: the compact raw scores of kCodePhase * 1024 tokens (see kScoreSteps), written to
     // HBM in one burst per phase; they share their LDS with the merge state, which is only needed
@@ -96,29 +97,71 @@ void decode_split_kernel(DecodeParams p) {
     __shared__ __attribute__((aligned(16))) half_t s_vt[WITH_V ? 4 : 1][WITH_V ? 16 * kVtStride : 8];
 
     const int g = blockIdx.x;       // the 8 KV heads of one token range are adjacent in dispatch order
-    const int split = blockIdx.y;
-    const int b = blockIdx.z;
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
     const int lane = tid & 63;
 
-    int seqlen = p.seqlens ? p.seqlens[b] : p.kv_stride_tokens;
-    // a length beyond what the block table covers must not index past the table
-    if (p.block_table) seqlen = min(seqlen, p.max_pages << p.page_shift);
-    seqlen = max(seqlen, 0);
-    int n;  // rows this (b, g) pair attends to
-    if (GATHER) {
+    // rows a (sequence, KV head) pair of length `len` attends to
+    auto rows_for = [&](int len) {
+        // a length beyond what the block table covers must not index past the table
+        if (p.block_table) len = min(len, p.max_pages << p.page_shift);
+        len = max(len, 0);
+        if (!GATHER) return len;
+        int n;
         if (p.topk_percent > 0.f) {
-            long long fl = (long long)floor((double)p.topk_percent * (double)seqlen / 100.0);
+            long long fl = (long long)floor((double)p.topk_percent * (double)len / 100.0);
             n = (int)(((fl + 127) / 128) * 128);
         } else {
             n = p.topk;
         }
         n = min(n, p.topk);
-        if (p.seqlens) n = min(n, seqlen);   // never more rows than the sequence holds
+        if (p.seqlens) n = min(n, len);   // never more rows than the sequence holds
+        return n;
+    };
+    // Which (sequence, split) this workgroup takes.  With per-sequence lengths the non-empty
+    // splits of all sequences are numbered consecutively (sequence-major; at least one split per
+    // sequence) and workgroup w of the launch takes number w: the workgroups left over -- a
+    // ragged batch has many -- come last in dispatch order and exit at once, instead of being
+    // scattered among the working ones, which left some compute units with several streams and
+    // others with none (four sequences of 131072..524288 tokens, 512 working workgroups: gather
+    // 101 -> 86 us).  One sequence needs none of this (and a decode step of a short one is all
+    // latency: the extra barrier would show).
+    int b, split, nsplit_b;
+    if (p.seqlens != nullptr && p.B > 1 && p.B <= 64) {
+        const int w = blockIdx.y + gridDim.y * blockIdx.z;
+        if (tid == 0) s_map[0] = -1;
+        if (wave == 0) {
+            int cnt = 0;
+            if (lane < p.B)
+                cnt = max(1, (rows_for(p.seqlens[lane]) + p.rows_per_split - 1) / p.rows_per_split);
+            int incl = cnt;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const int t = __shfl_up(incl, o);
+                if (lane >= o) incl += t;
+            }
+            const int excl = incl - cnt;
+            if (lane < p.B && w >= excl && w < incl) {
+                s_map[0] = lane;
+                s_map[1] = w - excl;
+                s_map[2] = cnt;
+            }
+        }
+        __syncthreads();
+        b = s_map[0];
+        if (b < 0) return;
+        split = s_map[1];
+        nsplit_b = s_map[2];
     } else {
-        n = seqlen;
+        b = blockIdx.z;
+        split = blockIdx.y;
+        nsplit_b = p.num_split;
     }
+
+    int seqlen = p.seqlens ? p.seqlens[b] : p.kv_stride_tokens;
+    if (p.block_table) seqlen = min(seqlen, p.max_pages << p.page_shift);
+    seqlen = max(seqlen, 0);
+    const int n = rows_for(seqlen);  // rows this (b, g) pair attends to
     // contiguous range of this split; every split covers rows_per_split rows, sequences
     // shorter than num_split*rows_per_split leave their last splits empty
     const long long r0l = (long long)split * p.rows_per_split;
@@ -499,6 +542,13 @@ void decode_split_kernel(DecodeParams p) {
             if (WITH_V) store_device2(p.opart + ph * kDim + d0, o0 * inv, o1 * inv);
         }
     }
+    // splits that no workgroup takes (sequences shorter than the longest) count as empty for
+    // the kernels that merge all num_split partial log-sums
+    if (split == 0) {
+        const int missing = p.num_split - nsplit_b;
+        for (int i = tid; i < kGroupSize * missing; i += kThreads)
+            p.glse[((size_t)b * kHeads + g * kGroupSize + i / missing) * p.num_split + nsplit_b + i % missing] = -INFINITY;
+    }
     // ---- fused combine: the last workgroup of (b, g) to arrive merges the splits ----
     // The partial results above are written through to device-coherent memory and the barrier
     // waits for those stores before thread 0 counts this workgroup in; the merging workgroup
@@ -509,7 +559,7 @@ void decode_split_kernel(DecodeParams p) {
     if (tid == 0) {
         const int arrived = __hip_atomic_fetch_add(&p.counters[b * kGroups + g], 1, __ATOMIC_RELAXED,
                                                    __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (arrived == p.num_split - 1);
+        s_last = (arrived == nsplit_b - 1);
     }
     __syncthreads();
     if (!s_last) return;
@@ -518,8 +568,8 @@ void decode_split_kernel(DecodeParams p) {
     if (tid < kThreads) {
         // wavefront -> head; lanes over the splits for the reductions, then two d's per lane
         const int head = g * kGroupSize + wave;
-        const int ns = p.num_split;
-        const size_t base = ((size_t)b * kHeads + head) * ns;
+        const int ns = nsplit_b;   // the splits of this sequence that exist
+        const size_t base = ((size_t)b * kHeads + head) * p.num_split;
         const float* gl = p.glse + base;
         const float* op = p.opart + base * kDim + lane * 2;
         // the first partial outputs are requested together with the log-sums, so that short

@@ -53,7 +53,7 @@ GATHER_ROWS_PER_SPLIT = 1664
 
 
 def default_num_split(total_rows: int, max_rows: int, wgs_per_cu: int = 2, min_rows: int = 512,
-                      cap_rows: Optional[int] = None) -> int:
+                      cap_rows: Optional[int] = None, row_counts=None, heads: int = G) -> int:
     """Split count for a decode launch.  Every split covers the same number of rows
     (ceil(max_rows/num_split)), so the number of non-empty workgroups is about
     total_rows / rows_per_split; aim at wgs_per_cu of them per compute unit without
@@ -62,9 +62,30 @@ def default_num_split(total_rows: int, max_rows: int, wgs_per_cu: int = 2, min_r
     cap_rows: upper limit on the rows of a split.  Gather launches keep a split at about
     GATHER_ROWS_PER_SPLIT rows: twice that is 1-3 % faster on uniform batches (batch 16 x 26240
     rows: 307 us against 316 us) but 6 % slower on the ragged batch of four long sequences
-    (109 us against 103 us); the streaming kernels do not care."""
+    (109 us against 103 us); the streaming kernels do not care.
+    row_counts: the rows of every sequence (per KV head), when the caller knows them."""
     cus = _lib.init().kascade_device_cu_count() or 256
     target_wgs = wgs_per_cu * cus
+    if row_counts is not None and len(row_counts) > 1 and total_rows / max(min_rows, 1) >= cus:
+        # Ragged batch with known lengths: count the workgroups exactly.  Each sequence rounds its
+        # split count up, and a few workgroups beyond what is resident at once run when almost
+        # everything else has finished, far below the device's bandwidth (four sequences of
+        # 131072..524288 tokens, 10 % gathered: 86 us with 512 workgroups, 100 us with 544).  So
+        # take the largest split count whose workgroups still fit `rounds` residencies, more
+        # than one only when a split would otherwise exceed about 4096 rows.
+        def count(ns):
+            rps = ((-(-max_rows // ns) + 63) // 64) * 64
+            return heads * sum(max(1, -(-int(n) // rps)) for n in row_counts), rps
+        rounds = 1
+        while True:
+            best = 1
+            for ns in range(1, 257):
+                wgs, rps = count(ns)
+                if wgs <= rounds * target_wgs and rps >= min(min_rows, max_rows):
+                    best = ns
+            if not cap_rows or count(best)[1] <= 4096 or rounds >= 8:
+                return best
+            rounds += 1
     rows_per_split = max(min_rows, total_rows / target_wgs)
     if cap_rows:
         rows_per_split = min(rows_per_split, cap_rows)

@@ -213,11 +213,14 @@ class PagedKascadeDecoder:
     def __init__(self, k: float, head_mapping: List[List[int]], recompute_layers: Sequence[int],
                  max_batch: int, max_seqlen: int, page_size: int = 16, device="cuda",
                  num_split_dense: Optional[int] = None, num_split_reuse: Optional[int] = None,
-                 total_tokens: Optional[int] = None, fused_combine: bool = True):
+                 total_tokens: Optional[int] = None, fused_combine: bool = True,
+                 seqlens_hint: Optional[Sequence[int]] = None):
         """fused_combine: merge the splits inside the split launch (one launch fewer per layer).
         total_tokens: expected sum of the sequence lengths of a batch (default
         max_batch*max_seqlen); with ragged batches it sizes the splits so that the non-empty
-        workgroups, not the grid, cover the device about twice."""
+        workgroups, not the grid, cover the device about twice.
+        seqlens_hint: the (approximate) lengths themselves, as a serving engine's scheduler knows
+        them; then the workgroups of a ragged batch are counted exactly."""
         self.k = k
         self.page_size = page_size
         self.recompute_layers = list(recompute_layers)
@@ -226,10 +229,15 @@ class PagedKascadeDecoder:
         self.max_batch, self.max_seqlen = max_batch, max_seqlen
         self.stride = ((max_seqlen + 7) // 8) * 8
         self.max_topk = budgets.decode_budget(max_seqlen, k)
+        if seqlens_hint is not None and total_tokens is None:
+            total_tokens = sum(seqlens_hint)
         total = total_tokens if total_tokens is not None else max_batch * max_seqlen
-        self.ns_dense = num_split_dense or kernels.default_num_split(G * total, max_seqlen)
+        dense_rows = list(seqlens_hint) if seqlens_hint is not None else None
+        reuse_rows = [budgets.decode_budget(n, k) for n in seqlens_hint] if seqlens_hint is not None else None
+        self.ns_dense = num_split_dense or kernels.default_num_split(G * total, max_seqlen, row_counts=dense_rows)
         self.ns_reuse = num_split_reuse or kernels.default_num_split(
-            G * budgets.decode_budget(total, k), self.max_topk, cap_rows=kernels.GATHER_ROWS_PER_SPLIT)
+            G * budgets.decode_budget(total, k), self.max_topk, cap_rows=kernels.GATHER_ROWS_PER_SPLIT,
+            row_counts=reuse_rows)
         ns = max(self.ns_dense, self.ns_reuse)
         dev = self.device
         self._glse = torch.empty(max_batch * H * ns, device=dev, dtype=torch.float32)

@@ -103,6 +103,37 @@ def test_default_num_split_heuristic(monkeypatch):
     assert kernels.default_num_split(128 * 6656, 6656, cap_rows=kernels.GATHER_ROWS_PER_SPLIT) == 4
 
 
+def test_split_count_of_a_ragged_batch_with_known_lengths(monkeypatch):
+    """With the lengths known, the non-empty workgroups are counted exactly: as many splits as
+    fit two workgroups per compute unit, every sequence's count rounded up."""
+    from kascade_amd import kernels, _lib
+
+    class FakeLib:
+        def kascade_device_cu_count(self):
+            return 256
+    monkeypatch.setattr(_lib, "init", lambda: FakeLib())
+    cus = 256
+    seq = [131072, 196608, 262144, 524288]
+
+    def wgs(ns, rows, longest):
+        rps = ((-(-longest // ns) + 63) // 64) * 64
+        return 8 * sum(max(1, -(-n // rps)) for n in rows)
+
+    ns = kernels.default_num_split(8 * sum(seq), max(seq), row_counts=seq)
+    assert wgs(ns, seq, max(seq)) <= 2 * cus < wgs(ns + 1, seq, max(seq))
+    rows = [budgets.decode_budget(n, 10) for n in seq]
+    ns = kernels.default_num_split(8 * sum(rows), max(rows), cap_rows=kernels.GATHER_ROWS_PER_SPLIT, row_counts=rows)
+    assert wgs(ns, rows, max(rows)) <= 2 * cus < wgs(ns + 1, rows, max(rows))
+    # uniform batches: whole residencies, a second one once a split would pass ~4096 rows
+    assert kernels.default_num_split(128 * 13184, 13184, cap_rows=kernels.GATHER_ROWS_PER_SPLIT,
+                                     row_counts=[13184] * 16) == 4
+    assert kernels.default_num_split(128 * 26240, 26240, cap_rows=kernels.GATHER_ROWS_PER_SPLIT,
+                                     row_counts=[26240] * 16) == 8
+    # a single sequence and launches too small to fill the device keep the plain rule
+    assert kernels.default_num_split(8 * 1664, 1664, row_counts=[1664]) == 13
+    assert kernels.default_num_split(8 * 600, 300, row_counts=[300, 300]) == kernels.default_num_split(8 * 600, 300)
+
+
 def test_workloads_are_seeded_and_shaped():
     a = workloads.prefill_inputs(1, 256, seed=3)
     b = workloads.prefill_inputs(1, 256, seed=3)
