@@ -289,7 +289,7 @@ def main():
                       for i in range(n_caches)]
             c0 = caches[0]
             dec = PagedKascadeDecoder(PCT, head_map, ANCHORS, B, max_len, page_size=16, device=dev,
-                                      seqlens_hint=seqlens if ragged else None, total_tokens=sum(seqlens))
+                                      seqlens_hint=seqlens)
             calls = [0]
 
             def cache():
