@@ -72,7 +72,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2)))
 void decode_split_kernel(DecodeParams p) {
     __shared__ int s_row[GATHER ? kSubChunk : 1];
     __shared__ int s_last;
-    __shared__ int s_map[3];
     __shared__ int s_found;   // gather mode: sub-chunk whose index list names the newest token
     // anchor mode: the compact raw scores of kCodePhase * 1024 tokens (see kScoreSteps), written to
     // HBM in one burst per phase; they share their LDS with the merge state, which is only needed
@@ -124,41 +123,34 @@ void decode_split_kernel(DecodeParams p) {
     // ragged batch has many -- come last in dispatch order and exit at once, instead of being
     // scattered among the working ones, which left some compute units with several streams and
     // others with none (four sequences of 131072..524288 tokens, 512 working workgroups: gather
-    // 101 -> 86 us).  One sequence needs none of this (and a decode step of a short one is all
-    // latency: the extra barrier would show).
-    int b, split, nsplit_b;
+    // 101 -> 86 us).  One sequence needs none of this.
+    int b, split, nsplit_b, seqlen;
     if (p.seqlens != nullptr && p.B > 1 && p.B <= 64) {
+        // every wavefront works it out for itself: lane l holds sequence l, no LDS, no barrier,
+        // and the sequence's length comes out of the same load
         const int w = blockIdx.y + gridDim.y * blockIdx.z;
-        if (tid == 0) s_map[0] = -1;
-        if (wave == 0) {
-            int cnt = 0;
-            if (lane < p.B)
-                cnt = max(1, (rows_for(p.seqlens[lane]) + p.rows_per_split - 1) / p.rows_per_split);
-            int incl = cnt;
+        const int len = lane < p.B ? p.seqlens[lane] : 0;
+        const int cnt = lane < p.B ? max(1, (rows_for(len) + p.rows_per_split - 1) / p.rows_per_split) : 0;
+        int incl = cnt;
 #pragma unroll
-            for (int o = 1; o < 64; o <<= 1) {
-                const int t = __shfl_up(incl, o);
-                if (lane >= o) incl += t;
-            }
-            const int excl = incl - cnt;
-            if (lane < p.B && w >= excl && w < incl) {
-                s_map[0] = lane;
-                s_map[1] = w - excl;
-                s_map[2] = cnt;
-            }
+        for (int o = 1; o < 64; o <<= 1) {
+            const int t = __shfl_up(incl, o);
+            if (lane >= o) incl += t;
         }
-        __syncthreads();
-        b = s_map[0];
-        if (b < 0) return;
-        split = s_map[1];
-        nsplit_b = s_map[2];
+        const int excl = incl - cnt;
+        const unsigned long long mine = __ballot(lane < p.B && w >= excl && w < incl);
+        if (mine == 0) return;   // beyond the last working workgroup
+        const int src = __ffsll((long long)mine) - 1;
+        b = src;
+        split = __builtin_amdgcn_readfirstlane(w - __shfl(excl, src));
+        nsplit_b = __builtin_amdgcn_readfirstlane(__shfl(cnt, src));
+        seqlen = __builtin_amdgcn_readfirstlane(__shfl(len, src));
     } else {
         b = blockIdx.z;
         split = blockIdx.y;
         nsplit_b = p.num_split;
+        seqlen = p.seqlens ? p.seqlens[b] : p.kv_stride_tokens;
     }
-
-    int seqlen = p.seqlens ? p.seqlens[b] : p.kv_stride_tokens;
     if (p.block_table) seqlen = min(seqlen, p.max_pages << p.page_shift);
     seqlen = max(seqlen, 0);
     const int n = rows_for(seqlen);  // rows this (b, g) pair attends to
