@@ -164,6 +164,28 @@ def test_decode_recompute_long_ranges(cuda, seqlens, ns, layer):
         assert_close(o, o_want, "anchor-0 decode output")
 
 
+def test_many_short_sequences(cuda):
+    """More sequences than the in-kernel numbering of working splits handles (64): the plain
+    grid mapping takes over; and a batch where most splits are empty."""
+    from kascade_amd import kernels
+    gen = torch.Generator().manual_seed(77)
+    for B, lo, hi, ns in ((70, 40, 400, 3), (9, 16, 3000, 12)):
+        seqlens = torch.randint(lo, hi, (B,), generator=gen).tolist()
+        seqlens[0] = hi          # one long sequence, the rest leave trailing splits empty
+        w = _paged_case(seqlens, seed=B)
+        kc = orc.paged_to_contiguous(w.k_pages, w.block_table, seqlens)
+        vc = orc.paged_to_contiguous(w.v_pages, w.block_table, seqlens)
+        want, _ = orc.dense_decode(w.q, kc, vc, seqlens)
+        for sync in (None, torch.zeros(B * G, dtype=torch.int32, device=cuda)):
+            glse, part = _scratch(B, ns, cuda)
+            got = kernels.decode_dense_paged(w.q.to(cuda), w.k_pages.to(cuda), w.v_pages.to(cuda),
+                                             w.seqlens.to(cuda), glse, part, w.block_table.to(cuda), w.page_size,
+                                             sync=sync)
+            assert_close(got, want, f"dense decode, {B} sequences, fused={sync is not None}")
+            if sync is not None:
+                assert int(sync.abs().sum()) == 0, "arrival counters must be back at zero"
+
+
 def test_decode_reuse_paged_ragged_head_mapping(cuda):
     """Reuse layer on a ragged paged batch through a random head map, indices from the oracle anchor."""
     from kascade_amd import kernels
