@@ -9,11 +9,7 @@ from __future__ import annotations
 import ctypes as C
 from pathlib import Path
 
-import os
-
-# KASCADE_HIP_LIB points the loader at another build of the same library (kernel tuning runs).
-LIB_PATH = Path(os.environ.get("KASCADE_HIP_LIB") or
-                Path(__file__).resolve().parent / "libkascade_hip.so")
+LIB_PATH = Path(__file__).resolve().parent / "libkascade_hip.so"
 
 
 class KascadeError(RuntimeError):

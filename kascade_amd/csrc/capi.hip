@@ -244,6 +244,9 @@ int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_hal
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (check_hip(launch_decode_split(p, false, with_output != 0, true, s), "decode_recompute split"))
         return -1;
+    // the kernels cut every sequence length down to this (decode_split_kernel's safe_len)
+    long long len_cap = block_table ? (long long)max_pages * page_size : (long long)kv_stride_tokens;
+    if (len_cap > scores_stride) len_cap = scores_stride;
     // Without an output the only thing left to merge is the log-sums, which the aggregate
     // launch does for itself: no combine launch.
     const bool merge_in_aggregate = !sync_counters && !with_output;
@@ -254,7 +257,7 @@ int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_hal
     return check_hip(launch_decode_aggregate(scores, merge_in_aggregate ? nullptr : row_sums,
                                              merge_in_aggregate ? glse : nullptr, num_split, row_sums,
                                              cache_seqlens, H(aggregated_scores), batch, scores_stride,
-                                             kv_stride_tokens, s),
+                                             kv_stride_tokens, (int)len_cap, s),
                      "decode_recompute aggregate");
 }
 

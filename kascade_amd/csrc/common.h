@@ -40,23 +40,6 @@ __device__ __forceinline__ float row16_sum(float x) {
     return x;
 }
 
-// Maximum over the 16 lanes of a DPP row; every lane of the row receives it.
-__device__ __forceinline__ float row16_max(float x) {
-    x = fmaxf(x, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, false)));
-    x = fmaxf(x, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, false)));
-    x = fmaxf(x, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x141, 0xF, 0xF, false)));
-    x = fmaxf(x, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x140, 0xF, 0xF, false)));
-    return x;
-}
-
-__device__ __forceinline__ float dot8(const Pack16& a, const Pack16& b, float acc) {
-    acc = __builtin_amdgcn_fdot2(a.h2[0], b.h2[0], acc, false);
-    acc = __builtin_amdgcn_fdot2(a.h2[1], b.h2[1], acc, false);
-    acc = __builtin_amdgcn_fdot2(a.h2[2], b.h2[2], acc, false);
-    acc = __builtin_amdgcn_fdot2(a.h2[3], b.h2[3], acc, false);
-    return acc;
-}
-
 __device__ __forceinline__ uint4_t ld_global_16(const void* p) {
     return *reinterpret_cast<const uint4_t*>(p);
 }

@@ -49,10 +49,11 @@ hipError_t launch_decode_combine(const float* glse, const float* opart, half_t* 
                                  float* row_sums, int batch, int num_split, bool with_v,
                                  hipStream_t stream);
 // Log-sums per head: merged (row_sums_in), or glse [B,H,num_split] to be merged by the kernel,
-// which then also writes them to row_sums_out.
+// which then also writes them to row_sums_out.  len_cap: the bound the streaming launch put on
+// every sequence length (block-table coverage or cache length, and the score row width).
 hipError_t launch_decode_aggregate(const float* scores, const float* row_sums_in, const float* glse,
                                    int num_split, float* row_sums_out, const int* seqlens,
                                    half_t* agg, int batch, int scores_stride, int uniform_len,
-                                   hipStream_t stream);
+                                   int len_cap, hipStream_t stream);
 
 }  // namespace kascade

@@ -100,11 +100,18 @@ void decode_split_kernel(DecodeParams p) {
     const int wave = tid >> 6;
     const int lane = tid & 63;
 
-    // rows a (sequence, KV head) pair of length `len` attends to
-    auto rows_for = [&](int len) {
-        // a length beyond what the block table covers must not index past the table
+    // The longest context memory allows a sequence that claims `len` tokens: lengths live in device
+    // memory, the host sized every buffer from its own arguments, so each length is cut down to
+    // what the block table covers (or the cache holds) and, on an anchor pass, to the row width of
+    // the score scratch.  Nothing is read or written beyond those bounds whatever the lengths say.
+    auto safe_len = [&](int len) {
         if (p.block_table) len = min(len, p.max_pages << p.page_shift);
-        len = max(len, 0);
+        else if (p.kv_stride_tokens > 0) len = min(len, p.kv_stride_tokens);
+        if (WRITE_SCORES) len = min(len, p.scores_stride);
+        return max(len, 0);
+    };
+    // rows a (sequence, KV head) pair of (safe) length `len` attends to
+    auto rows_for = [&](int len) {
         if (!GATHER) return len;
         int n;
         if (p.topk_percent > 0.f) {
@@ -117,54 +124,86 @@ void decode_split_kernel(DecodeParams p) {
         if (p.seqlens) n = min(n, len);   // never more rows than the sequence holds
         return n;
     };
+    // Splits a sequence of `rows` rows occupies: never more than the launch has per sequence.  A
+    // sequence longer than the host sized the splits for (its length exceeds the caller's bound)
+    // keeps num_split splits and its last split takes every row that is left.
+    auto split_count = [&](int rows) {
+        return max(1, min(p.num_split, (rows + p.rows_per_split - 1) / p.rows_per_split));
+    };
     // Which (sequence, split) this workgroup takes.  With per-sequence lengths the non-empty
     // splits of all sequences are numbered consecutively (sequence-major; at least one split per
     // sequence) and workgroup w of the launch takes number w: the workgroups left over -- a
     // ragged batch has many -- come last in dispatch order and exit at once, instead of being
     // scattered among the working ones, which left some compute units with several streams and
     // others with none (four sequences of 131072..524288 tokens, 512 working workgroups: gather
-    // 101 -> 86 us).  One sequence needs none of this.
+    // 101 -> 86 us).  One sequence needs none of this; beyond 64 * kMapRounds sequences the
+    // workgroups keep their grid position.
+    constexpr int kMapRounds = 4;
     int b, split, nsplit_b, seqlen;
-    if (p.seqlens != nullptr && p.B > 1 && p.B <= 64) {
-        // every wavefront works it out for itself: lane l holds sequence l, no LDS, no barrier,
-        // and the sequence's length comes out of the same load
+    bool len_cut;
+    if (p.seqlens != nullptr && p.B > 1 && p.B <= 64 * kMapRounds) {
+        // every wavefront works it out for itself: lane l holds sequences l, l + 64, ...; no LDS,
+        // no barrier, and the sequence's length comes out of the same loads (all issued first)
         const int w = blockIdx.y + gridDim.y * blockIdx.z;
-        const int len = lane < p.B ? p.seqlens[lane] : 0;
-        const int cnt = lane < p.B ? max(1, (rows_for(len) + p.rows_per_split - 1) / p.rows_per_split) : 0;
-        int incl = cnt;
+        int lens[kMapRounds];
+        unsigned long long cut[kMapRounds];   // sequences whose length had to be cut down
 #pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-            const int t = __shfl_up(incl, o);
-            if (lane >= o) incl += t;
+        for (int r = 0; r < kMapRounds; ++r) {
+            const int bi = 64 * r + lane;
+            const int raw = bi < p.B ? p.seqlens[bi] : 0;
+            lens[r] = safe_len(raw);
+            cut[r] = __ballot(lens[r] != raw);
         }
-        const int excl = incl - cnt;
-        const unsigned long long mine = __ballot(lane < p.B && w >= excl && w < incl);
-        if (mine == 0) return;   // beyond the last working workgroup
-        const int src = __ffsll((long long)mine) - 1;
-        b = src;
-        split = __builtin_amdgcn_readfirstlane(w - __shfl(excl, src));
-        nsplit_b = __builtin_amdgcn_readfirstlane(__shfl(cnt, src));
-        seqlen = __builtin_amdgcn_readfirstlane(__shfl(len, src));
+        int carry = 0;   // splits of the sequences of earlier rounds (wavefront-uniform)
+        b = -1; split = 0; nsplit_b = 1; seqlen = 0; len_cut = false;
+#pragma unroll
+        for (int r = 0; r < kMapRounds; ++r) {
+            if (64 * r < p.B && b < 0) {   // uniform
+                const int bi = 64 * r + lane;
+                const int cnt = bi < p.B ? split_count(rows_for(lens[r])) : 0;
+                int incl = cnt;
+#pragma unroll
+                for (int o = 1; o < 64; o <<= 1) {
+                    const int t = __shfl_up(incl, o);
+                    if (lane >= o) incl += t;
+                }
+                const int excl = carry + incl - cnt;
+                const unsigned long long mine = __ballot(bi < p.B && w >= excl && w < excl + cnt);
+                if (mine != 0) {
+                    const int src = __ffsll((long long)mine) - 1;
+                    b = 64 * r + src;
+                    split = __builtin_amdgcn_readfirstlane(w - __shfl(excl, src));
+                    nsplit_b = __builtin_amdgcn_readfirstlane(__shfl(cnt, src));
+                    seqlen = __builtin_amdgcn_readfirstlane(__shfl(lens[r], src));
+                    len_cut = (cut[r] >> src) & 1;
+                }
+                carry += __builtin_amdgcn_readfirstlane(__shfl(incl, 63));
+            }
+        }
+        if (b < 0) return;   // beyond the last working workgroup
     } else {
         b = blockIdx.z;
         split = blockIdx.y;
         nsplit_b = p.num_split;
-        seqlen = p.seqlens ? p.seqlens[b] : p.kv_stride_tokens;
+        const int raw = p.seqlens ? p.seqlens[b] : p.kv_stride_tokens;
+        seqlen = safe_len(raw);
+        len_cut = seqlen != raw;
     }
-    if (p.block_table) seqlen = min(seqlen, p.max_pages << p.page_shift);
-    seqlen = max(seqlen, 0);
     const int n = rows_for(seqlen);  // rows this (b, g) pair attends to
     // contiguous range of this split; every split covers rows_per_split rows, sequences
-    // shorter than num_split*rows_per_split leave their last splits empty
+    // shorter than num_split*rows_per_split leave their last splits empty, and the last split of
+    // a sequence runs to the sequence's end
     const long long r0l = (long long)split * p.rows_per_split;
     const int r0 = (int)min((long long)n, r0l);
-    const int r1 = (int)min((long long)n, r0l + p.rows_per_split);
+    const int r1 = (split == nsplit_b - 1) ? n : (int)min((long long)n, r0l + p.rows_per_split);
 
     // Fused append.  With k_new/v_new the K/V rows of the newest token (position seqlen-1)
     // arrive beside the cache and have to end up in it.  A workgroup that is going to read that
     // row writes it first and waits for its own stores at a barrier; what other workgroups write
     // there is the same bytes.  `write_newest` is uniform over the workgroup.
+    // A length that had to be cut down names a slot that does not exist: nothing is appended.
     const int newest = seqlen - 1;
+    const bool can_append = p.k_new != nullptr && newest >= 0 && !len_cut;
     auto write_newest = [&]() {
         if (tid < 32) {
             const int part = tid >> 4, c = tid & 15;
@@ -181,7 +220,7 @@ void decode_split_kernel(DecodeParams p) {
             *reinterpret_cast<uint4_t*>(dst) = ld_global_16(src);
         }
     };
-    if (p.k_new != nullptr && newest >= 0) {
+    if (can_append) {
         if (!GATHER) {
             if (newest >= r0 && newest < r1) {   // the split that streams the newest row
                 write_newest();
@@ -392,7 +431,7 @@ void decode_split_kernel(DecodeParams p) {
             else if (cn <= 4 * kThreads) stage(std::integral_constant<int, 4>{});
             else stage(std::integral_constant<int, kSubChunk / kThreads>{});
             __syncthreads();
-            if (p.k_new != nullptr && s_found == c0) {   // c0 differs per sub-chunk: no reset needed
+            if (can_append && s_found == c0) {   // c0 differs per sub-chunk: no reset needed
                 write_newest();
                 __syncthreads();
             }
@@ -547,6 +586,11 @@ void decode_split_kernel(DecodeParams p) {
     // reads them back with device-coherent loads.  No device-wide fence is involved: one per
     // workgroup would write back and invalidate the L2 that the K/V stream lives in.
     if (p.counters == nullptr) return;
+    // Every wavefront waits until its own stores above have been acknowledged (they are
+    // write-through at device scope, so an acknowledged store is in device-coherent memory) and
+    // only then joins the barrier.  The barrier by itself does not do this: at workgroup scope
+    // the compiler may leave the wait for outstanding stores out of the barrier's fences.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (tid == 0) {
         const int arrived = __hip_atomic_fetch_add(&p.counters[b * kGroups + g], 1, __ATOMIC_RELAXED,
@@ -688,11 +732,13 @@ __global__ __launch_bounds__(256) void decode_aggregate_kernel(const float* __re
                                                               float* __restrict__ row_sums_out,
                                                               const int* __restrict__ seqlens,
                                                               half_t* __restrict__ agg,
-                                                              int scores_stride, int uniform_len) {
+                                                              int scores_stride, int uniform_len,
+                                                              int len_cap) {
     __shared__ float s_lse[kGroupSize];
     const int g = blockIdx.y;
     const int b = blockIdx.z;
-    const int len = seqlens ? seqlens[b] : uniform_len;
+    // the same bound the streaming launch applied to the length: codes beyond it were never written
+    const int len = max(0, min(seqlens ? seqlens[b] : uniform_len, len_cap));
     const int j0 = (blockIdx.x * 256 + threadIdx.x) * 8;
     float lse[kGroupSize];
     if (glse != nullptr) {   // uniform over the launch
@@ -793,10 +839,10 @@ hipError_t launch_decode_combine(const float* glse, const float* opart, half_t* 
 hipError_t launch_decode_aggregate(const float* scores, const float* row_sums_in, const float* glse,
                                    int num_split, float* row_sums_out, const int* seqlens,
                                    half_t* agg, int batch, int scores_stride, int uniform_len,
-                                   hipStream_t stream) {
+                                   int len_cap, hipStream_t stream) {
     dim3 grid((scores_stride + 2047) / 2048, kGroups, batch), block(256);
     hipLaunchKernelGGL(decode_aggregate_kernel, grid, block, 0, stream, scores, row_sums_in, glse,
-                       num_split, row_sums_out, seqlens, agg, scores_stride, uniform_len);
+                       num_split, row_sums_out, seqlens, agg, scores_stride, uniform_len, len_cap);
     return hipGetLastError();
 }
 

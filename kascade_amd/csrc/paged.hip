@@ -20,6 +20,9 @@ __global__ __launch_bounds__(256) void paged_kv_append_kernel(
     const int t = (int)(bt % n_new);
     const int b = (int)(bt / n_new);
     const int tok = start_pos[b] + t;
+    // a position before the sequence or beyond what the block table covers has no slot: skipped,
+    // like rope_append_kernel does (reading the table there would land in another sequence's row)
+    if (tok < 0 || (tok >> page_shift) >= max_pages) return;
     const int pg = block_table[(long long)b * max_pages + (tok >> page_shift)];
     const long long row = ((long long)pg << page_shift) + (tok & ((1 << page_shift) - 1));
     const long long dst = (row * kGroups + g) * kDim + col * 8;

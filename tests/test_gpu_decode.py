@@ -165,11 +165,12 @@ def test_decode_recompute_long_ranges(cuda, seqlens, ns, layer):
 
 
 def test_many_short_sequences(cuda):
-    """More sequences than the in-kernel numbering of working splits handles (64): the plain
-    grid mapping takes over; and a batch where most splits are empty."""
+    """Batches beyond one wavefront of sequences: the in-kernel numbering of the working splits
+    takes several rounds (70, 130 sequences), beyond 256 the plain grid mapping takes over; and a
+    batch where most splits are empty."""
     from kascade_amd import kernels
     gen = torch.Generator().manual_seed(77)
-    for B, lo, hi, ns in ((70, 40, 400, 3), (9, 16, 3000, 12)):
+    for B, lo, hi, ns in ((70, 40, 400, 3), (130, 20, 300, 2), (260, 20, 200, 2), (9, 16, 3000, 12)):
         seqlens = torch.randint(lo, hi, (B,), generator=gen).tolist()
         seqlens[0] = hi          # one long sequence, the rest leave trailing splits empty
         w = _paged_case(seqlens, seed=B)
@@ -531,3 +532,142 @@ def test_page_sizes(cuda, page_size):
     got = kernels.decode_reuse_paged(q, kp, vp, lens, idx, hm, float(p), glse, part, block_table=bt,
                                      page_size=page_size)
     assert_close(got, orc.reuse_decode(w.q, kc, vc, idx.cpu(), w.head_mapping, counts), f"reuse decode, page {page_size}")
+
+
+GUARD = 1234.5
+
+
+def _guarded(shape_lead, n_valid, n_guard, dev, dtype=torch.float32):
+    """A buffer of n_valid + n_guard elements per leading index, guard part preset; returns
+    (whole, view of the valid part as a fresh contiguous-looking tensor is not possible, so the
+    kernels get the leading n_valid*prod(lead) elements of a flat buffer followed by the guard)."""
+    lead = 1
+    for x in shape_lead:
+        lead *= x
+    whole = torch.full((lead * n_valid + n_guard,), GUARD, device=dev, dtype=dtype)
+    return whole, whole[:lead * n_valid].view(*shape_lead, n_valid)
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_lengths_beyond_the_callers_bound(cuda, fused):
+    """Sequence lengths live in device memory; the host sizes the splits from the caller's bound.
+    A length above that bound must stay inside every buffer: behind a block table the last
+    split takes the rest of the sequence (same attention, one long split), the partial-result
+    rows of other (sequence, head) pairs and the memory behind the buffers stay untouched, and
+    the arrival counters return to zero."""
+    from kascade_amd import kernels
+    seqlens = [1000, 3000, 515]
+    bound, ns = 1024, 4                      # splits sized for 1024 tokens: 256 rows each
+    w = _paged_case(seqlens, seed=51)
+    B = len(seqlens)
+    kc = orc.paged_to_contiguous(w.k_pages, w.block_table, seqlens)
+    vc = orc.paged_to_contiguous(w.v_pages, w.block_table, seqlens)
+    q, kp, vp = w.q.to(cuda), w.k_pages.to(cuda), w.v_pages.to(cuda)
+    lens, bt = w.seqlens.to(cuda), w.block_table.to(cuda)
+    sync = torch.zeros(B * G, dtype=torch.int32, device=cuda) if fused else None
+    g_whole, glse = _guarded((B, H), ns, 64, cuda)
+    p_whole, part = _guarded((B, H), ns * D, 64 * D, cuda)
+    part = part.view(B, H, ns, D)
+    want, _ = orc.dense_decode(w.q, kc, vc, seqlens)
+    got = kernels.decode_dense_paged(q, kp, vp, lens, glse, part, bt, w.page_size, kv_len=bound, sync=sync)
+    torch.cuda.synchronize()
+    assert_close(got, want, "dense decode with a length above the bound")
+    assert bool((g_whole[B * H * ns:] == GUARD).all()) and bool((p_whole[B * H * ns * D:] == GUARD).all()), \
+        "partial results written past their buffers"
+    if fused:
+        assert int(sync.abs().sum()) == 0, "arrival counters must be back at zero"
+    # anchor pass: the score rows are 1024 wide, so every length is cut to 1024 tokens there
+    stride = bound
+    s_whole, scores = _guarded((B, H), stride, 4096, cuda)
+    row_sums = torch.empty(B, H, device=cuda, dtype=torch.float32)
+    cut = [min(n, stride) for n in seqlens]
+    for layer in (0, 1):
+        o, agg = kernels.decode_recompute(q, kp, vp, glse, part, row_sums, scores, layer, cache_seqlens=lens,
+                                          block_table=bt, page_size=w.page_size, kv_len=bound, sync=sync)
+        torch.cuda.synchronize()
+        assert bool((s_whole[B * H * stride:] == GUARD).all()), "raw scores written past their buffer"
+        assert bool((g_whole[B * H * ns:] == GUARD).all()) and bool((p_whole[B * H * ns * D:] == GUARD).all())
+        assert_close(agg.cpu(), orc.pooled_decode_scores(w.q, kc[:, :stride], cut), "agg over the cut lengths",
+                     atol=2e-6, rtol=2e-3)
+        if layer == 0:
+            assert_close(o, orc.dense_decode(w.q, kc[:, :stride], vc[:, :stride], cut)[0], "anchor-0 output, cut")
+        if fused:
+            assert int(sync.abs().sum()) == 0
+    # contiguous cache of 900 tokens per sequence, lengths claiming more
+    L = 900
+    kcc, vcc = kc[:, :L].contiguous().to(cuda), vc[:, :L].contiguous().to(cuda)
+    got = kernels.decode_dense_paged(q, kcc, vcc, lens, glse, part, sync=sync)
+    cut = [min(n, L) for n in seqlens]
+    assert_close(got, orc.dense_decode(w.q, kc[:, :L], vc[:, :L], cut)[0], "contiguous cache, lengths cut to its size")
+    # gather: indices are clamped into the (cut) sequence, budgets follow the cut length
+    gen = torch.Generator().manual_seed(6)
+    idx = _rand_idx(B, 500, 256, gen).to(cuda)
+    hm = torch.arange(G, dtype=torch.int32, device=cuda)
+    got = kernels.decode_reuse_paged(q, kcc, vcc, lens, idx, hm, 0.0, glse, part, sync=sync)
+    assert_close(got, orc.reuse_decode(w.q, kc[:, :L], vc[:, :L], idx.cpu(), list(range(G))), "reuse, lengths cut")
+    assert bool((g_whole[B * H * ns:] == GUARD).all()) and bool((p_whole[B * H * ns * D:] == GUARD).all())
+    # a fused append to a slot that does not exist is dropped: the cache keeps its contents
+    k_new = torch.full((B, G, D), 7.0, dtype=torch.float16, device=cuda)
+    before_k, before_v = kcc.clone(), vcc.clone()
+    kernels.decode_dense_paged(q, kcc, vcc, lens, glse, part, sync=sync, k_new=k_new, v_new=k_new)
+    torch.cuda.synchronize()
+    for b, n in enumerate(seqlens):
+        if n > L:
+            assert torch.equal(kcc[b], before_k[b]) and torch.equal(vcc[b], before_v[b]), "append beyond the cache"
+        else:
+            assert float(kcc[b, n - 1].float().mean()) == 7.0
+
+
+def test_fused_merge_random_shapes(cuda):
+    """Bounded sweep: the in-launch merge against the combine launch over random batch sizes,
+    lengths and split counts; stops at the first mismatch."""
+    from kascade_amd import kernels
+    gen = torch.Generator().manual_seed(2024)
+    for case in range(24):
+        B = int(torch.randint(1, 7, (1,), generator=gen))
+        seqlens = torch.randint(1, 5000, (B,), generator=gen).tolist()
+        ns = int(torch.randint(1, 33, (1,), generator=gen))
+        w = _paged_case(seqlens, seed=100 + case, peaked=bool(case % 2))
+        q, kp, vp = w.q.to(cuda), w.k_pages.to(cuda), w.v_pages.to(cuda)
+        lens, bt = w.seqlens.to(cuda), w.block_table.to(cuda)
+        glse, part = _scratch(B, ns, cuda)
+        sync = torch.zeros(B * G, dtype=torch.int32, device=cuda)
+        two = kernels.decode_dense_paged(q, kp, vp, lens, glse, part, bt, w.page_size).clone()
+        one = kernels.decode_dense_paged(q, kp, vp, lens, glse, part, bt, w.page_size, sync=sync)
+        torch.cuda.synchronize()
+        assert int(sync.abs().sum()) == 0, f"case {case} {seqlens} ns={ns}: counters"
+        assert_close(one, two, f"case {case} {seqlens} ns={ns}: fused vs combine", atol=1e-3, rtol=2e-3)
+        k = min(min(seqlens), 1 + int(torch.randint(0, 2000, (1,), generator=gen)))
+        idx = _rand_idx(B, min(seqlens), k, gen).to(cuda)
+        hm = torch.randint(0, G, (G,), generator=gen).to(torch.int32).to(cuda)
+        two = kernels.decode_reuse_paged(q, kp, vp, lens, idx, hm, 0.0, glse, part, block_table=bt,
+                                         page_size=w.page_size).clone()
+        one = kernels.decode_reuse_paged(q, kp, vp, lens, idx, hm, 0.0, glse, part, block_table=bt,
+                                         page_size=w.page_size, sync=sync)
+        torch.cuda.synchronize()
+        assert int(sync.abs().sum()) == 0, f"case {case}: counters (reuse)"
+        assert_close(one, two, f"case {case} {seqlens} k={k} ns={ns}: fused vs combine (reuse)", atol=1e-3, rtol=2e-3)
+
+
+def test_kv_append_beyond_the_block_table(cuda):
+    """Tokens whose position has no block-table entry are dropped, not scattered into other pages."""
+    from kascade_amd import kernels
+    gen = torch.Generator().manual_seed(3)
+    B, page, n_new, P, max_pages = 2, 16, 40, 16, 4
+    Kp = torch.zeros(P, page, G, D, dtype=torch.float16, device=cuda)
+    Vp = torch.zeros_like(Kp)
+    bt = torch.randperm(P, generator=gen)[:B * max_pages].view(B, max_pages).to(torch.int32)
+    start = torch.tensor([40, -3], dtype=torch.int32)           # 40+40 overruns 64 slots by one page
+    kn = torch.randn(B, n_new, G, D, generator=gen).half()
+    vn = torch.randn(B, n_new, G, D, generator=gen).half()
+    kernels.paged_kv_append(Kp, Vp, kn.to(cuda), vn.to(cuda), start.to(cuda), bt.to(cuda), page)
+    torch.cuda.synchronize()
+    Kc, Vc = Kp.cpu(), Vp.cpu()
+    want_k, want_v = torch.zeros_like(Kc), torch.zeros_like(Vc)
+    for b in range(B):
+        for t in range(n_new):
+            tok = int(start[b]) + t
+            if 0 <= tok < max_pages * page:
+                want_k[int(bt[b, tok // page]), tok % page] = kn[b, t]
+                want_v[int(bt[b, tok // page]), tok % page] = vn[b, t]
+    assert torch.equal(Kc, want_k) and torch.equal(Vc, want_v)
