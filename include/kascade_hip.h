@@ -111,6 +111,27 @@ int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K
                                     const kascade_half* k_new, const kascade_half* v_new,
                                     int32_t* sync_counters, void* stream);
 
+/* kascade_decode_reuse_paged_call for callers that cannot allocate device memory and have no
+ * scratch of their own to pass: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  No counterpart in the reference.  The partial results of the splits
+ * (glse, Output_partial) live in a buffer built into the library instead of in caller memory; the
+ * splits are merged by the combine launch.  Everything else is the argument list above.
+ *   Limit: batch * num_split <= 1024 (a 16.9 MB buffer per device, held until the process ends);
+ *   larger launches are rejected with an error.  The call allocates and frees nothing.
+ *   Every call on a device uses that device's one buffer, on whatever stream: calls that overlap
+ *   in time on one device race.  Nothing in the buffer has to be cleared between calls (every
+ *   entry a launch reads it has written itself).  kascade_init() on the device prepares the
+ *   buffer's address; without it the first call does. */
+int kascade_decode_reuse_paged_noalloc_call(const kascade_half* Q, const kascade_half* K,
+                                            const kascade_half* V, const int32_t* cache_seqlens,
+                                            const int32_t* topk_indices, const int32_t* head_mapping,
+                                            float topk_percent, kascade_half* Output, int batch,
+                                            int kv_stride_tokens, int topk, int num_split,
+                                            const int32_t* block_table, int max_pages, int page_size,
+                                            const kascade_strides* kv_strides,
+                                            const kascade_half* k_new, const kascade_half* v_new,
+                                            void* stream);
+
 /* Dense split-K decode (the reference's TileLang dense baseline, gqa_decode.py:117-254 and
  * gqa_decode_with_kvcache.py:118-257), same cache conventions as above.
  * cache_seqlens may be NULL (all sequences have kv_stride_tokens tokens).  With a block

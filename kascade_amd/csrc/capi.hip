@@ -21,6 +21,17 @@ namespace {
 thread_local char g_err[1024] = "";
 int g_cu_count = 0;
 
+// Scratch of kascade_decode_reuse_paged_noalloc_call: the partial log-sums [batch,32,num_split]
+// and partial outputs [batch,32,num_split,128] of the splits, fp32, for up to kNoAllocUnits
+// (sequence, split) pairs.  Every device the library runs on holds its own copy of the array at
+// its own address until the process ends; host code never uses the array's name as an address but
+// the pointer hipGetSymbolAddress returns for the current device (g_noalloc_ptr).
+constexpr int kNoAllocUnits = 1024;
+constexpr size_t kNoAllocFloats = (size_t)kNoAllocUnits * kHeads * (1 + kDim);   // 16.9 MB
+static __device__ __align__(256) float scratch[kNoAllocFloats];
+constexpr int kMaxDevices = 64;
+float* g_noalloc_ptr[kMaxDevices] = {};
+
 int fail(const char* fmt, ...) {
     va_list ap;
     va_start(ap, fmt);
@@ -41,6 +52,22 @@ int check_hip(hipError_t e, const char* what) {
 
 inline const half_t* H(const kascade_half* p) { return reinterpret_cast<const half_t*>(p); }
 inline half_t* H(kascade_half* p) { return reinterpret_cast<half_t*>(p); }
+
+// Device address of `scratch` on the current device, looked up once per device.
+int noalloc_scratch(float** out) {
+    int dev = 0;
+    if (check_hip(hipGetDevice(&dev), "hipGetDevice")) return -1;
+    REQUIRE(dev >= 0 && dev < kMaxDevices, "device ordinal %d out of range", dev);
+    if (!g_noalloc_ptr[dev]) {
+        void* ptr = nullptr;
+        if (check_hip(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)"))
+            return -1;
+        REQUIRE(ptr != nullptr, "hipGetSymbolAddress(scratch) returned a null address");
+        g_noalloc_ptr[dev] = static_cast<float*>(ptr);
+    }
+    *out = g_noalloc_ptr[dev];
+    return 0;
+}
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
@@ -104,7 +131,7 @@ int set_append(DecodeParams& p, const kascade_half* k_new, const kascade_half* v
 
 extern "C" {
 
-int kascade_abi_version(void) { return 5; }
+int kascade_abi_version(void) { return 6; }
 
 const char* kascade_get_last_error(void) { return g_err; }
 
@@ -118,7 +145,8 @@ int kascade_init(void) {
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail("libkascade_hip is built for gfx950 only; device is %s", prop.gcnArchName);
     g_cu_count = prop.multiProcessorCount;
-    return 0;
+    float* ptr;
+    return noalloc_scratch(&ptr);   // this device's copy of the scratch array
 }
 
 int kascade_decode_reuse_call(const kascade_half* Q, const kascade_half* K, const kascade_half* V,
@@ -166,6 +194,30 @@ int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K
     if (sync_counters) return 0;   // the split kernel's last workgroups have combined
     return check_hip(launch_decode_combine(glse, Output_partial, H(Output), nullptr, batch,
                                            num_split, true, s), "decode_reuse combine");
+}
+
+int kascade_decode_reuse_paged_noalloc_call(const kascade_half* Q, const kascade_half* K,
+                                            const kascade_half* V, const int32_t* cache_seqlens,
+                                            const int32_t* topk_indices, const int32_t* head_mapping,
+                                            float topk_percent, kascade_half* Output, int batch,
+                                            int kv_stride_tokens, int topk, int num_split,
+                                            const int32_t* block_table, int max_pages, int page_size,
+                                            const kascade_strides* kv_strides,
+                                            const kascade_half* k_new, const kascade_half* v_new,
+                                            void* stream) {
+    REQUIRE(batch > 0 && num_split > 0, "decode_reuse_noalloc: batch, num_split must be > 0");
+    REQUIRE((long long)batch * num_split <= kNoAllocUnits,
+            "decode_reuse_noalloc: batch * num_split = %lld exceeds the built-in scratch (%d); "
+            "use kascade_decode_reuse_paged_call with caller-provided scratch",
+            (long long)batch * num_split, kNoAllocUnits);
+    float* base;
+    if (noalloc_scratch(&base)) return -1;
+    float* glse = base;                                           // [batch,32,num_split]
+    float* opart = base + (size_t)kNoAllocUnits * kHeads;         // [batch,32,num_split,128]
+    return kascade_decode_reuse_paged_call(Q, K, V, cache_seqlens, topk_indices, head_mapping,
+                                           topk_percent, glse, opart, Output, batch,
+                                           kv_stride_tokens, topk, num_split, block_table, max_pages,
+                                           page_size, kv_strides, k_new, v_new, nullptr, stream);
 }
 
 int kascade_decode_dense_paged_call(const kascade_half* Q, const kascade_half* K,

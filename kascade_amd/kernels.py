@@ -227,6 +227,35 @@ def decode_reuse_paged(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_
     return out
 
 
+NOALLOC_MAX_UNITS = 1024   # batch * num_split the library's built-in scratch holds
+
+
+def decode_reuse_paged_noalloc(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_percent,
+                               num_split: int, out: torch.Tensor, block_table=None, page_size: int = 16,
+                               k_new=None, v_new=None) -> torch.Tensor:
+    """``decode_reuse_paged`` for callers that cannot allocate: the splits' partial results live in
+    a buffer built into the library (batch * num_split <= NOALLOC_MAX_UNITS), the output buffer is
+    the caller's, and nothing is allocated on the way -- not by this wrapper either."""
+    lib = _lib.init()
+    B = Q.shape[0]
+    _req(Q, torch.float16, "Q")
+    kv_strides = _decode_kv(K, V, block_table)
+    _req(topk_indices, torch.int32, "topk_indices"); _req(head_mapping, torch.int32, "head_mapping")
+    if cache_seqlens is not None:
+        _req(cache_seqlens, torch.int32, "cache_seqlens")
+    if block_table is not None:
+        _req(block_table, torch.int32, "block_table")
+        stride_tokens, max_pages = 0, block_table.shape[1]
+    else:
+        stride_tokens, max_pages = K.shape[1], 0
+    out = _out_buffer(out, B, Q.device)
+    _lib.check(lib.kascade_decode_reuse_paged_noalloc_call(
+        _ptr(Q), _ptr(K), _ptr(V), _ptr(cache_seqlens), _ptr(topk_indices), _ptr(head_mapping),
+        float(topk_percent), _ptr(out), B, stride_tokens, topk_indices.shape[-1], int(num_split),
+        _ptr(block_table), max_pages, page_size, kv_strides, *_new_rows(k_new, v_new, B), _stream()))
+    return out
+
+
 def decode_dense_paged(Q, K, V, cache_seqlens, glse, Output_partial, block_table=None,
                        page_size: int = 16, kv_len: Optional[int] = None, out=None,
                        sync=None, k_new=None, v_new=None) -> torch.Tensor:
