@@ -60,6 +60,15 @@ class KascadeAttentionStack:
         self.length = length
         self.seqlens.fill_(length)
 
+    def set_lengths(self, lengths: Sequence[int]):
+        """Per-sequence lengths for decoding a batch whose caches were filled sequence by
+        sequence (``kernels.paged_kv_append`` into ``k_pages`` / ``v_pages`` through
+        ``block_table``).  Chunked prefill through ``prefill_chunk`` needs a common length."""
+        if len(lengths) != self.batch or max(lengths) > self.max_seqlen or min(lengths) < 0:
+            raise KascadeError("set_lengths: one length per sequence, each within max_seqlen")
+        self.length = int(max(lengths))
+        self.seqlens.copy_(torch.tensor(list(lengths), dtype=torch.int32))
+
     # ------------------------------------------------------------------ prefill
     def prefill_chunk(self, q: Sequence[torch.Tensor], k_new: Sequence[torch.Tensor],
                       v_new: Sequence[torch.Tensor]) -> List[torch.Tensor]:
@@ -67,6 +76,8 @@ class KascadeAttentionStack:
         starts at the current length, which must be a multiple of 32.  Returns O[l] [B,Lq,H,D]."""
         Lq = q[0].shape[1]
         q_start = self.length
+        if self.batch > 1 and int(self.seqlens.min()) != q_start:
+            raise KascadeError("chunked prefill of a batch needs sequences of one common length")
         if q_start % TILE:
             raise KascadeError("a prefill chunk must start at a multiple of 32 tokens")
         if q_start + Lq > self.max_seqlen:
