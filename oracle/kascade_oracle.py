@@ -417,6 +417,39 @@ def topk_agreement(scores_row: torch.Tensor, got: torch.Tensor, n: int, valid: i
     return ok, recall, msg
 
 
+def topk_set_quality(scores_row: torch.Tensor, got: torch.Tensor, n: int, valid: int,
+                     ulps: float = 1.0) -> Tuple[bool, float, float, float, str]:
+    """Graded form of ``topk_agreement`` for selections made on scores that may differ from
+    ``scores_row`` by one fp16 rounding step (a kernel's own pooled scores against the oracle's).
+    With tau the n-th largest oracle score and u its fp16 spacing it returns
+      structural_ok  n distinct indices inside [0, valid)
+      recall         fraction of the indices scoring above tau + ulps*u that were selected
+      precision      fraction of the selected indices scoring at least tau - ulps*u
+      worst          largest distance, in units of u, of a selected index below tau or of a
+                     missing index above tau (0 when the set is an exact top-n set)
+    A score error of one step moves an entry by one step and the threshold by at most one, so an
+    honest selection has worst <= 2 and recall / precision close to 1."""
+    s = scores_row[:valid].float()
+    n = min(n, valid)
+    g = got[:n].long()
+    if n == 0:
+        return True, 1.0, 1.0, 0.0, ""
+    if g.numel() != n or int(g.min()) < 0 or int(g.max()) >= valid or torch.unique(g).numel() != n:
+        return False, 0.0, 0.0, float("inf"), "short row, index out of range or duplicate indices"
+    tau = torch.topk(s, n).values[-1]
+    u = fp16_ulp(tau)
+    present = torch.zeros(valid, dtype=torch.bool)
+    present[g] = True
+    must = s > tau + ulps * u
+    recall = float(present[must].float().mean()) if bool(must.any()) else 1.0
+    precision = float((s[g] >= tau - ulps * u).float().mean())
+    low = float(((tau - s[g]) / u).max())
+    missing = s[~present]
+    high = float(((missing - tau) / u).max()) if missing.numel() else 0.0
+    worst = max(low, high, 0.0)
+    return True, recall, precision, worst, f"recall={recall:.6f} precision={precision:.6f} worst={worst:.2f} ulp"
+
+
 # --------------------------------------------------------------------------
 # strategy semantics (KascadeStrategy.py), used for the CPU plumbing config
 # --------------------------------------------------------------------------

@@ -1,5 +1,5 @@
-"""GPU tests of the strategy inside a Hugging Face decoder: a random-init Llama-shaped model built
-from a local config object (nothing is downloaded), switched to the registered attention function
+"""GPU tests of the strategy inside a Hugging Face decoder: random-init Llama-shaped and
+Qwen3-shaped (query/key head normalisation) models built from a local config object (nothing is downloaded), switched to the registered attention function
 the way the reference's eval script does it (`model.config._attn_implementation = strategy.name`,
 eval_script.py:126), and driven through `generate` (prefill, then decode steps over HF's own
 cache).  Every attention call the model makes is recorded and checked against the CPU oracle on
@@ -17,18 +17,29 @@ ANCHORS = [0, 2]
 HEAD_MAPS = [list(range(G)), [5, 0, 0, 3, 7, 1, 6, 2], list(range(G)), [1, 2, 3, 4, 5, 6, 7, 0]]
 
 
-def _tiny_llama(cuda):
-    from transformers import LlamaConfig, LlamaForCausalLM
-    cfg = LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=len(HEAD_MAPS),
-                      num_attention_heads=H, num_key_value_heads=G, head_dim=D, vocab_size=256,
-                      max_position_embeddings=4096, pad_token_id=0, bos_token_id=1, eos_token_id=None)
+def _tiny_model(cuda, family="llama"):
+    """Random-init decoder from a local config: Llama-shaped, or Qwen3-shaped (RMS-normalised
+    query and key heads before the rotary embedding)."""
+    kw = dict(hidden_size=256, intermediate_size=512, num_hidden_layers=len(HEAD_MAPS),
+              num_attention_heads=H, num_key_value_heads=G, head_dim=D, vocab_size=256,
+              max_position_embeddings=4096, pad_token_id=0, bos_token_id=1, eos_token_id=None)
     torch.manual_seed(0)
-    model = LlamaForCausalLM(cfg).eval()
-    # larger q/k projections so the random model's attention is not uniform over the keys
+    if family == "llama":
+        from transformers import LlamaConfig, LlamaForCausalLM
+        model = LlamaForCausalLM(LlamaConfig(**kw)).eval()
+    else:
+        from transformers import Qwen3Config, Qwen3ForCausalLM
+        model = Qwen3ForCausalLM(Qwen3Config(**kw)).eval()
+    # sharper attention than the default initialisation gives (it would be uniform over the keys):
+    # larger q/k projections; with head normalisation, larger normalisation weights instead
     with torch.no_grad():
         for layer in model.model.layers:
-            layer.self_attn.q_proj.weight.mul_(6.0)
-            layer.self_attn.k_proj.weight.mul_(6.0)
+            if family == "llama":
+                layer.self_attn.q_proj.weight.mul_(6.0)
+                layer.self_attn.k_proj.weight.mul_(6.0)
+            else:
+                layer.self_attn.q_norm.weight.mul_(2.5)
+                layer.self_attn.k_norm.weight.mul_(2.0)
     return model.half().to(cuda)
 
 
@@ -36,10 +47,11 @@ def _bld(x):   # HF layout [B,h,L,D] -> [B,L,h,D] on the CPU
     return x.detach().cpu().transpose(1, 2).contiguous()
 
 
-def test_generate_through_registered_attention(cuda):
+@pytest.mark.parametrize("family", ["llama", "qwen3"])
+def test_generate_through_registered_attention(cuda, family):
     from kascade_amd.strategy import EfficientKascadeStrategy
     p, L, B, new_tokens = 10, 700, 2, 3
-    model = _tiny_llama(cuda)
+    model = _tiny_model(cuda, family)
     s = EfficientKascadeStrategy(ANCHORS, None, k=p, tile_size=TILE, rolling_prefill=True,
                                  head_mapping=HEAD_MAPS, register=True)
     model.config._attn_implementation = s.name
@@ -94,13 +106,14 @@ def test_generate_through_registered_attention(cuda):
             assert_close(o[:, 0], want, what)
 
 
-def test_full_budget_equals_sdpa_model(cuda):
+@pytest.mark.parametrize("family", ["llama", "qwen3"])
+def test_full_budget_equals_sdpa_model(cuda, family):
     """With k = 100 % every layer kind attends to all keys, so the model's logits must equal the
     same weights run with the library's SDPA attention: prefill, then two teacher-forced decode
     steps over the cache each implementation filled itself."""
     from kascade_amd.strategy import EfficientKascadeStrategy
     L, B = 500, 2
-    model = _tiny_llama(cuda)
+    model = _tiny_model(cuda, family)
     s = EfficientKascadeStrategy(ANCHORS, None, k=100, tile_size=TILE, rolling_prefill=True,
                                  head_mapping=HEAD_MAPS, register=True)
     gen = torch.Generator().manual_seed(2)

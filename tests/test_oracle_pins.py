@@ -292,6 +292,19 @@ def test_topk_agreement_metric():
     assert not ok
     ok, _, _ = orc.topk_agreement(s, torch.tensor([0, 2, 6]), 3, 6)       # out of the valid range
     assert not ok
+    # graded form: scores one fp16 step (2^-11 at 0.5..1) apart around the threshold 0.75
+    u = 2.0 ** -11
+    s = torch.tensor([0.9, 0.75 + 2 * u, 0.75, 0.75 - u, 0.75 - 3 * u, 0.1])
+    ok, rec, prec, worst, _ = orc.topk_set_quality(s, torch.tensor([0, 1, 2]), 3, 6)
+    assert ok and rec == 1.0 and prec == 1.0 and worst == 0.0
+    ok, rec, prec, worst, _ = orc.topk_set_quality(s, torch.tensor([0, 1, 3]), 3, 6)       # tie within 1 ulp
+    assert ok and rec == 1.0 and prec == 1.0 and worst == 1.0
+    ok, rec, prec, worst, _ = orc.topk_set_quality(s, torch.tensor([0, 2, 3]), 3, 6)       # misses tau + 2 ulp
+    assert ok and rec == 0.5 and prec == 1.0 and worst == 2.0
+    ok, rec, prec, worst, _ = orc.topk_set_quality(s, torch.tensor([0, 1, 4]), 3, 6)       # 3 ulps low
+    assert ok and rec == 1.0 and abs(prec - 2 / 3) < 1e-6 and worst == 3.0
+    ok, *_ = orc.topk_set_quality(s, torch.tensor([0, 0, 1]), 3, 6)
+    assert not ok
 
 
 # ----------------------------------------------------- strategy semantics
@@ -456,3 +469,57 @@ def test_rope_and_head_norm_vs_library():
         _, b = orc.rope_append(qa, ka, pk, cos_t, sin_t)
         dots.append(float((a * b).sum()))
     assert abs(dots[0] - dots[1]) < 2e-3 and abs(dots[0] - dots[2]) < 2e-3   # fp32 angles
+
+
+def test_attention_blocks_vs_library_decoder_layers():
+    """The oracle's stack of decoder attention blocks equals the attention halves of the
+    transformers library's own Qwen3 decoder layers (input norm, q/k/v projection, head norm,
+    rotary embedding, causal attention, output projection, residual) run in fp32 on shared
+    weights: a wrong row order in the packed projection, the norm after the rotation, a missing
+    residual or head norm would each fail."""
+    qwen3 = pytest.importorskip("transformers.models.qwen3.modeling_qwen3")
+    from transformers import Qwen3Config
+    D, Hh, Gg, B, L, hidden, layers = 16, 4, 2, 2, 21, 48, 3
+    cfg = Qwen3Config(hidden_size=hidden, num_attention_heads=Hh, num_key_value_heads=Gg, head_dim=D,
+                      rope_theta=1e6, max_position_embeddings=128, num_hidden_layers=layers,
+                      intermediate_size=64, vocab_size=32, rms_norm_eps=1e-6, attention_bias=False)
+    cfg._attn_implementation = "eager"
+    theta = cfg.rope_parameters["rope_theta"] if getattr(cfg, "rope_parameters", None) else cfg.rope_theta
+    torch.manual_seed(11)
+    mods = [qwen3.Qwen3DecoderLayer(cfg, layer_idx=l).eval() for l in range(layers)]
+    gen = torch.Generator().manual_seed(12)
+    with torch.no_grad():
+        for m in mods:       # non-trivial norm weights; sharper attention than the default init gives
+            for w in (m.input_layernorm.weight, m.self_attn.q_norm.weight, m.self_attn.k_norm.weight):
+                w.copy_(1 + 0.3 * torch.randn(w.shape, generator=gen))
+            m.self_attn.q_norm.weight.mul_(2.0)
+            for lin in (m.self_attn.q_proj, m.self_attn.k_proj, m.self_attn.v_proj, m.self_attn.o_proj):
+                lin.weight.copy_(torch.randn(lin.weight.shape, generator=gen) * lin.weight.shape[1] ** -0.5)
+    x = torch.randn(B, L, hidden, generator=gen)
+    pos = torch.arange(L)[None].expand(B, L)
+    rot = qwen3.Qwen3RotaryEmbedding(cfg)
+    mask = torch.zeros(L, L).masked_fill(torch.arange(L)[None] > torch.arange(L)[:, None], float("-inf"))[None, None]
+    want = x
+    with torch.no_grad():
+        pe = rot(x, pos)
+        for m in mods:       # the attention half of Qwen3DecoderLayer.forward
+            a = m.self_attn(hidden_states=m.input_layernorm(want), position_embeddings=pe,
+                            attention_mask=mask.expand(B, 1, L, L))[0]
+            want = want + a
+    d = lambda t: t.detach()
+    w_qkv = [torch.cat((d(m.self_attn.q_proj.weight), d(m.self_attn.k_proj.weight), d(m.self_attn.v_proj.weight)))
+             for m in mods]
+    cos, sin = orc.rope_angles(torch.arange(128), D, theta)
+    got = orc.attention_blocks_dense(x, w_qkv, [d(m.self_attn.o_proj.weight) for m in mods],
+                                     [d(m.input_layernorm.weight) for m in mods],
+                                     [d(m.self_attn.q_norm.weight) for m in mods],
+                                     [d(m.self_attn.k_norm.weight) for m in mods], cos, sin, Hh, Gg, 1e-6)
+    assert float(want.std()) > 0.5 and float((want - x).abs().max()) > 0.1
+    assert torch.allclose(got, want, atol=2e-5, rtol=1e-5), float((got - want).abs().max())
+    # sensitivity: the same oracle with key and value rows swapped in the packed projection is far off
+    swapped = [torch.cat((w[:Hh * D], w[(Hh + Gg) * D:], w[Hh * D:(Hh + Gg) * D])) for w in w_qkv]
+    bad = orc.attention_blocks_dense(x, swapped, [d(m.self_attn.o_proj.weight) for m in mods],
+                                     [d(m.input_layernorm.weight) for m in mods],
+                                     [d(m.self_attn.q_norm.weight) for m in mods],
+                                     [d(m.self_attn.k_norm.weight) for m in mods], cos, sin, Hh, Gg, 1e-6)
+    assert float((bad - want).abs().max()) > 1e-2
