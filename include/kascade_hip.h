@@ -111,6 +111,25 @@ int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K
                                     const kascade_half* k_new, const kascade_half* v_new,
                                     int32_t* sync_counters, void* stream);
 
+/* Reuse-layer decode over a paged cache whose index lists were translated to cache rows once, at
+ * the anchor (kascade_translate_indices_call): cache_rows [B,G,topk] holds page * page_size + slot
+ * of every selected token, so the path from a list entry to its K/V row has one dependent load
+ * instead of two (list -> block table -> row).  An anchor's selection serves every reuse layer up
+ * to the next anchor, all over the same block table, so the translation is paid once per anchor.
+ * No counterpart in the reference (its caches are contiguous).  Otherwise as
+ * kascade_decode_reuse_paged_call: sequence b consumes the first n(b) entries of its rows (n(b)
+ * from topk_percent and cache_seqlens, or topk).  cache_seqlens may be NULL when topk_percent
+ * <= 0 and nothing is appended.  The block table is used by the fused append only.  Entries are
+ * clamped to [0, num_pages * page_size). */
+int kascade_decode_reuse_rows_call(const kascade_half* Q, const kascade_half* K_pages,
+                                   const kascade_half* V_pages, const int32_t* cache_seqlens,
+                                   const int32_t* cache_rows, const int32_t* head_mapping,
+                                   float topk_percent, float* glse, float* Output_partial,
+                                   kascade_half* Output, int batch, int topk, int num_split,
+                                   const int32_t* block_table, int max_pages, int page_size,
+                                   int num_pages, const kascade_half* k_new,
+                                   const kascade_half* v_new, int32_t* sync_counters, void* stream);
+
 /* kascade_decode_reuse_paged_call for callers that cannot allocate device memory and have no
  * scratch of their own to pass: code under HIP graph capture, tight serving loops, harnesses
  * that forbid hipMalloc.  No counterpart in the reference.  The partial results of the splits

@@ -36,6 +36,8 @@ SIGNATURES = {
     "kascade_decode_reuse_call": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _P]),
     "kascade_decode_reuse_paged_call": (_I, [_P, _P, _P, _P, _P, _P, _F, _P, _P, _P, _I, _I, _I, _I,
                                              _P, _I, _I, _SP, _P, _P, _P, _P]),
+    "kascade_decode_reuse_rows_call": (_I, [_P, _P, _P, _P, _P, _P, _F, _P, _P, _P, _I, _I, _I, _P, _I, _I, _I,
+                                            _P, _P, _P, _P]),
     "kascade_decode_reuse_paged_noalloc_call": (_I, [_P, _P, _P, _P, _P, _P, _F, _P, _I, _I, _I, _I,
                                                      _P, _I, _I, _SP, _P, _P, _P]),
     "kascade_decode_dense_paged_call": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _I, _I, _SP,

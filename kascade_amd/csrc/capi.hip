@@ -196,6 +196,45 @@ int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K
                                            num_split, true, s), "decode_reuse combine");
 }
 
+int kascade_decode_reuse_rows_call(const kascade_half* Q, const kascade_half* K_pages,
+                                   const kascade_half* V_pages, const int32_t* cache_seqlens,
+                                   const int32_t* cache_rows, const int32_t* head_mapping,
+                                   float topk_percent, float* glse, float* Output_partial,
+                                   kascade_half* Output, int batch, int topk, int num_split,
+                                   const int32_t* block_table, int max_pages, int page_size,
+                                   int num_pages, const kascade_half* k_new,
+                                   const kascade_half* v_new, int32_t* sync_counters, void* stream) {
+    REQUIRE(Q && K_pages && V_pages && cache_rows && head_mapping && glse && Output_partial && Output &&
+                block_table, "decode_reuse_rows: null pointer argument");
+    REQUIRE(batch > 0 && topk > 0 && num_split > 0, "decode_reuse_rows: batch, topk, num_split must be > 0");
+    REQUIRE(batch <= 65535, "decode_reuse_rows: batch exceeds grid limit");
+    REQUIRE(!(topk_percent > 0.f) || cache_seqlens, "decode_reuse_rows: topk_percent needs cache_seqlens");
+    REQUIRE(!k_new || cache_seqlens, "decode_reuse_rows: the fused append needs cache_seqlens");
+    REQUIRE(aligned16(Q) && aligned16(K_pages) && aligned16(V_pages),
+            "decode_reuse_rows: Q/K/V must be 16-byte aligned");
+    int shift;
+    if (check_paging(block_table, max_pages, page_size, &shift)) return -1;
+    REQUIRE(num_pages > 0 && (long long)num_pages * page_size < (1LL << 31),
+            "decode_reuse_rows: num_pages out of range");
+    DecodeParams p{};
+    p.Q = H(Q); p.K = H(K_pages); p.V = H(V_pages);
+    p.seqlens = cache_seqlens; p.idx = cache_rows; p.head_map = head_mapping;
+    p.idx_physical = 1; p.max_row = num_pages * page_size - 1;
+    p.block_table = block_table; p.glse = glse; p.opart = Output_partial; p.scores = nullptr;
+    p.max_pages = max_pages; p.page_shift = shift; p.kv_stride_tokens = 0;
+    if (set_kv_strides(p, nullptr, block_table, 0)) return -1;
+    if (set_append(p, k_new, v_new, K_pages, V_pages)) return -1;
+    p.topk = topk; p.topk_percent = topk_percent; p.scores_stride = 0; p.num_split = num_split;
+    p.rows_per_split = rows_per_split(topk, num_split);
+    p.B = batch;
+    p.counters = sync_counters; p.out = H(Output);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (check_hip(launch_decode_split(p, true, true, false, s), "decode_reuse_rows split")) return -1;
+    if (sync_counters) return 0;
+    return check_hip(launch_decode_combine(glse, Output_partial, H(Output), nullptr, batch,
+                                           num_split, true, s), "decode_reuse_rows combine");
+}
+
 int kascade_decode_reuse_paged_noalloc_call(const kascade_half* Q, const kascade_half* K,
                                             const kascade_half* V, const int32_t* cache_seqlens,
                                             const int32_t* topk_indices, const int32_t* head_mapping,

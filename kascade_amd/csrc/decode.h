@@ -9,7 +9,7 @@ struct DecodeParams {
     const half_t* K;        // pages [P,page,G,D], or a strided [B,tokens,G,D] view
     const half_t* V;
     const int* seqlens;     // [B] or null
-    const int* idx;         // [B,G,topk] logical token ids (gather mode)
+    const int* idx;         // [B,G,topk] logical token ids (gather mode); physical cache rows with idx_physical
     const int* head_map;    // [G] (gather mode)
     const int* block_table; // [B,max_pages] or null
     float* glse;            // [B,H,num_split]
@@ -27,6 +27,8 @@ struct DecodeParams {
     int* counters;
     half_t* out;
     float* row_sums;
+    int idx_physical;       // gather mode over pages: idx holds cache rows (page * page_size + slot)
+    int max_row;            // ... each clamped to [0, max_row]
     int max_pages;
     int page_shift;
     int kv_stride_tokens;   // without seqlens: tokens per sequence; with: an upper bound

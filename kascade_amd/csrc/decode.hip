@@ -67,7 +67,10 @@ struct alignas(16) MergeState {  // one per wavefront after the in-wave merge
     float acc[kGroupSize][kDim];
 };
 
-template <bool GATHER, bool WITH_V, bool WRITE_SCORES>
+// PHYS (gather mode over a paged cache): the index lists hold physical cache rows
+// (page * page_size + slot, what translate_indices_kernel writes) instead of token positions, so
+// the block table is not on the path from a list entry to its K/V row.
+template <bool GATHER, bool WITH_V, bool WRITE_SCORES, bool PHYS = false>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2)))
 void decode_split_kernel(DecodeParams p) {
     __shared__ int s_row[GATHER ? kSubChunk : 1];
@@ -137,11 +140,14 @@ void decode_split_kernel(DecodeParams p) {
     // scattered among the working ones, which left some compute units with several streams and
     // others with none (four sequences of 131072..524288 tokens, 512 working workgroups: gather
     // 101 -> 86 us).  One sequence needs none of this; beyond 64 * kMapRounds sequences the
-    // workgroups keep their grid position.
+    // workgroups keep their grid position.  Neither do gather launches whose lists all have the
+    // same length (no per-sequence budget): every split of the grid has work, and leaving the
+    // numbering out takes one dependent trip to memory off the start of every workgroup.
     constexpr int kMapRounds = 4;
     int b, split, nsplit_b, seqlen;
     bool len_cut;
-    if (p.seqlens != nullptr && p.B > 1 && p.B <= 64 * kMapRounds) {
+    const bool ragged_rows = !GATHER || p.topk_percent > 0.f;
+    if (p.seqlens != nullptr && p.B > 1 && p.B <= 64 * kMapRounds && ragged_rows) {
         // every wavefront works it out for itself: lane l holds sequences l, l + 64, ...; no LDS,
         // no barrier, and the sequence's length comes out of the same loads (all issued first)
         const int w = blockIdx.y + gridDim.y * blockIdx.z;
@@ -204,6 +210,10 @@ void decode_split_kernel(DecodeParams p) {
     // A length that had to be cut down names a slot that does not exist: nothing is appended.
     const int newest = seqlen - 1;
     const bool can_append = p.k_new != nullptr && newest >= 0 && !len_cut;
+    int newest_row = -1;   // PHYS: the cache row of the newest token, what a list names it by
+    if (PHYS && can_append)
+        newest_row = (p.block_table[(size_t)b * p.max_pages + (newest >> p.page_shift)] << p.page_shift) +
+                     (newest & ((1 << p.page_shift) - 1));
     auto write_newest = [&]() {
         if (tid < 32) {
             const int part = tid >> 4, c = tid & 15;
@@ -403,6 +413,35 @@ void decode_split_kernel(DecodeParams p) {
         constexpr bool PAGED = decltype(paged_tag)::value;
         for (int c0 = r0; c0 < r1; c0 += kSubChunk) {
             const int cn = min(kSubChunk, r1 - c0);
+            Tile ta, tb;
+            // Physical rows, first sub-chunk: every wavefront fetches the rows of its first two
+            // tiles straight from the list and has their K/V loads in flight while the sub-chunk
+            // is being staged -- one trip to memory less before the first product.  Not when the
+            // launch appends the newest token: a tile that names it must be loaded after the write.
+            // Loads retire in order, so the order of issue is: these eight list entries, the
+            // staging's list loads, the K/V loads of the two tiles (which wait for the eight
+            // entries only), and then the staging consumes its entries with the K/V loads still
+            // in flight behind them.
+            const bool early = PHYS && c0 == r0 && !can_append;   // uniform over the workgroup
+            int er[2][4];
+            if (early) {
+#pragma unroll
+                for (int u = 0; u < 2; ++u)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        er[u][i] = idx_row[c0 + min(16 * (wave + 4 * u) + 4 * i + dq, cn - 1)];
+            }
+            auto early_tiles = [&]() {
+                if (early) {
+                    KASCADE_SCHED_FENCE();
+#pragma unroll
+                    for (int u = 0; u < 2; ++u)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            load_row(paged_tag, max(0, min(er[u][i], p.max_row)), u ? tb : ta, i);
+                    KASCADE_SCHED_FENCE();
+                }
+            };
             __syncthreads();
             // all of a thread's index loads first, then all of its block-table loads: two trips to
             // memory per sub-chunk instead of two per entry (the count per thread is a compile-time
@@ -412,17 +451,19 @@ void decode_split_kernel(DecodeParams p) {
                 int toks[kPer], rows[kPer];
 #pragma unroll
                 for (int j = 0; j < kPer; ++j) toks[j] = idx_row[c0 + min(tid + j * kThreads, cn - 1)];
+                early_tiles();
 #pragma unroll
                 for (int j = 0; j < kPer; ++j) {
-                    toks[j] = max(0, min(toks[j], seqlen - 1));   // a corrupt index must not leave the sequence
-                    rows[j] = PAGED ? p.block_table[(size_t)b * p.max_pages + (toks[j] >> p.page_shift)] : toks[j];
+                    // a corrupt entry must not leave the sequence (the cache, for physical rows)
+                    toks[j] = max(0, min(toks[j], PHYS ? p.max_row : seqlen - 1));
+                    rows[j] = (PAGED && !PHYS) ? p.block_table[(size_t)b * p.max_pages + (toks[j] >> p.page_shift)] : toks[j];
                 }
 #pragma unroll
                 for (int j = 0; j < kPer; ++j) {
                     const int i = tid + j * kThreads;
                     if (i < cn) {
-                        if (toks[j] == newest) s_found = c0;
-                        s_row[i] = PAGED ? (rows[j] << p.page_shift) + (toks[j] & page_mask) : rows[j];
+                        if (toks[j] == (PHYS ? newest_row : newest)) s_found = c0;
+                        s_row[i] = (PAGED && !PHYS) ? (rows[j] << p.page_shift) + (toks[j] & page_mask) : rows[j];
                     }
                 }
             };
@@ -440,10 +481,20 @@ void decode_split_kernel(DecodeParams p) {
                 for (int i = 0; i < 4; ++i)      // past the end: clamped, masked later
                     load_row(paged_tag, s_row[min(16 * t + 4 * i + dq, cn - 1)], tb, i);
             };
-            Tile ta, tb;
-            issue(wave, ta);
             const int ntiles = (cn + 15) / 16;
-            for (int t = wave; t < ntiles; t += 8) {
+            int t_first = wave;
+            if (early) {   // tiles wave and wave + 4 are in flight already
+                compute_tile(ta, 16 * wave + 4 * dq, cn);
+                KASCADE_SCHED_FENCE();
+                issue(wave + 8, ta);
+                KASCADE_SCHED_FENCE();
+                compute_tile(tb, 16 * (wave + 4) + 4 * dq, cn);
+                KASCADE_SCHED_FENCE();
+                t_first = wave + 8;
+            } else {
+                issue(wave, ta);
+            }
+            for (int t = t_first; t < ntiles; t += 8) {
                 issue(t + 4, tb);
                 KASCADE_SCHED_FENCE();   // the scheduler otherwise sinks the loads down to their first use
                 compute_tile(ta, 16 * t + 4 * dq, cn);
@@ -810,7 +861,9 @@ __global__ __launch_bounds__(256) void decode_aggregate_kernel(const float* __re
 hipError_t launch_decode_split(const DecodeParams& p, bool gather, bool with_v, bool write_scores,
                                hipStream_t stream) {
     dim3 grid(kGroups, p.num_split, p.B), block(kThreads);
-    if (gather) {
+    if (gather && p.idx_physical) {
+        hipLaunchKernelGGL((decode_split_kernel<true, true, false, true>), grid, block, 0, stream, p);
+    } else if (gather) {
         hipLaunchKernelGGL((decode_split_kernel<true, true, false>), grid, block, 0, stream, p);
     } else if (write_scores) {
         if (with_v)

@@ -227,6 +227,33 @@ def decode_reuse_paged(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_
     return out
 
 
+def decode_reuse_rows(Q, K_pages, V_pages, cache_seqlens, cache_rows, head_mapping, topk_percent, glse,
+                      Output_partial, block_table, page_size: int = 16, out=None, sync=None,
+                      k_new=None, v_new=None) -> torch.Tensor:
+    """Reuse decode over a paged cache from index lists already translated to cache rows
+    (``translate_indices`` of the anchor's selection): one dependent load fewer per row than
+    ``decode_reuse_paged``.  cache_rows [B,G,topk] int32."""
+    lib = _lib.init()
+    B = Q.shape[0]
+    _req(Q, torch.float16, "Q"); _req(K_pages, torch.float16, "K_pages"); _req(V_pages, torch.float16, "V_pages")
+    _req(cache_rows, torch.int32, "cache_rows"); _req(head_mapping, torch.int32, "head_mapping")
+    _req(glse, torch.float32, "glse"); _req(Output_partial, torch.float32, "Output_partial")
+    _req(block_table, torch.int32, "block_table")
+    if cache_seqlens is not None:
+        _req(cache_seqlens, torch.int32, "cache_seqlens")
+    if K_pages.dim() != 4 or K_pages.shape[1] != page_size or tuple(K_pages.shape[2:]) != (G, D) \
+            or K_pages.shape != V_pages.shape:
+        raise KascadeError(f"pages must be [num_pages,{page_size},{G},{D}]")
+    ns = glse.shape[2]
+    out = _out_buffer(out, B, Q.device)
+    _lib.check(lib.kascade_decode_reuse_rows_call(
+        _ptr(Q), _ptr(K_pages), _ptr(V_pages), _ptr(cache_seqlens), _ptr(cache_rows), _ptr(head_mapping),
+        float(topk_percent), _ptr(glse), _ptr(Output_partial), _ptr(out), B, cache_rows.shape[-1], ns,
+        _ptr(block_table), block_table.shape[1], page_size, K_pages.shape[0], *_new_rows(k_new, v_new, B),
+        _sync_arg(sync, B), _stream()))
+    return out
+
+
 NOALLOC_MAX_UNITS = 1024   # batch * num_split the library's built-in scratch holds
 
 

@@ -247,7 +247,10 @@ class PagedKascadeDecoder:
         self._hm = {None: torch.arange(G, device=dev, dtype=torch.int32)}
         for l, row in enumerate(head_mapping):
             self._hm[l] = torch.tensor(row, device=dev, dtype=torch.int32)
-        self._topk_to_reuse = None
+        self._topk_to_reuse = None      # the last anchor's selection as token positions
+        self._rows_to_reuse = None      # ... translated to cache rows, what the reuse launches gather from
+        widest = max(self.max_topk, budgets.topk_width(max_seqlen, k), budgets.CHUNK)
+        self._rows_buf = torch.empty(max_batch * G * widest, device=dev, dtype=torch.int32)
         self._counts = None
         self._valid_rows = torch.empty(max_batch * G, device=dev, dtype=torch.int32)
         self._nsel_rows = torch.empty(max_batch * G, device=dev, dtype=torch.int32)
@@ -304,6 +307,11 @@ class PagedKascadeDecoder:
             width = budgets.topk_width(max_len, self.k)
             self._topk_to_reuse = kernels.topk_indices(agg[:, :, :max_len], width, fill_value=0)
             self._pct = 0.0
+        # One translation per anchor: every reuse launch up to the next anchor reads the same block
+        # table, so the lists are turned into cache rows here and the gathers skip the table.
+        self._rows_to_reuse = kernels.translate_indices(
+            self._topk_to_reuse, block_table, max_len, self.page_size,
+            out=self._rows_buf[:self._topk_to_reuse.numel()].view(self._topk_to_reuse.shape))
         if layer != 0:
             o = self._reuse(q, k_pages, v_pages, block_table, seqlens, self._hm[None], out)
         return o
@@ -321,9 +329,9 @@ class PagedKascadeDecoder:
     def _reuse(self, q, k_pages, v_pages, block_table, seqlens, hm, out=None, k_new=None, v_new=None):
         B = q.shape[0]
         glse, part = self._scratch(B, self.ns_reuse)
-        return kernels.decode_reuse_paged(q, k_pages, v_pages, seqlens, self._topk_to_reuse, hm, self._pct,
-                                          glse, part, block_table=block_table, page_size=self.page_size, out=out,
-                                          sync=self._sync_reuse, k_new=k_new, v_new=v_new)
+        return kernels.decode_reuse_rows(q, k_pages, v_pages, seqlens, self._rows_to_reuse, hm, self._pct,
+                                         glse, part, block_table, page_size=self.page_size, out=out,
+                                         sync=self._sync_reuse, k_new=k_new, v_new=v_new)
 
     def reuse(self, layer, q, k_pages, v_pages, block_table, seqlens, out=None, k_new=None, v_new=None):
         """Reuse layer: attends to rows head_mapping[layer] of the last anchor's indices."""

@@ -671,3 +671,63 @@ def test_kv_append_beyond_the_block_table(cuda):
                 want_k[int(bt[b, tok // page]), tok % page] = kn[b, t]
                 want_v[int(bt[b, tok // page]), tok % page] = vn[b, t]
     assert torch.equal(Kc, want_k) and torch.equal(Vc, want_v)
+
+
+@pytest.mark.parametrize("seqlens,k,ns,pct", [([5000, 2100, 3300], 1792, 3, 0.0), ([9000], 4300, 1, 0.0),
+                                              ([2600, 1400, 700], 256, 2, 10.0), ([130], 100, 4, 0.0)])
+def test_reuse_from_translated_rows_equals_reuse_from_token_lists(cuda, seqlens, k, ns, pct):
+    """Lists translated to cache rows once (translate_indices) and gathered without the block
+    table give bit-identical outputs to the token lists through the table: same rows, same order
+    of accumulation; uniform and per-sequence budgets, several staged sub-chunks per split, the
+    fused merge, and the fused append with the newest token named in front, deep, or not at all."""
+    from kascade_amd import kernels
+    w = _paged_case(seqlens, seed=61)
+    B = len(seqlens)
+    gen = torch.Generator().manual_seed(k)
+    q, kp, vp = w.q.to(cuda), w.k_pages.to(cuda), w.v_pages.to(cuda)
+    lens, bt = w.seqlens.to(cuda), w.block_table.to(cuda)
+    hm = torch.randint(0, G, (G,), generator=gen).to(torch.int32).to(cuda)
+    glse, part = _scratch(B, ns, cuda)
+    sync = torch.zeros(B * G, dtype=torch.int32, device=cuda)
+    idx = _rand_idx(B, min(seqlens) - 1, k, gen).to(cuda)
+    rows = kernels.translate_indices(idx, bt, max(seqlens), w.page_size)
+    ps = w.page_size
+    want_rows = (bt.long().gather(1, (idx.long() // ps).view(B, -1)).view(idx.shape) * ps + idx.long() % ps)
+    assert torch.equal(rows.long(), want_rows)
+    for s in (None, sync):
+        a = kernels.decode_reuse_paged(q, kp, vp, lens, idx, hm, pct, glse, part, block_table=bt, page_size=ps, sync=s)
+        b = kernels.decode_reuse_rows(q, kp, vp, lens, rows, hm, pct, glse, part, bt, page_size=ps, sync=s)
+        assert torch.equal(a, b), f"rows vs token lists (fused merge: {s is not None})"
+    assert int(sync.abs().sum()) == 0
+    kc = orc.paged_to_contiguous(w.k_pages, w.block_table, seqlens)
+    vc = orc.paged_to_contiguous(w.v_pages, w.block_table, seqlens)
+    counts = [min(orc.n_kvcache(n, pct), k) for n in seqlens] if pct > 0 else None
+    assert_close(b, orc.reuse_decode(w.q, kc, vc, idx.cpu(), hm.tolist(), counts), "reuse from rows vs oracle")
+    # fused append
+    k_new = torch.empty(B, G, D, dtype=torch.float16, device=cuda)
+    v_new = torch.empty_like(k_new)
+    k_hole, v_hole = kp.clone(), vp.clone()
+    for bb, n in enumerate(seqlens):
+        pg, slot = int(w.block_table[bb, (n - 1) // ps]), (n - 1) % ps
+        k_new[bb], v_new[bb] = kp[pg, slot], vp[pg, slot]
+        k_hole[pg, slot] = float("nan"); v_hole[pg, slot] = float("nan")
+    for where in ("front", "deep", "absent"):
+        idx2 = idx.clone()
+        if where != "absent":
+            for bb, n in enumerate(seqlens):
+                idx2[bb, :, 0 if where == "front" else min(k, 128) - 3] = n - 1
+        rows2 = kernels.translate_indices(idx2, bt, max(seqlens), ps)
+        want = kernels.decode_reuse_paged(q, kp, vp, lens, idx2, hm, pct, glse, part, block_table=bt, page_size=ps)
+        kc2, vc2 = k_hole.clone(), v_hole.clone()
+        got = kernels.decode_reuse_rows(q, kc2, vc2, lens, rows2, hm, pct, glse, part, bt, page_size=ps,
+                                        k_new=k_new, v_new=v_new)
+        torch.cuda.synchronize()
+        assert torch.isfinite(got).all() and torch.equal(got, want), f"rows with fused append, newest {where}"
+        assert torch.equal(kc2, kp) and torch.equal(vc2, vp), f"cache after the fused append ({where})"
+    # entries outside the cache are clamped, never followed
+    bad = rows.clone()
+    bad[:, :, 1] = 2 ** 30
+    bad[:, :, 2] = -5
+    out = kernels.decode_reuse_rows(q, kp, vp, lens, bad, hm, pct, glse, part, bt, page_size=ps)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()
