@@ -683,21 +683,19 @@ void decode_split_kernel(DecodeParams p) {
             const float lref = (lse == -INFINITY) ? 0.f : lse;
             float o0 = 0.f, o1 = 0.f;
             float wl = fast_exp2(g0 - lref);   // 0 in lanes beyond the split count
+            // batches of kEarly partial outputs, every load of a batch in flight before the first
+            // is used (the first batch has been since before the log-sums were read)
+            for (int s0 = 0; s0 < ns; s0 += kEarly) {
+                if (s0 > 0) {
+                    if ((s0 & 63) == 0) wl = (s0 + lane < ns) ? fast_exp2(load_device(gl + s0 + lane) - lref) : 0.f;
 #pragma unroll
-            for (int j = 0; j < kEarly; ++j) {
-                const float w = __shfl(wl, j);
-                o0 += w * xe[j].x;
-                o1 += w * xe[j].y;
-            }
-            for (int s0 = 0; s0 < ns; s0 += 64) {
-                if (s0 > 0) wl = (s0 + lane < ns) ? fast_exp2(load_device(gl + s0 + lane) - lref) : 0.f;
-                const int cnt = min(64, ns - s0);
-#pragma unroll 8
-                for (int j = (s0 == 0 ? kEarly : 0); j < cnt; ++j) {
-                    const float w = __shfl(wl, j);
-                    const float2 x = load_device2(op + (size_t)(s0 + j) * kDim);
-                    o0 += w * x.x;
-                    o1 += w * x.y;
+                    for (int j = 0; j < kEarly; ++j) xe[j] = load_device2(op + (size_t)min(s0 + j, ns - 1) * kDim);
+                }
+#pragma unroll
+                for (int j = 0; j < kEarly; ++j) {
+                    const float w = __shfl(wl, (s0 & 63) + j);   // 0 for splits that do not exist
+                    o0 += w * xe[j].x;
+                    o1 += w * xe[j].y;
                 }
             }
             half2_t o = {(half_t)o0, (half_t)o1};

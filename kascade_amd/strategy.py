@@ -34,6 +34,7 @@ from . import budgets, kernels
 from ._lib import KascadeError
 
 H, G, D, TILE = 32, 8, 128, 32
+FUSED_MERGE_MAX_SPLITS = 32
 
 
 def get_head_mapping(model_name: str, recompute_layers: Sequence[int],
@@ -256,11 +257,11 @@ class PagedKascadeDecoder:
         self._nsel_rows = torch.empty(max_batch * G, device=dev, dtype=torch.int32)
         # arrival counters of the fused combine: zero now, set back to zero by every launch
         self._sync = torch.zeros(max_batch * G, device=dev, dtype=torch.int32) if fused_combine else None
-        # one workgroup merges all splits of a (sequence, KV head): a win up to about 16 splits
-        # (one trip to memory); beyond that the combine launch, which spreads the merge over
-        # 32 workgroups per sequence, is faster
-        self._sync_dense = self._sync if self.ns_dense <= 16 else None
-        self._sync_reuse = self._sync if self.ns_reuse <= 16 else None
+        # one workgroup merges all splits of a (sequence, KV head), 16 partial outputs per trip to
+        # memory: a win up to about 32 splits; beyond that the combine launch, which spreads the
+        # merge over 32 workgroups per sequence, is faster
+        self._sync_dense = self._sync if self.ns_dense <= FUSED_MERGE_MAX_SPLITS else None
+        self._sync_reuse = self._sync if self.ns_reuse <= FUSED_MERGE_MAX_SPLITS else None
 
     def _scratch(self, B, ns):
         return self._glse[:B * H * ns].view(B, H, ns), self._part[:B * H * ns * D].view(B, H, ns, D)
