@@ -36,19 +36,54 @@ N_LAYERS = 32
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 MFMA_PEAK_TFLOPS = 2500.0      # MI355X published dense fp16 MFMA rate
 H100_PREFILL_32K_MS = 6.42     # reference's published Kascade prefill ms @32768 (H100)
-# rocprofv3 FETCH_SIZE*2.0 + WRITE_SIZE*1.0 per launch at config 1 (profiles/prefill_reuse.md)
-MEASURED_TRAFFIC_BYTES = {"prefill_attn_reuse": 1.199e9}
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+
+
+def profiled_traffic(kernel):
+    """HBM bytes per launch of ``kernel`` from the committed rocprofv3 counter summary
+    (profiles/traffic.json: FETCH_SIZE and WRITE_SIZE per dispatch, each scaled by what the same
+    counter reads for a plain copy of known size), with the commit the profile was taken at; None
+    when the summary does not cover the kernel."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            table = json.load(f)
+        e = table["kernels"][kernel]
+        return {"bytes": e["hbm_bytes_per_launch"], "source": f"profiles/traffic.json@{table.get('commit', '?')}",
+                "workload": e.get("workload")}
+    except (OSError, KeyError, ValueError):
+        return None
 
 
 def log(msg):
     print(msg, file=sys.stderr, flush=True)
 
 
+N_SETS = 3
+
+
+def make_prefill_sets(L, dev):
+    """Every layer of a model has its own Q/K/V, so consecutive layers must not find each other's
+    K/V in the 256 MB last-level cache: anchors rotate over N_SETS independent input sets and the
+    reuse layers behind an anchor over N_SETS variants correlated with that anchor's set (its Q/K
+    plus 0.3-scaled noise, own V) -- more than 1 GB of other tensors pass between two uses of one.
+    Returns [(anchor_inputs, [(q, k, v) reuse variants])]."""
+    from kascade_amd import workloads
+    sets = []
+    for si in range(N_SETS):
+        a = workloads.prefill_inputs(1, L, seed=si, device=dev)
+        variants = [(a.q_reuse, a.k_reuse, a.v)]
+        for r in range(1, N_SETS):
+            variants.append((workloads.perturb(a.q, seed=3000 + 10 * si + r), workloads.perturb(a.k, seed=4000 + 10 * si + r),
+                             workloads.gaussian((1, L, G, D), seed=5000 + 10 * si + r, device=dev)))
+        sets.append((a, variants))
+    return sets
+
+
 SINGLE_KERNELS = ("membw_copy", "prefill_dense", "prefill_scores", "prefill_aggregate", "prefill_topk", "prefill_reuse",
                   "decode_dense", "decode_anchor0", "decode_anchor", "decode_topk", "decode_reuse", "rope_append")
 
 
-def run_single_kernel(name, iters, seq_len, dev, head_map):
+def run_single_kernel(name, iters, seq_len, dev, head_map, decode_len=65536):
     """Profiling mode (rocprofv3 -- python3 bench.py --kernel NAME): the named kernel alone on its
     benchmark workload -- prefill kernels on config 1 (32K), decode kernels on config 2 (B=16,
     L=65536, paged) rotating over three layer caches so the K/V rows come from HBM."""
@@ -85,44 +120,53 @@ def run_single_kernel(name, iters, seq_len, dev, head_map):
         print(json.dumps({"kernel": name, "iters": iters}), flush=True)
         return
     if name.startswith("prefill"):
+        # the named kernel on config 1, every call on the next of the rotating input sets
         L = seq_len
         T = math.ceil(L / TILE)
-        w = workloads.prefill_inputs(1, L, seed=0, device=dev)
+        sets = make_prefill_sets(L, dev)
         width = budgets.topk_width(L, PCT)
         valid, nsel = budgets.prefill_tile_budgets(L, TILE, PCT, True, width)
         valid = torch.tensor(valid, dtype=torch.int32, device=dev)
         nsel = torch.tensor(nsel, dtype=torch.int32, device=dev)
-        log_sum = kernels.prefill_recompute1(w.q, w.k)
-        scores = torch.empty(1, G, T, L, device=dev, dtype=torch.float16)
-        kernels.prefill_aggregate(w.q, w.k, log_sum, scores)
-        idx = kernels.topk_indices(scores, width, valid_len=valid, n_sel=nsel)
+        log_sums = [kernels.prefill_recompute1(a.q, a.k) for a, _ in sets]
+        scores = [torch.empty(1, G, T, L, device=dev, dtype=torch.float16) for _ in sets]
+        for (a, _), ls, sc in zip(sets, log_sums, scores):
+            kernels.prefill_aggregate(a.q, a.k, ls, sc)
+        idxs = [kernels.topk_indices(sc, width, valid_len=valid, n_sel=nsel) for sc in scores]
         hm = torch.tensor(head_map[1], dtype=torch.int32, device=dev)
-        fn = {"prefill_dense": lambda: kernels.prefill_recompute0(w.q, w.k, w.v),
-              "prefill_scores": lambda: kernels.prefill_recompute1(w.q, w.k),
-              "prefill_aggregate": lambda: kernels.prefill_aggregate(w.q, w.k, log_sum, scores),
-              "prefill_topk": lambda: kernels.topk_indices(scores, width, valid_len=valid, n_sel=nsel),
-              "prefill_reuse": lambda: kernels.prefill_reuse(w.q_reuse, w.k_reuse, w.v, idx, hm, float(PCT), True),
-              }[name]
-        for _ in range(iters):
-            fn()
+        for it in range(iters):
+            i, r = it % N_SETS, it // N_SETS % N_SETS
+            a = sets[i][0]
+            if name == "prefill_dense":
+                kernels.prefill_recompute0(a.q, a.k, a.v)
+            elif name == "prefill_scores":
+                kernels.prefill_recompute1(a.q, a.k)
+            elif name == "prefill_aggregate":
+                kernels.prefill_aggregate(a.q, a.k, log_sums[i], scores[i])
+            elif name == "prefill_topk":
+                kernels.topk_indices(scores[i], width, valid_len=valid, n_sel=nsel)
+            else:
+                q, k, v = sets[i][1][r]
+                kernels.prefill_reuse(q, k, v, idxs[i], hm, float(PCT), True)
     else:
-        seqlens = [65536] * 16
+        Ld = decode_len
+        seqlens = [Ld] * 16
         caches = [workloads.paged_decode_inputs(seqlens, seed=10 + i, device=dev, reuse_keys=False)
                   for i in range(3)]
         c0 = caches[0]
-        dec = PagedKascadeDecoder(PCT, head_map, ANCHORS, 16, 65536, device=dev)
-        dec.anchor(0, c0.q, c0.k_pages, c0.v_pages, c0.block_table, c0.seqlens, 65536, ragged=False)
-        agg = torch.rand(16, G, 65536, device=dev).half()
+        dec = PagedKascadeDecoder(PCT, head_map, ANCHORS, 16, Ld, device=dev)
+        dec.anchor(0, c0.q, c0.k_pages, c0.v_pages, c0.block_table, c0.seqlens, Ld, ragged=False)
+        agg = torch.rand(16, G, Ld, device=dev).half()
         for i in range(iters):
             c = caches[i % 3]
             if name == "decode_dense":
-                dec.dense(c.q, c.k_pages, c.v_pages, c0.block_table, c0.seqlens, 65536)
+                dec.dense(c.q, c.k_pages, c.v_pages, c0.block_table, c0.seqlens, Ld)
             elif name == "decode_anchor0":
-                dec.anchor(0, c.q, c.k_pages, c.v_pages, c0.block_table, c0.seqlens, 65536, ragged=False)
+                dec.anchor(0, c.q, c.k_pages, c.v_pages, c0.block_table, c0.seqlens, Ld, ragged=False)
             elif name == "decode_anchor":
-                dec.anchor(2, c.q, c.k_pages, c.v_pages, c0.block_table, c0.seqlens, 65536, ragged=False)
+                dec.anchor(2, c.q, c.k_pages, c.v_pages, c0.block_table, c0.seqlens, Ld, ragged=False)
             elif name == "decode_topk":
-                kernels.topk_indices(agg, budgets.topk_width(65536, PCT), fill_value=0)
+                kernels.topk_indices(agg, budgets.topk_width(Ld, PCT), fill_value=0)
             else:
                 dec.reuse(1, c.q, c.k_pages, c.v_pages, c0.block_table, c0.seqlens)
     torch.cuda.synchronize()
@@ -143,6 +187,8 @@ def main():
     ap.add_argument("--kernel", choices=sorted(SINGLE_KERNELS), default=None,
                     help="profiling mode: run only this kernel --iters times on its benchmark workload")
     ap.add_argument("--iters", type=int, default=5)
+    ap.add_argument("--decode-len", type=int, default=65536,
+                    help="profiling mode: context length of the 16 sequences of the decode kernels")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
@@ -157,8 +203,11 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    last_mean = [0.0]
+
     def ev_time(fn, n=5, warm=1, reps=1):
-        """Median duration (us) of fn() measured with events on the stream the kernels launch on.
+        """Median duration (us) of fn() measured with events on the stream the kernels launch on
+        (the mean of the same samples is left in last_mean[0]).
         reps > 1: that many calls back to back between the two events (for calls so short that
         the host's launch path would otherwise be part of what is timed), divided by reps."""
         for _ in range(warm):
@@ -174,27 +223,33 @@ def main():
             e.synchronize()
             ts.append(s.elapsed_time(e) * 1e3 / reps)
         ts.sort()
+        last_mean[0] = sum(ts) / len(ts)
         return ts[len(ts) // 2]
 
     head_map = get_head_mapping("Meta-Llama-3.1-8B-Instruct", list(ANCHORS))
 
     if args.kernel:
-        run_single_kernel(args.kernel, args.iters, args.seq_len, dev, head_map)
+        run_single_kernel(args.kernel, args.iters, args.seq_len, dev, head_map, args.decode_len)
         return
 
     # ------------------------------------------------------------------ prefill, 32K
     L = args.seq_len
-    log(f"[bench] generating prefill inputs L={L}")
-    w = workloads.prefill_inputs(1, L, seed=0, device=dev)
+    log(f"[bench] generating prefill inputs L={L}: {N_SETS} anchor sets x {N_SETS} reuse variants")
+    sets = make_prefill_sets(L, dev)
+    w = sets[0][0]
     strat = EfficientKascadeStrategy(list(ANCHORS), None, k=PCT, tile_size=TILE, rolling_prefill=True,
                                      head_mapping=head_map, register=False)
     width = budgets.topk_width(L, PCT)
     T = math.ceil(L / TILE)
+    anchor_order = sorted(ANCHORS)
 
     def prefill_layer(layer):
         if layer in ANCHORS:
-            return strat._prefill_recomp_forward(w.q, w.k, w.v, width, TILE, layer, PCT)
-        return strat._prefill_reuse_forward(w.q_reuse, w.k_reuse, w.v, PCT, layer)
+            a = sets[anchor_order.index(layer) % N_SETS][0]
+            return strat._prefill_recomp_forward(a.q, a.k, a.v, width, TILE, layer, PCT)
+        gov = max(x for x in anchor_order if x < layer)
+        q, k, v = sets[anchor_order.index(gov) % N_SETS][1][layer % N_SETS]
+        return strat._prefill_reuse_forward(q, k, v, PCT, layer)
 
     def prefill_step():
         for layer in range(N_LAYERS):
@@ -227,34 +282,65 @@ def main():
             gathered += n
     flop_reuse = 4.0 * D * (H // G) * TILE * G * sum_m
     if not args.decode_only:
-        t_dense = ev_time(lambda: kernels.prefill_dense(w.q, w.k, w.v), n=3)
-        t_p0 = ev_time(lambda: kernels.prefill_recompute0(w.q, w.k, w.v), n=3)
-        t_p1 = ev_time(lambda: kernels.prefill_recompute1(w.q, w.k), n=3)
-        log_sum = kernels.prefill_recompute1(w.q, w.k)
-        scores = torch.empty(1, G, T, L, device=dev, dtype=torch.float16)
-        t_agg = ev_time(lambda: kernels.prefill_aggregate(w.q, w.k, log_sum, scores), n=3)
-        valid, nsel = strat._tile_budgets(L, width, dev)
-        t_topk = ev_time(lambda: kernels.topk_indices(scores, width, valid_len=valid, n_sel=nsel), n=3, reps=3)
-        idx = kernels.topk_indices(scores, width, valid_len=valid, n_sel=nsel)
-        hm = strat._hm(1, dev)
-        t_reuse = ev_time(lambda: kernels.prefill_reuse(w.q_reuse, w.k_reuse, w.v, idx, hm, float(PCT), True), n=5, reps=3)
-        del scores, idx, log_sum
+        # every call of a timed kernel takes the next input set (cold caches, as in the timed step)
+        turn = [0]
 
-        def mfma(flop, us):
+        def nxt():
+            turn[0] += 1
+            return turn[0] % N_SETS
+
+        def anchor_set():
+            return sets[nxt()][0]
+
+        means = {}
+
+        def timed(name, fn, **kw):
+            t = ev_time(fn, **kw)
+            means[name] = last_mean[0]
+            return t
+        t_dense = timed("dense", lambda: (lambda a: kernels.prefill_dense(a.q, a.k, a.v))(anchor_set()), n=4)
+        t_p0 = timed("p0", lambda: (lambda a: kernels.prefill_recompute0(a.q, a.k, a.v))(anchor_set()), n=4)
+        t_p1 = timed("p1", lambda: (lambda a: kernels.prefill_recompute1(a.q, a.k))(anchor_set()), n=4)
+        valid, nsel = strat._tile_budgets(L, width, dev)
+        log_sums = [kernels.prefill_recompute1(a.q, a.k) for a, _ in sets]
+        # pooled scores and selections of the three sets (1.5 GiB of scores: also what keeps the
+        # selection kernel's input cold)
+        scores = [torch.empty(1, G, T, L, device=dev, dtype=torch.float16) for _ in sets]
+
+        def agg_call():
+            i = nxt()
+            kernels.prefill_aggregate(sets[i][0].q, sets[i][0].k, log_sums[i], scores[i])
+        t_agg = timed("agg", agg_call, n=4)
+        for i in range(N_SETS):
+            kernels.prefill_aggregate(sets[i][0].q, sets[i][0].k, log_sums[i], scores[i])
+        t_topk = timed("topk", lambda: kernels.topk_indices(scores[nxt()], width, valid_len=valid, n_sel=nsel), n=5, reps=3)
+        idxs = [kernels.topk_indices(sc, width, valid_len=valid, n_sel=nsel) for sc in scores]
+        hm = strat._hm(1, dev)
+
+        def reuse_call():
+            i, r = nxt(), turn[0] // N_SETS % N_SETS
+            q, k, v = sets[i][1][r]
+            kernels.prefill_reuse(q, k, v, idxs[i], hm, float(PCT), True)
+        t_reuse = timed("reuse", reuse_call, n=7, reps=3)
+        del scores, idxs, log_sums
+
+        def mfma(flop, us, mean_us):
             a = flop / us / 1e6
             return {"bound": "mfma", "achieved": round(a, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                    "frac": round(a / MFMA_PEAK_TFLOPS, 4), "us": round(us, 1)}
-        kern["prefill_attn_dense(QK+PV+lse)"] = mfma(flop_dense, t_p0)
-        kern["prefill_attn_dense(baseline, no lse)"] = mfma(flop_dense, t_dense)
-        kern["prefill_attn_scores(QK only)"] = mfma(flop_qk, t_p1)
-        kern["prefill_aggregate"] = mfma(flop_qk, t_agg)
-        kern["prefill_attn_reuse"] = mfma(flop_reuse, t_reuse)
-        kern["prefill_attn_reuse"]["gathered_GBps"] = round(gathered * G * D * 2 * 2 / t_reuse / 1e3, 1)
+                    "frac": round(a / MFMA_PEAK_TFLOPS, 4), "us": round(us, 1), "us_mean": round(mean_us, 1)}
+        kern["prefill_attn_dense(QK+PV+lse)"] = mfma(flop_dense, t_p0, means["p0"])
+        kern["prefill_attn_dense(baseline, no lse)"] = mfma(flop_dense, t_dense, means["dense"])
+        kern["prefill_attn_scores(QK only)"] = mfma(flop_qk, t_p1, means["p1"])
+        kern["prefill_aggregate"] = mfma(flop_qk, t_agg, means["agg"])
+        kern["prefill_attn_reuse"] = mfma(flop_reuse, t_reuse, means["reuse"])
+        # rows gathered per second; the rows of one launch add up to 7.1 GB out of 128 MB of K/V, so
+        # this is mostly cache bandwidth (L2 and the 256 MB last-level cache), not HBM
+        kern["prefill_attn_reuse"]["gathered_cache_GBps"] = round(gathered * G * D * 2 * 2 / t_reuse / 1e3, 1)
         sel_bytes = G * sum(32 * t for t in range(T)) * 2
         kern["topk_select(prefill)"] = {"bound": "hbm", "achieved": round(sel_bytes / t_topk / 1e3, 1),
                                         "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                         "frac": round(sel_bytes / t_topk / 1e3 / HBM_PEAK_GBS, 4),
-                                        "us": round(t_topk, 1)}
+                                        "us": round(t_topk, 1), "us_mean": round(means["topk"], 1)}
         t_a0 = t_p0 + t_agg + t_topk
         t_a = t_p1 + t_agg + t_topk + t_reuse
         prefill = {"seq_len": L, "dense_ms": round(t_dense / 1e3, 3), "anchor0_ms": round(t_a0 / 1e3, 3),
@@ -268,16 +354,19 @@ def main():
         roofline = dict(kern[dom])
         roofline["kernel"] = dom
         # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of the same kernel
-        # on this workload (scaled by the plain-copy calibration): summaries under profiles/.
-        roofline["traffic"] = MEASURED_TRAFFIC_BYTES.get(dom) if L == 32768 else None
+        # on this workload (scaled by the plain-copy calibration), read from the committed summary
+        tr = profiled_traffic(dom) if L == 32768 else None
+        roofline["traffic"] = tr["bytes"] if tr else None
+        roofline["traffic_source"] = tr["source"] if tr else None
     else:
         prefill, roofline = {}, {"bound": "mfma", "achieved": None, "peak": MFMA_PEAK_TFLOPS,
                                  "unit": "TFLOP/s", "frac": None, "traffic": None}
-    del w
+    del w, sets
     torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ paged decode
     decode = {}
+    roofline_decode = {}
     if not args.skip_decode:
         cases = [("cfg2_B16_L65536", [65536] * 16, False, 4),
                  ("B16_L131072", [131072] * 16, False, 3),
@@ -322,6 +411,15 @@ def main():
             counts = [budgets.decode_budget(n, PCT) if ragged else budgets.topk_width(n, PCT) for n in seqlens]
             reuse_bytes = sum(G * n * D * 2 * 2 + G * n * 4 for n in counts) + 2 * B * H * D * 2
             dense_bytes = sum(n * G * D * 2 * 2 for n in seqlens)
+            if name == "B16_L131072":
+                # the decode side's dominant kernel: the reuse gather (27 of 32 layers), one launch per call
+                tr = profiled_traffic("decode_reuse_B16_L131072")
+                roofline_decode.update({
+                    "bound": "hbm", "kernel": "decode_split_kernel<gather over cache rows>",
+                    "achieved": round(reuse_bytes / t_r / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(reuse_bytes / t_r / 1e3 / HBM_PEAK_GBS, 4), "us": round(t_r, 1),
+                    "traffic": tr["bytes"] if tr else None, "traffic_source": tr["source"] if tr else None,
+                    "workload": "reuse paged decode, batch 16 x 131072 tokens, 13184 gathered rows per (sequence, KV head)"})
             decode[name] = {
                 "dense_us": round(t_dense, 1), "anchor0_us": round(t_a0, 1), "anchor_us": round(t_a, 1),
                 "reuse_us": round(t_r, 1), "kascade_us_per_layer": round(t_kas, 1),
@@ -608,7 +706,7 @@ def main():
                                "32 layers (1 anchor-0, 4 anchor, 27 reuse)",
                    "seq_len": L, "layers_per_step": N_LAYERS,
                    "baseline_note": "vs_baseline = value / 6.42 ms, the reference's published H100 figure"},
-        "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "decode": decode, "stack": stack_res,
+        "roofline": roofline, "roofline_decode": roofline_decode or None, "cpu_baseline": cpu, "prefill": prefill, "decode": decode, "stack": stack_res,
         "library_ceilings": ceilings,
         "kernels": kern,
     }
