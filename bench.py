@@ -180,6 +180,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--seq-len", type=int, default=32768)
     ap.add_argument("--skip-decode", action="store_true")
+    ap.add_argument("--skip-long", action="store_true", help="skip the 65536- and 131072-token prefill timings")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-stack", action="store_true", help="skip the 36-layer chunked-prefill + decode stack")
     ap.add_argument("--skip-ceilings", action="store_true", help="skip the library copy / gather / GEMM rates")
@@ -363,6 +364,30 @@ def main():
                                  "unit": "TFLOP/s", "frac": None, "traffic": None}
     del w, sets
     torch.cuda.empty_cache()
+
+    # ---- longer prompts (the reference publishes 65536 and 131072 on H100: dense FA3 53.77 / 215.76 ms,
+    # Kascade 24.63 / 98.55 ms): the same layer kinds through the strategy; beyond 65536 tokens the
+    # anchors pool and select 512 tiles at a time
+    prefill_long = {}
+    if not args.decode_only and not args.skip_long:
+        for Ll in (65536, 131072):
+            log(f"[bench] prefill L={Ll}")
+            a = workloads.prefill_inputs(1, Ll, seed=7, device=dev)
+            wl = budgets.topk_width(Ll, PCT)
+            t_d = ev_time(lambda: kernels.prefill_dense(a.q, a.k, a.v), n=2)
+            t_a0 = ev_time(lambda: strat._prefill_recomp_forward(a.q, a.k, a.v, wl, TILE, 0, PCT), n=2)
+            t_a = ev_time(lambda: strat._prefill_recomp_forward(a.q, a.k, a.v, wl, TILE, 2, PCT), n=2)
+            t_r = ev_time(lambda: strat._prefill_reuse_forward(a.q_reuse, a.k_reuse, a.v, PCT, 1), n=3)
+            kas = (t_a0 + 4 * t_a + 27 * t_r) / 32
+            prefill_long[str(Ll)] = {"dense_ms": round(t_d / 1e3, 2), "anchor0_ms": round(t_a0 / 1e3, 2),
+                                     "anchor_ms": round(t_a / 1e3, 2), "reuse_ms": round(t_r / 1e3, 3),
+                                     "kascade_ms_per_layer": round(kas / 1e3, 2),
+                                     "speedup_vs_dense": round(t_d / kas, 3),
+                                     "dense_frac_mfma": round(2.0 * H * Ll * Ll * D / t_d / 1e6 / MFMA_PEAK_TFLOPS, 4)}
+            log(f"[bench] prefill L={Ll}: {prefill_long[str(Ll)]}")
+            strat._topk_to_reuse = None
+            del a
+            torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ paged decode
     decode = {}
@@ -706,7 +731,7 @@ def main():
                                "32 layers (1 anchor-0, 4 anchor, 27 reuse)",
                    "seq_len": L, "layers_per_step": N_LAYERS,
                    "baseline_note": "vs_baseline = value / 6.42 ms, the reference's published H100 figure"},
-        "roofline": roofline, "roofline_decode": roofline_decode or None, "cpu_baseline": cpu, "prefill": prefill, "decode": decode, "stack": stack_res,
+        "roofline": roofline, "roofline_decode": roofline_decode or None, "cpu_baseline": cpu, "prefill": prefill, "prefill_long": prefill_long, "decode": decode, "stack": stack_res,
         "library_ceilings": ceilings,
         "kernels": kern,
     }

@@ -237,6 +237,21 @@ int kascade_prefill_aggregate_call(const kascade_half* Q, const kascade_half* K,
                                    int seq_len, kascade_strides q_strides,
                                    kascade_strides kv_strides, int fill_invalid, void* stream);
 
+/* kascade_prefill_aggregate_call for a range of query tiles of a long prompt, so that the pooled
+ * scores of a prompt never have to exist all at once (they take L^2/4 bytes per sequence: 8 GiB at
+ * 131072 tokens).  The reference chunks only its torch.topk call, by rows, above 131072 tokens
+ * (EfficientKascadeStrategy.py:83-90) and keeps the whole score tensor.
+ *   Q        the q_len query rows at positions q_start .. q_start+q_len-1 (q_start a multiple of
+ *            32): a view into the prompt's Q, [B,q_len,H,D] through q_strides
+ *   K        the prompt's keys [B,>=q_start+q_len,G,D] through kv_strides
+ *   log_sum  [B,q_len,H] f32, the rows of the log-sum pass that belong to these queries
+ *   aggregate_scores [B,G,ceil(q_len/32),q_start+q_len] f16; row t is valid for keys < q_start+32t */
+int kascade_prefill_aggregate_range_call(const kascade_half* Q, const kascade_half* K,
+                                         const float* log_sum, kascade_half* aggregate_scores,
+                                         int batch, int q_start, int q_len,
+                                         kascade_strides q_strides, kascade_strides kv_strides,
+                                         int fill_invalid, void* stream);
+
 /* Reuse-layer prefill.  Same argument list as the reference's reuse `call`s
  * (…reuse_cp_async_ts32…groups8_rolling.cu:268 and …groups8.cu:260; DSL
  * reuse_kascade_gqa_prefill.py:147-198) plus strides and the rolling switch that

@@ -48,6 +48,7 @@ SIGNATURES = {
     "kascade_topk_call": (_I, [_P, _P, _I, _L, _I, _P, _P, _I, _I, _I, _P, _P]),
     "kascade_prefill_dense_call": (_I, [_P, _P, _P, _P, _P, _I, _I, Strides, Strides, _I, _P]),
     "kascade_prefill_aggregate_call": (_I, [_P, _P, _P, _P, _I, _I, Strides, Strides, _I, _P]),
+    "kascade_prefill_aggregate_range_call": (_I, [_P, _P, _P, _P, _I, _I, _I, Strides, Strides, _I, _P]),
     "kascade_prefill_reuse_call": (_I, [_P, _P, _P, _P, _P, _F, _P, _I, _I, _I, _I, Strides, Strides,
                                         _P]),
     "kascade_paged_kv_append_call": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, Strides, _P]),

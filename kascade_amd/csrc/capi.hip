@@ -411,6 +411,27 @@ int kascade_prefill_aggregate_call(const kascade_half* Q, const kascade_half* K,
                      "prefill_aggregate");
 }
 
+int kascade_prefill_aggregate_range_call(const kascade_half* Q, const kascade_half* K,
+                                         const float* log_sum, kascade_half* aggregate_scores,
+                                         int batch, int q_start, int q_len,
+                                         kascade_strides q_strides, kascade_strides kv_strides,
+                                         int fill_invalid, void* stream) {
+    REQUIRE(Q && K && log_sum && aggregate_scores, "prefill_aggregate_range: null pointer argument");
+    REQUIRE(batch > 0 && q_len > 0 && batch <= 65535, "prefill_aggregate_range: bad batch/q_len");
+    REQUIRE(q_start >= 0 && q_start % kTile == 0, "prefill_aggregate_range: q_start must be a multiple of 32");
+    REQUIRE((long long)q_start + q_len < (1LL << 31), "prefill_aggregate_range: q_start + q_len out of range");
+    REQUIRE(aligned16(Q) && aligned16(K), "prefill_aggregate_range: Q/K must be 16-byte aligned");
+    if (check_strides(q_strides, "Q") || check_strides(kv_strides, "K")) return -1;
+    PrefillParams p{};
+    p.Q = H(Q); p.K = H(K); p.V = H(K); p.log_sum_in = log_sum; p.agg = H(aggregate_scores);
+    p.q_sb = q_strides.b; p.q_sl = q_strides.l; p.q_sh = q_strides.h;
+    p.k_sb = kv_strides.b; p.k_sl = kv_strides.l; p.k_sh = kv_strides.h;
+    p.B = batch; p.L = q_start + q_len; p.Lq = q_len; p.q_start = q_start;
+    p.T = (q_len + kTile - 1) / kTile; p.fill_invalid = fill_invalid;
+    return check_hip(launch_prefill_aggregate(p, static_cast<hipStream_t>(stream)),
+                     "prefill_aggregate_range");
+}
+
 int kascade_prefill_reuse_call(const kascade_half* Q, const kascade_half* K, const kascade_half* V,
                                const int32_t* topk_indices, const int32_t* head_mapping,
                                float topk_percent, kascade_half* Output, int batch, int seq_len,

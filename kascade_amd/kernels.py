@@ -460,6 +460,27 @@ def prefill_aggregate(Q, K, log_sum, scores, fill_invalid: bool = False) -> None
                                                   qs, ks, 1 if fill_invalid else 0, _stream()))
 
 
+def prefill_aggregate_range(Q, K, log_sum, scores, q_start: int, q_len: int, fill_invalid: bool = False) -> None:
+    """``aggregate_kernel`` for the query tiles of rows [q_start, q_start+q_len) of a long prompt:
+    Q [B,L,H,D] and log_sum [B,L,H] are the whole prompt's, scores is
+    [B,G,ceil(q_len/32),q_start+q_len] fp16.  Lets an anchor layer pool and select a few hundred
+    tiles at a time instead of holding L^2/4 bytes of scores."""
+    lib = _lib.init()
+    _req(Q, torch.float16, "Q", False); _req(K, torch.float16, "K", False)
+    _req(log_sum, torch.float32, "log_sum"); _req(scores, torch.float16, "scores")
+    B, L = Q.shape[0], Q.shape[1]
+    if q_start % TILE or q_start < 0 or q_len <= 0 or q_start + q_len > L:
+        raise KascadeError("q_start must be a multiple of 32 and the range must lie inside the prompt")
+    T = (q_len + TILE - 1) // TILE
+    if tuple(scores.shape) != (B, G, T, q_start + q_len) or tuple(log_sum.shape) != (B, L, H):
+        raise KascadeError("scores must be [B,G,ceil(q_len/32),q_start+q_len] and log_sum [B,L,H]")
+    qs, ks = _blhd_strides(Q, "Q"), _blhd_strides(K, "K")
+    q_rows = Q[:, q_start:q_start + q_len]
+    ls_rows = log_sum[:, q_start:q_start + q_len].contiguous()      # a view for batch 1
+    _lib.check(lib.kascade_prefill_aggregate_range_call(_ptr(q_rows), _ptr(K), _ptr(ls_rows), _ptr(scores), B,
+                                                        q_start, q_len, qs, ks, 1 if fill_invalid else 0, _stream()))
+
+
 def prefill_reuse(Q, K, V, topk_idx, head_mapping, topk_percent, rolling: bool) -> torch.Tensor:
     """``prefill_reuse_kernel(Q, K, V, topk_indices, head_mapping, topk_percent) -> O``
     (out_idx=[6]; EfficientKascadeStrategy.py:61-70, 92, 97); ``rolling`` selects between the

@@ -56,6 +56,9 @@ def get_head_mapping(model_name: str, recompute_layers: Sequence[int],
 class EfficientKascadeStrategy:
     """Drop-in for the reference's EfficientKascadeStrategy (name ``efficient_kascade``)."""
 
+    WHOLE_PROMPT_SCORES = 65536   # prompts up to this length pool their tile scores in one tensor
+    SCORE_CHUNK_TILES = 512       # longer ones this many query tiles (16384 queries) at a time
+
     def __init__(self, recompute_layers: List[int], model_name: Optional[str], k=1, tile_size=1,
                  rolling_prefill=False, block_size=12288, head_mapping: Optional[List[List[int]]] = None,
                  register: bool = True):
@@ -109,10 +112,28 @@ class EfficientKascadeStrategy:
             log_sum, o = kernels.prefill_recompute0(Q, K, V)
         else:
             log_sum = kernels.prefill_recompute1(Q, K)
-        scores = torch.empty((B, G, T, L), device=Q.device, dtype=torch.float16)
-        kernels.prefill_aggregate(Q, K, log_sum, scores)
         valid, nsel = self._tile_budgets(L, topk, Q.device)
-        self._topk_to_reuse = kernels.topk_indices(scores, topk, valid_len=valid, n_sel=nsel)
+        if L <= self.WHOLE_PROMPT_SCORES:
+            scores = torch.empty((B, G, T, L), device=Q.device, dtype=torch.float16)
+            kernels.prefill_aggregate(Q, K, log_sum, scores)
+            self._topk_to_reuse = kernels.topk_indices(scores, topk, valid_len=valid, n_sel=nsel)
+        else:
+            # Long prompts: pool and select SCORE_CHUNK_TILES tiles at a time.  The whole score
+            # tensor would take L^2/4 bytes (8 GiB at 131072 tokens), and rows beyond 65536 entries
+            # go to the multi-workgroup selection, which takes a few thousand rows per call.  The
+            # reference keeps the whole tensor and chunks its torch.topk by rows above 131072
+            # tokens (EfficientKascadeStrategy.py:83-90); the indices are the same.
+            idx = torch.empty((B, G, T, topk), device=Q.device, dtype=torch.int32)
+            step = max(32, self.SCORE_CHUNK_TILES // B)
+            buf = torch.empty(B * G * step * L, device=Q.device, dtype=torch.float16)
+            for t0 in range(0, T, step):
+                t1 = min(t0 + step, T)
+                s, e = t0 * tile_size, min(t1 * tile_size, L)
+                scores = buf[:B * G * (t1 - t0) * e].view(B, G, t1 - t0, e)
+                kernels.prefill_aggregate_range(Q, K, log_sum, scores, s, e - s)
+                idx[:, :, t0:t1] = kernels.topk_indices(scores, topk, valid_len=valid[t0:t1].contiguous(),
+                                                        n_sel=nsel[t0:t1].contiguous(), fill_value=L - 1)
+            self._topk_to_reuse = idx
         if layer != 0:
             o = kernels.prefill_reuse(Q, K, V, self._topk_to_reuse, self._hm(None, Q.device), topk_percent,
                                       self.rolling_prefill)

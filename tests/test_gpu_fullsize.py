@@ -293,3 +293,49 @@ def test_config4_stack_36_layers_prefill_and_256_replayed_decode_steps(cuda):
             assert_close(gq[20], orc.reuse_decode(qs[20][:, t].cpu(), *kv[20], idx14, maps[20], [count]),
                          f"step {step} reuse layer 20")
     assert int(graph.seqlens[0]) == n_tok == graph.length
+
+
+@pytest.mark.parametrize("L", [65536, 131072])
+def test_prefill_beyond_32k(cuda, L):
+    """Prompts of 65536 and 131072 tokens (the reference publishes both): an anchor layer > 0
+    through the strategy -- at 131072 pooled and selected 512 tiles at a time, rows longer than
+    65536 entries on the multi-workgroup selection -- and a reuse layer through a head map, against
+    the oracle on sampled tiles; every tile's selection against the kernel's own pooled scores on
+    one chunk of tiles."""
+    from kascade_amd import kernels, budgets, workloads
+    from kascade_amd.strategy import EfficientKascadeStrategy
+    T = L // TILE
+    w = workloads.prefill_inputs(1, L, seed=6, device=cuda)
+    hm = [list(range(G)), w.head_mapping]
+    K = budgets.topk_width(L, P)
+    assert K == {65536: 6656, 131072: 13184}[L]
+    s = EfficientKascadeStrategy([0], None, k=P, tile_size=TILE, rolling_prefill=True, head_mapping=hm, register=False)
+    o_anchor = s._prefill_recomp_forward(w.q, w.k, w.v, K, TILE, 1, P)         # anchor > 0: own indices, sparse pass
+    idx = s._topk_to_reuse
+    assert tuple(idx.shape) == (1, G, T, K)
+    o_reuse = s._prefill_reuse_forward(w.q_reuse, w.k_reuse, w.v, P, 1)
+    q, k, v = w.q.cpu(), w.k.cpu(), w.v.cpu()
+    idx_c = idx.cpu()
+    for ta in (5, T // 2 + 3, T - 1):
+        n = min(K, orc.prefill_budget(ta, TILE, L, P, True, K))
+        pooled = orc.pooled_prefill_scores(q, k, TILE, tiles=(ta, ta + 1))[0, :, 0]          # [G, L]
+        for g in range(G):
+            ok, rec, prec, worst, msg = orc.topk_set_quality(pooled[g], idx_c[0, g, ta], n, ta * TILE)
+            assert ok and worst <= 2.0 and rec >= 0.999 and prec >= 0.999, f"tile {ta} head {g}: {msg}"
+        want = orc.reuse_prefill(q, k, v, idx_c, list(range(G)), TILE, True, P, tiles=(ta, ta + 1))
+        assert_close(o_anchor[:, ta * TILE:(ta + 1) * TILE], want, f"L={L}: anchor output, tile {ta}")
+        want = orc.reuse_prefill(w.q_reuse.cpu(), w.k_reuse.cpu(), v, idx_c, w.head_mapping, TILE, True, P,
+                                 tiles=(ta, ta + 1))
+        assert_close(o_reuse[:, ta * TILE:(ta + 1) * TILE], want, f"L={L}: reuse output, tile {ta}")
+    # the last 256 tiles: exact selection on the kernel's own pooled scores, every row
+    t0 = T - 256
+    log_sum = kernels.prefill_recompute1(w.q, w.k)
+    scores = torch.empty(1, G, 256, L, device=cuda, dtype=torch.float16)
+    kernels.prefill_aggregate_range(w.q, w.k, log_sum, scores, t0 * TILE, 256 * TILE, fill_invalid=True)
+    valid, nsel = budgets.prefill_tile_budgets(L, TILE, P, True, K)
+    vl = torch.tensor(valid[t0:], dtype=torch.int64, device=cuda).repeat(G)
+    ns = torch.tensor(nsel[t0:], dtype=torch.int64, device=cuda).repeat(G)
+    for g0 in range(0, G, 2):        # two KV heads at a time keeps the checker's temporaries small
+        rows = slice(g0 * 256, (g0 + 2) * 256)
+        _check_selection_on_device(scores.view(G * 256, L)[rows], idx[0, :, t0:].reshape(G * 256, K)[rows],
+                                   ns[rows], vl[rows])

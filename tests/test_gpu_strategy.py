@@ -153,3 +153,32 @@ def test_results_are_deterministic(cuda):
         outs.append((a, idx, r))
     for a, b in zip(*outs):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("L,B", [(1300, 1), (2050, 2)])
+def test_anchor_prefill_in_tile_chunks_equals_whole_prompt(cuda, L, B):
+    """Pooling and selecting a few tiles at a time (the path long prompts take) gives the index
+    tensor and the outputs of the whole-prompt path, bit for bit."""
+    from kascade_amd import workloads
+    from kascade_amd.strategy import EfficientKascadeStrategy
+    p = 10
+    w = workloads.prefill_inputs(B, L, seed=15, device=cuda)
+    hm = [list(range(G)), w.head_mapping]
+    K = orc.k_kern(L, p)
+    runs = []
+    for chunked in (False, True):
+        s = EfficientKascadeStrategy([0], None, k=p, tile_size=TILE, rolling_prefill=True, head_mapping=hm, register=False)
+        if chunked:
+            s.WHOLE_PROMPT_SCORES, s.SCORE_CHUNK_TILES = 256, 36
+        o0 = s._prefill_recomp_forward(w.q, w.k, w.v, K, TILE, 0, p)
+        i0 = s._topk_to_reuse.clone()
+        o1 = s._prefill_recomp_forward(w.q_reuse, w.k_reuse, w.v, K, TILE, 1, p)
+        runs.append((o0, i0, o1, s._topk_to_reuse.clone()))
+    T = (L + TILE - 1) // TILE
+    nsel = torch.tensor([min(K, orc.prefill_budget(t, TILE, L, p, True, K)) for t in range(T)])
+    live = torch.arange(K).view(1, -1) < torch.minimum(nsel, torch.arange(T) * TILE).view(-1, 1)     # consumed slots
+    for a, b in zip(*runs):
+        if a.dtype == torch.int32:
+            assert torch.equal(torch.where(live.to(a.device), a, 0), torch.where(live.to(a.device), b, 0))
+        else:
+            assert torch.equal(a, b)
