@@ -213,6 +213,19 @@ int kascade_topk_call(const kascade_half* scores, int32_t* out_idx, int rows, in
                       int uniform_len, const int32_t* valid_len, const int32_t* n_sel, int period,
                       int k, int fill_value, void* workspace, void* stream);
 
+/* kascade_topk_call with a second output: every selected position also as a row of a paged
+ * cache, out_rows[r, i] = block_table[r / rows_per_sequence, t / page_size] * page_size +
+ * t % page_size for t = out_idx[r, i] (fill slots included), which is what
+ * kascade_decode_reuse_rows_call and kascade_prefill_chunk_reuse_call gather from -- the
+ * translation of kascade_translate_indices_call without its launch.  out_rows [rows, k] i32 or
+ * NULL (then the block-table arguments are ignored); rows_per_sequence consecutive score rows
+ * belong to one sequence (8 for decode rows, 8 * tiles for prefill rows). */
+int kascade_topk_rows_call(const kascade_half* scores, int32_t* out_idx, int rows, int64_t row_stride,
+                           int uniform_len, const int32_t* valid_len, const int32_t* n_sel, int period,
+                           int k, int fill_value, void* workspace, int32_t* out_rows,
+                           const int32_t* block_table, int max_pages, int page_size,
+                           int rows_per_sequence, void* stream);
+
 /* ----------------------------------------------------------------- prefill */
 
 /* Anchor layer 0: dense causal GQA flash attention that also emits the log2

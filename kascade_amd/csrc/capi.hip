@@ -359,7 +359,26 @@ int64_t kascade_topk_workspace_bytes(int rows, int64_t row_len) {
 int kascade_topk_call(const kascade_half* scores, int32_t* out_idx, int rows, int64_t row_stride,
                       int uniform_len, const int32_t* valid_len, const int32_t* n_sel, int period,
                       int k, int fill_value, void* workspace, void* stream) {
+    return kascade_topk_rows_call(scores, out_idx, rows, row_stride, uniform_len, valid_len, n_sel,
+                                  period, k, fill_value, workspace, nullptr, nullptr, 0, 1, 1, stream);
+}
+
+int kascade_topk_rows_call(const kascade_half* scores, int32_t* out_idx, int rows, int64_t row_stride,
+                           int uniform_len, const int32_t* valid_len, const int32_t* n_sel, int period,
+                           int k, int fill_value, void* workspace, int32_t* out_rows,
+                           const int32_t* block_table, int max_pages, int page_size,
+                           int rows_per_sequence, void* stream) {
     REQUIRE(scores && out_idx, "topk: null pointer argument");
+    TopkRows tr{};
+    if (out_rows) {
+        REQUIRE(block_table && rows_per_sequence > 0, "topk: out_rows needs a block table and rows_per_sequence > 0");
+        int shift;
+        if (check_paging(block_table, max_pages, page_size, &shift)) return -1;
+        REQUIRE((long long)max_pages * page_size >= uniform_len,
+                "topk: block table shorter than the rows it is to translate");
+        tr.out_rows = out_rows; tr.block_table = block_table; tr.max_pages = max_pages;
+        tr.page_shift = shift; tr.rows_per_seq = rows_per_sequence;
+    }
     REQUIRE(rows >= 0 && k > 0 && row_stride > 0, "topk: rows >= 0, k > 0, row_stride > 0 required");
     REQUIRE(uniform_len >= 0 && uniform_len <= row_stride,
             "topk: uniform_len must be within [0, row_stride]");
@@ -369,9 +388,9 @@ int kascade_topk_call(const kascade_half* scores, int32_t* out_idx, int rows, in
     if (workspace && topk_split_workspace_bytes(rows, uniform_len) > 0)
         return check_hip(launch_topk_split(H(scores), out_idx, rows, row_stride, uniform_len,
                                            uniform_len, valid_len, n_sel, period, k, fill_value,
-                                           workspace, s), "topk (split)");
+                                           workspace, &tr, s), "topk (split)");
     return check_hip(launch_topk(H(scores), out_idx, rows, row_stride, uniform_len, valid_len, n_sel,
-                                 period, k, fill_value, s), "topk");
+                                 period, k, fill_value, &tr, s), "topk");
 }
 
 int kascade_prefill_dense_call(const kascade_half* Q, const kascade_half* K, const kascade_half* V,

@@ -68,23 +68,6 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
     const int q0 = p.q_start + q0l;     // its global position
     const int head = g * kGroupSize + wave;
 
-    // ---- Q fragments (B operand of S^T): query li (+32 qb), d chunk 16*ks + 8*lg ----
-    half8_t qf[NQB][8];
-#pragma unroll
-    for (int qb = 0; qb < NQB; ++qb) {
-        const int ql = q0l + 32 * qb + li;
-        const bool ok = ql < Lq;
-        const half_t* qp = p.Q + (long long)b * p.q_sb + (long long)min(ql, Lq - 1) * p.q_sl +
-                           (long long)head * p.q_sh + lg * 8;
-#pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
-            Pack16 t;
-            t.u = ld_global_16(qp + ks * 16);
-            if (!ok) t.u = uint4_t{0, 0, 0, 0};
-            qf[qb][ks] = t.h8;
-        }
-    }
-
     // ---- key regime of this block ----
     bool sparse = false;
     int n = 0, ng = 0;
@@ -171,20 +154,46 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
             for (int v = 0; v < 16; ++v) oT[qb][db][v] = 0.f;
     }
 
-    fetch_ids(0);
+    // Order of the tiles.  A sparse unit takes its diagonal tile first: the keys q0 .. q0+31 need
+    // no index list, so their loads leave at once and the first products run while the list of
+    // the first gathered tile and then its rows are still on their way -- one dependent trip to
+    // memory less before the first product of every unit, and units are short (28 tiles on
+    // average under rolling budgets).  Softmax is accumulated online, so the order is free.
+    auto tile_at = [&](int s) { return (REUSE && sparse) ? (s == 0 ? ng : s - 1) : s; };
+    fetch_ids(tile_at(0));
     issue_loads();
-    if (ntiles > 1) fetch_ids(1);
+    if (ntiles > 1) fetch_ids(tile_at(1));
 
-    // The diagonal tile of a sparse unit (32 keys, half the products) runs as a second phase of
-    // the tile loop; the phase loop is unrolled, so each phase is compiled with its key-block
-    // count as a constant and the tiles before the diagonal run straight-line code (with a
-    // run-time count every matrix instruction of the second half sits behind a branch).
+    // ---- Q fragments (B operand of S^T): query li (+32 qb), d chunk 16*ks + 8*lg; requested after
+    // the first tile's rows, which the first barrier waits for ----
+    half8_t qf[NQB][8];
+#pragma unroll
+    for (int qb = 0; qb < NQB; ++qb) {
+        const int ql = q0l + 32 * qb + li;
+        const bool ok = ql < Lq;
+        const half_t* qp = p.Q + (long long)b * p.q_sb + (long long)min(ql, Lq - 1) * p.q_sl +
+                           (long long)head * p.q_sh + lg * 8;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            Pack16 t;
+            t.u = ld_global_16(qp + ks * 16);
+            if (!ok) t.u = uint4_t{0, 0, 0, 0};
+            qf[qb][ks] = t.h8;
+        }
+    }
+
+
+    // The diagonal tile of a sparse unit (32 keys, half the products) runs as a phase of its own
+    // of the tile loop; the phase loop is unrolled, so each phase is compiled with its key-block
+    // count as a constant and the gathered tiles run straight-line code (with a run-time count
+    // every matrix instruction of the second half sits behind a branch).
 #pragma unroll
     for (int phase = 0; phase < (REUSE ? 2 : 1); ++phase) {
-    const bool diag_phase = (phase == 1);
-    const int t_begin = diag_phase ? ng : 0;
-    const int t_end = diag_phase ? (sparse ? ng + 1 : ng) : (REUSE && sparse ? ng : ntiles);
-    for (int ti = t_begin; ti < t_end; ++ti) {
+    const bool diag_phase = REUSE && (phase == 0);
+    const int s_begin = (REUSE && !diag_phase && sparse) ? 1 : 0;
+    const int s_end = diag_phase ? (sparse ? 1 : 0) : ntiles;
+    for (int sq = s_begin; sq < s_end; ++sq) {
+        const int ti = tile_at(sq);
         __syncthreads();
         // ---- registers -> LDS ----
 #pragma unroll
@@ -205,9 +214,9 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
             }
         }
         __syncthreads();
-        if (ti + 1 < ntiles) {
+        if (sq + 1 < ntiles) {
             issue_loads();
-            if (ti + 2 < ntiles) fetch_ids(ti + 2);
+            if (sq + 2 < ntiles) fetch_ids(tile_at(sq + 2));
         }
 
         // ---- S^T = K_tile Q^T ----

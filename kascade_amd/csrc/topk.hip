@@ -21,6 +21,23 @@ constexpr int kSplitMinLen = 65537;   // longer than a workgroup's registers hol
 constexpr int kSplitMaxRows = 4096;   // workspace is 8 KB per row for the coarse histogram
 namespace {
 
+// Optional second output: every selected position translated to its row of a paged cache
+// (block_table[sequence][pos / page] * page + pos % page), sequence = row / rows_per_seq.  What the
+// gather kernels of the reuse layers read, produced here so that no separate launch is needed.
+struct RowsOut {
+    int* rows;               // [rows, k] or null
+    const int* block_table;  // [sequences, max_pages]
+    int max_pages;
+    int page_shift;
+    int rows_per_seq;
+};
+
+__device__ __forceinline__ int to_cache_row(const RowsOut& ro, long long row, int pos) {
+    const int* bt = ro.block_table + (row / ro.rows_per_seq) * ro.max_pages;
+    pos = max(0, min(pos, (ro.max_pages << ro.page_shift) - 1));
+    return (bt[pos >> ro.page_shift] << ro.page_shift) + (pos & ((1 << ro.page_shift) - 1));
+}
+
 __device__ __forceinline__ uint32_t order_key(uint16_t bits) {
     // monotone map fp16 -> u16: negatives below positives, -inf lowest finite order
     return (bits & 0x8000u) ? (uint32_t)(uint16_t)~bits : (uint32_t)(bits | 0x8000u);
@@ -72,7 +89,7 @@ __device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t* s_wave
 __global__ __launch_bounds__(kThreads) void topk_select_kernel(
     const uint16_t* __restrict__ scores, int* __restrict__ out, long long row_stride,
     int uniform_len, const int* __restrict__ valid_len, const int* __restrict__ n_sel, int period,
-    int k, int fill) {
+    int k, int fill, RowsOut ro) {
     __shared__ uint32_t s_hist[kBins1];
     __shared__ uint32_t s_hist2[32];
     __shared__ uint32_t s_wave[kWaves];
@@ -86,9 +103,14 @@ __global__ __launch_bounds__(kThreads) void topk_select_kernel(
     n = max(0, min(n, k));
     const uint16_t* src = scores + row * row_stride;
     int* dst = out + row * (long long)k;
+    int* rdst = ro.rows ? ro.rows + row * (long long)k : nullptr;
+    auto put = [&](int slot, int pos) {
+        dst[slot] = pos;
+        if (rdst) rdst[slot] = to_cache_row(ro, row, pos);
+    };
 
     if (len <= n || n == 0) {
-        for (int i = tid; i < k; i += kThreads) dst[i] = (i < n) ? i : fill;
+        for (int i = tid; i < k; i += kThreads) put(i, (i < n) ? i : fill);
         return;
     }
     const bool aligned = ((reinterpret_cast<uintptr_t>(src) & 15) == 0);
@@ -171,10 +193,10 @@ __global__ __launch_bounds__(kThreads) void topk_select_kernel(
         for (int e = 0; e < 8; ++e) {
             if (e < nv) {
                 if (keys[e] > T) {
-                    dst[my_gt + min(my_eq, r)] = base + e;
+                    put(my_gt + min(my_eq, r), base + e);
                     ++my_gt;
                 } else if (keys[e] == T) {
-                    if (my_eq < r) dst[my_gt + my_eq] = base + e;
+                    if (my_eq < r) put(my_gt + my_eq, base + e);
                     ++my_eq;
                 }
             }
@@ -182,7 +204,7 @@ __global__ __launch_bounds__(kThreads) void topk_select_kernel(
         gt_base += total & 0xFFFFu;
         eq_base += total >> 16;
     }
-    for (int i = n + tid; i < k; i += kThreads) dst[i] = fill;
+    for (int i = n + tid; i < k; i += kThreads) put(i, fill);
 }
 
 
@@ -205,7 +227,7 @@ template <int MAXC>
 __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
     const uint16_t* __restrict__ scores, int* __restrict__ out, long long row_stride,
     int uniform_len, const int* __restrict__ valid_len, const int* __restrict__ n_sel, int period,
-    int k, int fill) {
+    int k, int fill, RowsOut ro) {
     constexpr int kCopies = 4;
     constexpr int kStage = kBins1 * kCopies;       // selected indices staged in the histogram's LDS
     __shared__ uint32_t s_hist[kBins1 * kCopies];
@@ -225,9 +247,14 @@ __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
     n = max(0, min(n, k));
     const uint16_t* src = scores + row * row_stride;
     int* dst = out + row * (long long)k;
+    int* rdst = ro.rows ? ro.rows + row * (long long)k : nullptr;
+    auto put = [&](int slot, int pos) {
+        dst[slot] = pos;
+        if (rdst) rdst[slot] = to_cache_row(ro, row, pos);
+    };
 
     if (len <= n || n == 0) {
-        for (int i = tid; i < k; i += kThreads) dst[i] = (i < n) ? i : fill;
+        for (int i = tid; i < k; i += kThreads) put(i, (i < n) ? i : fill);
         return;
     }
     const int nchunks = (len + kChunk - 1) / kChunk;   // <= MAXC (host)
@@ -421,7 +448,7 @@ __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
                 const int pos = (int)(my_gt + min(my_eq, r));
                 if (is_gt || (is_eq && my_eq < r)) {
                     if (staged) stage[pos] = base + e;
-                    else dst[pos] = base + e;
+                    else put(pos, base + e);
                 }
                 my_gt += is_gt ? 1u : 0u;
                 my_eq += is_eq ? 1u : 0u;
@@ -439,12 +466,24 @@ __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
                 v.z = (i + 2 < n) ? stage[i + 2] : fill;
                 v.w = (i + 3 < n) ? stage[i + 3] : fill;
                 *reinterpret_cast<int4*>(dst + i) = v;
+                if (rdst) {   // k % 4 == 0 here; the rows tensor has the layout of the index tensor
+                    int4 w;
+                    w.x = to_cache_row(ro, row, v.x);
+                    w.y = to_cache_row(ro, row, v.y);
+                    w.z = to_cache_row(ro, row, v.z);
+                    w.w = to_cache_row(ro, row, v.w);
+                    if ((reinterpret_cast<uintptr_t>(ro.rows) & 15) == 0) {
+                        *reinterpret_cast<int4*>(rdst + i) = w;
+                    } else {
+                        rdst[i] = w.x; rdst[i + 1] = w.y; rdst[i + 2] = w.z; rdst[i + 3] = w.w;
+                    }
+                }
             }
         } else {
-            for (int i = tid; i < k; i += kThreads) dst[i] = (i < n) ? stage[i] : fill;
+            for (int i = tid; i < k; i += kThreads) put(i, (i < n) ? stage[i] : fill);
         }
     } else {
-        for (int i = n + tid; i < k; i += kThreads) dst[i] = fill;
+        for (int i = n + tid; i < k; i += kThreads) put(i, fill);
     }
 }
 
@@ -629,7 +668,7 @@ __global__ __launch_bounds__(64) void topk_split_scan2_kernel(int max_chunks, Sp
 
 __global__ __launch_bounds__(kThreads) void topk_split_write_kernel(
     const uint16_t* __restrict__ scores, int* __restrict__ out, long long row_stride, int k,
-    int fill, int max_chunks, SplitWs ws) {
+    int fill, int max_chunks, SplitWs ws, RowsOut ro) {
     __shared__ uint32_t s_wave[kWaves];
     const int tid = threadIdx.x;
     const long long row = blockIdx.y;
@@ -637,13 +676,18 @@ __global__ __launch_bounds__(kThreads) void topk_split_write_kernel(
     const int len = (int)sel[6];
     const int n = (int)sel[5];
     int* dst = out + row * (long long)k;
+    int* rdst = ro.rows ? ro.rows + row * (long long)k : nullptr;
+    auto put = [&](int slot, int pos) {
+        dst[slot] = pos;
+        if (rdst) rdst[slot] = to_cache_row(ro, row, pos);
+    };
     const int c0 = blockIdx.x * kSplitChunk;
     if (blockIdx.x == 0) {
         if (sel[0] == 0) {
-            for (int i = tid; i < k; i += kThreads) dst[i] = (i < n) ? i : fill;
+            for (int i = tid; i < k; i += kThreads) put(i, (i < n) ? i : fill);
             return;
         }
-        for (int i = n + tid; i < k; i += kThreads) dst[i] = fill;
+        for (int i = n + tid; i < k; i += kThreads) put(i, fill);
     }
     if (sel[0] == 0 || c0 >= len) return;
     const int c1 = min(len, c0 + kSplitChunk);
@@ -673,10 +717,10 @@ __global__ __launch_bounds__(kThreads) void topk_split_write_kernel(
         for (int e = 0; e < 8; ++e) {
             if (e < nv) {
                 if (keys[e] > T) {
-                    dst[my_gt + min(my_eq, r)] = base + e;
+                    put(my_gt + min(my_eq, r), base + e);
                     ++my_gt;
                 } else if (keys[e] == T) {
-                    if (my_eq < r) dst[my_gt + my_eq] = base + e;
+                    if (my_eq < r) put(my_gt + my_eq, base + e);
                     ++my_eq;
                 }
             }
@@ -704,10 +748,23 @@ long long topk_split_workspace_bytes(int rows, long long row_len) {
     return 4ll * rows * (kBins1 + kSelWords + chunks * (kInfoWords + 2));
 }
 
+namespace {
+RowsOut rows_out(const TopkRows* tr) {
+    RowsOut ro{};
+    if (tr && tr->out_rows) {
+        ro.rows = tr->out_rows; ro.block_table = tr->block_table; ro.max_pages = tr->max_pages;
+        ro.page_shift = tr->page_shift; ro.rows_per_seq = tr->rows_per_seq;
+    }
+    return ro;
+}
+}  // namespace
+
 hipError_t launch_topk_split(const half_t* scores, int* out_idx, int rows, long long row_stride,
                              int max_len, int uniform_len, const int* valid_len, const int* n_sel,
-                             int period, int k, int fill, void* workspace, hipStream_t stream) {
+                             int period, int k, int fill, void* workspace, const TopkRows* tr,
+                             hipStream_t stream) {
     if (rows == 0) return hipSuccess;
+    const RowsOut ro = rows_out(tr);
     const int max_chunks = (max_len + kSplitChunk - 1) / kSplitChunk;
     SplitWs ws = carve_ws(workspace, rows, max_chunks);
     const uint16_t* src = reinterpret_cast<const uint16_t*>(scores);
@@ -723,27 +780,28 @@ hipError_t launch_topk_split(const half_t* scores, int* out_idx, int rows, long 
                        max_chunks, ws);
     hipLaunchKernelGGL(topk_split_scan2_kernel, dim3(rows), dim3(64), 0, stream, max_chunks, ws);
     hipLaunchKernelGGL(topk_split_write_kernel, grid, dim3(kThreads), 0, stream, src, out_idx,
-                       row_stride, k, fill, max_chunks, ws);
+                       row_stride, k, fill, max_chunks, ws, ro);
     return hipGetLastError();
 }
 
 hipError_t launch_topk(const half_t* scores, int* out_idx, int rows, long long row_stride,
                        int uniform_len, const int* valid_len, const int* n_sel, int period, int k,
-                       int fill, hipStream_t stream) {
+                       int fill, const TopkRows* tr, hipStream_t stream) {
     if (rows == 0) return hipSuccess;
+    const RowsOut ro = rows_out(tr);
     const uint16_t* src = reinterpret_cast<const uint16_t*>(scores);
     // rows that start 16-byte aligned and fit the register file of a workgroup are selected
     // from registers; anything else streams the row three times
     const bool aligned_rows = (reinterpret_cast<uintptr_t>(scores) & 15) == 0 && row_stride % 8 == 0;
     if (aligned_rows && uniform_len <= 4 * kChunk)
         hipLaunchKernelGGL(topk_select_reg_kernel<4>, dim3(rows), dim3(kThreads), 0, stream, src, out_idx,
-                           row_stride, uniform_len, valid_len, n_sel, period, k, fill);
+                           row_stride, uniform_len, valid_len, n_sel, period, k, fill, ro);
     else if (aligned_rows && uniform_len <= 8 * kChunk)
         hipLaunchKernelGGL(topk_select_reg_kernel<8>, dim3(rows), dim3(kThreads), 0, stream, src, out_idx,
-                           row_stride, uniform_len, valid_len, n_sel, period, k, fill);
+                           row_stride, uniform_len, valid_len, n_sel, period, k, fill, ro);
     else
         hipLaunchKernelGGL(topk_select_kernel, dim3(rows), dim3(kThreads), 0, stream, src, out_idx,
-                           row_stride, uniform_len, valid_len, n_sel, period, k, fill);
+                           row_stride, uniform_len, valid_len, n_sel, period, k, fill, ro);
     return hipGetLastError();
 }
 

@@ -357,13 +357,17 @@ def _topk_workspace(nbytes: int, device) -> torch.Tensor:
 
 
 def topk_indices(scores: torch.Tensor, k: int, valid_len=None, n_sel=None,
-                 uniform_len: Optional[int] = None, fill_value: Optional[int] = None
-                 ) -> torch.Tensor:
+                 uniform_len: Optional[int] = None, fill_value: Optional[int] = None,
+                 block_table: Optional[torch.Tensor] = None, page_size: int = 16,
+                 rows_out: Optional[torch.Tensor] = None):
     """Stands for ``torch.topk(scores, k, dim=-1).indices.to(int32)``
     (EfficientKascadeStrategy.py:82, 111) as an exact selection: row r delivers the
     n_sel largest of its first valid_len entries in slots [0, n_sel), ascending by
     index; remaining slots hold fill_value.  valid_len / n_sel are int32 device
-    tensors indexed by (row % len) or None for uniform rows."""
+    tensors indexed by (row % len) or None for uniform rows.
+    With ``block_table`` [B,max_pages] (scores [B, ..., L]) the call returns (indices, cache_rows):
+    the same selection also as rows of the paged cache (``translate_indices`` without its
+    launch), written to ``rows_out`` when given."""
     lib = _lib.init()
     _req(scores, torch.float16, "scores", contiguous=False)
     if scores.stride(-1) != 1:
@@ -394,11 +398,26 @@ def topk_indices(scores: torch.Tensor, k: int, valid_len=None, n_sel=None,
     ulen = Lrow if uniform_len is None else uniform_len
     ws_bytes = lib.kascade_topk_workspace_bytes(rows, ulen)
     ws = _topk_workspace(ws_bytes, scores.device) if ws_bytes > 0 else None
-    _lib.check(lib.kascade_topk_call(
-        _ptr(scores), _ptr(out), rows, row_stride, ulen,
-        _ptr(valid_len), _ptr(n_sel), period, k, (Lrow - 1) if fill_value is None else fill_value,
-        _ptr(ws), _stream()))
-    return out
+    fill = (Lrow - 1) if fill_value is None else fill_value
+    if block_table is None:
+        _lib.check(lib.kascade_topk_call(
+            _ptr(scores), _ptr(out), rows, row_stride, ulen,
+            _ptr(valid_len), _ptr(n_sel), period, k, fill, _ptr(ws), _stream()))
+        return out
+    _req(block_table, torch.int32, "block_table")
+    nseq = block_table.shape[0]
+    if scores.shape[0] != nseq or rows % nseq:
+        raise KascadeError("block_table needs one row per sequence (the leading dimension of scores)")
+    if rows_out is None:
+        rows_out = torch.empty_like(out)
+    else:
+        _req(rows_out, torch.int32, "rows_out")
+        if tuple(rows_out.shape) != tuple(out.shape):
+            raise KascadeError("rows_out must have the shape of the index tensor")
+    _lib.check(lib.kascade_topk_rows_call(
+        _ptr(scores), _ptr(out), rows, row_stride, ulen, _ptr(valid_len), _ptr(n_sel), period, k, fill,
+        _ptr(ws), _ptr(rows_out), _ptr(block_table), block_table.shape[1], page_size, rows // nseq, _stream()))
+    return out, rows_out
 
 
 # --------------------------------------------------------------- prefill

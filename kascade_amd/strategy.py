@@ -322,18 +322,17 @@ class PagedKascadeDecoder:
         if ragged:
             width = budgets.decode_budget(max_len, self.k)
             lens_rows, counts = self._row_budgets(seqlens)
-            self._topk_to_reuse = kernels.topk_indices(agg[:, :, :max_len], width, valid_len=lens_rows,
-                                                       n_sel=counts, fill_value=0)
-            self._pct = float(self.k)
         else:
             width = budgets.topk_width(max_len, self.k)
-            self._topk_to_reuse = kernels.topk_indices(agg[:, :, :max_len], width, fill_value=0)
-            self._pct = 0.0
-        # One translation per anchor: every reuse launch up to the next anchor reads the same block
-        # table, so the lists are turned into cache rows here and the gathers skip the table.
-        self._rows_to_reuse = kernels.translate_indices(
-            self._topk_to_reuse, block_table, max_len, self.page_size,
-            out=self._rows_buf[:self._topk_to_reuse.numel()].view(self._topk_to_reuse.shape))
+            lens_rows = counts = None
+        # One translation per anchor, inside the selection launch: every reuse launch up to the
+        # next anchor reads the same block table, so the selection also leaves its lists as cache
+        # rows and the gathers skip the table.
+        self._topk_to_reuse, self._rows_to_reuse = kernels.topk_indices(
+            agg[:, :, :max_len], width, valid_len=lens_rows, n_sel=counts, fill_value=0,
+            block_table=block_table, page_size=self.page_size,
+            rows_out=self._rows_buf[:B * G * width].view(B, G, width))
+        self._pct = float(self.k) if ragged else 0.0
         if layer != 0:
             o = self._reuse(q, k_pages, v_pages, block_table, seqlens, self._hm[None], out)
         return o
@@ -426,8 +425,8 @@ class PagedKascadePrefill:
         scores = self._score_buffer(B, T, Lk)
         kernels.prefill_chunk_aggregate(q, k_pages, log_sum, scores, block_table, q_start, self.page_size)
         valid, nsel = self._tile_budgets(q_start, Lq, width)
-        self._topk_to_reuse = kernels.topk_indices(scores, width, valid_len=valid, n_sel=nsel)
-        self._rows_to_reuse = kernels.translate_indices(self._topk_to_reuse, block_table, Lk, self.page_size)
+        self._topk_to_reuse, self._rows_to_reuse = kernels.topk_indices(
+            scores, width, valid_len=valid, n_sel=nsel, block_table=block_table, page_size=self.page_size)
         if layer != 0:
             o = self._reuse(q, k_pages, v_pages, block_table, q_start, self._hm[None])
         return o

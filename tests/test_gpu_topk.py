@@ -150,3 +150,24 @@ def test_topk_crowded_thresholds_and_special_values(cuda, L, K):
     torch.cuda.synchronize()
     # signed zeros compare equal as values; the multiset check works on values, so it holds either way
     _check_exact_sets(sc, idx, K, f"L={L} K={K}")
+
+
+@pytest.mark.parametrize("L,k,rows_per_seq", [(5000, 512, 8), (70016, 7040, 8), (20000, 2048, 16), (1000, 128, 8)])
+def test_topk_second_output_as_cache_rows(cuda, L, k, rows_per_seq):
+    """The selection's second output equals the translation launch applied to its first output
+    (register kernel, streaming kernel for unaligned rows, multi-workgroup path for long rows)."""
+    from kascade_amd import kernels
+    gen = torch.Generator().manual_seed(L + k)
+    nseq, page = 3, 16
+    pages = (L + page - 1) // page
+    scores = torch.rand(nseq, rows_per_seq, L, generator=gen).half().to(cuda)
+    bt = torch.randperm(nseq * pages, generator=gen).to(torch.int32).view(nseq, pages).to(cuda)
+    valid = torch.randint(L // 2, L + 1, (nseq * rows_per_seq,), generator=gen).to(torch.int32).to(cuda)
+    nsel = torch.randint(1, k + 1, (nseq * rows_per_seq,), generator=gen).to(torch.int32).to(cuda)
+    for view in (scores, scores[:, :, 1:]):          # the second view has rows that are not 16-byte aligned
+        Lv = view.shape[-1]
+        want = kernels.topk_indices(view, k, valid_len=valid.clamp(max=Lv), n_sel=nsel, fill_value=0)
+        got, rows = kernels.topk_indices(view, k, valid_len=valid.clamp(max=Lv), n_sel=nsel, fill_value=0,
+                                         block_table=bt, page_size=page)
+        assert torch.equal(got, want)
+        assert torch.equal(rows, kernels.translate_indices(want, bt, Lv, page))
