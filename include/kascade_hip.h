@@ -45,6 +45,20 @@ typedef struct {
     int64_t b, l, h;
 } kascade_strides;
 
+/* Tensor shape of a call.  The reference kernels exist for one shape only (32 query heads, 8 KV
+ * heads, head dimension 128, fp16: EfficientKascadeStrategy.py:19-21, README.md:74-75), and the
+ * entry points named after them take no shape.  Their `*_shaped_call` twins take this descriptor
+ * as first argument and the argument list of the plain entry after it; every size that the
+ * comments give as 32 / 8 / 128 reads 4*kv_heads / kv_heads / head_dim there, and kascade_half
+ * means an element of `dtype`.  A KV head always serves four query heads.  Pooled scores stay
+ * fp16 for both element types.  No counterpart in the reference. */
+enum { KASCADE_F16 = 0, KASCADE_BF16 = 1 };
+typedef struct {
+    int32_t kv_heads; /* >= 1; query heads = 4 * kv_heads */
+    int32_t head_dim; /* 64 or 128 */
+    int32_t dtype;    /* KASCADE_F16 or KASCADE_BF16 */
+} kascade_shape;
+
 /* Replaces `init()` of every reference kernel object (e.g. decode reuse .cu:253-258):
  * one-time device query and kernel attribute set-up for the current device. */
 int kascade_init(void);

@@ -52,6 +52,9 @@ int check_hip(hipError_t e, const char* what) {
 
 inline const half_t* H(const kascade_half* p) { return reinterpret_cast<const half_t*>(p); }
 inline half_t* H(kascade_half* p) { return reinterpret_cast<half_t*>(p); }
+// element tensors whose type (fp16 or bf16) the shape decides
+inline const void* E(const kascade_half* p) { return p; }
+inline void* E(kascade_half* p) { return p; }
 
 // Device address of `scratch` on the current device, looked up once per device.
 int noalloc_scratch(float** out) {
@@ -79,6 +82,23 @@ int check_strides(const kascade_strides& s, const char* name) {
     return 0;
 }
 
+// Shape of the tensors a call works on: KV heads, head dimension, element kind.  Query heads are
+// always kGroupSize per KV head.  The entry points without a shape argument use the reference's.
+struct Shape {
+    int G, D, elem;
+    int H() const { return G * kGroupSize; }
+};
+const Shape kRefShape{kGroups, kDim, kElemF16};
+
+int get_shape(const kascade_shape* in, Shape* out) {
+    REQUIRE(in, "shape: null pointer argument");
+    REQUIRE(in->kv_heads >= 1 && in->kv_heads <= 65535, "shape: kv_heads out of range");
+    REQUIRE(in->head_dim == 64 || in->head_dim == 128, "shape: head_dim must be 64 or 128, got %d", in->head_dim);
+    REQUIRE(in->dtype == KASCADE_F16 || in->dtype == KASCADE_BF16, "shape: dtype must be KASCADE_F16 or KASCADE_BF16");
+    out->G = in->kv_heads; out->D = in->head_dim; out->elem = in->dtype == KASCADE_BF16 ? kElemBF16 : kElemF16;
+    return 0;
+}
+
 int rows_per_split(long long max_rows, int num_split) {
     long long r = (max_rows + num_split - 1) / num_split;
     return (int)(((r + 63) / 64) * 64);
@@ -98,12 +118,13 @@ int check_paging(const int32_t* block_table, int max_pages, int page_size, int* 
 
 // K/V addressing of the decode calls without a block table: `strides` (elements, may be NULL
 // for the contiguous [B,kv_stride_tokens,G,D] cache).
-int set_kv_strides(DecodeParams& p, const kascade_strides* strides, const int32_t* block_table,
-                   int kv_stride_tokens) {
+int set_kv_strides(DecodeParams& p, const Shape& sh, const kascade_strides* strides,
+                   const int32_t* block_table, int kv_stride_tokens) {
+    p.G = sh.G; p.head_dim = sh.D; p.elem = sh.elem;
     if (!strides) {
-        p.kv_stride_b = (long long)kv_stride_tokens * kGroups * kDim;
-        p.kv_stride_l = kGroups * kDim;
-        p.kv_stride_h = kDim;
+        p.kv_stride_b = (long long)kv_stride_tokens * sh.G * sh.D;
+        p.kv_stride_l = sh.G * sh.D;
+        p.kv_stride_h = sh.D;
         return 0;
     }
     REQUIRE(!block_table, "kv_strides and block_table exclude each other");
@@ -160,7 +181,9 @@ int kascade_decode_reuse_call(const kascade_half* Q, const kascade_half* K, cons
                                            stream);
 }
 
-int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K,
+}  // extern "C"
+namespace {
+int decode_reuse_paged_impl(const Shape& sh, const kascade_half* Q, const kascade_half* K,
                                     const kascade_half* V, const int32_t* cache_seqlens,
                                     const int32_t* topk_indices, const int32_t* head_mapping,
                                     float topk_percent, float* glse, float* Output_partial,
@@ -183,7 +206,7 @@ int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K
     p.seqlens = cache_seqlens; p.idx = topk_indices; p.head_map = head_mapping;
     p.block_table = block_table; p.glse = glse; p.opart = Output_partial; p.scores = nullptr;
     p.max_pages = max_pages; p.page_shift = shift; p.kv_stride_tokens = kv_stride_tokens;
-    if (set_kv_strides(p, kv_strides, block_table, kv_stride_tokens)) return -1;
+    if (set_kv_strides(p, sh, kv_strides, block_table, kv_stride_tokens)) return -1;
     if (set_append(p, k_new, v_new, K, V)) return -1;
     p.topk = topk; p.topk_percent = topk_percent; p.scores_stride = 0; p.num_split = num_split;
     p.rows_per_split = rows_per_split(topk, num_split);
@@ -192,11 +215,40 @@ int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (check_hip(launch_decode_split(p, true, true, false, s), "decode_reuse split")) return -1;
     if (sync_counters) return 0;   // the split kernel's last workgroups have combined
-    return check_hip(launch_decode_combine(glse, Output_partial, H(Output), nullptr, batch,
-                                           num_split, true, s), "decode_reuse combine");
+    return check_hip(launch_decode_combine(glse, Output_partial, E(Output), nullptr, batch, sh.H(), num_split, true, sh.D, sh.elem, s), "decode_reuse combine");
+}
+}  // namespace
+extern "C" {
+
+int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K,
+                                    const kascade_half* V, const int32_t* cache_seqlens,
+                                    const int32_t* topk_indices, const int32_t* head_mapping,
+                                    float topk_percent, float* glse, float* Output_partial,
+                                    kascade_half* Output, int batch, int kv_stride_tokens,
+                                    int topk, int num_split, const int32_t* block_table,
+                                    int max_pages, int page_size, const kascade_strides* kv_strides,
+                                    const kascade_half* k_new, const kascade_half* v_new,
+                                    int32_t* sync_counters, void* stream) {
+    return decode_reuse_paged_impl(kRefShape, Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_percent, glse, Output_partial, Output, batch, kv_stride_tokens, topk, num_split, block_table, max_pages, page_size, kv_strides, k_new, v_new, sync_counters, stream);
 }
 
-int kascade_decode_reuse_rows_call(const kascade_half* Q, const kascade_half* K_pages,
+int kascade_decode_reuse_paged_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K,
+                                    const kascade_half* V, const int32_t* cache_seqlens,
+                                    const int32_t* topk_indices, const int32_t* head_mapping,
+                                    float topk_percent, float* glse, float* Output_partial,
+                                    kascade_half* Output, int batch, int kv_stride_tokens,
+                                    int topk, int num_split, const int32_t* block_table,
+                                    int max_pages, int page_size, const kascade_strides* kv_strides,
+                                    const kascade_half* k_new, const kascade_half* v_new,
+                                    int32_t* sync_counters, void* stream) {
+    Shape sh;
+    if (get_shape(shape, &sh)) return -1;
+    return decode_reuse_paged_impl(sh, Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_percent, glse, Output_partial, Output, batch, kv_stride_tokens, topk, num_split, block_table, max_pages, page_size, kv_strides, k_new, v_new, sync_counters, stream);
+}
+
+}  // extern "C"
+namespace {
+int decode_reuse_rows_impl(const Shape& sh, const kascade_half* Q, const kascade_half* K_pages,
                                    const kascade_half* V_pages, const int32_t* cache_seqlens,
                                    const int32_t* cache_rows, const int32_t* head_mapping,
                                    float topk_percent, float* glse, float* Output_partial,
@@ -222,7 +274,7 @@ int kascade_decode_reuse_rows_call(const kascade_half* Q, const kascade_half* K_
     p.idx_physical = 1; p.max_row = num_pages * page_size - 1;
     p.block_table = block_table; p.glse = glse; p.opart = Output_partial; p.scores = nullptr;
     p.max_pages = max_pages; p.page_shift = shift; p.kv_stride_tokens = 0;
-    if (set_kv_strides(p, nullptr, block_table, 0)) return -1;
+    if (set_kv_strides(p, sh, nullptr, block_table, 0)) return -1;
     if (set_append(p, k_new, v_new, K_pages, V_pages)) return -1;
     p.topk = topk; p.topk_percent = topk_percent; p.scores_stride = 0; p.num_split = num_split;
     p.rows_per_split = rows_per_split(topk, num_split);
@@ -231,8 +283,33 @@ int kascade_decode_reuse_rows_call(const kascade_half* Q, const kascade_half* K_
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (check_hip(launch_decode_split(p, true, true, false, s), "decode_reuse_rows split")) return -1;
     if (sync_counters) return 0;
-    return check_hip(launch_decode_combine(glse, Output_partial, H(Output), nullptr, batch,
-                                           num_split, true, s), "decode_reuse_rows combine");
+    return check_hip(launch_decode_combine(glse, Output_partial, E(Output), nullptr, batch, sh.H(), num_split, true, sh.D, sh.elem, s), "decode_reuse_rows combine");
+}
+}  // namespace
+extern "C" {
+
+int kascade_decode_reuse_rows_call(const kascade_half* Q, const kascade_half* K_pages,
+                                   const kascade_half* V_pages, const int32_t* cache_seqlens,
+                                   const int32_t* cache_rows, const int32_t* head_mapping,
+                                   float topk_percent, float* glse, float* Output_partial,
+                                   kascade_half* Output, int batch, int topk, int num_split,
+                                   const int32_t* block_table, int max_pages, int page_size,
+                                   int num_pages, const kascade_half* k_new,
+                                   const kascade_half* v_new, int32_t* sync_counters, void* stream) {
+    return decode_reuse_rows_impl(kRefShape, Q, K_pages, V_pages, cache_seqlens, cache_rows, head_mapping, topk_percent, glse, Output_partial, Output, batch, topk, num_split, block_table, max_pages, page_size, num_pages, k_new, v_new, sync_counters, stream);
+}
+
+int kascade_decode_reuse_rows_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K_pages,
+                                   const kascade_half* V_pages, const int32_t* cache_seqlens,
+                                   const int32_t* cache_rows, const int32_t* head_mapping,
+                                   float topk_percent, float* glse, float* Output_partial,
+                                   kascade_half* Output, int batch, int topk, int num_split,
+                                   const int32_t* block_table, int max_pages, int page_size,
+                                   int num_pages, const kascade_half* k_new,
+                                   const kascade_half* v_new, int32_t* sync_counters, void* stream) {
+    Shape sh;
+    if (get_shape(shape, &sh)) return -1;
+    return decode_reuse_rows_impl(sh, Q, K_pages, V_pages, cache_seqlens, cache_rows, head_mapping, topk_percent, glse, Output_partial, Output, batch, topk, num_split, block_table, max_pages, page_size, num_pages, k_new, v_new, sync_counters, stream);
 }
 
 int kascade_decode_reuse_paged_noalloc_call(const kascade_half* Q, const kascade_half* K,
@@ -253,13 +330,15 @@ int kascade_decode_reuse_paged_noalloc_call(const kascade_half* Q, const kascade
     if (noalloc_scratch(&base)) return -1;
     float* glse = base;                                           // [batch,32,num_split]
     float* opart = base + (size_t)kNoAllocUnits * kHeads;         // [batch,32,num_split,128]
-    return kascade_decode_reuse_paged_call(Q, K, V, cache_seqlens, topk_indices, head_mapping,
+    return decode_reuse_paged_impl(kRefShape, Q, K, V, cache_seqlens, topk_indices, head_mapping,
                                            topk_percent, glse, opart, Output, batch,
                                            kv_stride_tokens, topk, num_split, block_table, max_pages,
                                            page_size, kv_strides, k_new, v_new, nullptr, stream);
 }
 
-int kascade_decode_dense_paged_call(const kascade_half* Q, const kascade_half* K,
+}  // extern "C"
+namespace {
+int decode_dense_paged_impl(const Shape& sh, const kascade_half* Q, const kascade_half* K,
                                     const kascade_half* V, const int32_t* cache_seqlens,
                                     float* glse, float* Output_partial, kascade_half* Output,
                                     int batch, int kv_stride_tokens, int num_split,
@@ -279,7 +358,7 @@ int kascade_decode_dense_paged_call(const kascade_half* Q, const kascade_half* K
     p.Q = H(Q); p.K = H(K); p.V = H(V);
     p.seqlens = cache_seqlens; p.block_table = block_table; p.glse = glse; p.opart = Output_partial;
     p.max_pages = max_pages; p.page_shift = shift; p.kv_stride_tokens = kv_stride_tokens;
-    if (set_kv_strides(p, kv_strides, block_table, kv_stride_tokens)) return -1;
+    if (set_kv_strides(p, sh, kv_strides, block_table, kv_stride_tokens)) return -1;
     if (set_append(p, k_new, v_new, K, V)) return -1;
     p.num_split = num_split; p.B = batch;
     const long long max_rows = kv_stride_tokens > 0 ? kv_stride_tokens : (long long)max_pages * page_size;
@@ -288,11 +367,38 @@ int kascade_decode_dense_paged_call(const kascade_half* Q, const kascade_half* K
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (check_hip(launch_decode_split(p, false, true, false, s), "decode_dense split")) return -1;
     if (sync_counters) return 0;
-    return check_hip(launch_decode_combine(glse, Output_partial, H(Output), nullptr, batch,
-                                           num_split, true, s), "decode_dense combine");
+    return check_hip(launch_decode_combine(glse, Output_partial, E(Output), nullptr, batch, sh.H(), num_split, true, sh.D, sh.elem, s), "decode_dense combine");
+}
+}  // namespace
+extern "C" {
+
+int kascade_decode_dense_paged_call(const kascade_half* Q, const kascade_half* K,
+                                    const kascade_half* V, const int32_t* cache_seqlens,
+                                    float* glse, float* Output_partial, kascade_half* Output,
+                                    int batch, int kv_stride_tokens, int num_split,
+                                    const int32_t* block_table, int max_pages, int page_size,
+                                    const kascade_strides* kv_strides, const kascade_half* k_new,
+                                    const kascade_half* v_new, int32_t* sync_counters,
+                                    void* stream) {
+    return decode_dense_paged_impl(kRefShape, Q, K, V, cache_seqlens, glse, Output_partial, Output, batch, kv_stride_tokens, num_split, block_table, max_pages, page_size, kv_strides, k_new, v_new, sync_counters, stream);
 }
 
-int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_half* K,
+int kascade_decode_dense_paged_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K,
+                                    const kascade_half* V, const int32_t* cache_seqlens,
+                                    float* glse, float* Output_partial, kascade_half* Output,
+                                    int batch, int kv_stride_tokens, int num_split,
+                                    const int32_t* block_table, int max_pages, int page_size,
+                                    const kascade_strides* kv_strides, const kascade_half* k_new,
+                                    const kascade_half* v_new, int32_t* sync_counters,
+                                    void* stream) {
+    Shape sh;
+    if (get_shape(shape, &sh)) return -1;
+    return decode_dense_paged_impl(sh, Q, K, V, cache_seqlens, glse, Output_partial, Output, batch, kv_stride_tokens, num_split, block_table, max_pages, page_size, kv_strides, k_new, v_new, sync_counters, stream);
+}
+
+}  // extern "C"
+namespace {
+int decode_recompute_paged_impl(const Shape& sh, const kascade_half* Q, const kascade_half* K,
                                         const kascade_half* V, const int32_t* cache_seqlens,
                                         float* glse, float* Output_partial, float* row_sums,
                                         float* scores, kascade_half* Output,
@@ -325,7 +431,7 @@ int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_hal
     p.seqlens = cache_seqlens; p.block_table = block_table; p.glse = glse; p.opart = Output_partial;
     p.scores = scores; p.scores_stride = scores_stride;
     p.max_pages = max_pages; p.page_shift = shift; p.kv_stride_tokens = kv_stride_tokens;
-    if (set_kv_strides(p, kv_strides, block_table, kv_stride_tokens)) return -1;
+    if (set_kv_strides(p, sh, kv_strides, block_table, kv_stride_tokens)) return -1;
     if (set_append(p, k_new, v_new, K, V)) return -1;
     p.num_split = num_split; p.B = batch;
     long long max_rows = kv_stride_tokens > 0 ? kv_stride_tokens : (long long)max_pages * page_size;
@@ -342,14 +448,45 @@ int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_hal
     // launch does for itself: no combine launch.
     const bool merge_in_aggregate = !sync_counters && !with_output;
     if (!sync_counters && with_output &&
-        check_hip(launch_decode_combine(glse, Output_partial, H(Output), row_sums, batch, num_split,
-                                        true, s), "decode_recompute combine"))
+        check_hip(launch_decode_combine(glse, Output_partial, E(Output), row_sums, batch, sh.H(), num_split, true, sh.D, sh.elem, s), "decode_recompute combine"))
         return -1;
     return check_hip(launch_decode_aggregate(scores, merge_in_aggregate ? nullptr : row_sums,
                                              merge_in_aggregate ? glse : nullptr, num_split, row_sums,
-                                             cache_seqlens, H(aggregated_scores), batch, scores_stride,
+                                             cache_seqlens, H(aggregated_scores), batch, sh.G, scores_stride,
                                              kv_stride_tokens, (int)len_cap, s),
                      "decode_recompute aggregate");
+}
+}  // namespace
+extern "C" {
+
+int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_half* K,
+                                        const kascade_half* V, const int32_t* cache_seqlens,
+                                        float* glse, float* Output_partial, float* row_sums,
+                                        float* scores, kascade_half* Output,
+                                        kascade_half* aggregated_scores, int batch,
+                                        int kv_stride_tokens, int scores_stride, int num_split,
+                                        int with_output, const int32_t* block_table,
+                                        int max_pages, int page_size,
+                                        const kascade_strides* kv_strides,
+                                        const kascade_half* k_new, const kascade_half* v_new,
+                                        int32_t* sync_counters, void* stream) {
+    return decode_recompute_paged_impl(kRefShape, Q, K, V, cache_seqlens, glse, Output_partial, row_sums, scores, Output, aggregated_scores, batch, kv_stride_tokens, scores_stride, num_split, with_output, block_table, max_pages, page_size, kv_strides, k_new, v_new, sync_counters, stream);
+}
+
+int kascade_decode_recompute_paged_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K,
+                                        const kascade_half* V, const int32_t* cache_seqlens,
+                                        float* glse, float* Output_partial, float* row_sums,
+                                        float* scores, kascade_half* Output,
+                                        kascade_half* aggregated_scores, int batch,
+                                        int kv_stride_tokens, int scores_stride, int num_split,
+                                        int with_output, const int32_t* block_table,
+                                        int max_pages, int page_size,
+                                        const kascade_strides* kv_strides,
+                                        const kascade_half* k_new, const kascade_half* v_new,
+                                        int32_t* sync_counters, void* stream) {
+    Shape sh;
+    if (get_shape(shape, &sh)) return -1;
+    return decode_recompute_paged_impl(sh, Q, K, V, cache_seqlens, glse, Output_partial, row_sums, scores, Output, aggregated_scores, batch, kv_stride_tokens, scores_stride, num_split, with_output, block_table, max_pages, page_size, kv_strides, k_new, v_new, sync_counters, stream);
 }
 
 int64_t kascade_topk_workspace_bytes(int rows, int64_t row_len) {

@@ -21,6 +21,54 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
 
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef short short4_t __attribute__((ext_vector_type(4)));
+
+// Element types of Q, K, V and the attention output (pooled scores are fp16 for both).
+enum ElemKind { kElemF16 = 0, kElemBF16 = 1 };
+
+// D^-0.5 * log2(e) for the head dimensions the kernels are built for
+template <int D> struct ScaleLog2;
+template <> struct ScaleLog2<128> { static constexpr float value = 0.12751743082459868f; };
+template <> struct ScaleLog2<64> { static constexpr float value = 0.18033688011112042f; };
+
+// Vector types and matrix instructions per element type.  Both types have the same operand
+// layouts, so the kernels are written once over Elem<T>.
+template <typename T> struct Elem;
+template <> struct Elem<half_t> {
+    typedef half2_t x2; typedef half4_t x4; typedef half8_t x8;
+    static __device__ __forceinline__ float4_t mma_16x16x32(x8 a, x8 b, float4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float4_t mma_16x16x16(short4_t a, x4 b, float4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(x4, a), b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float16_t mma_32x32x16(x8 a, x8 b, float16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+template <> struct Elem<bf16_t> {
+    typedef bf16x2_t x2; typedef bf16x4_t x4; typedef bf16x8_t x8;
+    static __device__ __forceinline__ float4_t mma_16x16x32(x8 a, x8 b, float4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float4_t mma_16x16x16(short4_t a, x4 b, float4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, __builtin_bit_cast(short4_t, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float16_t mma_32x32x16(x8 a, x8 b, float16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+};
+
+template <typename T> union PackT {  // one 16-byte transaction seen as 8 elements of type T
+    uint4_t u;
+    typename Elem<T>::x8 v8;
+    T e[8];
+};
+
 union Pack16 {  // one 16-byte global/LDS transaction seen as 8 halves
     uint4_t u;
     half8_t h8;

@@ -5,9 +5,11 @@
 namespace kascade {
 
 struct DecodeParams {
-    const half_t* Q;        // [B,H,D]
-    const half_t* K;        // pages [P,page,G,D], or a strided [B,tokens,G,D] view
-    const half_t* V;
+    // Q, K, V, the new rows and the output hold elements of kind `elem` (fp16 or bf16); G KV heads,
+    // H = 4 G query heads, head dimension head_dim (64 or 128).
+    const void* Q;          // [B,H,D]
+    const void* K;          // pages [P,page,G,D], or a strided [B,tokens,G,D] view
+    const void* V;
     const int* seqlens;     // [B] or null
     const int* idx;         // [B,G,topk] logical token ids (gather mode); physical cache rows with idx_physical
     const int* head_map;    // [G] (gather mode)
@@ -20,12 +22,12 @@ struct DecodeParams {
     // out [B,H,D] and row_sums [B,H] (either may be null), and no combine launch is needed.
     // Fused append: with k_new != null the rows k_new/v_new [B,G,D] of each sequence's newest
     // token (position seqlen-1) are written into k_cache / v_cache by the launch itself.
-    const half_t* k_new;
-    const half_t* v_new;
-    half_t* k_cache;
-    half_t* v_cache;
+    const void* k_new;
+    const void* v_new;
+    void* k_cache;
+    void* v_cache;
     int* counters;
-    half_t* out;
+    void* out;
     float* row_sums;
     int idx_physical;       // gather mode over pages: idx holds cache rows (page * page_size + slot)
     int max_row;            // ... each clamped to [0, max_row]
@@ -43,19 +45,22 @@ struct DecodeParams {
     int num_split;
     int rows_per_split;     // multiple of 64; num_split*rows_per_split >= longest row list
     int B;
+    int G;                  // KV heads
+    int head_dim;           // 64 or 128
+    int elem;               // kElemF16 or kElemBF16
 };
 
 hipError_t launch_decode_split(const DecodeParams& p, bool gather, bool with_v, bool write_scores,
                                hipStream_t stream);
-hipError_t launch_decode_combine(const float* glse, const float* opart, half_t* out,
-                                 float* row_sums, int batch, int num_split, bool with_v,
+hipError_t launch_decode_combine(const float* glse, const float* opart, void* out, float* row_sums,
+                                 int batch, int heads, int num_split, bool with_v, int head_dim, int elem,
                                  hipStream_t stream);
 // Log-sums per head: merged (row_sums_in), or glse [B,H,num_split] to be merged by the kernel,
 // which then also writes them to row_sums_out.  len_cap: the bound the streaming launch put on
 // every sequence length (block-table coverage or cache length, and the score row width).
 hipError_t launch_decode_aggregate(const float* scores, const float* row_sums_in, const float* glse,
                                    int num_split, float* row_sums_out, const int* seqlens,
-                                   half_t* agg, int batch, int scores_stride, int uniform_len,
+                                   half_t* agg, int batch, int groups, int scores_stride, int uniform_len,
                                    int len_cap, hipStream_t stream);
 
 }  // namespace kascade

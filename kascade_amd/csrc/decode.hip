@@ -61,18 +61,27 @@ __device__ __forceinline__ float2 load_device2(const float* p) {
     return make_float2(x.f[0], x.f[1]);
 }
 
+template <int D>
 struct alignas(16) MergeState {  // one per wavefront after the in-wave merge
     float m[kGroupSize];
     float l[kGroupSize];
-    float acc[kGroupSize][kDim];
+    float acc[kGroupSize][D];
 };
 
 // PHYS (gather mode over a paged cache): the index lists hold physical cache rows
 // (page * page_size + slot, what translate_indices_kernel writes) instead of token positions, so
 // the block table is not on the path from a list entry to its K/V row.
-template <bool GATHER, bool WITH_V, bool WRITE_SCORES, bool PHYS = false>
+// D, T: head dimension (64 or 128) and element type (fp16 or bf16) of Q, K, V and the output; the
+// number of KV heads is a launch parameter, a KV head always serves kGroupSize query heads.
+template <bool GATHER, bool WITH_V, bool WRITE_SCORES, bool PHYS, int D, typename T>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2)))
 void decode_split_kernel(DecodeParams p) {
+    typedef typename Elem<T>::x8 x8_t;
+    typedef typename Elem<T>::x4 x4_t;
+    typedef typename Elem<T>::x2 x2_t;
+    constexpr float kScaleLog2 = ScaleLog2<D>::value;
+    const int kvh = p.G;                 // KV heads
+    const int nheads = p.G * kGroupSize; // query heads
     __shared__ int s_row[GATHER ? kSubChunk : 1];
     __shared__ int s_last;
     __shared__ int s_found;   // gather mode: sub-chunk whose index list names the newest token
@@ -82,21 +91,21 @@ void decode_split_kernel(DecodeParams p) {
     constexpr int kCodePhase = WITH_V ? 5 : 7;             // what fits beside two workgroups' tiles
     constexpr int kPhaseRows = WRITE_SCORES ? kCodePhase * 4 * kStripRows : 64;
     union Shared {
-        MergeState merge[4];
+        MergeState<D> merge[4];
         struct {
             uint16_t code[kGroupSize][kPhaseRows];
             float ref[kGroupSize][kPhaseRows / 64];
         } sc;
     };
     __shared__ __attribute__((aligned(16))) Shared s_u;
-    MergeState* s_merge = s_u.merge;
+    MergeState<D>* s_merge = s_u.merge;
     auto& s_code = s_u.sc.code;
     auto& s_ref = s_u.sc.ref;
     // per wavefront one tile of 16 K rows (and V rows) on its way into the matrix layouts
-    constexpr int kKtStride = 136;   // halves per K row (128 + 8): rows 272 bytes apart, conflict-free both ways
-    constexpr int kVtStride = 144;   // halves per V row: 288 bytes, conflict-free for the transposing reads
-    __shared__ __attribute__((aligned(16))) half_t s_kt[4][16 * kKtStride];
-    __shared__ __attribute__((aligned(16))) half_t s_vt[WITH_V ? 4 : 1][WITH_V ? 16 * kVtStride : 8];
+    constexpr int kKtStride = D + 8;    // elements per K row: rows 272 (144) bytes apart, conflict-free both ways
+    constexpr int kVtStride = D + 16;   // elements per V row: 288 (160) bytes, conflict-free for the transposing reads
+    __shared__ __attribute__((aligned(16))) T s_kt[4][16 * kKtStride];
+    __shared__ __attribute__((aligned(16))) T s_vt[WITH_V ? 4 : 1][WITH_V ? 16 * kVtStride : 8];
 
     const int g = blockIdx.x;       // the 8 KV heads of one token range are adjacent in dispatch order
     const int tid = threadIdx.x;
@@ -215,18 +224,18 @@ void decode_split_kernel(DecodeParams p) {
         newest_row = (p.block_table[(size_t)b * p.max_pages + (newest >> p.page_shift)] << p.page_shift) +
                      (newest & ((1 << p.page_shift) - 1));
     auto write_newest = [&]() {
-        if (tid < 32) {
-            const int part = tid >> 4, c = tid & 15;
+        if (tid < 2 * (D / 8)) {   // one 16-byte chunk of the K row or of the V row per thread
+            const int part = tid / (D / 8), c = tid % (D / 8);
             size_t off;
             if (p.block_table) {
                 const int pg = p.block_table[(size_t)b * p.max_pages + (newest >> p.page_shift)];
                 const int row = (pg << p.page_shift) + (newest & ((1 << p.page_shift) - 1));
-                off = (size_t)row * (kGroups * kDim) + (size_t)g * kDim + c * 8;
+                off = (size_t)row * (kvh * D) + (size_t)g * D + c * 8;
             } else {
                 off = (size_t)b * p.kv_stride_b + (size_t)g * p.kv_stride_h + (size_t)newest * p.kv_stride_l + c * 8;
             }
-            const half_t* src = (part ? p.v_new : p.k_new) + ((size_t)b * kGroups + g) * kDim + c * 8;
-            half_t* dst = (part ? p.v_cache : p.k_cache) + off;
+            const T* src = (part ? (const T*)p.v_new : (const T*)p.k_new) + ((size_t)b * kvh + g) * D + c * 8;
+            T* dst = (part ? (T*)p.v_cache : (T*)p.k_cache) + off;
             *reinterpret_cast<uint4_t*>(dst) = ld_global_16(src);
         }
     };
@@ -254,32 +263,40 @@ void decode_split_kernel(DecodeParams p) {
     // a cross-lane reduction: ~10 vector instructions per row, where dot products on the vector
     // unit needed ~110 and bounded every variant of this kernel.
     const int col = lane & 15, dq = lane >> 4;
-    half8_t qb[4];   // B operand of the first product: Q[col][32*st + 8*dq, +8)
+    // Loading role: a row is D/8 chunks of 16 bytes, so a wavefront instruction fetches kRowsPerLoad
+    // whole rows (4 at D = 128, 8 at D = 64) and a tile of 16 rows takes kLoads of them; lane
+    // (lr, lc) takes chunk lc of rows kRowsPerLoad * i + lr.
+    constexpr int kChunks = D / 8, kRowsPerLoad = 64 / kChunks, kLoads = 16 / kRowsPerLoad;
+    const int lc = lane % kChunks, lr = lane / kChunks;
+    x8_t qb[D / 32];   // B operand of the first product: Q[col][32*st + 8*dq, +8)
 #pragma unroll
-    for (int st = 0; st < 4; ++st) {
-        Pack16 t;
-        t.u = ld_global_16(p.Q + ((size_t)b * kHeads + g * kGroupSize + (col & 3)) * kDim + 32 * st + 8 * dq);
+    for (int st = 0; st < D / 32; ++st) {
+        PackT<T> t;
+        t.u = ld_global_16((const T*)p.Q + ((size_t)b * nheads + g * kGroupSize + (col & 3)) * D + 32 * st + 8 * dq);
         if (col >= kGroupSize) t.u = uint4_t{0, 0, 0, 0};
-        qb[st] = t.h8;
+        qb[st] = t.v8;
     }
     // Online softmax state of this lane's column.  With V one running maximum per column (the
     // second product needs a common reference: two cross-lane exchanges per tile); without V
     // every lane keeps the maximum and sum of its own keys and the four parts meet at the end.
     float mcol = -INFINITY, lcol = 0.f;
-    float4_t oacc[WITH_V ? 8 : 1];   // O^T[16*blk + 4*dq + r][col]
+    constexpr int kOBlocks = D / 16;
+    float4_t oacc[WITH_V ? kOBlocks : 1];   // O^T[16*blk + 4*dq + r][col]
 #pragma unroll
-    for (int blk = 0; blk < (WITH_V ? 8 : 1); ++blk) oacc[blk] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int blk = 0; blk < (WITH_V ? kOBlocks : 1); ++blk) oacc[blk] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     const int* idx_row = nullptr;
-    if (GATHER) idx_row = p.idx + ((size_t)b * kGroups + p.head_map[g]) * p.topk;
+    if (GATHER) idx_row = p.idx + ((size_t)b * kvh + p.head_map[g]) * p.topk;
     const int page_mask = (1 << p.page_shift) - 1;
     const unsigned stride_l = p.kv_stride_l;
-    half_t* kt = &s_kt[wave][0];
-    half_t* vt = &s_vt[wave][0];
+    T* kt = &s_kt[wave][0];
+    T* vt = &s_vt[wave][0];
+    const T* Kc = (const T*)p.K;
+    const T* Vc = (const T*)p.V;
 
     struct Tile {
-        uint4_t k[4];
-        uint4_t v[WITH_V ? 4 : 1];
+        uint4_t k[kLoads];
+        uint4_t v[WITH_V ? kLoads : 1];
     };
     // `row`: physical row (page * page_size + slot) behind a block table; otherwise the token
     // number of sequence b behind the caller's (batch, token, head) strides, so that a head-major
@@ -288,11 +305,11 @@ void decode_split_kernel(DecodeParams p) {
     // the raw scores of an anchor pass).
     auto load_row = [&](auto paged_tag, int row, Tile& tb, int i) {
         constexpr bool PAGED = decltype(paged_tag)::value;
-        const size_t off = PAGED ? ((size_t)row * kGroups + g) * kDim + 8 * col
+        const size_t off = PAGED ? ((size_t)row * kvh + g) * D + 8 * lc
                                  : (size_t)b * p.kv_stride_b + (size_t)g * p.kv_stride_h +
-                                       (size_t)(unsigned)row * stride_l + 8 * col;
-        tb.k[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.K + off));
-        if (WITH_V) tb.v[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.V + off));
+                                       (size_t)(unsigned)row * stride_l + 8 * lc;
+        tb.k[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(Kc + off));
+        if (WITH_V) tb.v[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(Vc + off));
     };
     // One tile: `key0` is the position of this lane's first key within the range, `cn` the number
     // of rows of the range (keys at or beyond it are masked).  Returns this lane's four raw scores.
@@ -300,16 +317,16 @@ void decode_split_kernel(DecodeParams p) {
     // consuming them makes the compiler wait for every load in flight.
     auto compute_tile = [&](const Tile& tb, int key0, int cn) -> float4_t {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            *reinterpret_cast<uint4_t*>(&kt[(4 * i + dq) * kKtStride + 8 * col]) = tb.k[i];
-            if (WITH_V) *reinterpret_cast<uint4_t*>(&vt[(4 * i + dq) * kVtStride + 8 * col]) = tb.v[i];
+        for (int i = 0; i < kLoads; ++i) {
+            *reinterpret_cast<uint4_t*>(&kt[(kRowsPerLoad * i + lr) * kKtStride + 8 * lc]) = tb.k[i];
+            if (WITH_V) *reinterpret_cast<uint4_t*>(&vt[(kRowsPerLoad * i + lr) * kVtStride + 8 * lc]) = tb.v[i];
         }
         __builtin_amdgcn_wave_barrier();   // the reads below are other lanes' writes (same wavefront: in order)
         float4_t sc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int st = 0; st < 4; ++st) {
-            const half8_t a = *reinterpret_cast<const half8_t*>(&kt[col * kKtStride + 32 * st + 8 * dq]);
-            sc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qb[st], sc, 0, 0, 0);
+        for (int st = 0; st < D / 32; ++st) {
+            const x8_t a = *reinterpret_cast<const x8_t*>(&kt[col * kKtStride + 32 * st + 8 * dq]);
+            sc = Elem<T>::mma_16x16x32(a, qb[st], sc);
         }
 #pragma unroll
         for (int e = 0; e < 4; ++e)
@@ -334,18 +351,17 @@ void decode_split_kernel(DecodeParams p) {
         if (WITH_V) {
             if (__any(corr != 1.f)) {   // wavefront-uniform: skip when no maximum moved
 #pragma unroll
-                for (int blk = 0; blk < 8; ++blk) oacc[blk] *= corr;
+                for (int blk = 0; blk < kOBlocks; ++blk) oacc[blk] *= corr;
             }
-            const half4_t pb = {(half_t)pe[0], (half_t)pe[1], (half_t)pe[2], (half_t)pe[3]};
-            typedef short short4_t __attribute__((ext_vector_type(4)));
+            const x4_t pb = {(T)pe[0], (T)pe[1], (T)pe[2], (T)pe[3]};
             // ds_read_b64_tr_b16: lane (dq, col) points at V[row 4dq + col/4][16blk + 4(col%4), +4)
             // and receives V[rows 4dq .. 4dq+3][16blk + col]
-            const half_t* vp = &vt[(4 * dq + (col >> 2)) * kVtStride + 4 * (col & 3)];
+            const T* vp = &vt[(4 * dq + (col >> 2)) * kVtStride + 4 * (col & 3)];
 #pragma unroll
-            for (int blk = 0; blk < 8; ++blk) {
+            for (int blk = 0; blk < kOBlocks; ++blk) {
                 const short4_t raw = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                     (__attribute__((address_space(3))) short4_t*)(vp + 16 * blk));
-                oacc[blk] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4_t, raw), pb, oacc[blk], 0, 0, 0);
+                oacc[blk] = Elem<T>::mma_16x16x16(raw, pb, oacc[blk]);
             }
         }
         __builtin_amdgcn_wave_barrier();
@@ -390,7 +406,7 @@ void decode_split_kernel(DecodeParams p) {
         if (nrows > 0) {
 #pragma unroll
             for (int h = 0; h < kGroupSize; ++h) {
-                float* row = p.scores + ((size_t)b * kHeads + g * kGroupSize + h) * p.scores_stride;
+                float* row = p.scores + ((size_t)b * nheads + g * kGroupSize + h) * p.scores_stride;
                 uint16_t* dst = reinterpret_cast<uint16_t*>(row) + r0 + lo;
                 for (int i = tid * 8; i < nrows; i += kThreads * 8) {
                     if (i + 8 <= nrows) {
@@ -423,13 +439,13 @@ void decode_split_kernel(DecodeParams p) {
             // entries only), and then the staging consumes its entries with the K/V loads still
             // in flight behind them.
             const bool early = PHYS && c0 == r0 && !can_append;   // uniform over the workgroup
-            int er[2][4];
+            int er[2][kLoads];
             if (early) {
 #pragma unroll
                 for (int u = 0; u < 2; ++u)
 #pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        er[u][i] = idx_row[c0 + min(16 * (wave + 4 * u) + 4 * i + dq, cn - 1)];
+                    for (int i = 0; i < kLoads; ++i)
+                        er[u][i] = idx_row[c0 + min(16 * (wave + 4 * u) + kRowsPerLoad * i + lr, cn - 1)];
             }
             auto early_tiles = [&]() {
                 if (early) {
@@ -437,7 +453,7 @@ void decode_split_kernel(DecodeParams p) {
 #pragma unroll
                     for (int u = 0; u < 2; ++u)
 #pragma unroll
-                        for (int i = 0; i < 4; ++i)
+                        for (int i = 0; i < kLoads; ++i)
                             load_row(paged_tag, max(0, min(er[u][i], p.max_row)), u ? tb : ta, i);
                     KASCADE_SCHED_FENCE();
                 }
@@ -478,8 +494,8 @@ void decode_split_kernel(DecodeParams p) {
             }
             auto issue = [&](int t, Tile& tb) {   // tile t: rows [16t, 16t+16) of the sub-chunk
 #pragma unroll
-                for (int i = 0; i < 4; ++i)      // past the end: clamped, masked later
-                    load_row(paged_tag, s_row[min(16 * t + 4 * i + dq, cn - 1)], tb, i);
+                for (int i = 0; i < kLoads; ++i)      // past the end: clamped, masked later
+                    load_row(paged_tag, s_row[min(16 * t + kRowsPerLoad * i + lr, cn - 1)], tb, i);
             };
             const int ntiles = (cn + 15) / 16;
             int t_first = wave;
@@ -521,14 +537,14 @@ void decode_split_kernel(DecodeParams p) {
         constexpr bool PAGED = decltype(paged_tag)::value;
         // tile k of this wavefront: 16 keys from row (k / 16) * 1024 + wave * 256 + (k % 16) * 16
         auto tile_row = [&](int k) { return (k / kTilesPerStrip) * (4 * kStripRows) + wave * kStripRows + (k % kTilesPerStrip) * 16; };
-        auto tok_of = [&](int k, int i) { return min(r0 + tile_row(k) + 4 * i + dq, r1 - 1); };   // past the end: clamped, masked later
-        auto fetch_pages = [&](int k, int (&pg)[4]) {
+        auto tok_of = [&](int k, int i) { return min(r0 + tile_row(k) + kRowsPerLoad * i + lr, r1 - 1); };   // past the end: clamped, masked later
+        auto fetch_pages = [&](int k, int (&pg)[kLoads]) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) pg[i] = PAGED ? bt_row[tok_of(k, i) >> p.page_shift] : 0;
+            for (int i = 0; i < kLoads; ++i) pg[i] = PAGED ? bt_row[tok_of(k, i) >> p.page_shift] : 0;
         };
-        auto issue = [&](int k, const int (&pg)[4], Tile& tb) {
+        auto issue = [&](int k, const int (&pg)[kLoads], Tile& tb) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
+            for (int i = 0; i < kLoads; ++i) {
                 const int tok = tok_of(k, i);
                 load_row(paged_tag, PAGED ? (pg[i] << p.page_shift) + (tok & page_mask) : tok, tb, i);
             }
@@ -537,7 +553,7 @@ void decode_split_kernel(DecodeParams p) {
             const int nsup = (cn + 4 * kStripRows - 1) / (4 * kStripRows);
             const int ntile = nsup * kTilesPerStrip;   // the same for every wavefront
             Tile buf[kDepth];
-            int pgn[kDepth][4];
+            int pgn[kDepth][kLoads];
 #pragma unroll
             for (int j = 0; j < kDepth; ++j) {
                 fetch_pages(j, pgn[j]);
@@ -589,15 +605,16 @@ void decode_split_kernel(DecodeParams p) {
         }
         if (WITH_V) {
 #pragma unroll
-            for (int blk = 0; blk < 8; ++blk)
+            for (int blk = 0; blk < kOBlocks; ++blk)
                 *reinterpret_cast<float4_t*>(&s_merge[wave].acc[col][16 * blk + 4 * dq]) = oacc[blk];
         }
     }
     __syncthreads();
     // ---- merge the four wavefronts; thread -> (head, two d's) ----
-    if (tid < kThreads) {
+    {
         const int h = tid >> 6;
-        const int d0 = (tid & 63) * 2;
+        const bool has_d = (tid & 63) * 2 < D;           // at D = 64 half of the lanes have no output element
+        const int d0 = has_d ? (tid & 63) * 2 : 0;
         float mx = -INFINITY;
 #pragma unroll
         for (int w = 0; w < 4; ++w) mx = fmaxf(mx, s_merge[w].m[h]);
@@ -612,16 +629,16 @@ void decode_split_kernel(DecodeParams p) {
                 o1 += s_merge[w].acc[h][d0 + 1] * c;
             }
         }
-        const size_t ph = ((size_t)b * kHeads + g * kGroupSize + h) * p.num_split + split;
+        const size_t ph = ((size_t)b * nheads + g * kGroupSize + h) * p.num_split + split;
         const float lse_part = (L > 0.f) ? (fast_log2(L) + mref) : -INFINITY;
         const float inv = (L > 0.f) ? 1.f / L : 0.f;
         if (p.counters == nullptr) {
             if ((tid & 63) == 0) p.glse[ph] = lse_part;
-            if (WITH_V) *reinterpret_cast<float2*>(p.opart + ph * kDim + d0) = make_float2(o0 * inv, o1 * inv);
+            if (WITH_V && has_d) *reinterpret_cast<float2*>(p.opart + ph * D + d0) = make_float2(o0 * inv, o1 * inv);
         } else {
             // read by another workgroup of this launch: device-coherent stores
             if ((tid & 63) == 0) store_device(p.glse + ph, lse_part);
-            if (WITH_V) store_device2(p.opart + ph * kDim + d0, o0 * inv, o1 * inv);
+            if (WITH_V && has_d) store_device2(p.opart + ph * D + d0, o0 * inv, o1 * inv);
         }
     }
     // splits that no workgroup takes (sequences shorter than the longest) count as empty for
@@ -629,7 +646,7 @@ void decode_split_kernel(DecodeParams p) {
     if (split == 0) {
         const int missing = p.num_split - nsplit_b;
         for (int i = tid; i < kGroupSize * missing; i += kThreads)
-            p.glse[((size_t)b * kHeads + g * kGroupSize + i / missing) * p.num_split + nsplit_b + i % missing] = -INFINITY;
+            p.glse[((size_t)b * nheads + g * kGroupSize + i / missing) * p.num_split + nsplit_b + i % missing] = -INFINITY;
     }
     // ---- fused combine: the last workgroup of (b, g) to arrive merges the splits ----
     // The partial results above are written through to device-coherent memory and the barrier
@@ -644,28 +661,29 @@ void decode_split_kernel(DecodeParams p) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (tid == 0) {
-        const int arrived = __hip_atomic_fetch_add(&p.counters[b * kGroups + g], 1, __ATOMIC_RELAXED,
+        const int arrived = __hip_atomic_fetch_add(&p.counters[b * kvh + g], 1, __ATOMIC_RELAXED,
                                                    __HIP_MEMORY_SCOPE_AGENT);
         s_last = (arrived == nsplit_b - 1);
     }
     __syncthreads();
     if (!s_last) return;
     if (tid == 0)   // ready for the next launch
-        __hip_atomic_store(&p.counters[b * kGroups + g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (tid < kThreads) {
+        __hip_atomic_store(&p.counters[b * kvh + g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    {
         // wavefront -> head; lanes over the splits for the reductions, then two d's per lane
         const int head = g * kGroupSize + wave;
         const int ns = nsplit_b;   // the splits of this sequence that exist
-        const size_t base = ((size_t)b * kHeads + head) * p.num_split;
+        const size_t base = ((size_t)b * nheads + head) * p.num_split;
         const float* gl = p.glse + base;
-        const float* op = p.opart + base * kDim + lane * 2;
+        const bool has_d = lane * 2 < D;
+        const float* op = p.opart + base * D + (has_d ? lane * 2 : 0);
         // the first partial outputs are requested together with the log-sums, so that short
         // split lists cost one trip to memory, not two
         constexpr int kEarly = 16;
         float2 xe[kEarly];
         if (WITH_V) {
 #pragma unroll
-            for (int j = 0; j < kEarly; ++j) xe[j] = load_device2(op + (size_t)min(j, ns - 1) * kDim);
+            for (int j = 0; j < kEarly; ++j) xe[j] = load_device2(op + (size_t)min(j, ns - 1) * D);
         }
         const float g0 = (lane < ns) ? load_device(gl + lane) : -INFINITY;   // splits [0, 64)
         float mx = g0;
@@ -678,7 +696,7 @@ void decode_split_kernel(DecodeParams p) {
 #pragma unroll
         for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
         const float lse = (sum > 0.f) ? fast_log2(sum) + mref : -INFINITY;
-        if (p.row_sums && lane == 0) p.row_sums[(size_t)b * kHeads + head] = lse;
+        if (p.row_sums && lane == 0) p.row_sums[(size_t)b * nheads + head] = lse;
         if (WITH_V) {
             const float lref = (lse == -INFINITY) ? 0.f : lse;
             float o0 = 0.f, o1 = 0.f;
@@ -689,7 +707,7 @@ void decode_split_kernel(DecodeParams p) {
                 if (s0 > 0) {
                     if ((s0 & 63) == 0) wl = (s0 + lane < ns) ? fast_exp2(load_device(gl + s0 + lane) - lref) : 0.f;
 #pragma unroll
-                    for (int j = 0; j < kEarly; ++j) xe[j] = load_device2(op + (size_t)min(s0 + j, ns - 1) * kDim);
+                    for (int j = 0; j < kEarly; ++j) xe[j] = load_device2(op + (size_t)min(s0 + j, ns - 1) * D);
                 }
 #pragma unroll
                 for (int j = 0; j < kEarly; ++j) {
@@ -698,8 +716,8 @@ void decode_split_kernel(DecodeParams p) {
                     o1 += w * xe[j].y;
                 }
             }
-            half2_t o = {(half_t)o0, (half_t)o1};
-            *reinterpret_cast<half2_t*>(p.out + ((size_t)b * kHeads + head) * kDim + lane * 2) = o;
+            x2_t o = {(T)o0, (T)o1};
+            if (has_d) *reinterpret_cast<x2_t*>((T*)p.out + ((size_t)b * nheads + head) * D + lane * 2) = o;
         }
     }
 }
@@ -721,18 +739,19 @@ __device__ __forceinline__ float combine_reduce(float x, bool is_max, float* s_r
     return is_max ? fmaxf(s_red[0], s_red[1]) : s_red[0] + s_red[1];
 }
 
-template <bool WITH_V>
+template <bool WITH_V, int D, typename T>
 __global__ __launch_bounds__(128) void decode_combine_kernel(const float* __restrict__ glse,
                                                             const float* __restrict__ opart,
-                                                            half_t* __restrict__ out,
+                                                            T* __restrict__ out,
                                                             float* __restrict__ row_sums,
                                                             int num_split) {
     __shared__ float s_w[kCombineLds];
     __shared__ float s_red[2];
     const int h = blockIdx.x;
     const int b = blockIdx.y;
-    const int d = threadIdx.x;
-    const size_t base = ((size_t)b * kHeads + h) * num_split;
+    const int nheads = gridDim.x;
+    const int d = threadIdx.x;            // threads beyond D only take part in the reductions
+    const size_t base = ((size_t)b * nheads + h) * num_split;
     float mx = -INFINITY;
     for (int s = d; s < num_split; s += 128) mx = fmaxf(mx, glse[base + s]);
     mx = combine_reduce(mx, true, s_red);
@@ -741,19 +760,20 @@ __global__ __launch_bounds__(128) void decode_combine_kernel(const float* __rest
     for (int s = d; s < num_split; s += 128) sum += fast_exp2(glse[base + s] - mref);
     sum = combine_reduce(sum, false, s_red);
     const float lse = (sum > 0.f) ? fast_log2(sum) + mref : -INFINITY;
-    if (row_sums && d == 0) row_sums[(size_t)b * kHeads + h] = lse;
+    if (row_sums && d == 0) row_sums[(size_t)b * nheads + h] = lse;
     if (WITH_V) {
         const float lref = (lse == -INFINITY) ? 0.f : lse;
         for (int s = d; s < min(num_split, kCombineLds); s += 128) s_w[s] = fast_exp2(glse[base + s] - lref);
         __syncthreads();
-        const float* op = opart + base * kDim + d;
+        if (d >= D) return;
+        const float* op = opart + base * D + d;
         float o = 0.f;
         int s = 0;
         // a split that saw no rows leaves its partial output unwritten: select, never multiply
         for (; s + 8 <= min(num_split, kCombineLds); s += 8) {
             float x[8];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) x[e] = op[(size_t)(s + e) * kDim];
+            for (int e = 0; e < 8; ++e) x[e] = op[(size_t)(s + e) * D];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const float w = s_w[s + e];
@@ -762,10 +782,10 @@ __global__ __launch_bounds__(128) void decode_combine_kernel(const float* __rest
         }
         for (; s < num_split; ++s) {
             const float w = (s < kCombineLds) ? s_w[s] : fast_exp2(glse[base + s] - lref);
-            const float x = op[(size_t)s * kDim];
+            const float x = op[(size_t)s * D];
             o += (w > 0.f) ? w * x : 0.f;
         }
-        out[((size_t)b * kHeads + h) * kDim + d] = (half_t)o;
+        out[((size_t)b * nheads + h) * D + d] = (T)o;
     }
 }
 
@@ -786,13 +806,14 @@ __global__ __launch_bounds__(256) void decode_aggregate_kernel(const float* __re
     __shared__ float s_lse[kGroupSize];
     const int g = blockIdx.y;
     const int b = blockIdx.z;
+    const int kvh = gridDim.y, nheads = gridDim.y * kGroupSize;
     // the same bound the streaming launch applied to the length: codes beyond it were never written
     const int len = max(0, min(seqlens ? seqlens[b] : uniform_len, len_cap));
     const int j0 = (blockIdx.x * 256 + threadIdx.x) * 8;
     float lse[kGroupSize];
     if (glse != nullptr) {   // uniform over the launch
         const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-        const float* gl = glse + ((size_t)b * kHeads + g * kGroupSize + wave) * num_split;
+        const float* gl = glse + ((size_t)b * nheads + g * kGroupSize + wave) * num_split;
         float mx = -INFINITY;
         for (int sidx = lane; sidx < num_split; sidx += 64) mx = fmaxf(mx, gl[sidx]);
 #pragma unroll
@@ -805,14 +826,14 @@ __global__ __launch_bounds__(256) void decode_aggregate_kernel(const float* __re
         const float v = (sum > 0.f) ? fast_log2(sum) + mref : -INFINITY;
         if (lane == 0) {
             s_lse[wave] = v;
-            if (blockIdx.x == 0 && row_sums_out) row_sums_out[(size_t)b * kHeads + g * kGroupSize + wave] = v;
+            if (blockIdx.x == 0 && row_sums_out) row_sums_out[(size_t)b * nheads + g * kGroupSize + wave] = v;
         }
         __syncthreads();
 #pragma unroll
         for (int h = 0; h < kGroupSize; ++h) lse[h] = s_lse[h];
     } else {
 #pragma unroll
-        for (int h = 0; h < kGroupSize; ++h) lse[h] = row_sums_in[(size_t)b * kHeads + g * kGroupSize + h];
+        for (int h = 0; h < kGroupSize; ++h) lse[h] = row_sums_in[(size_t)b * nheads + g * kGroupSize + h];
     }
     if (j0 >= scores_stride) return;
     float sum[8];
@@ -822,7 +843,7 @@ __global__ __launch_bounds__(256) void decode_aggregate_kernel(const float* __re
     if (j0 < len) {   // codes and references beyond the sequence were never written
 #pragma unroll
         for (int h = 0; h < kGroupSize; ++h) {
-            const float* row = scores + ((size_t)b * kHeads + g * kGroupSize + h) * scores_stride;
+            const float* row = scores + ((size_t)b * nheads + g * kGroupSize + h) * scores_stride;
             const uint16_t* sp = reinterpret_cast<const uint16_t*>(row) + j0;
             const float ref = row[scores_stride / 2 + (j0 >> 6)] - lse[h];
             uint32_t q[8];
@@ -841,7 +862,7 @@ __global__ __launch_bounds__(256) void decode_aggregate_kernel(const float* __re
             }
         }
     }
-    half_t* ap = agg + ((size_t)b * kGroups + g) * scores_stride + j0;
+    half_t* ap = agg + ((size_t)b * kvh + g) * scores_stride + j0;
     if (full && ((scores_stride & 7) == 0)) {
         Pack16 o;
 #pragma unroll
@@ -856,42 +877,68 @@ __global__ __launch_bounds__(256) void decode_aggregate_kernel(const float* __re
 
 }  // namespace
 
-hipError_t launch_decode_split(const DecodeParams& p, bool gather, bool with_v, bool write_scores,
-                               hipStream_t stream) {
-    dim3 grid(kGroups, p.num_split, p.B), block(kThreads);
+namespace {
+
+template <int D, typename T>
+hipError_t launch_split_t(const DecodeParams& p, bool gather, bool with_v, bool write_scores, hipStream_t stream) {
+    dim3 grid(p.G, p.num_split, p.B), block(kThreads);
     if (gather && p.idx_physical) {
-        hipLaunchKernelGGL((decode_split_kernel<true, true, false, true>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((decode_split_kernel<true, true, false, true, D, T>), grid, block, 0, stream, p);
     } else if (gather) {
-        hipLaunchKernelGGL((decode_split_kernel<true, true, false>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((decode_split_kernel<true, true, false, false, D, T>), grid, block, 0, stream, p);
     } else if (write_scores) {
         if (with_v)
-            hipLaunchKernelGGL((decode_split_kernel<false, true, true>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((decode_split_kernel<false, true, true, false, D, T>), grid, block, 0, stream, p);
         else
-            hipLaunchKernelGGL((decode_split_kernel<false, false, true>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((decode_split_kernel<false, false, true, false, D, T>), grid, block, 0, stream, p);
     } else {
-        hipLaunchKernelGGL((decode_split_kernel<false, true, false>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((decode_split_kernel<false, true, false, false, D, T>), grid, block, 0, stream, p);
     }
     return hipGetLastError();
 }
 
-hipError_t launch_decode_combine(const float* glse, const float* opart, half_t* out,
-                                 float* row_sums, int batch, int num_split, bool with_v,
-                                 hipStream_t stream) {
-    dim3 grid(kHeads, batch), block(128);
+template <int D, typename T>
+hipError_t launch_combine_t(const float* glse, const float* opart, void* out, float* row_sums, int batch, int heads,
+                            int num_split, bool with_v, hipStream_t stream) {
+    dim3 grid(heads, batch), block(128);
     if (with_v)
-        hipLaunchKernelGGL((decode_combine_kernel<true>), grid, block, 0, stream, glse, opart, out,
-                           row_sums, num_split);
+        hipLaunchKernelGGL((decode_combine_kernel<true, D, T>), grid, block, 0, stream, glse, opart,
+                           static_cast<T*>(out), row_sums, num_split);
     else
-        hipLaunchKernelGGL((decode_combine_kernel<false>), grid, block, 0, stream, glse, opart, out,
-                           row_sums, num_split);
+        hipLaunchKernelGGL((decode_combine_kernel<false, D, T>), grid, block, 0, stream, glse, opart,
+                           static_cast<T*>(out), row_sums, num_split);
     return hipGetLastError();
+}
+
+}  // namespace
+
+// head_dim in {64, 128}, elem in {kElemF16, kElemBF16}: checked by the callers
+hipError_t launch_decode_split(const DecodeParams& p, bool gather, bool with_v, bool write_scores,
+                               hipStream_t stream) {
+    if (p.head_dim == 128)
+        return p.elem == kElemBF16 ? launch_split_t<128, bf16_t>(p, gather, with_v, write_scores, stream)
+                                   : launch_split_t<128, half_t>(p, gather, with_v, write_scores, stream);
+    return p.elem == kElemBF16 ? launch_split_t<64, bf16_t>(p, gather, with_v, write_scores, stream)
+                               : launch_split_t<64, half_t>(p, gather, with_v, write_scores, stream);
+}
+
+hipError_t launch_decode_combine(const float* glse, const float* opart, void* out, float* row_sums,
+                                 int batch, int heads, int num_split, bool with_v, int head_dim, int elem,
+                                 hipStream_t stream) {
+    if (head_dim == 128)
+        return elem == kElemBF16
+                   ? launch_combine_t<128, bf16_t>(glse, opart, out, row_sums, batch, heads, num_split, with_v, stream)
+                   : launch_combine_t<128, half_t>(glse, opart, out, row_sums, batch, heads, num_split, with_v, stream);
+    return elem == kElemBF16
+               ? launch_combine_t<64, bf16_t>(glse, opart, out, row_sums, batch, heads, num_split, with_v, stream)
+               : launch_combine_t<64, half_t>(glse, opart, out, row_sums, batch, heads, num_split, with_v, stream);
 }
 
 hipError_t launch_decode_aggregate(const float* scores, const float* row_sums_in, const float* glse,
                                    int num_split, float* row_sums_out, const int* seqlens,
-                                   half_t* agg, int batch, int scores_stride, int uniform_len,
+                                   half_t* agg, int batch, int groups, int scores_stride, int uniform_len,
                                    int len_cap, hipStream_t stream) {
-    dim3 grid((scores_stride + 2047) / 2048, kGroups, batch), block(256);
+    dim3 grid((scores_stride + 2047) / 2048, groups, batch), block(256);
     hipLaunchKernelGGL(decode_aggregate_kernel, grid, block, 0, stream, scores, row_sums_in, glse,
                        num_split, row_sums_out, seqlens, agg, scores_stride, uniform_len, len_cap);
     return hipGetLastError();
