@@ -124,6 +124,16 @@ int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K
                                     int max_pages, int page_size, const kascade_strides* kv_strides,
                                     const kascade_half* k_new, const kascade_half* v_new,
                                     int32_t* sync_counters, void* stream);
+/* kascade_decode_reuse_paged_call for any kascade_shape. */
+int kascade_decode_reuse_paged_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K,
+                                    const kascade_half* V, const int32_t* cache_seqlens,
+                                    const int32_t* topk_indices, const int32_t* head_mapping,
+                                    float topk_percent, float* glse, float* Output_partial,
+                                    kascade_half* Output, int batch, int kv_stride_tokens,
+                                    int topk, int num_split, const int32_t* block_table,
+                                    int max_pages, int page_size, const kascade_strides* kv_strides,
+                                    const kascade_half* k_new, const kascade_half* v_new,
+                                    int32_t* sync_counters, void* stream);
 
 /* Reuse-layer decode over a paged cache whose index lists were translated to cache rows once, at
  * the anchor (kascade_translate_indices_call): cache_rows [B,G,topk] holds page * page_size + slot
@@ -136,6 +146,15 @@ int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K
  * <= 0 and nothing is appended.  The block table is used by the fused append only.  Entries are
  * clamped to [0, num_pages * page_size). */
 int kascade_decode_reuse_rows_call(const kascade_half* Q, const kascade_half* K_pages,
+                                   const kascade_half* V_pages, const int32_t* cache_seqlens,
+                                   const int32_t* cache_rows, const int32_t* head_mapping,
+                                   float topk_percent, float* glse, float* Output_partial,
+                                   kascade_half* Output, int batch, int topk, int num_split,
+                                   const int32_t* block_table, int max_pages, int page_size,
+                                   int num_pages, const kascade_half* k_new,
+                                   const kascade_half* v_new, int32_t* sync_counters, void* stream);
+/* kascade_decode_reuse_rows_call for any kascade_shape. */
+int kascade_decode_reuse_rows_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K_pages,
                                    const kascade_half* V_pages, const int32_t* cache_seqlens,
                                    const int32_t* cache_rows, const int32_t* head_mapping,
                                    float topk_percent, float* glse, float* Output_partial,
@@ -178,6 +197,15 @@ int kascade_decode_dense_paged_call(const kascade_half* Q, const kascade_half* K
                                     const kascade_strides* kv_strides, const kascade_half* k_new,
                                     const kascade_half* v_new, int32_t* sync_counters,
                                     void* stream);
+/* kascade_decode_dense_paged_call for any kascade_shape. */
+int kascade_decode_dense_paged_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K,
+                                    const kascade_half* V, const int32_t* cache_seqlens,
+                                    float* glse, float* Output_partial, kascade_half* Output,
+                                    int batch, int kv_stride_tokens, int num_split,
+                                    const int32_t* block_table, int max_pages, int page_size,
+                                    const kascade_strides* kv_strides, const kascade_half* k_new,
+                                    const kascade_half* v_new, int32_t* sync_counters,
+                                    void* stream);
 
 /* Anchor-layer decode: split QK^T (+PV when with_output != 0), log-sum merge and
  * pooled post-softmax scores.  Replaces the three launches of the reference's
@@ -194,6 +222,18 @@ int kascade_decode_dense_paged_call(const kascade_half* Q, const kascade_half* K
  *                     of softmax probabilities; 0 at positions >= cache_seqlens[b]
  *   Output            [B,H,D] f16, written only when with_output != 0. */
 int kascade_decode_recompute_paged_call(const kascade_half* Q, const kascade_half* K,
+                                        const kascade_half* V, const int32_t* cache_seqlens,
+                                        float* glse, float* Output_partial, float* row_sums,
+                                        float* scores, kascade_half* Output,
+                                        kascade_half* aggregated_scores, int batch,
+                                        int kv_stride_tokens, int scores_stride, int num_split,
+                                        int with_output, const int32_t* block_table,
+                                        int max_pages, int page_size,
+                                        const kascade_strides* kv_strides,
+                                        const kascade_half* k_new, const kascade_half* v_new,
+                                        int32_t* sync_counters, void* stream);
+/* kascade_decode_recompute_paged_call for any kascade_shape. */
+int kascade_decode_recompute_paged_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K,
                                         const kascade_half* V, const int32_t* cache_seqlens,
                                         float* glse, float* Output_partial, float* row_sums,
                                         float* scores, kascade_half* Output,
@@ -251,6 +291,11 @@ int kascade_prefill_dense_call(const kascade_half* Q, const kascade_half* K, con
                                float* log_sum, kascade_half* Output, int batch, int seq_len,
                                kascade_strides q_strides, kascade_strides kv_strides,
                                int with_output, void* stream);
+/* kascade_prefill_dense_call for any kascade_shape. */
+int kascade_prefill_dense_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K, const kascade_half* V,
+                               float* log_sum, kascade_half* Output, int batch, int seq_len,
+                               kascade_strides q_strides, kascade_strides kv_strides,
+                               int with_output, void* stream);
 
 /* Pooled tile scores.  Same argument list as the reference's aggregate `call`
  * (dynamic_alllen_aggregate_cp_async_ts32_dim128_gsize4_heads32_groups8.cu:138;
@@ -260,6 +305,11 @@ int kascade_prefill_dense_call(const kascade_half* Q, const kascade_half* K, con
  *   exp2(q.k*scale - log_sum).  With fill_invalid != 0 the entries j >= 32 t are
  *   written as -inf (the reference pre-fills the tensor on the host instead). */
 int kascade_prefill_aggregate_call(const kascade_half* Q, const kascade_half* K,
+                                   const float* log_sum, kascade_half* aggregate_scores, int batch,
+                                   int seq_len, kascade_strides q_strides,
+                                   kascade_strides kv_strides, int fill_invalid, void* stream);
+/* kascade_prefill_aggregate_call for any kascade_shape. */
+int kascade_prefill_aggregate_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K,
                                    const float* log_sum, kascade_half* aggregate_scores, int batch,
                                    int seq_len, kascade_strides q_strides,
                                    kascade_strides kv_strides, int fill_invalid, void* stream);
@@ -278,6 +328,12 @@ int kascade_prefill_aggregate_range_call(const kascade_half* Q, const kascade_ha
                                          int batch, int q_start, int q_len,
                                          kascade_strides q_strides, kascade_strides kv_strides,
                                          int fill_invalid, void* stream);
+/* kascade_prefill_aggregate_range_call for any kascade_shape. */
+int kascade_prefill_aggregate_range_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K,
+                                         const float* log_sum, kascade_half* aggregate_scores,
+                                         int batch, int q_start, int q_len,
+                                         kascade_strides q_strides, kascade_strides kv_strides,
+                                         int fill_invalid, void* stream);
 
 /* Reuse-layer prefill.  Same argument list as the reference's reuse `call`s
  * (…reuse_cp_async_ts32…groups8_rolling.cu:268 and …groups8.cu:260; DSL
@@ -291,6 +347,12 @@ int kascade_prefill_reuse_call(const kascade_half* Q, const kascade_half* K, con
                                float topk_percent, kascade_half* Output, int batch, int seq_len,
                                int max_topk_num, int rolling, kascade_strides q_strides,
                                kascade_strides kv_strides, void* stream);
+/* kascade_prefill_reuse_call for any kascade_shape. */
+int kascade_prefill_reuse_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K, const kascade_half* V,
+                               const int32_t* topk_indices, const int32_t* head_mapping,
+                               float topk_percent, kascade_half* Output, int batch, int seq_len,
+                               int max_topk_num, int rolling, kascade_strides q_strides,
+                               kascade_strides kv_strides, void* stream);
 
 /* --------------------------------------------------------------- KV append */
 
@@ -300,6 +362,12 @@ int kascade_prefill_reuse_call(const kascade_half* Q, const kascade_half* K, con
  * this is the step right before the decode path.
  *   k_new, v_new [B,n_new,G,D] with strides new_strides (b, l, h=g). */
 int kascade_paged_kv_append_call(kascade_half* K_pages, kascade_half* V_pages,
+                                 const kascade_half* k_new, const kascade_half* v_new,
+                                 const int32_t* start_pos, const int32_t* block_table, int batch,
+                                 int n_new, int max_pages, int page_size,
+                                 kascade_strides new_strides, void* stream);
+/* kascade_paged_kv_append_call for any kascade_shape. */
+int kascade_paged_kv_append_shaped_call(const kascade_shape* shape, kascade_half* K_pages, kascade_half* V_pages,
                                  const kascade_half* k_new, const kascade_half* v_new,
                                  const int32_t* start_pos, const int32_t* block_table, int batch,
                                  int n_new, int max_pages, int page_size,

@@ -67,6 +67,17 @@ SIGNATURES = {
     "kascade_diag_gather_rows_call": (_I, [_P, _P, _P, _L, _L, _P, _P]),
 }
 
+class Shape(C.Structure):
+    """kascade_shape: KV heads, head dimension, element type (0 fp16, 1 bf16)."""
+    _fields_ = [("kv_heads", C.c_int32), ("head_dim", C.c_int32), ("dtype", C.c_int32)]
+
+
+# every *_shaped_call takes a kascade_shape* followed by the arguments of the plain entry
+for _name in ("decode_reuse_paged", "decode_reuse_rows", "decode_dense_paged", "decode_recompute_paged",
+              "prefill_dense", "prefill_aggregate", "prefill_aggregate_range", "prefill_reuse", "paged_kv_append"):
+    _res, _args = SIGNATURES[f"kascade_{_name}_call"]
+    SIGNATURES[f"kascade_{_name}_shaped_call"] = (_res, [C.POINTER(Shape)] + list(_args))
+
 _lib = None
 _initialised = False
 

@@ -152,7 +152,7 @@ int set_append(DecodeParams& p, const kascade_half* k_new, const kascade_half* v
 
 extern "C" {
 
-int kascade_abi_version(void) { return 6; }
+int kascade_abi_version(void) { return 7; }
 
 const char* kascade_get_last_error(void) { return g_err; }
 
@@ -530,7 +530,9 @@ int kascade_topk_rows_call(const kascade_half* scores, int32_t* out_idx, int row
                                  period, k, fill_value, &tr, s), "topk");
 }
 
-int kascade_prefill_dense_call(const kascade_half* Q, const kascade_half* K, const kascade_half* V,
+}  // extern "C"
+namespace {
+int prefill_dense_impl(const Shape& sh, const kascade_half* Q, const kascade_half* K, const kascade_half* V,
                                float* log_sum, kascade_half* Output, int batch, int seq_len,
                                kascade_strides q_strides, kascade_strides kv_strides,
                                int with_output, void* stream) {
@@ -542,15 +544,36 @@ int kascade_prefill_dense_call(const kascade_half* Q, const kascade_half* K, con
             "prefill_dense: tensors must be 16-byte aligned");
     if (check_strides(q_strides, "Q") || check_strides(kv_strides, "K/V")) return -1;
     PrefillParams p{};
+    p.G = sh.G; p.head_dim = sh.D; p.elem = sh.elem;
     p.Q = H(Q); p.K = H(K); p.V = with_output ? H(V) : H(K); p.log_sum = log_sum; p.O = H(Output);
     p.q_sb = q_strides.b; p.q_sl = q_strides.l; p.q_sh = q_strides.h;
     p.k_sb = kv_strides.b; p.k_sl = kv_strides.l; p.k_sh = kv_strides.h;
     p.B = batch; p.L = seq_len; p.Lq = seq_len; p.T = (seq_len + kTile - 1) / kTile;
-    return check_hip(launch_prefill_attn(p, false, with_output != 0, with_output ? 1 : 2,
+    return check_hip(launch_prefill_attn(p, false, with_output != 0, (with_output || sh.D != 128) ? 1 : 2,
                                          static_cast<hipStream_t>(stream)), "prefill_dense");
 }
+}  // namespace
+extern "C" {
 
-int kascade_prefill_aggregate_call(const kascade_half* Q, const kascade_half* K,
+int kascade_prefill_dense_call(const kascade_half* Q, const kascade_half* K, const kascade_half* V,
+                               float* log_sum, kascade_half* Output, int batch, int seq_len,
+                               kascade_strides q_strides, kascade_strides kv_strides,
+                               int with_output, void* stream) {
+    return prefill_dense_impl(kRefShape, Q, K, V, log_sum, Output, batch, seq_len, q_strides, kv_strides, with_output, stream);
+}
+
+int kascade_prefill_dense_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K, const kascade_half* V,
+                               float* log_sum, kascade_half* Output, int batch, int seq_len,
+                               kascade_strides q_strides, kascade_strides kv_strides,
+                               int with_output, void* stream) {
+    Shape sh;
+    if (get_shape(shape, &sh)) return -1;
+    return prefill_dense_impl(sh, Q, K, V, log_sum, Output, batch, seq_len, q_strides, kv_strides, with_output, stream);
+}
+
+}  // extern "C"
+namespace {
+int prefill_aggregate_impl(const Shape& sh, const kascade_half* Q, const kascade_half* K,
                                    const float* log_sum, kascade_half* aggregate_scores, int batch,
                                    int seq_len, kascade_strides q_strides,
                                    kascade_strides kv_strides, int fill_invalid, void* stream) {
@@ -559,6 +582,7 @@ int kascade_prefill_aggregate_call(const kascade_half* Q, const kascade_half* K,
     REQUIRE(aligned16(Q) && aligned16(K), "prefill_aggregate: Q/K must be 16-byte aligned");
     if (check_strides(q_strides, "Q") || check_strides(kv_strides, "K")) return -1;
     PrefillParams p{};
+    p.G = sh.G; p.head_dim = sh.D; p.elem = sh.elem;
     p.Q = H(Q); p.K = H(K); p.V = H(K); p.log_sum_in = log_sum; p.agg = H(aggregate_scores);
     p.q_sb = q_strides.b; p.q_sl = q_strides.l; p.q_sh = q_strides.h;
     p.k_sb = kv_strides.b; p.k_sl = kv_strides.l; p.k_sh = kv_strides.h;
@@ -566,8 +590,28 @@ int kascade_prefill_aggregate_call(const kascade_half* Q, const kascade_half* K,
     return check_hip(launch_prefill_aggregate(p, static_cast<hipStream_t>(stream)),
                      "prefill_aggregate");
 }
+}  // namespace
+extern "C" {
 
-int kascade_prefill_aggregate_range_call(const kascade_half* Q, const kascade_half* K,
+int kascade_prefill_aggregate_call(const kascade_half* Q, const kascade_half* K,
+                                   const float* log_sum, kascade_half* aggregate_scores, int batch,
+                                   int seq_len, kascade_strides q_strides,
+                                   kascade_strides kv_strides, int fill_invalid, void* stream) {
+    return prefill_aggregate_impl(kRefShape, Q, K, log_sum, aggregate_scores, batch, seq_len, q_strides, kv_strides, fill_invalid, stream);
+}
+
+int kascade_prefill_aggregate_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K,
+                                   const float* log_sum, kascade_half* aggregate_scores, int batch,
+                                   int seq_len, kascade_strides q_strides,
+                                   kascade_strides kv_strides, int fill_invalid, void* stream) {
+    Shape sh;
+    if (get_shape(shape, &sh)) return -1;
+    return prefill_aggregate_impl(sh, Q, K, log_sum, aggregate_scores, batch, seq_len, q_strides, kv_strides, fill_invalid, stream);
+}
+
+}  // extern "C"
+namespace {
+int prefill_aggregate_range_impl(const Shape& sh, const kascade_half* Q, const kascade_half* K,
                                          const float* log_sum, kascade_half* aggregate_scores,
                                          int batch, int q_start, int q_len,
                                          kascade_strides q_strides, kascade_strides kv_strides,
@@ -579,6 +623,7 @@ int kascade_prefill_aggregate_range_call(const kascade_half* Q, const kascade_ha
     REQUIRE(aligned16(Q) && aligned16(K), "prefill_aggregate_range: Q/K must be 16-byte aligned");
     if (check_strides(q_strides, "Q") || check_strides(kv_strides, "K")) return -1;
     PrefillParams p{};
+    p.G = sh.G; p.head_dim = sh.D; p.elem = sh.elem;
     p.Q = H(Q); p.K = H(K); p.V = H(K); p.log_sum_in = log_sum; p.agg = H(aggregate_scores);
     p.q_sb = q_strides.b; p.q_sl = q_strides.l; p.q_sh = q_strides.h;
     p.k_sb = kv_strides.b; p.k_sl = kv_strides.l; p.k_sh = kv_strides.h;
@@ -587,8 +632,30 @@ int kascade_prefill_aggregate_range_call(const kascade_half* Q, const kascade_ha
     return check_hip(launch_prefill_aggregate(p, static_cast<hipStream_t>(stream)),
                      "prefill_aggregate_range");
 }
+}  // namespace
+extern "C" {
 
-int kascade_prefill_reuse_call(const kascade_half* Q, const kascade_half* K, const kascade_half* V,
+int kascade_prefill_aggregate_range_call(const kascade_half* Q, const kascade_half* K,
+                                         const float* log_sum, kascade_half* aggregate_scores,
+                                         int batch, int q_start, int q_len,
+                                         kascade_strides q_strides, kascade_strides kv_strides,
+                                         int fill_invalid, void* stream) {
+    return prefill_aggregate_range_impl(kRefShape, Q, K, log_sum, aggregate_scores, batch, q_start, q_len, q_strides, kv_strides, fill_invalid, stream);
+}
+
+int kascade_prefill_aggregate_range_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K,
+                                         const float* log_sum, kascade_half* aggregate_scores,
+                                         int batch, int q_start, int q_len,
+                                         kascade_strides q_strides, kascade_strides kv_strides,
+                                         int fill_invalid, void* stream) {
+    Shape sh;
+    if (get_shape(shape, &sh)) return -1;
+    return prefill_aggregate_range_impl(sh, Q, K, log_sum, aggregate_scores, batch, q_start, q_len, q_strides, kv_strides, fill_invalid, stream);
+}
+
+}  // extern "C"
+namespace {
+int prefill_reuse_impl(const Shape& sh, const kascade_half* Q, const kascade_half* K, const kascade_half* V,
                                const int32_t* topk_indices, const int32_t* head_mapping,
                                float topk_percent, kascade_half* Output, int batch, int seq_len,
                                int max_topk_num, int rolling, kascade_strides q_strides,
@@ -602,6 +669,7 @@ int kascade_prefill_reuse_call(const kascade_half* Q, const kascade_half* K, con
             "prefill_reuse: tensors must be 16-byte aligned");
     if (check_strides(q_strides, "Q") || check_strides(kv_strides, "K/V")) return -1;
     PrefillParams p{};
+    p.G = sh.G; p.head_dim = sh.D; p.elem = sh.elem;
     p.Q = H(Q); p.K = H(K); p.V = H(V); p.idx = topk_indices; p.head_map = head_mapping;
     p.O = H(Output); p.log_sum = nullptr;
     p.q_sb = q_strides.b; p.q_sl = q_strides.l; p.q_sh = q_strides.h;
@@ -611,8 +679,30 @@ int kascade_prefill_reuse_call(const kascade_half* Q, const kascade_half* K, con
     return check_hip(launch_prefill_attn(p, true, true, 1, static_cast<hipStream_t>(stream)),
                      "prefill_reuse");
 }
+}  // namespace
+extern "C" {
 
-int kascade_paged_kv_append_call(kascade_half* K_pages, kascade_half* V_pages,
+int kascade_prefill_reuse_call(const kascade_half* Q, const kascade_half* K, const kascade_half* V,
+                               const int32_t* topk_indices, const int32_t* head_mapping,
+                               float topk_percent, kascade_half* Output, int batch, int seq_len,
+                               int max_topk_num, int rolling, kascade_strides q_strides,
+                               kascade_strides kv_strides, void* stream) {
+    return prefill_reuse_impl(kRefShape, Q, K, V, topk_indices, head_mapping, topk_percent, Output, batch, seq_len, max_topk_num, rolling, q_strides, kv_strides, stream);
+}
+
+int kascade_prefill_reuse_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K, const kascade_half* V,
+                               const int32_t* topk_indices, const int32_t* head_mapping,
+                               float topk_percent, kascade_half* Output, int batch, int seq_len,
+                               int max_topk_num, int rolling, kascade_strides q_strides,
+                               kascade_strides kv_strides, void* stream) {
+    Shape sh;
+    if (get_shape(shape, &sh)) return -1;
+    return prefill_reuse_impl(sh, Q, K, V, topk_indices, head_mapping, topk_percent, Output, batch, seq_len, max_topk_num, rolling, q_strides, kv_strides, stream);
+}
+
+}  // extern "C"
+namespace {
+int paged_kv_append_impl(const Shape& sh, kascade_half* K_pages, kascade_half* V_pages,
                                  const kascade_half* k_new, const kascade_half* v_new,
                                  const int32_t* start_pos, const int32_t* block_table, int batch,
                                  int n_new, int max_pages, int page_size,
@@ -628,9 +718,29 @@ int kascade_paged_kv_append_call(kascade_half* K_pages, kascade_half* V_pages,
             "paged_kv_append: tensors must be 16-byte aligned");
     return check_hip(launch_paged_kv_append(H(K_pages), H(V_pages), H(k_new), H(v_new), start_pos,
                                             block_table, batch, n_new, max_pages, shift,
-                                            new_strides.b, new_strides.l, new_strides.h,
+                                            new_strides.b, new_strides.l, new_strides.h, sh.G, sh.D,
                                             static_cast<hipStream_t>(stream)),
                      "paged_kv_append");
+}
+}  // namespace
+extern "C" {
+
+int kascade_paged_kv_append_call(kascade_half* K_pages, kascade_half* V_pages,
+                                 const kascade_half* k_new, const kascade_half* v_new,
+                                 const int32_t* start_pos, const int32_t* block_table, int batch,
+                                 int n_new, int max_pages, int page_size,
+                                 kascade_strides new_strides, void* stream) {
+    return paged_kv_append_impl(kRefShape, K_pages, V_pages, k_new, v_new, start_pos, block_table, batch, n_new, max_pages, page_size, new_strides, stream);
+}
+
+int kascade_paged_kv_append_shaped_call(const kascade_shape* shape, kascade_half* K_pages, kascade_half* V_pages,
+                                 const kascade_half* k_new, const kascade_half* v_new,
+                                 const int32_t* start_pos, const int32_t* block_table, int batch,
+                                 int n_new, int max_pages, int page_size,
+                                 kascade_strides new_strides, void* stream) {
+    Shape sh;
+    if (get_shape(shape, &sh)) return -1;
+    return paged_kv_append_impl(sh, K_pages, V_pages, k_new, v_new, start_pos, block_table, batch, n_new, max_pages, page_size, new_strides, stream);
 }
 
 int kascade_rope_append_paged_call(const kascade_half* q_in, const kascade_strides* q_strides,
@@ -698,6 +808,7 @@ static int chunk_params(PrefillParams& p, const char* what, const kascade_half* 
     REQUIRE((long long)max_pages * page_size >= (long long)q_start + q_len,
             "prefill_chunk: block table shorter than q_start + q_len");
     (void)what;
+    p.G = kRefShape.G; p.head_dim = kRefShape.D; p.elem = kRefShape.elem;
     p.Q = H(Q);
     p.q_sb = q_strides.b; p.q_sl = q_strides.l; p.q_sh = q_strides.h;
     p.B = batch; p.L = q_start + q_len; p.Lq = q_len; p.q_start = q_start;

@@ -1,5 +1,6 @@
 // Paged KV-cache append: scatter the new tokens' K/V rows into their page slots.
-// One 16-byte chunk per thread; grid covers B * n_new * G * 16 chunks for K and V.
+// One 16-byte chunk per thread; grid covers B * n_new * G * (D/8) chunks for K and V.  Elements are
+// 16 bits wide (fp16 or bf16: the kernel only moves them).
 #include "paged.h"
 
 namespace kascade {
@@ -10,13 +11,14 @@ __global__ __launch_bounds__(256) void paged_kv_append_kernel(
     half_t* __restrict__ Kp, half_t* __restrict__ Vp, const half_t* __restrict__ k_new,
     const half_t* __restrict__ v_new, const int* __restrict__ start_pos,
     const int* __restrict__ block_table, int batch, int n_new, int max_pages, int page_shift,
-    long long sb, long long sl, long long sh) {
-    const long long total = (long long)batch * n_new * kGroups * 16;
+    long long sb, long long sl, long long sh, int groups, int head_dim) {
+    const int chunks = head_dim / 8;
+    const long long total = (long long)batch * n_new * groups * chunks;
     const long long c = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= total) return;
-    const int col = (int)(c & 15);
-    const int g = (int)((c >> 4) % kGroups);
-    const long long bt = c / (16 * kGroups);
+    const int col = (int)(c % chunks);
+    const int g = (int)((c / chunks) % groups);
+    const long long bt = c / (chunks * groups);
     const int t = (int)(bt % n_new);
     const int b = (int)(bt / n_new);
     const int tok = start_pos[b] + t;
@@ -25,7 +27,7 @@ __global__ __launch_bounds__(256) void paged_kv_append_kernel(
     if (tok < 0 || (tok >> page_shift) >= max_pages) return;
     const int pg = block_table[(long long)b * max_pages + (tok >> page_shift)];
     const long long row = ((long long)pg << page_shift) + (tok & ((1 << page_shift) - 1));
-    const long long dst = (row * kGroups + g) * kDim + col * 8;
+    const long long dst = (row * groups + g) * head_dim + col * 8;
     const long long src = b * sb + t * sl + g * sh + col * 8;
     *reinterpret_cast<uint4_t*>(Kp + dst) = ld_global_16(k_new + src);
     *reinterpret_cast<uint4_t*>(Vp + dst) = ld_global_16(v_new + src);
@@ -136,12 +138,13 @@ hipError_t launch_decode_budgets(int* seqlens, int advance, float percent, int b
 hipError_t launch_paged_kv_append(half_t* Kp, half_t* Vp, const half_t* k_new, const half_t* v_new,
                                   const int* start_pos, const int* block_table, int batch,
                                   int n_new, int max_pages, int page_shift, long long sb,
-                                  long long sl, long long sh, hipStream_t stream) {
-    const long long total = (long long)batch * n_new * kGroups * 16;
+                                  long long sl, long long sh, int groups, int head_dim,
+                                  hipStream_t stream) {
+    const long long total = (long long)batch * n_new * groups * (head_dim / 8);
     if (total == 0) return hipSuccess;
     dim3 grid((unsigned)((total + 255) / 256)), block(256);
     hipLaunchKernelGGL(paged_kv_append_kernel, grid, block, 0, stream, Kp, Vp, k_new, v_new,
-                       start_pos, block_table, batch, n_new, max_pages, page_shift, sb, sl, sh);
+                       start_pos, block_table, batch, n_new, max_pages, page_shift, sb, sl, sh, groups, head_dim);
     return hipGetLastError();
 }
 

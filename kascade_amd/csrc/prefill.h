@@ -7,14 +7,16 @@ namespace kascade {
 struct PrefillParams {
     // Queries are rows [0, Lq) of Q at global positions q_start + row; keys are positions
     // [0, L), L = q_start + Lq.  A whole-prompt call has q_start = 0 and Lq = L.
-    const half_t* Q;          // [B,Lq,H,D] through (q_sb, q_sl, q_sh)
-    const half_t* K;          // [B,L,G,D] through (k_sb, k_sl, k_sh); V shares the strides.
-    const half_t* V;          //   Paged: [num_pages, page, G, D] contiguous, strides unused
+    // Q, K, V and O hold elements of kind `elem` (fp16 or bf16); G KV heads, H = 4 G query heads,
+    // head dimension head_dim (64 or 128).
+    const void* Q;            // [B,Lq,H,D] through (q_sb, q_sl, q_sh)
+    const void* K;            // [B,L,G,D] through (k_sb, k_sl, k_sh); V shares the strides.
+    const void* V;            //   Paged: [num_pages, page, G, D] contiguous, strides unused
     const int* idx;           // [B,G,T,max_topk] (reuse); physical rows when paged
     const int* head_map;      // [G] (reuse)
     const float* log_sum_in;  // [B,Lq,H] (aggregate)
     float* log_sum;           // [B,Lq,H] or null (attention kernel output)
-    half_t* O;                // [B,Lq,H,D] contiguous
+    void* O;                  // [B,Lq,H,D] contiguous
     half_t* agg;              // [B,G,T,L] (aggregate)
     const int* block_table;   // [B,max_pages] or null (strided K/V)
     long long q_sb, q_sl, q_sh;
@@ -26,6 +28,9 @@ struct PrefillParams {
     int rolling;
     float topk_percent;
     int fill_invalid;
+    int G;                    // KV heads
+    int head_dim;             // 64 or 128
+    int elem;                 // kElemF16 or kElemBF16
 };
 
 hipError_t launch_prefill_attn(const PrefillParams& p, bool reuse, bool with_v, int nqb,

@@ -31,10 +31,22 @@ namespace kascade {
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kKT = 64;           // keys per tile (attention kernel)
-constexpr int kKStride = 136;      // halves per K row in LDS (128 + 8 pad)
-constexpr int kVStride = 64;       // halves per V^T row in LDS (one 64-key tile)
 constexpr int kAggKT = 128;        // keys per tile (aggregate kernel)
+
+// Tile geometry of the attention kernel per head dimension.  A tile is 16 KB of K (and of V)
+// whatever D: 64 keys at D = 128, 128 keys at D = 64, so a thread always stages four consecutive
+// keys of one 16-byte column, both products issue 16 matrix instructions per tile and wavefront,
+// and the score registers a narrower head frees hold the extra keys.
+template <int D> struct AttnTile {
+    static constexpr int kKT = 64 * 128 / D;     // keys per tile
+    static constexpr int kKStride = D + 8;       // elements per K row in LDS (padded)
+    static constexpr int kVStride = kKT;         // elements per V^T row in LDS (one tile of keys)
+    static constexpr int kKS = D / 16;           // contraction steps of S^T = K Q^T
+    static constexpr int kDB = D / 32;           // 32-row blocks of O^T
+    static constexpr int kKB = kKT / 32;         // 32-key blocks of a tile
+    static constexpr int kS = kKT / 16;          // contraction steps of O^T = V^T P^T
+    static constexpr int kChunks = D / 8;        // 16-byte columns of a row
+};
 
 __device__ __forceinline__ int swap_bits23(int x) {
     return (x & ~0xC) | ((x & 4) << 1) | ((x & 8) >> 1);
@@ -49,8 +61,18 @@ __device__ __forceinline__ int rolling_budget(float pct, int tile_start) {
 // Queries are rows [0, Lq) of Q at global positions q_start + row (q_start a multiple of 32);
 // keys are positions [0, L) with L = q_start + Lq.  PAGED: K/V are pages [P, page, G, D]
 // addressed through the block table, and gathered index rows hold physical row numbers.
-template <int NQB, bool REUSE, bool WITH_V, bool PAGED>
-__device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t* sK, half_t* sV) {
+template <int NQB, bool REUSE, bool WITH_V, bool PAGED, int D, typename T>
+__device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK, T* sV) {
+    typedef typename Elem<T>::x8 x8_t;
+    typedef typename Elem<T>::x4 x4_t;
+    typedef AttnTile<D> G_;
+    constexpr int kKT = G_::kKT, kKStride = G_::kKStride, kVStride = G_::kVStride;
+    constexpr int kKS = G_::kKS, kDB = G_::kDB, kKB = G_::kKB, kS = G_::kS, kChunks = G_::kChunks;
+    constexpr float kScaleLog2 = ScaleLog2<D>::value;
+    const int kvh = p.G, nheads = p.G * kGroupSize;
+    const T* Qp = (const T*)p.Q;
+    const T* Kp = (const T*)p.K;
+    const T* Vp = (const T*)p.V;
 
     constexpr int QT = 32 * NQB;
     const int L = p.L;
@@ -78,17 +100,17 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
         if (q0 > n) {
             sparse = true;
             ng = (n + kKT - 1) / kKT;
-            idx_row = p.idx + (((long long)b * kGroups + p.head_map[g]) * p.T + tq) * p.max_topk;
+            idx_row = p.idx + (((long long)b * kvh + p.head_map[g]) * p.T + tq) * p.max_topk;
         }
     }
     const int ntiles = sparse ? ng + 1 : (min(q0 + QT, L) + kKT - 1) / kKT;
 
-    const int krow = tid >> 4;   // tile positions 4*krow + i, 16-byte column kcol
-    const int kcol = tid & 15;
-    const half_t* kbase = PAGED ? p.K + (long long)g * kDim + kcol * 8
-                                : p.K + (long long)b * p.k_sb + (long long)g * p.k_sh + kcol * 8;
-    const half_t* vbase = PAGED ? p.V + (long long)g * kDim + kcol * 8
-                                : p.V + (long long)b * p.k_sb + (long long)g * p.k_sh + kcol * 8;
+    const int krow = tid / kChunks;   // tile positions 4*krow + i, 16-byte column kcol
+    const int kcol = tid % kChunks;
+    const T* kbase = PAGED ? Kp + (long long)g * D + kcol * 8
+                           : Kp + (long long)b * p.k_sb + (long long)g * p.k_sh + kcol * 8;
+    const T* vbase = PAGED ? Vp + (long long)g * D + kcol * 8
+                           : Vp + (long long)b * p.k_sb + (long long)g * p.k_sh + kcol * 8;
     const int* bt_row = PAGED ? p.block_table + (long long)b * p.max_pages : nullptr;
     const int page_mask = (1 << p.page_shift) - 1;
     const int max_row = PAGED ? (p.num_pages << p.page_shift) - 1 : 0;
@@ -107,7 +129,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
     int ids[4];
     int pend_ti = 0;        // tile the ids belong to
     uint4_t kr[4], vr[4];   // tile data in flight
-    const unsigned row_stride = PAGED ? (unsigned)(kGroups * kDim) : (unsigned)p.k_sl;   // host checks < 2^31
+    const unsigned row_stride = PAGED ? (unsigned)(kvh * D) : (unsigned)p.k_sl;   // host checks < 2^31
     auto fetch_ids = [&](int ti) {
         pend_ti = ti;
         if (sparse && ti < ng) {
@@ -143,13 +165,13 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
     };
 
     float m[NQB], l[NQB];
-    float16_t oT[NQB][4];
+    float16_t oT[NQB][kDB];
 #pragma unroll
     for (int qb = 0; qb < NQB; ++qb) {
         m[qb] = -INFINITY;
         l[qb] = 0.f;
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
+        for (int db = 0; db < kDB; ++db)
 #pragma unroll
             for (int v = 0; v < 16; ++v) oT[qb][db][v] = 0.f;
     }
@@ -166,19 +188,19 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
 
     // ---- Q fragments (B operand of S^T): query li (+32 qb), d chunk 16*ks + 8*lg; requested after
     // the first tile's rows, which the first barrier waits for ----
-    half8_t qf[NQB][8];
+    x8_t qf[NQB][kKS];
 #pragma unroll
     for (int qb = 0; qb < NQB; ++qb) {
         const int ql = q0l + 32 * qb + li;
         const bool ok = ql < Lq;
-        const half_t* qp = p.Q + (long long)b * p.q_sb + (long long)min(ql, Lq - 1) * p.q_sl +
-                           (long long)head * p.q_sh + lg * 8;
+        const T* qp = Qp + (long long)b * p.q_sb + (long long)min(ql, Lq - 1) * p.q_sl +
+                      (long long)head * p.q_sh + lg * 8;
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
-            Pack16 t;
+        for (int ks = 0; ks < kKS; ++ks) {
+            PackT<T> t;
             t.u = ld_global_16(qp + ks * 16);
             if (!ok) t.u = uint4_t{0, 0, 0, 0};
-            qf[qb][ks] = t.h8;
+            qf[qb][ks] = t.v8;
         }
     }
 
@@ -202,15 +224,15 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
             *reinterpret_cast<uint4_t*>(&sK[slot * kKStride + kcol * 8]) = kr[i];
         }
         if (WITH_V) {
-            Pack16 v0, v1, v2, v3;
+            PackT<T> v0, v1, v2, v3;
             v0.u = vr[0]; v1.u = vr[1]; v2.u = vr[2]; v3.u = vr[3];
             const int kq = krow;   // keys 4*kq .. 4*kq+3
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
                 const int d = kcol * 8 + r;
                 const int sw = (r ^ kcol) & 7;    // = ((d & 7) ^ (d >> 3)) & 7
-                half4_t w = {v0.h[r], v1.h[r], v2.h[r], v3.h[r]};
-                *reinterpret_cast<half4_t*>(&sV[d * kVStride + (((kq >> 1) ^ sw) * 8) + (kq & 1) * 4]) = w;
+                x4_t w = {v0.e[r], v1.e[r], v2.e[r], v3.e[r]};
+                *reinterpret_cast<x4_t*>(&sV[d * kVStride + (((kq >> 1) ^ sw) * 8) + (kq & 1) * 4]) = w;
             }
         }
         __syncthreads();
@@ -221,22 +243,21 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
 
         // ---- S^T = K_tile Q^T ----
         const bool diag_tile = diag_phase;
-        const int nkb = (diag_tile && QT == 32) ? 1 : 2;
-        float16_t sT[NQB][2];
+        const int nkb = (diag_tile && QT == 32) ? 1 : kKB;
+        float16_t sT[NQB][kKB];
         float16_t zero16;
 #pragma unroll
         for (int v = 0; v < 16; ++v) zero16[v] = 0.f;
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
+        for (int kb = 0; kb < kKB; ++kb) {
             if (kb < nkb) {
 #pragma unroll
-                for (int ks = 0; ks < 8; ++ks) {
-                    half8_t a = *reinterpret_cast<const half8_t*>(
+                for (int ks = 0; ks < kKS; ++ks) {
+                    x8_t a = *reinterpret_cast<const x8_t*>(
                         &sK[(32 * kb + li) * kKStride + ks * 16 + lg * 8]);
 #pragma unroll
                     for (int qb = 0; qb < NQB; ++qb)   // the first product starts from a constant zero
-                        sT[qb][kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[qb][ks],
-                                                                            ks == 0 ? zero16 : sT[qb][kb], 0, 0, 0);
+                        sT[qb][kb] = Elem<T>::mma_32x32x16(a, qf[qb][ks], ks == 0 ? zero16 : sT[qb][kb]);
                 }
             } else {   // second key block of a 32-key diagonal tile: nothing there
 #pragma unroll
@@ -253,7 +274,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
                 for (int qb = 0; qb < NQB; ++qb) {
                     const int q = q0 + 32 * qb + li;   // global position
 #pragma unroll
-                    for (int kb = 0; kb < 2; ++kb)
+                    for (int kb = 0; kb < kKB; ++kb)
 #pragma unroll
                         for (int v = 0; v < 16; ++v) {
                             const int key = kstart + 32 * kb + 16 * (v >> 3) + 8 * lg + (v & 7);
@@ -265,7 +286,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
 #pragma unroll
             for (int qb = 0; qb < NQB; ++qb)
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
+                for (int kb = 0; kb < kKB; ++kb)
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
                         const int pos = ti * kKT + 32 * kb + 16 * (v >> 3) + 8 * lg + (v & 7);
@@ -273,12 +294,12 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
                     }
         }
         // ---- online softmax (one query column per lane) ----
-        half8_t pf[NQB][4];
+        x8_t pf[NQB][kS];
 #pragma unroll
         for (int qb = 0; qb < NQB; ++qb) {
             float mx = -INFINITY;
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+            for (int kb = 0; kb < kKB; ++kb)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) mx = fmaxf(mx, sT[qb][kb][v]);
             mx = fmaxf(mx, __shfl_xor(mx, 32));
@@ -288,7 +309,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
             m[qb] = mnew;
             float sum = 0.f;
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+            for (int kb = 0; kb < kKB; ++kb)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const float e = fast_exp2(sT[qb][kb][v] * kScaleLog2 - mref);
@@ -299,15 +320,15 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
             if (WITH_V) {
                 if (__any(corr != 1.f)) {   // wavefront-uniform: skip when no maximum moved
 #pragma unroll
-                    for (int db = 0; db < 4; ++db)
+                    for (int db = 0; db < kDB; ++db)
 #pragma unroll
                         for (int v = 0; v < 16; ++v) oT[qb][db][v] *= corr;
                 }
 #pragma unroll
-                for (int s = 0; s < 4; ++s) {
-                    half8_t t;
+                for (int s = 0; s < kS; ++s) {
+                    x8_t t;
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) t[e] = (half_t)sT[qb][s >> 1][8 * (s & 1) + e];
+                    for (int e = 0; e < 8; ++e) t[e] = (T)sT[qb][s >> 1][8 * (s & 1) + e];
                     pf[qb][s] = t;
                 }
             }
@@ -315,17 +336,17 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
         // ---- O^T += V^T P^T ----
         if (WITH_V) {
 #pragma unroll
-            for (int db = 0; db < 4; ++db) {
+            for (int db = 0; db < kDB; ++db) {
                 const int d = 32 * db + li;
                 const int sw = ((d & 7) ^ (d >> 3)) & 7;
 #pragma unroll
-                for (int s = 0; s < 4; ++s) {
+                for (int s = 0; s < kS; ++s) {
                     if (s < 2 * nkb) {
-                        half8_t a = *reinterpret_cast<const half8_t*>(
+                        x8_t a = *reinterpret_cast<const x8_t*>(
                             &sV[d * kVStride + (((2 * s + lg) ^ sw) * 8)]);
 #pragma unroll
                         for (int qb = 0; qb < NQB; ++qb)
-                            oT[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pf[qb][s], oT[qb][db], 0, 0, 0);
+                            oT[qb][db] = Elem<T>::mma_32x32x16(a, pf[qb][s], oT[qb][db]);
                     }
                 }
             }
@@ -340,17 +361,17 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
         const float lt = l[qb] + __shfl_xor(l[qb], 32);
         if (ql < Lq) {
             if (p.log_sum && lg == 0)
-                p.log_sum[((long long)b * Lq + ql) * kHeads + head] = fast_log2(lt) + m[qb] * kScaleLog2;
+                p.log_sum[((long long)b * Lq + ql) * nheads + head] = fast_log2(lt) + m[qb] * kScaleLog2;
             if (WITH_V) {
                 const float inv = 1.f / lt;
-                half_t* op = p.O + (((long long)b * Lq + ql) * kHeads + head) * kDim;
+                T* op = (T*)p.O + (((long long)b * Lq + ql) * nheads + head) * D;
 #pragma unroll
-                for (int db = 0; db < 4; ++db)
+                for (int db = 0; db < kDB; ++db)
 #pragma unroll
                     for (int v4 = 0; v4 < 4; ++v4) {
-                        half4_t o = {(half_t)(oT[qb][db][4 * v4 + 0] * inv), (half_t)(oT[qb][db][4 * v4 + 1] * inv),
-                                     (half_t)(oT[qb][db][4 * v4 + 2] * inv), (half_t)(oT[qb][db][4 * v4 + 3] * inv)};
-                        *reinterpret_cast<half4_t*>(op + 32 * db + 8 * v4 + 4 * lg) = o;
+                        x4_t o = {(T)(oT[qb][db][4 * v4 + 0] * inv), (T)(oT[qb][db][4 * v4 + 1] * inv),
+                                  (T)(oT[qb][db][4 * v4 + 2] * inv), (T)(oT[qb][db][4 * v4 + 3] * inv)};
+                        *reinterpret_cast<x4_t*>(op + 32 * db + 8 * v4 + 4 * lg) = o;
                     }
             }
         }
@@ -360,31 +381,38 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, half_t
 
 // 32 queries per wavefront: register budget capped so that two workgroups share a
 // compute unit and hide each other's LDS staging and gather latency.
-template <bool REUSE, bool WITH_V, bool PAGED>
+template <bool REUSE, bool WITH_V, bool PAGED, int D, typename T>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2)))
 void prefill_attn_kernel_q32(PrefillParams p) {
-    __shared__ __attribute__((aligned(16))) half_t sK[kKT * kKStride];
-    __shared__ __attribute__((aligned(16))) half_t sV[WITH_V ? kDim * kVStride : 8];
-    prefill_attn_body<1, REUSE, WITH_V, PAGED>(p, sK, sV);
+    __shared__ __attribute__((aligned(16))) T sK[AttnTile<D>::kKT * AttnTile<D>::kKStride];
+    __shared__ __attribute__((aligned(16))) T sV[WITH_V ? D * AttnTile<D>::kVStride : 8];
+    prefill_attn_body<1, REUSE, WITH_V, PAGED, D, T>(p, sK, sV);
 }
 
 // 64 queries per wavefront for the K-only log-sum pass, whose state fits 256 registers: two
 // workgroups per compute unit, and the MFMA results stay in ordinary registers (with the full
 // 512-register budget the compiler parks them in accumulation registers and copies each one out
 // before the softmax).
+template <int D, typename T>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2)))
 void prefill_attn_kernel_q64(PrefillParams p) {
-    __shared__ __attribute__((aligned(16))) half_t sK[kKT * kKStride];
-    prefill_attn_body<2, false, false, false>(p, sK, nullptr);
+    __shared__ __attribute__((aligned(16))) T sK[AttnTile<D>::kKT * AttnTile<D>::kKStride];
+    prefill_attn_body<2, false, false, false, D, T>(p, sK, static_cast<T*>(nullptr));
 }
 
 // Pooled tile scores: out[b,g,t,key] = sum over the 32 queries of tile t and the 4 q-heads of g
 // of exp2(s*scale - log_sum), for keys before the tile's first (global) position.
 // Two workgroups per compute unit (register budget 256): one wavefront's exponentials run
 // under the other's matrix instructions.
-template <bool PAGED>
+template <bool PAGED, int D, typename T>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2)))
 void prefill_aggregate_kernel(PrefillParams p) {
+    typedef typename Elem<T>::x8 x8_t;
+    constexpr int kKS = D / 16;
+    constexpr float kScaleLog2 = ScaleLog2<D>::value;
+    const int kvh = p.G, nheads = p.G * kGroupSize;
+    const T* Qp = (const T*)p.Q;
+    const T* Kp = (const T*)p.K;
     __shared__ __attribute__((aligned(16))) float s_lse[128];
 
     const int L = p.L;
@@ -399,30 +427,30 @@ void prefill_aggregate_kernel(PrefillParams p) {
     const int lg = lane >> 5;
     const int tl = t * kTile;            // first query row of the tile
     const int ts = p.q_start + tl;       // its global position
-    half_t* out = p.agg + (((long long)b * kGroups + g) * p.T + t) * L;
+    half_t* out = p.agg + (((long long)b * kvh + g) * p.T + t) * L;
     const half_t neg_inf = (half_t)(-INFINITY);
 
     const int ntiles = (ts + kAggKT - 1) / kAggKT;
     if (ntiles > 0) {
         // A operands: row block rb = q-head 4g+rb, row li = query tl+li
-        half8_t qa[kGroupSize][8];
+        x8_t qa[kGroupSize][kKS];
 #pragma unroll
         for (int rb = 0; rb < kGroupSize; ++rb) {
             const int q = tl + li;
             const bool ok = q < Lq;
-            const half_t* qp = p.Q + (long long)b * p.q_sb + (long long)min(q, Lq - 1) * p.q_sl +
-                               (long long)(g * kGroupSize + rb) * p.q_sh + lg * 8;
+            const T* qp = Qp + (long long)b * p.q_sb + (long long)min(q, Lq - 1) * p.q_sl +
+                          (long long)(g * kGroupSize + rb) * p.q_sh + lg * 8;
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks) {
-                Pack16 x;
+            for (int ks = 0; ks < kKS; ++ks) {
+                PackT<T> x;
                 x.u = ld_global_16(qp + ks * 16);
                 if (!ok) x.u = uint4_t{0, 0, 0, 0};
-                qa[rb][ks] = x.h8;
+                qa[rb][ks] = x.v8;
             }
         }
         if (tid < 128) {
             const int q = tl + (tid & 31);
-            s_lse[tid] = (q < Lq) ? p.log_sum_in[((long long)b * Lq + q) * kHeads + g * kGroupSize + (tid >> 5)]
+            s_lse[tid] = (q < Lq) ? p.log_sum_in[((long long)b * Lq + q) * nheads + g * kGroupSize + (tid >> 5)]
                                   : INFINITY;
         }
         // A wavefront takes 32 keys of every 128-key tile and nobody else reads them, so its B
@@ -431,14 +459,14 @@ void prefill_aggregate_kernel(PrefillParams p) {
         // tile loop.  The registers of operand ks are refilled with the next tile's data as soon
         // as the products that read them have been issued, which leaves the rest of the tile
         // (remaining products, exponentials) to cover the load latency.
-        const half_t* kbase = PAGED ? p.K + (long long)g * kDim + lg * 8
-                                    : p.K + (long long)b * p.k_sb + (long long)g * p.k_sh + lg * 8;
+        const T* kbase = PAGED ? Kp + (long long)g * D + lg * 8
+                               : Kp + (long long)b * p.k_sb + (long long)g * p.k_sh + lg * 8;
         const int* bt_row = PAGED ? p.block_table + (long long)b * p.max_pages : nullptr;
         const int page_mask = (1 << p.page_shift) - 1;
         auto key_of = [&](int ti) { return min(ti * kAggKT + 32 * wave + li, L - 1); };
         auto row_ptr = [&](int ti, int pgv) {
             const int key = key_of(ti);
-            return PAGED ? kbase + (long long)((pgv << p.page_shift) + (key & page_mask)) * (kGroups * kDim)
+            return PAGED ? kbase + (long long)((pgv << p.page_shift) + (key & page_mask)) * (kvh * D)
                          : kbase + (long long)key * p.k_sl;
         };
         int pg_next = 0;    // block-table entry of this lane's key in the tile after the current one
@@ -447,14 +475,14 @@ void prefill_aggregate_kernel(PrefillParams p) {
             pg_next = bt_row[key_of(0) >> p.page_shift];
             if (ntiles > 1) pg_after = bt_row[key_of(1) >> p.page_shift];
         }
-        half8_t kb[8];
+        x8_t kb[kKS];
         {
-            const half_t* rp = row_ptr(0, pg_next);
+            const T* rp = row_ptr(0, pg_next);
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks) {
-                Pack16 x;
+            for (int ks = 0; ks < kKS; ++ks) {
+                PackT<T> x;
                 x.u = ld_global_16(rp + ks * 16);
-                kb[ks] = x.h8;
+                kb[ks] = x.v8;
             }
         }
         __syncthreads();   // s_lse
@@ -464,27 +492,26 @@ void prefill_aggregate_kernel(PrefillParams p) {
                 pg_next = pg_after;
                 if (ti + 2 < ntiles) pg_after = bt_row[key_of(ti + 2) >> p.page_shift];
             }
-            const half_t* rp = row_ptr(more ? ti + 1 : ti, pg_next);
+            const T* rp = row_ptr(more ? ti + 1 : ti, pg_next);
 
             float16_t acc[kGroupSize];
             float16_t zero16;   // the first product of a tile starts from a constant zero
 #pragma unroll
             for (int v = 0; v < 16; ++v) zero16[v] = 0.f;
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks) {
+            for (int ks = 0; ks < kKS; ++ks) {
 #pragma unroll
                 for (int rb = 0; rb < kGroupSize; ++rb)
-                    acc[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa[rb][ks], kb[ks],
-                                                                     ks == 0 ? zero16 : acc[rb], 0, 0, 0);
+                    acc[rb] = Elem<T>::mma_32x32x16(qa[rb][ks], kb[ks], ks == 0 ? zero16 : acc[rb]);
                 if (more) {
                     // the refill must stay behind the products that read the old contents, or
                     // the compiler hoists all eight loads and needs a second set of registers:
                     // its address is made to depend on the last product of this step
                     long long off = ks * 16;
                     asm volatile("" : "+v"(off) : "v"(acc[kGroupSize - 1][0]));
-                    Pack16 x;
+                    PackT<T> x;
                     x.u = ld_global_16(rp + off);
-                    kb[ks] = x.h8;
+                    kb[ks] = x.v8;
                 }
             }
             // accumulator v of row block rb is query row 8(v/4) + 4lg + v%4, column = key li
@@ -515,38 +542,59 @@ void prefill_aggregate_kernel(PrefillParams p) {
 
 }  // namespace
 
-hipError_t launch_prefill_attn(const PrefillParams& p, bool reuse, bool with_v, int nqb,
-                               hipStream_t stream) {
+namespace {
+
+template <int D, typename T>
+hipError_t launch_attn_t(const PrefillParams& p, bool reuse, bool with_v, int nqb, hipStream_t stream) {
     const int qt = 32 * nqb;
     const bool paged = p.block_table != nullptr;
-    dim3 grid((p.Lq + qt - 1) / qt, kGroups, p.B), block(kThreads);
+    dim3 grid((p.Lq + qt - 1) / qt, p.G, p.B), block(kThreads);
     if (paged) {
         if (reuse)
-            hipLaunchKernelGGL((prefill_attn_kernel_q32<true, true, true>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((prefill_attn_kernel_q32<true, true, true, D, T>), grid, block, 0, stream, p);
         else if (with_v)
-            hipLaunchKernelGGL((prefill_attn_kernel_q32<false, true, true>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((prefill_attn_kernel_q32<false, true, true, D, T>), grid, block, 0, stream, p);
         else
-            hipLaunchKernelGGL((prefill_attn_kernel_q32<false, false, true>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((prefill_attn_kernel_q32<false, false, true, D, T>), grid, block, 0, stream, p);
     } else if (reuse) {
-        hipLaunchKernelGGL((prefill_attn_kernel_q32<true, true, false>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((prefill_attn_kernel_q32<true, true, false, D, T>), grid, block, 0, stream, p);
     } else if (nqb == 2) {   // K-only log-sum pass
-        hipLaunchKernelGGL(prefill_attn_kernel_q64, grid, block, 0, stream, p);
+        hipLaunchKernelGGL((prefill_attn_kernel_q64<D, T>), grid, block, 0, stream, p);
     } else {
         if (with_v)
-            hipLaunchKernelGGL((prefill_attn_kernel_q32<false, true, false>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((prefill_attn_kernel_q32<false, true, false, D, T>), grid, block, 0, stream, p);
         else
-            hipLaunchKernelGGL((prefill_attn_kernel_q32<false, false, false>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((prefill_attn_kernel_q32<false, false, false, D, T>), grid, block, 0, stream, p);
     }
     return hipGetLastError();
 }
 
-hipError_t launch_prefill_aggregate(const PrefillParams& p, hipStream_t stream) {
-    dim3 grid(p.T, kGroups, p.B), block(kThreads);
+template <int D, typename T>
+hipError_t launch_aggregate_t(const PrefillParams& p, hipStream_t stream) {
+    dim3 grid(p.T, p.G, p.B), block(kThreads);
     if (p.block_table)
-        hipLaunchKernelGGL(prefill_aggregate_kernel<true>, grid, block, 0, stream, p);
+        hipLaunchKernelGGL((prefill_aggregate_kernel<true, D, T>), grid, block, 0, stream, p);
     else
-        hipLaunchKernelGGL(prefill_aggregate_kernel<false>, grid, block, 0, stream, p);
+        hipLaunchKernelGGL((prefill_aggregate_kernel<false, D, T>), grid, block, 0, stream, p);
     return hipGetLastError();
+}
+
+}  // namespace
+
+// p.head_dim in {64, 128}, p.elem in {kElemF16, kElemBF16}: checked by the callers
+hipError_t launch_prefill_attn(const PrefillParams& p, bool reuse, bool with_v, int nqb,
+                               hipStream_t stream) {
+    if (p.head_dim == 128)
+        return p.elem == kElemBF16 ? launch_attn_t<128, bf16_t>(p, reuse, with_v, nqb, stream)
+                                   : launch_attn_t<128, half_t>(p, reuse, with_v, nqb, stream);
+    return p.elem == kElemBF16 ? launch_attn_t<64, bf16_t>(p, reuse, with_v, nqb, stream)
+                               : launch_attn_t<64, half_t>(p, reuse, with_v, nqb, stream);
+}
+
+hipError_t launch_prefill_aggregate(const PrefillParams& p, hipStream_t stream) {
+    if (p.head_dim == 128)
+        return p.elem == kElemBF16 ? launch_aggregate_t<128, bf16_t>(p, stream) : launch_aggregate_t<128, half_t>(p, stream);
+    return p.elem == kElemBF16 ? launch_aggregate_t<64, bf16_t>(p, stream) : launch_aggregate_t<64, half_t>(p, stream);
 }
 
 // idx[i] (token position) -> physical row of the paged cache, in place or to another buffer.

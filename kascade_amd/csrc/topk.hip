@@ -8,6 +8,8 @@
 // The row is streamed from L2/HBM three times as 16-byte loads.
 #include "topk.h"
 
+#include "prefill.h"   // launch_translate_indices
+
 namespace kascade {
 
 namespace {
@@ -764,7 +766,10 @@ hipError_t launch_topk_split(const half_t* scores, int* out_idx, int rows, long 
                              int period, int k, int fill, void* workspace, const TopkRows* tr,
                              hipStream_t stream) {
     if (rows == 0) return hipSuccess;
-    const RowsOut ro = rows_out(tr);
+    // The chunk workgroups write their selections to scattered slots, where a block-table lookup
+    // per element would sit in the middle of the compaction (+40 us on four rows of 131072 to
+    // 524288 entries); the long-row path translates in a launch of its own at the end instead.
+    const RowsOut ro{};
     const int max_chunks = (max_len + kSplitChunk - 1) / kSplitChunk;
     SplitWs ws = carve_ws(workspace, rows, max_chunks);
     const uint16_t* src = reinterpret_cast<const uint16_t*>(scores);
@@ -781,6 +786,10 @@ hipError_t launch_topk_split(const half_t* scores, int* out_idx, int rows, long 
     hipLaunchKernelGGL(topk_split_scan2_kernel, dim3(rows), dim3(64), 0, stream, max_chunks, ws);
     hipLaunchKernelGGL(topk_split_write_kernel, grid, dim3(kThreads), 0, stream, src, out_idx,
                        row_stride, k, fill, max_chunks, ws, ro);
+    if (tr && tr->out_rows)
+        return launch_translate_indices(out_idx, tr->out_rows, tr->block_table, rows / tr->rows_per_seq,
+                                        (long long)tr->rows_per_seq * k, tr->max_pages, tr->page_shift,
+                                        tr->max_pages << tr->page_shift, stream);
     return hipGetLastError();
 }
 

@@ -22,7 +22,30 @@ from . import _lib
 from ._lib import Strides, KascadeError
 from . import budgets
 
-H, G, D, TILE = 32, 8, 128, 32
+H, G, D, TILE = 32, 8, 128, 32      # the reference's shape (EfficientKascadeStrategy.py:19-21)
+GROUP = 4                             # query heads per KV head, for every shape
+_ELEM = {torch.float16: 0, torch.bfloat16: 1}
+
+
+def _shape(Q: torch.Tensor, K: torch.Tensor):
+    """(query heads, KV heads, head_dim, dtype) of a call, from Q [..., H, D] and K [..., G, D]:
+    fp16 or bf16, head_dim 64 or 128, four query heads per KV head."""
+    Hq, Dh, Gk = Q.shape[-2], Q.shape[-1], K.shape[-2]
+    if Q.dtype not in _ELEM or K.dtype != Q.dtype:
+        raise KascadeError(f"Q and K must both be float16 or bfloat16, got {Q.dtype} / {K.dtype}")
+    if Dh not in (64, 128) or K.shape[-1] != Dh:
+        raise KascadeError(f"head_dim must be 64 or 128 for Q and K, got {Dh} / {K.shape[-1]}")
+    if Gk < 1 or Hq != GROUP * Gk:
+        raise KascadeError(f"need {GROUP} query heads per KV head, got {Hq} query / {Gk} KV heads")
+    return Hq, Gk, Dh, Q.dtype
+
+
+def _call(lib, name: str, shape, *args):
+    """The plain entry point for the reference's shape, its *_shaped_call twin otherwise."""
+    _, Gk, Dh, dt = shape
+    if (Gk, Dh, dt) == (G, D, torch.float16):
+        return getattr(lib, f"kascade_{name}_call")(*args)
+    return getattr(lib, f"kascade_{name}_shaped_call")(ctypes.byref(_lib.Shape(Gk, Dh, _ELEM[dt])), *args)
 
 
 def _stream() -> int:
@@ -44,8 +67,8 @@ def _req(t: torch.Tensor, dtype, name: str, contiguous: bool = True):
 
 def _blhd_strides(t: torch.Tensor, name: str) -> Strides:
     """Strides of a [B,L,heads,D] view whose innermost dimension is contiguous."""
-    if t.dim() != 4 or t.shape[-1] != D or t.stride(-1) != 1:
-        raise KascadeError(f"{name} must be [B,L,heads,{D}] with a contiguous last dimension")
+    if t.dim() != 4 or t.stride(-1) != 1:
+        raise KascadeError(f"{name} must be [B,L,heads,D] with a contiguous last dimension")
     return Strides(t.stride(0), t.stride(1), t.stride(2))
 
 
@@ -99,41 +122,46 @@ def default_num_split(total_rows: int, max_rows: int, wgs_per_cu: int = 2, min_r
 
 
 # ---------------------------------------------------------------- decode
-def _out_buffer(out, B, device) -> torch.Tensor:
-    """The caller's [B,H,D] fp16 output buffer, or a fresh one."""
+def _out_buffer(out, B, device, shape=(H, G, D, torch.float16)) -> torch.Tensor:
+    """The caller's [B,H,D] output buffer, or a fresh one."""
+    Hq, _, Dh, dt = shape
     if out is None:
-        return torch.empty(B, H, D, device=device, dtype=torch.float16)
-    _req(out, torch.float16, "out")
-    if tuple(out.shape) != (B, H, D):
-        raise KascadeError(f"out must be [{B},{H},{D}]")
+        return torch.empty(B, Hq, Dh, device=device, dtype=dt)
+    _req(out, dt, "out")
+    if tuple(out.shape) != (B, Hq, Dh):
+        raise KascadeError(f"out must be [{B},{Hq},{Dh}]")
     return out
 
 
-def _decode_kv(K, V, block_table):
+def _decode_kv(K, V, block_table, shape=(H, G, D, torch.float16)):
     """dtype / layout check of the decode K and V operands; returns the optional strides argument.
     Pages must be contiguous.  Without a block table any [B,L,G,D] view with a contiguous last
     dimension is read in place (e.g. a head-major [B,G,L,D] cache transposed), and the strides
     are passed only when the view is not the plain contiguous layout."""
+    _, Gk, Dh, dt = shape
     for t, name in ((K, "K"), (V, "V")):
-        _req(t, torch.float16, name, contiguous=block_table is not None)
+        _req(t, dt, name, contiguous=block_table is not None)
+    if K.shape != V.shape or tuple(K.shape[-2:]) != (Gk, Dh):
+        raise KascadeError(f"K and V must share one [..., {Gk}, {Dh}] shape")
     if block_table is not None or (K.is_contiguous() and V.is_contiguous()):
         return None
     ks, vs = _blhd_strides(K, "K"), _blhd_strides(V, "V")
-    if (ks.b, ks.l, ks.h) != (vs.b, vs.l, vs.h) or K.shape != V.shape or K.shape[2] != G:
-        raise KascadeError("K and V must share one [B,L,8,128] shape and one set of strides")
+    if (ks.b, ks.l, ks.h) != (vs.b, vs.l, vs.h):
+        raise KascadeError("K and V must share one set of strides")
     return ctypes.byref(ks)
 
 
-def _new_rows(k_new, v_new, B):
+def _new_rows(k_new, v_new, B, shape=(H, G, D, torch.float16)):
     """Optional [B,G,D] rows of the newest token for the fused append (both or neither)."""
     if k_new is None and v_new is None:
         return None, None
     if k_new is None or v_new is None:
         raise KascadeError("k_new and v_new come together")
+    _, Gk, Dh, dt = shape
     for t, name in ((k_new, "k_new"), (v_new, "v_new")):
-        _req(t, torch.float16, name)
-        if tuple(t.shape) != (B, G, D):
-            raise KascadeError(f"{name} must be [{B},{G},{D}]")
+        _req(t, dt, name)
+        if tuple(t.shape) != (B, Gk, Dh):
+            raise KascadeError(f"{name} must be [{B},{Gk},{Dh}]")
     return _ptr(k_new), _ptr(v_new)
 
 
@@ -158,13 +186,13 @@ def decode_budgets(cache_seqlens, topk_percent: float, advance: int = 0, valid_o
     return valid_out[:B * G], n_sel_out[:B * G]
 
 
-def _sync_arg(sync, B):
+def _sync_arg(sync, B, groups: int = G):
     """Optional [B*G] int32 counter array for the fused combine (zero-initialised by the caller)."""
     if sync is None:
         return None
     _req(sync, torch.int32, "sync_counters")
-    if sync.numel() < B * G:
-        raise KascadeError(f"sync_counters needs {B * G} entries")
+    if sync.numel() < B * groups:
+        raise KascadeError(f"sync_counters needs {B * groups} entries")
     return _ptr(sync)
 
 
@@ -173,27 +201,27 @@ def decode_reuse(Q, K, V, topk_indices, head_mapping, glse, Output_partial, sync
     (out_idx=[7]; EfficientKascadeStrategy.py:30-38, 113, 122).  Contiguous cache
     K,V [B,L,G,D]; the split count is glse.shape[2]."""
     lib = _lib.init()
-    B, Hq, Dq = Q.shape
+    B = Q.shape[0]
     L = K.shape[1]
-    _req(Q, torch.float16, "Q")
-    kv_strides = _decode_kv(K, V, None)
+    shape = _shape(Q, K)
+    Hq, Gk, Dh, dt = shape
+    _req(Q, dt, "Q")
+    kv_strides = _decode_kv(K, V, None, shape)
     _req(topk_indices, torch.int32, "topk_indices"); _req(head_mapping, torch.int32, "head_mapping")
     _req(glse, torch.float32, "glse"); _req(Output_partial, torch.float32, "Output_partial")
-    if (Hq, Dq, K.shape[2]) != (H, D, G):
-        raise KascadeError("decode_reuse supports H=32, G=8, D=128 only")
     ns = glse.shape[2]
-    if tuple(glse.shape) != (B, H, ns) or tuple(Output_partial.shape) != (B, H, ns, D):
+    if tuple(glse.shape) != (B, Hq, ns) or tuple(Output_partial.shape) != (B, Hq, ns, Dh):
         raise KascadeError("glse must be [B,H,S] and Output_partial [B,H,S,D]")
-    out = torch.empty(B, H, D, device=Q.device, dtype=torch.float16)
-    if kv_strides is None:
+    out = torch.empty(B, Hq, Dh, device=Q.device, dtype=dt)
+    if kv_strides is None and shape == (H, G, D, torch.float16):
         _lib.check(lib.kascade_decode_reuse_call(
             _ptr(Q), _ptr(K), _ptr(V), _ptr(topk_indices), _ptr(head_mapping), _ptr(glse),
             _ptr(Output_partial), _ptr(out), B, L, topk_indices.shape[-1], ns, _sync_arg(sync, B), _stream()))
     else:
-        _lib.check(lib.kascade_decode_reuse_paged_call(
+        _lib.check(_call(lib, "decode_reuse_paged", shape,
             _ptr(Q), _ptr(K), _ptr(V), None, _ptr(topk_indices), _ptr(head_mapping), 0.0, _ptr(glse),
             _ptr(Output_partial), _ptr(out), B, L, topk_indices.shape[-1], ns, None, 0, 1, kv_strides,
-            None, None, _sync_arg(sync, B), _stream()))
+            None, None, _sync_arg(sync, B, Gk), _stream()))
     return out
 
 
@@ -206,8 +234,9 @@ def decode_reuse_paged(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_
     with one they are pages [P,page_size,G,D]."""
     lib = _lib.init()
     B = Q.shape[0]
-    _req(Q, torch.float16, "Q")
-    kv_strides = _decode_kv(K, V, block_table)
+    shape = _shape(Q, K)
+    _req(Q, shape[3], "Q")
+    kv_strides = _decode_kv(K, V, block_table, shape)
     _req(topk_indices, torch.int32, "topk_indices"); _req(head_mapping, torch.int32, "head_mapping")
     _req(glse, torch.float32, "glse"); _req(Output_partial, torch.float32, "Output_partial")
     if cache_seqlens is not None:
@@ -218,12 +247,12 @@ def decode_reuse_paged(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_
         stride_tokens, max_pages = 0, block_table.shape[1]
     else:
         stride_tokens, max_pages = K.shape[1], 0
-    out = _out_buffer(out, B, Q.device)
-    _lib.check(lib.kascade_decode_reuse_paged_call(
+    out = _out_buffer(out, B, Q.device, shape)
+    _lib.check(_call(lib, "decode_reuse_paged", shape,
         _ptr(Q), _ptr(K), _ptr(V), _ptr(cache_seqlens), _ptr(topk_indices), _ptr(head_mapping),
         float(topk_percent), _ptr(glse), _ptr(Output_partial), _ptr(out), B, stride_tokens,
         topk_indices.shape[-1], ns, _ptr(block_table), max_pages, page_size, kv_strides,
-        *_new_rows(k_new, v_new, B), _sync_arg(sync, B), _stream()))
+        *_new_rows(k_new, v_new, B, shape), _sync_arg(sync, B, shape[1]), _stream()))
     return out
 
 
@@ -235,22 +264,23 @@ def decode_reuse_rows(Q, K_pages, V_pages, cache_seqlens, cache_rows, head_mappi
     ``decode_reuse_paged``.  cache_rows [B,G,topk] int32."""
     lib = _lib.init()
     B = Q.shape[0]
-    _req(Q, torch.float16, "Q"); _req(K_pages, torch.float16, "K_pages"); _req(V_pages, torch.float16, "V_pages")
+    shape = _shape(Q, K_pages)
+    Hq, Gk, Dh, dt = shape
+    _req(Q, dt, "Q"); _req(K_pages, dt, "K_pages"); _req(V_pages, dt, "V_pages")
     _req(cache_rows, torch.int32, "cache_rows"); _req(head_mapping, torch.int32, "head_mapping")
     _req(glse, torch.float32, "glse"); _req(Output_partial, torch.float32, "Output_partial")
     _req(block_table, torch.int32, "block_table")
     if cache_seqlens is not None:
         _req(cache_seqlens, torch.int32, "cache_seqlens")
-    if K_pages.dim() != 4 or K_pages.shape[1] != page_size or tuple(K_pages.shape[2:]) != (G, D) \
-            or K_pages.shape != V_pages.shape:
-        raise KascadeError(f"pages must be [num_pages,{page_size},{G},{D}]")
+    if K_pages.dim() != 4 or K_pages.shape[1] != page_size or K_pages.shape != V_pages.shape:
+        raise KascadeError(f"pages must be [num_pages,{page_size},{Gk},{Dh}]")
     ns = glse.shape[2]
-    out = _out_buffer(out, B, Q.device)
-    _lib.check(lib.kascade_decode_reuse_rows_call(
+    out = _out_buffer(out, B, Q.device, shape)
+    _lib.check(_call(lib, "decode_reuse_rows", shape,
         _ptr(Q), _ptr(K_pages), _ptr(V_pages), _ptr(cache_seqlens), _ptr(cache_rows), _ptr(head_mapping),
         float(topk_percent), _ptr(glse), _ptr(Output_partial), _ptr(out), B, cache_rows.shape[-1], ns,
-        _ptr(block_table), block_table.shape[1], page_size, K_pages.shape[0], *_new_rows(k_new, v_new, B),
-        _sync_arg(sync, B), _stream()))
+        _ptr(block_table), block_table.shape[1], page_size, K_pages.shape[0], *_new_rows(k_new, v_new, B, shape),
+        _sync_arg(sync, B, Gk), _stream()))
     return out
 
 
@@ -290,8 +320,9 @@ def decode_dense_paged(Q, K, V, cache_seqlens, glse, Output_partial, block_table
     ``kernel(Q, K, V, [cache_seqlens,] glse, Output_partial) -> O``."""
     lib = _lib.init()
     B = Q.shape[0]
-    _req(Q, torch.float16, "Q")
-    kv_strides = _decode_kv(K, V, block_table)
+    shape = _shape(Q, K)
+    _req(Q, shape[3], "Q")
+    kv_strides = _decode_kv(K, V, block_table, shape)
     _req(glse, torch.float32, "glse"); _req(Output_partial, torch.float32, "Output_partial")
     ns = glse.shape[2]
     if block_table is not None:
@@ -299,11 +330,11 @@ def decode_dense_paged(Q, K, V, cache_seqlens, glse, Output_partial, block_table
         stride_tokens, max_pages = (kv_len or 0), block_table.shape[1]
     else:
         stride_tokens, max_pages = K.shape[1], 0
-    out = _out_buffer(out, B, Q.device)
-    _lib.check(lib.kascade_decode_dense_paged_call(
+    out = _out_buffer(out, B, Q.device, shape)
+    _lib.check(_call(lib, "decode_dense_paged", shape,
         _ptr(Q), _ptr(K), _ptr(V), _ptr(cache_seqlens), _ptr(glse), _ptr(Output_partial), _ptr(out),
         B, stride_tokens, ns, _ptr(block_table), max_pages, page_size, kv_strides,
-        *_new_rows(k_new, v_new, B), _sync_arg(sync, B), _stream()))
+        *_new_rows(k_new, v_new, B, shape), _sync_arg(sync, B, shape[1]), _stream()))
     return out
 
 
@@ -319,8 +350,9 @@ def decode_recompute(Q, K, V, glse, Output_partial, row_sums, scores, layer: int
     otherwise O is None."""
     lib = _lib.init()
     B = Q.shape[0]
-    _req(Q, torch.float16, "Q")
-    kv_strides = _decode_kv(K, V, block_table)
+    shape = _shape(Q, K)
+    _req(Q, shape[3], "Q")
+    kv_strides = _decode_kv(K, V, block_table, shape)
     _req(glse, torch.float32, "glse"); _req(row_sums, torch.float32, "row_sums")
     _req(scores, torch.float32, "scores")
     with_out = 1 if layer == 0 else 0
@@ -331,13 +363,13 @@ def decode_recompute(Q, K, V, glse, Output_partial, row_sums, scores, layer: int
         stride_tokens, max_pages = (kv_len or 0), block_table.shape[1]
     else:
         stride_tokens, max_pages = K.shape[1], 0
-    out = _out_buffer(out, B, Q.device) if with_out else None
-    agg = torch.empty(B, G, stride, device=Q.device, dtype=torch.float16)
-    _lib.check(lib.kascade_decode_recompute_paged_call(
+    out = _out_buffer(out, B, Q.device, shape) if with_out else None
+    agg = torch.empty(B, shape[1], stride, device=Q.device, dtype=torch.float16)
+    _lib.check(_call(lib, "decode_recompute_paged", shape,
         _ptr(Q), _ptr(K), _ptr(V), _ptr(cache_seqlens), _ptr(glse), _ptr(Output_partial),
         _ptr(row_sums), _ptr(scores), _ptr(out), _ptr(agg), B, stride_tokens, stride, ns, with_out,
-        _ptr(block_table), max_pages, page_size, kv_strides, *_new_rows(k_new, v_new, B),
-        _sync_arg(sync, B), _stream()))
+        _ptr(block_table), max_pages, page_size, kv_strides, *_new_rows(k_new, v_new, B, shape),
+        _sync_arg(sync, B, shape[1]), _stream()))
     return out, agg
 
 
@@ -425,27 +457,30 @@ def prefill_recompute0(Q, K, V) -> Tuple[torch.Tensor, torch.Tensor]:
     """``prefill_recomp0_kernel(Q, K, V) -> (log_sum, O)`` (out_idx=[3,4];
     EfficientKascadeStrategy.py:40-43, 78).  Q [B,L,H,D], K,V [B,L,G,D] (strided views allowed)."""
     lib = _lib.init()
-    _req(Q, torch.float16, "Q", False); _req(K, torch.float16, "K", False); _req(V, torch.float16, "V", False)
+    shape = _shape(Q, K)
+    Hq, _, Dh, dt = shape
+    _req(Q, dt, "Q", False); _req(K, dt, "K", False); _req(V, dt, "V", False)
     B, L = Q.shape[0], Q.shape[1]
     qs, ks = _blhd_strides(Q, "Q"), _blhd_strides(K, "K")
-    if tuple(V.stride()) != tuple(K.stride()):
-        raise KascadeError("K and V must share strides")
-    log_sum = torch.empty(B, L, H, device=Q.device, dtype=torch.float32)
-    out = torch.empty(B, L, H, D, device=Q.device, dtype=torch.float16)
-    _lib.check(lib.kascade_prefill_dense_call(_ptr(Q), _ptr(K), _ptr(V), _ptr(log_sum), _ptr(out),
-                                              B, L, qs, ks, 1, _stream()))
+    if tuple(V.stride()) != tuple(K.stride()) or V.shape != K.shape:
+        raise KascadeError("K and V must share shape and strides")
+    log_sum = torch.empty(B, L, Hq, device=Q.device, dtype=torch.float32)
+    out = torch.empty(B, L, Hq, Dh, device=Q.device, dtype=dt)
+    _lib.check(_call(lib, "prefill_dense", shape, _ptr(Q), _ptr(K), _ptr(V), _ptr(log_sum), _ptr(out),
+                     B, L, qs, ks, 1, _stream()))
     return log_sum, out
 
 
 def prefill_recompute1(Q, K) -> torch.Tensor:
     """``prefill_recomp1_kernel(Q, K) -> log_sum`` (out_idx=[2]; EfficientKascadeStrategy.py:44-47, 80)."""
     lib = _lib.init()
-    _req(Q, torch.float16, "Q", False); _req(K, torch.float16, "K", False)
+    shape = _shape(Q, K)
+    _req(Q, shape[3], "Q", False); _req(K, shape[3], "K", False)
     B, L = Q.shape[0], Q.shape[1]
     qs, ks = _blhd_strides(Q, "Q"), _blhd_strides(K, "K")
-    log_sum = torch.empty(B, L, H, device=Q.device, dtype=torch.float32)
-    _lib.check(lib.kascade_prefill_dense_call(_ptr(Q), _ptr(K), None, _ptr(log_sum), None,
-                                              B, L, qs, ks, 0, _stream()))
+    log_sum = torch.empty(B, L, shape[0], device=Q.device, dtype=torch.float32)
+    _lib.check(_call(lib, "prefill_dense", shape, _ptr(Q), _ptr(K), None, _ptr(log_sum), None,
+                     B, L, qs, ks, 0, _stream()))
     return log_sum
 
 
@@ -453,14 +488,16 @@ def prefill_dense(Q, K, V) -> torch.Tensor:
     """Dense causal prefill baseline (example_gqa_fwd_bshd_wgmma_pipelined.py:121-166):
     ``kernel(Q, K, V) -> O``; no log-sum is written."""
     lib = _lib.init()
-    _req(Q, torch.float16, "Q", False); _req(K, torch.float16, "K", False); _req(V, torch.float16, "V", False)
+    shape = _shape(Q, K)
+    Hq, _, Dh, dt = shape
+    _req(Q, dt, "Q", False); _req(K, dt, "K", False); _req(V, dt, "V", False)
     B, L = Q.shape[0], Q.shape[1]
     qs, ks = _blhd_strides(Q, "Q"), _blhd_strides(K, "K")
-    if tuple(V.stride()) != tuple(K.stride()):
-        raise KascadeError("K and V must share strides")
-    out = torch.empty(B, L, H, D, device=Q.device, dtype=torch.float16)
-    _lib.check(lib.kascade_prefill_dense_call(_ptr(Q), _ptr(K), _ptr(V), None, _ptr(out),
-                                              B, L, qs, ks, 1, _stream()))
+    if tuple(V.stride()) != tuple(K.stride()) or V.shape != K.shape:
+        raise KascadeError("K and V must share shape and strides")
+    out = torch.empty(B, L, Hq, Dh, device=Q.device, dtype=dt)
+    _lib.check(_call(lib, "prefill_dense", shape, _ptr(Q), _ptr(K), _ptr(V), None, _ptr(out),
+                     B, L, qs, ks, 1, _stream()))
     return out
 
 
@@ -468,15 +505,17 @@ def prefill_aggregate(Q, K, log_sum, scores, fill_invalid: bool = False) -> None
     """``aggregate_kernel(Q, K, log_sum, scores)`` (out_idx=None; in place;
     EfficientKascadeStrategy.py:49-59, 81).  scores [B,G,ceil(L/32),L] fp16."""
     lib = _lib.init()
-    _req(Q, torch.float16, "Q", False); _req(K, torch.float16, "K", False)
+    shape = _shape(Q, K)
+    Hq, Gk, _, dt = shape
+    _req(Q, dt, "Q", False); _req(K, dt, "K", False)
     _req(log_sum, torch.float32, "log_sum"); _req(scores, torch.float16, "scores")
     B, L = Q.shape[0], Q.shape[1]
     T = (L + TILE - 1) // TILE
-    if tuple(scores.shape) != (B, G, T, L) or tuple(log_sum.shape) != (B, L, H):
+    if tuple(scores.shape) != (B, Gk, T, L) or tuple(log_sum.shape) != (B, L, Hq):
         raise KascadeError("scores must be [B,G,ceil(L/32),L] and log_sum [B,L,H]")
     qs, ks = _blhd_strides(Q, "Q"), _blhd_strides(K, "K")
-    _lib.check(lib.kascade_prefill_aggregate_call(_ptr(Q), _ptr(K), _ptr(log_sum), _ptr(scores), B, L,
-                                                  qs, ks, 1 if fill_invalid else 0, _stream()))
+    _lib.check(_call(lib, "prefill_aggregate", shape, _ptr(Q), _ptr(K), _ptr(log_sum), _ptr(scores), B, L,
+                     qs, ks, 1 if fill_invalid else 0, _stream()))
 
 
 def prefill_aggregate_range(Q, K, log_sum, scores, q_start: int, q_len: int, fill_invalid: bool = False) -> None:
@@ -485,19 +524,21 @@ def prefill_aggregate_range(Q, K, log_sum, scores, q_start: int, q_len: int, fil
     [B,G,ceil(q_len/32),q_start+q_len] fp16.  Lets an anchor layer pool and select a few hundred
     tiles at a time instead of holding L^2/4 bytes of scores."""
     lib = _lib.init()
-    _req(Q, torch.float16, "Q", False); _req(K, torch.float16, "K", False)
+    shape = _shape(Q, K)
+    Hq, Gk, _, dt = shape
+    _req(Q, dt, "Q", False); _req(K, dt, "K", False)
     _req(log_sum, torch.float32, "log_sum"); _req(scores, torch.float16, "scores")
     B, L = Q.shape[0], Q.shape[1]
     if q_start % TILE or q_start < 0 or q_len <= 0 or q_start + q_len > L:
         raise KascadeError("q_start must be a multiple of 32 and the range must lie inside the prompt")
     T = (q_len + TILE - 1) // TILE
-    if tuple(scores.shape) != (B, G, T, q_start + q_len) or tuple(log_sum.shape) != (B, L, H):
+    if tuple(scores.shape) != (B, Gk, T, q_start + q_len) or tuple(log_sum.shape) != (B, L, Hq):
         raise KascadeError("scores must be [B,G,ceil(q_len/32),q_start+q_len] and log_sum [B,L,H]")
     qs, ks = _blhd_strides(Q, "Q"), _blhd_strides(K, "K")
     q_rows = Q[:, q_start:q_start + q_len]
     ls_rows = log_sum[:, q_start:q_start + q_len].contiguous()      # a view for batch 1
-    _lib.check(lib.kascade_prefill_aggregate_range_call(_ptr(q_rows), _ptr(K), _ptr(ls_rows), _ptr(scores), B,
-                                                        q_start, q_len, qs, ks, 1 if fill_invalid else 0, _stream()))
+    _lib.check(_call(lib, "prefill_aggregate_range", shape, _ptr(q_rows), _ptr(K), _ptr(ls_rows), _ptr(scores), B,
+                     q_start, q_len, qs, ks, 1 if fill_invalid else 0, _stream()))
 
 
 def prefill_reuse(Q, K, V, topk_idx, head_mapping, topk_percent, rolling: bool) -> torch.Tensor:
@@ -505,17 +546,19 @@ def prefill_reuse(Q, K, V, topk_idx, head_mapping, topk_percent, rolling: bool) 
     (out_idx=[6]; EfficientKascadeStrategy.py:61-70, 92, 97); ``rolling`` selects between the
     reference's two compiled objects."""
     lib = _lib.init()
-    _req(Q, torch.float16, "Q", False); _req(K, torch.float16, "K", False); _req(V, torch.float16, "V", False)
+    shape = _shape(Q, K)
+    Hq, Gk, Dh, dt = shape
+    _req(Q, dt, "Q", False); _req(K, dt, "K", False); _req(V, dt, "V", False)
     _req(topk_idx, torch.int32, "topk_indices"); _req(head_mapping, torch.int32, "head_mapping")
     B, L = Q.shape[0], Q.shape[1]
     T = (L + TILE - 1) // TILE
-    if tuple(topk_idx.shape[:3]) != (B, G, T):
-        raise KascadeError("topk_indices must be [B,G,ceil(L/32),max_topk]")
+    if tuple(topk_idx.shape[:3]) != (B, Gk, T) or head_mapping.numel() != Gk:
+        raise KascadeError("topk_indices must be [B,G,ceil(L/32),max_topk] and head_mapping [G]")
     qs, ks = _blhd_strides(Q, "Q"), _blhd_strides(K, "K")
-    if tuple(V.stride()) != tuple(K.stride()):
-        raise KascadeError("K and V must share strides")
-    out = torch.empty(B, L, H, D, device=Q.device, dtype=torch.float16)
-    _lib.check(lib.kascade_prefill_reuse_call(
+    if tuple(V.stride()) != tuple(K.stride()) or V.shape != K.shape:
+        raise KascadeError("K and V must share shape and strides")
+    out = torch.empty(B, L, Hq, Dh, device=Q.device, dtype=dt)
+    _lib.check(_call(lib, "prefill_reuse", shape,
         _ptr(Q), _ptr(K), _ptr(V), _ptr(topk_idx), _ptr(head_mapping), float(topk_percent), _ptr(out),
         B, L, topk_idx.shape[-1], 1 if rolling else 0, qs, ks, _stream()))
     return out
@@ -525,14 +568,20 @@ def prefill_reuse(Q, K, V, topk_idx, head_mapping, topk_percent, rolling: bool) 
 def paged_kv_append(K_pages, V_pages, k_new, v_new, start_pos, block_table, page_size: int = 16):
     """Write k_new/v_new [B,n_new,G,D] into the paged cache at positions start_pos[b]+t."""
     lib = _lib.init()
-    _req(K_pages, torch.float16, "K_pages"); _req(V_pages, torch.float16, "V_pages")
-    _req(k_new, torch.float16, "k_new", False); _req(v_new, torch.float16, "v_new", False)
+    dt = K_pages.dtype
+    if dt not in _ELEM:
+        raise KascadeError("pages must be float16 or bfloat16")
+    _req(K_pages, dt, "K_pages"); _req(V_pages, dt, "V_pages")
+    _req(k_new, dt, "k_new", False); _req(v_new, dt, "v_new", False)
     _req(start_pos, torch.int32, "start_pos"); _req(block_table, torch.int32, "block_table")
     if tuple(k_new.stride()) != tuple(v_new.stride()):
         raise KascadeError("k_new and v_new must share strides")
+    Gk, Dh = K_pages.shape[-2], K_pages.shape[-1]
+    if Dh not in (64, 128) or tuple(k_new.shape[2:]) != (Gk, Dh) or K_pages.shape != V_pages.shape:
+        raise KascadeError("pages [num_pages,page,G,D] and new rows [B,n,G,D] must agree, D 64 or 128")
     B, n_new = k_new.shape[0], k_new.shape[1]
     st = _blhd_strides(k_new, "k_new")
-    _lib.check(lib.kascade_paged_kv_append_call(
+    _lib.check(_call(lib, "paged_kv_append", (GROUP * Gk, Gk, Dh, dt),
         _ptr(K_pages), _ptr(V_pages), _ptr(k_new), _ptr(v_new), _ptr(start_pos), _ptr(block_table),
         B, n_new, block_table.shape[1], page_size, st, _stream()))
 
@@ -683,19 +732,20 @@ def prefill_full_kernel(Q, K, V, topk, tile_size=TILE, layer=0, topk_percent=10,
     if tile_size != TILE:
         raise KascadeError(f"tile_size must be {TILE}")
     B, L = Q.shape[:2]
+    Gk = K.shape[2]
     T = (L + TILE - 1) // TILE
     if layer == 0:
         log_sum, o = prefill_recompute0(Q, K, V)
     else:
         log_sum = prefill_recompute1(Q, K)
-    scores = torch.empty(B, G, T, L, device=Q.device, dtype=torch.float16)
+    scores = torch.empty(B, Gk, T, L, device=Q.device, dtype=torch.float16)
     prefill_aggregate(Q, K, log_sum, scores, fill_invalid=fill_invalid)
     valid, nsel = budgets.prefill_tile_budgets(L, TILE, topk_percent, rolling, topk)
     indices = topk_indices(scores, topk,
                            valid_len=torch.tensor(valid, dtype=torch.int32, device=Q.device),
                            n_sel=torch.tensor(nsel, dtype=torch.int32, device=Q.device))
     if layer != 0:
-        o = prefill_reuse(Q, K, V, indices, torch.arange(G, device=Q.device, dtype=torch.int32),
+        o = prefill_reuse(Q, K, V, indices, torch.arange(Gk, device=Q.device, dtype=torch.int32),
                           topk_percent, rolling)
     return o, indices, scores
 
@@ -708,7 +758,7 @@ def decode_full_kernel(Q, K, V, topk, glse, Output_partial, row_sums, scores, la
     o, agg = decode_recompute(Q, K, V, glse, Output_partial, row_sums, scores, layer)
     indices = topk_indices(agg[:, :, :L], topk, fill_value=0)
     if layer != 0:
-        o = decode_reuse(Q, K, V, indices, torch.arange(G, device=Q.device, dtype=torch.int32), glse,
+        o = decode_reuse(Q, K, V, indices, torch.arange(K.shape[2], device=Q.device, dtype=torch.int32), glse,
                          Output_partial)
     return o, indices, agg[:, :, :L]
 
@@ -730,10 +780,11 @@ def decode_full_kernel_kvcache(Q, K, V, cache_seqlens, topk_percent, glse, Outpu
     else:
         fl = torch.floor(cache_seqlens.to(torch.float64) * float(topk_percent) / 100.0).to(torch.int64)
     counts = (((fl + 127) // 128) * 128).to(torch.int32)
-    indices = topk_indices(agg[:, :, :max_seqlen], width, valid_len=cache_seqlens.repeat_interleave(G),
-                           n_sel=counts.repeat_interleave(G), fill_value=0)
+    Gk = K.shape[-2]
+    indices = topk_indices(agg[:, :, :max_seqlen], width, valid_len=cache_seqlens.repeat_interleave(Gk),
+                           n_sel=counts.repeat_interleave(Gk), fill_value=0)
     if layer != 0:
         o = decode_reuse_paged(Q, K, V, cache_seqlens, indices,
-                               torch.arange(G, device=Q.device, dtype=torch.int32), topk_percent, glse,
+                               torch.arange(Gk, device=Q.device, dtype=torch.int32), topk_percent, glse,
                                Output_partial, block_table=block_table, page_size=page_size)
     return o, indices, agg[:, :, :max_seqlen]

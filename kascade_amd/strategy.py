@@ -86,10 +86,12 @@ class EfficientKascadeStrategy:
             self.register_attention()
 
     # ------------------------------------------------------------------ helpers
-    def _hm(self, layer, device) -> torch.Tensor:
-        key = (layer, str(device))
+    def _hm(self, layer, device, groups: int = G) -> torch.Tensor:
+        key = (layer, str(device), groups)
         if key not in self._hm_cache:
-            row = list(range(G)) if layer is None else self._head_mapping[layer]
+            row = list(range(groups)) if layer is None else self._head_mapping[layer]
+            if len(row) != groups:
+                raise KascadeError(f"head mapping of layer {layer} has {len(row)} entries for {groups} KV heads")
             self._hm_cache[key] = torch.tensor(row, device=device, dtype=torch.int32)
         return self._hm_cache[key]
 
@@ -107,6 +109,7 @@ class EfficientKascadeStrategy:
         layer 0), pooled tile scores, per-tile selection, and on layers > 0 the sparse pass with
         the fresh indices and the identity head map."""
         B, L = Q.shape[:2]
+        G = K.shape[2]                      # KV heads of this model (8 for the reference's shape)
         T = math.ceil(L / tile_size)
         if layer == 0:
             log_sum, o = kernels.prefill_recompute0(Q, K, V)
@@ -135,43 +138,45 @@ class EfficientKascadeStrategy:
                                                         n_sel=nsel[t0:t1].contiguous(), fill_value=L - 1)
             self._topk_to_reuse = idx
         if layer != 0:
-            o = kernels.prefill_reuse(Q, K, V, self._topk_to_reuse, self._hm(None, Q.device), topk_percent,
+            o = kernels.prefill_reuse(Q, K, V, self._topk_to_reuse, self._hm(None, Q.device, G), topk_percent,
                                       self.rolling_prefill)
         return o
 
     def _prefill_reuse_forward(self, Q, K, V, topk_percent, layer):
         """Reuse prefill (EfficientKascadeStrategy.py:95-98)."""
-        return kernels.prefill_reuse(Q, K, V, self._topk_to_reuse, self._hm(layer, Q.device), topk_percent,
+        return kernels.prefill_reuse(Q, K, V, self._topk_to_reuse, self._hm(layer, Q.device, K.shape[2]), topk_percent,
                                      self.rolling_prefill)
 
     # ------------------------------------------------------------------- decode
-    def _decode_scratch(self, B, ns, device):
-        return (torch.empty(B, H, ns, device=device, dtype=torch.float32),
-                torch.empty(B, H, ns, D, device=device, dtype=torch.float32))
+    def _decode_scratch(self, Q, ns):
+        B, heads, dim = Q.shape
+        return (torch.empty(B, heads, ns, device=Q.device, dtype=torch.float32),
+                torch.empty(B, heads, ns, dim, device=Q.device, dtype=torch.float32))
 
     def _decode_recomp_forward(self, Q, K, V, topk, layer):
         """Anchor decode (EfficientKascadeStrategy.py:100-115) over a contiguous [B,L,G,D] cache."""
-        B, L = K.shape[:2]
-        ns = kernels.default_num_split(B * G * L, L)
-        glse, part = self._decode_scratch(B, ns, Q.device)
+        B, L, G = K.shape[:3]
+        H = Q.shape[1]
+        ns = kernels.default_num_split(B * G * L, L, heads=G)
+        glse, part = self._decode_scratch(Q, ns)
         row_sums = torch.empty(B, H, device=Q.device, dtype=torch.float32)
         stride = ((L + 7) // 8) * 8
         scores = torch.empty(B, H, stride, device=Q.device, dtype=torch.float32)
         o, agg = kernels.decode_recompute(Q, K, V, glse, part, row_sums, scores, layer)
         self._topk_to_reuse = kernels.topk_indices(agg[:, :, :L], topk, fill_value=0)
         if layer != 0:
-            ns = kernels.default_num_split(B * G * topk, topk, cap_rows=kernels.GATHER_ROWS_PER_SPLIT)
-            glse, part = self._decode_scratch(B, ns, Q.device)
-            o = kernels.decode_reuse(Q, K, V, self._topk_to_reuse, self._hm(None, Q.device), glse, part)
+            ns = kernels.default_num_split(B * G * topk, topk, cap_rows=kernels.GATHER_ROWS_PER_SPLIT, heads=G)
+            glse, part = self._decode_scratch(Q, ns)
+            o = kernels.decode_reuse(Q, K, V, self._topk_to_reuse, self._hm(None, Q.device, G), glse, part)
         return o
 
     def _decode_reuse_forward(self, Q, K, V, layer):
         """Reuse decode (EfficientKascadeStrategy.py:117-123)."""
-        B = Q.shape[0]
+        B, G = Q.shape[0], K.shape[2]
         topk = self._topk_to_reuse.shape[-1]
-        ns = kernels.default_num_split(B * G * topk, topk, cap_rows=kernels.GATHER_ROWS_PER_SPLIT)
-        glse, part = self._decode_scratch(B, ns, Q.device)
-        return kernels.decode_reuse(Q, K, V, self._topk_to_reuse, self._hm(layer, Q.device), glse, part)
+        ns = kernels.default_num_split(B * G * topk, topk, cap_rows=kernels.GATHER_ROWS_PER_SPLIT, heads=G)
+        glse, part = self._decode_scratch(Q, ns)
+        return kernels.decode_reuse(Q, K, V, self._topk_to_reuse, self._hm(layer, Q.device, G), glse, part)
 
     # --------------------------------------------------------------- HF boundary
     def attention_forward(self, module, query, key, value, attention_mask, scaling, dropout=0.0, **kwargs):
@@ -180,8 +185,12 @@ class EfficientKascadeStrategy:
             from transformers.modeling_utils import ALL_ATTENTION_FUNCTIONS
             return ALL_ATTENTION_FUNCTIONS["sdpa"](module, query, key, value, attention_mask,
                                                    scaling=scaling, dropout=dropout, **kwargs)
-        if query.shape[1] != H or key.shape[1] != G or query.shape[-1] != D or query.dtype != torch.float16:
-            raise KascadeError("efficient_kascade supports fp16 with 32 query heads, 8 KV heads, head_dim 128")
+        # the reference's kernels exist for fp16, 32 query / 8 KV heads, head_dim 128 only
+        # (EfficientKascadeStrategy.py:19-21); here any model with four query heads per KV head,
+        # head_dim 64 or 128, in fp16 or bf16
+        if query.shape[1] != 4 * key.shape[1] or query.shape[-1] not in (64, 128) \
+                or query.dtype not in (torch.float16, torch.bfloat16):
+            raise KascadeError("efficient_kascade needs fp16 or bf16, four query heads per KV head, head_dim 64 or 128")
         is_decode = (query.shape[2] == 1)
         Lk = key.shape[-2]
         rounded_k = budgets.topk_width(Lk, self.k)
