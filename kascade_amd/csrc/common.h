@@ -49,6 +49,11 @@ template <> struct Elem<half_t> {
     static __device__ __forceinline__ float16_t mma_32x32x16(x8 a, x8 b, float16_t c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
     }
+    // acc + p.x + p.y in fp32 (one instruction for two elements)
+    static __device__ __forceinline__ float add_pair(x2 p, float acc) {
+        const x2 ones = {(half_t)1.f, (half_t)1.f};
+        return __builtin_amdgcn_fdot2(p, ones, acc, false);
+    }
 };
 template <> struct Elem<bf16_t> {
     typedef bf16x2_t x2; typedef bf16x4_t x4; typedef bf16x8_t x8;
@@ -60,6 +65,10 @@ template <> struct Elem<bf16_t> {
     }
     static __device__ __forceinline__ float16_t mma_32x32x16(x8 a, x8 b, float16_t c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float add_pair(x2 p, float acc) {
+        const x2 ones = {(bf16_t)1.f, (bf16_t)1.f};
+        return __builtin_amdgcn_fdot2_f32_bf16(p, ones, acc, false);
     }
 };
 
@@ -86,6 +95,18 @@ __device__ __forceinline__ float row16_sum(float x) {
     x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x141, 0xF, 0xF, false));  // row_half_mirror
     x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x140, 0xF, 0xF, false));  // row_mirror
     return x;
+}
+
+// max(x in this lane, x in lane ^ 32) without a trip through LDS (gfx950 lane-half swap)
+__device__ __forceinline__ float max_with_other_half(float x) {
+    const uint32_t u = __builtin_bit_cast(uint32_t, x);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);   // {low half twice, high half twice}
+    return fmaxf(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1]));
+}
+__device__ __forceinline__ float sum_with_other_half(float x) {
+    const uint32_t u = __builtin_bit_cast(uint32_t, x);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __builtin_bit_cast(float, (uint32_t)r[0]) + __builtin_bit_cast(float, (uint32_t)r[1]);
 }
 
 __device__ __forceinline__ uint4_t ld_global_16(const void* p) {

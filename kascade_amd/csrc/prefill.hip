@@ -25,6 +25,7 @@
 #include "prefill.h"
 
 #include <algorithm>
+#include <type_traits>
 
 namespace kascade {
 
@@ -65,6 +66,7 @@ template <int NQB, bool REUSE, bool WITH_V, bool PAGED, int D, typename T>
 __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK, T* sV) {
     typedef typename Elem<T>::x8 x8_t;
     typedef typename Elem<T>::x4 x4_t;
+    typedef typename Elem<T>::x2 x2_t;
     typedef AttnTile<D> G_;
     constexpr int kKT = G_::kKT, kKStride = G_::kKStride, kVStride = G_::kVStride;
     constexpr int kKS = G_::kKS, kDB = G_::kDB, kKB = G_::kKB, kS = G_::kS, kChunks = G_::kChunks;
@@ -135,10 +137,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
         if (sparse && ti < ng) {
             const int base = ti * kKT + 4 * krow;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int a = idx_row[min(base + i, n - 1)];
-                ids[i] = max(0, min(a, PAGED ? max_row : L - 1));
-            }
+            for (int i = 0; i < 4; ++i) ids[i] = idx_row[min(base + i, n - 1)];   // used (and bounded) a tile later
         } else if (PAGED) {
             ids[0] = bt_row[tile_key(ti, 4 * krow) >> p.page_shift];
         }
@@ -147,7 +146,10 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
         long long off[4];
         if (sparse && pend_ti < ng) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) off[i] = (long long)((unsigned long long)(unsigned)ids[i] * row_stride);
+            for (int i = 0; i < 4; ++i) {   // a corrupt index must not leave the tensor
+                const int row = max(0, min(ids[i], PAGED ? max_row : L - 1));
+                off[i] = (long long)((unsigned long long)(unsigned)row * row_stride);
+            }
         } else {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -164,6 +166,16 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
         }
     };
 
+    // Softmax state.  m[] is the reference the exponentials are taken against, in log2 units of
+    // the scaled scores.  It follows the running maximum lazily: a tile moves it only when one of
+    // its scores lies more than kRefSlack above it, so an exponential never exceeds 2^kRefSlack
+    // (representable in fp16 and bf16, sums and products are kept in fp32) and the rescaling of the
+    // accumulators -- 64 products per lane -- runs on the first tiles of a unit and then almost
+    // never.  The quotient is the same: numerator and denominator carry the same factor.
+    constexpr float kRefSlack = 8.f;
+    // Reuse units sum the exponentials as they enter the second product (rounded to the element
+    // type, two per instruction); the passes whose log-sum feeds the selection sum them in fp32.
+    constexpr bool kPairSum = REUSE && WITH_V;
     float m[NQB], l[NQB];
     float16_t oT[NQB][kDB];
 #pragma unroll
@@ -204,17 +216,14 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
         }
     }
 
-
-    // The diagonal tile of a sparse unit (32 keys, half the products) runs as a phase of its own
-    // of the tile loop; the phase loop is unrolled, so each phase is compiled with its key-block
-    // count as a constant and the gathered tiles run straight-line code (with a run-time count
-    // every matrix instruction of the second half sits behind a branch).
-#pragma unroll
-    for (int phase = 0; phase < (REUSE ? 2 : 1); ++phase) {
-    const bool diag_phase = REUSE && (phase == 0);
-    const int s_begin = (REUSE && !diag_phase && sparse) ? 1 : 0;
-    const int s_end = diag_phase ? (sparse ? 1 : 0) : ntiles;
-    for (int sq = s_begin; sq < s_end; ++sq) {
+    // One tile: registers -> LDS, next tile's loads, both products, softmax.  Three copies of
+    // the code, each straight-line: tiles that need no mask (all but one or two of a unit), tiles
+    // that do (the causal edge, the end of the sequence, a selection that ends inside a tile), and
+    // the diagonal tile of a sparse unit (32 keys: half the products).
+    constexpr int kFull = 0, kMasked = 1, kDiag = 2;
+    auto run_tile = [&](int sq, auto mode_c) {
+        constexpr int MODE = decltype(mode_c)::value;
+        constexpr int nkb = (MODE == kDiag && QT == 32) ? 1 : kKB;
         const int ti = tile_at(sq);
         __syncthreads();
         // ---- registers -> LDS ----
@@ -242,39 +251,39 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
         }
 
         // ---- S^T = K_tile Q^T ----
-        const bool diag_tile = diag_phase;
-        const int nkb = (diag_tile && QT == 32) ? 1 : kKB;
-        float16_t sT[NQB][kKB];
+        float16_t sT[NQB][nkb];
         float16_t zero16;
 #pragma unroll
         for (int v = 0; v < 16; ++v) zero16[v] = 0.f;
 #pragma unroll
-        for (int kb = 0; kb < kKB; ++kb) {
-            if (kb < nkb) {
+        for (int kb = 0; kb < nkb; ++kb) {
 #pragma unroll
-                for (int ks = 0; ks < kKS; ++ks) {
-                    x8_t a = *reinterpret_cast<const x8_t*>(
-                        &sK[(32 * kb + li) * kKStride + ks * 16 + lg * 8]);
+            for (int ks = 0; ks < kKS; ++ks) {
+                x8_t a = *reinterpret_cast<const x8_t*>(&sK[(32 * kb + li) * kKStride + ks * 16 + lg * 8]);
 #pragma unroll
-                    for (int qb = 0; qb < NQB; ++qb)   // the first product starts from a constant zero
-                        sT[qb][kb] = Elem<T>::mma_32x32x16(a, qf[qb][ks], ks == 0 ? zero16 : sT[qb][kb]);
-                }
-            } else {   // second key block of a 32-key diagonal tile: nothing there
-#pragma unroll
-                for (int qb = 0; qb < NQB; ++qb)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) sT[qb][kb][v] = -INFINITY;
+                for (int qb = 0; qb < NQB; ++qb)   // the first product starts from a constant zero
+                    sT[qb][kb] = Elem<T>::mma_32x32x16(a, qf[qb][ks], ks == 0 ? zero16 : sT[qb][kb]);
             }
         }
         // ---- masks: accumulator v of key block kb is tile position 32kb + 16(v/8) + 8lg + v%8 ----
-        if (!sparse || diag_tile) {
-            const int kstart = diag_tile ? q0 : ti * kKT;
-            if (kstart + kKT - 1 > q0 || kstart + kKT > L) {
+        if (MODE != kFull) {
+            if (MODE == kMasked && sparse) {   // a selection that ends inside this tile
+#pragma unroll
+                for (int qb = 0; qb < NQB; ++qb)
+#pragma unroll
+                    for (int kb = 0; kb < nkb; ++kb)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const int pos = ti * kKT + 32 * kb + 16 * (v >> 3) + 8 * lg + (v & 7);
+                            if (pos >= n) sT[qb][kb][v] = -INFINITY;
+                        }
+            } else {                           // the causal edge and the end of the sequence
+                const int kstart = (MODE == kDiag) ? q0 : ti * kKT;
 #pragma unroll
                 for (int qb = 0; qb < NQB; ++qb) {
                     const int q = q0 + 32 * qb + li;   // global position
 #pragma unroll
-                    for (int kb = 0; kb < kKB; ++kb)
+                    for (int kb = 0; kb < nkb; ++kb)
 #pragma unroll
                         for (int v = 0; v < 16; ++v) {
                             const int key = kstart + 32 * kb + 16 * (v >> 3) + 8 * lg + (v & 7);
@@ -282,56 +291,60 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
                         }
                 }
             }
-        } else if ((ti + 1) * kKT > n) {
-#pragma unroll
-            for (int qb = 0; qb < NQB; ++qb)
-#pragma unroll
-                for (int kb = 0; kb < kKB; ++kb)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int pos = ti * kKT + 32 * kb + 16 * (v >> 3) + 8 * lg + (v & 7);
-                        if (pos >= n) sT[qb][kb][v] = -INFINITY;
-                    }
         }
-        // ---- online softmax (one query column per lane) ----
-        x8_t pf[NQB][kS];
+        // ---- online softmax (one query column per lane pair: lanes li and li + 32) ----
+        x8_t pf[NQB][2 * nkb];
 #pragma unroll
         for (int qb = 0; qb < NQB; ++qb) {
             float mx = -INFINITY;
 #pragma unroll
-            for (int kb = 0; kb < kKB; ++kb)
+            for (int kb = 0; kb < nkb; ++kb)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) mx = fmaxf(mx, sT[qb][kb][v]);
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
-            const float mnew = fmaxf(m[qb], mx);
-            const float mref = (mnew == -INFINITY) ? 0.f : mnew * kScaleLog2;
-            const float corr = fast_exp2(m[qb] * kScaleLog2 - mref);
-            m[qb] = mnew;
-            float sum = 0.f;
-#pragma unroll
-            for (int kb = 0; kb < kKB; ++kb)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const float e = fast_exp2(sT[qb][kb][v] * kScaleLog2 - mref);
-                    sT[qb][kb][v] = e;
-                    sum += e;
-                }
-            l[qb] = l[qb] * corr + sum;   // per-lane partial sum (own key positions)
-            if (WITH_V) {
-                if (__any(corr != 1.f)) {   // wavefront-uniform: skip when no maximum moved
+            const float ms = mx * kScaleLog2;
+            if (__any(ms > m[qb] + kRefSlack)) {   // wavefront-uniform
+                const float mnew = fmaxf(m[qb], max_with_other_half(ms));   // the same in both lanes of a column
+                const float corr = (mnew == -INFINITY) ? 1.f : fast_exp2(m[qb] - mnew);
+                m[qb] = mnew;
+                l[qb] *= corr;
+                if (WITH_V) {
 #pragma unroll
                     for (int db = 0; db < kDB; ++db)
 #pragma unroll
                         for (int v = 0; v < 16; ++v) oT[qb][db][v] *= corr;
                 }
+            }
+            const float mu = (m[qb] == -INFINITY) ? 0.f : m[qb];
 #pragma unroll
-                for (int s = 0; s < kS; ++s) {
+            for (int kb = 0; kb < nkb; ++kb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    sT[qb][kb][v] = fast_exp2(__builtin_fmaf(sT[qb][kb][v], kScaleLog2, -mu));
+            float sum = 0.f;
+            if (WITH_V) {
+#pragma unroll
+                for (int s = 0; s < 2 * nkb; ++s) {
                     x8_t t;
 #pragma unroll
                     for (int e = 0; e < 8; ++e) t[e] = (T)sT[qb][s >> 1][8 * (s & 1) + e];
                     pf[qb][s] = t;
                 }
             }
+            if (kPairSum) {
+#pragma unroll
+                for (int s = 0; s < 2 * nkb; ++s)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const x2_t pr = {pf[qb][s][2 * e], pf[qb][s][2 * e + 1]};
+                        sum = Elem<T>::add_pair(pr, sum);
+                    }
+            } else {
+#pragma unroll
+                for (int kb = 0; kb < nkb; ++kb)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) sum += sT[qb][kb][v];
+            }
+            l[qb] += sum;   // per-lane partial sum (own key positions)
         }
         // ---- O^T += V^T P^T ----
         if (WITH_V) {
@@ -340,28 +353,36 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
                 const int d = 32 * db + li;
                 const int sw = ((d & 7) ^ (d >> 3)) & 7;
 #pragma unroll
-                for (int s = 0; s < kS; ++s) {
-                    if (s < 2 * nkb) {
-                        x8_t a = *reinterpret_cast<const x8_t*>(
-                            &sV[d * kVStride + (((2 * s + lg) ^ sw) * 8)]);
+                for (int s = 0; s < 2 * nkb; ++s) {
+                    x8_t a = *reinterpret_cast<const x8_t*>(&sV[d * kVStride + (((2 * s + lg) ^ sw) * 8)]);
 #pragma unroll
-                        for (int qb = 0; qb < NQB; ++qb)
-                            oT[qb][db] = Elem<T>::mma_32x32x16(a, pf[qb][s], oT[qb][db]);
-                    }
+                    for (int qb = 0; qb < NQB; ++qb)
+                        oT[qb][db] = Elem<T>::mma_32x32x16(a, pf[qb][s], oT[qb][db]);
                 }
             }
         }
-    }
+    };
+
+    {
+        int sq = 0;
+        if (REUSE && sparse) {
+            run_tile(0, std::integral_constant<int, kDiag>{});
+            sq = 1;
+        }
+        // tiles wholly below the unit's first query and inside the sequence / wholly inside the selection
+        const int full_end = (REUSE && sparse) ? 1 + n / kKT : min((q0 + 1) / kKT, L / kKT);
+        for (; sq < full_end; ++sq) run_tile(sq, std::integral_constant<int, kFull>{});
+        for (; sq < ntiles; ++sq) run_tile(sq, std::integral_constant<int, kMasked>{});
     }
 
     // ---- epilogue (rows are local to this call) ----
 #pragma unroll
     for (int qb = 0; qb < NQB; ++qb) {
         const int ql = q0l + 32 * qb + li;
-        const float lt = l[qb] + __shfl_xor(l[qb], 32);
+        const float lt = sum_with_other_half(l[qb]);
         if (ql < Lq) {
             if (p.log_sum && lg == 0)
-                p.log_sum[((long long)b * Lq + ql) * nheads + head] = fast_log2(lt) + m[qb] * kScaleLog2;
+                p.log_sum[((long long)b * Lq + ql) * nheads + head] = fast_log2(lt) + m[qb];
             if (WITH_V) {
                 const float inv = 1.f / lt;
                 T* op = (T*)p.O + (((long long)b * Lq + ql) * nheads + head) * D;
