@@ -26,6 +26,7 @@ typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef short short8_t __attribute__((ext_vector_type(8)));
 
 // Element types of Q, K, V and the attention output (pooled scores are fp16 for both).
 enum ElemKind { kElemF16 = 0, kElemBF16 = 1 };

@@ -1,4 +1,4 @@
-// Prefill attention kernels for gfx950 (fp16 MFMA 32x32x16, fp32 softmax).
+// Prefill attention kernels for gfx950 (fp16/bf16 MFMA 32x32x16, fp32 softmax).
 //
 // prefill_attn_kernel -- flash attention over one (query block, KV head, batch)
 //   per workgroup; 4 wavefronts, wavefront w owns q-head 4g+w and 32*NQB queries,
@@ -6,17 +6,20 @@
 //   Three key regimes (REUSE): dense causal, gathered top-k rows through the
 //   tile's index list, and the within-tile causal diagonal.
 //
+//   K/V tiles go from global memory straight into LDS (global_load_lds_dwordx4: no staging
+//   registers, no LDS store instructions) into one of two buffers, so a tile costs one
+//   barrier: wait for the own loads, barrier, start the next tile's loads into the other
+//   buffer, compute.  Rows lie in LDS as they lie in memory; the 16-byte chunk c of row R
+//   sits at chunk c ^ swz(R), chosen by the lane that fetches it (each lane picks the global
+//   chunk that belongs at its LDS position), which makes both read patterns below free of
+//   bank conflicts without padding.
+//
 //   The kernel works on S^T = K Q^T so that each lane owns one query column:
 //   row max / row sum are in-lane reductions plus one cross-half exchange, and
 //   the exponentiated scores are already in the B-operand layout of the second
-//   product O^T = V^T P^T -- P never leaves registers.  K rows are stored in LDS
-//   at a bit-swapped slot (bits 2 and 3 exchanged) which makes the accumulator
-//   registers of one lane cover 8 consecutive key positions, i.e. one 16-byte
-//   read of the transposed V tile per MFMA operand.  V is transposed on its way
-//   into LDS (4 keys x 8 d per thread, eight 8-byte writes) with the 16-byte chunks
-//   of each row XOR-swizzled by (d & 7) ^ (d >> 3); of the layouts measured with the
-//   LDS bank-conflict counter this one conflicts least (K rows padded to 272 bytes
-//   show no conflicts at all).
+//   product O^T = V^T P^T -- P never leaves registers.  The A operand of that product,
+//   V^T, comes out of the row-major V tile through the transposing LDS read
+//   ds_read_b64_tr_b16 (two per operand: four keys each).
 //
 // prefill_aggregate_kernel -- pooled tile scores: S = Q_tile K^T with the 128
 //   (query, head) rows of a tile held as A operands in registers by every
@@ -40,17 +43,53 @@ constexpr int kAggKT = 128;        // keys per tile (aggregate kernel)
 // and the score registers a narrower head frees hold the extra keys.
 template <int D> struct AttnTile {
     static constexpr int kKT = 64 * 128 / D;     // keys per tile
-    static constexpr int kKStride = D + 8;       // elements per K row in LDS (padded)
-    static constexpr int kVStride = kKT;         // elements per V^T row in LDS (one tile of keys)
     static constexpr int kKS = D / 16;           // contraction steps of S^T = K Q^T
     static constexpr int kDB = D / 32;           // 32-row blocks of O^T
     static constexpr int kKB = kKT / 32;         // 32-key blocks of a tile
-    static constexpr int kS = kKT / 16;          // contraction steps of O^T = V^T P^T
-    static constexpr int kChunks = D / 8;        // 16-byte columns of a row
+    static constexpr int kChunks = D / 8;        // 16-byte chunks of a row
+    static constexpr int kRowsPerLoad = 64 / kChunks;   // rows one wavefront-wide 16-byte load covers
+    static constexpr int kTileElems = kKT * D;   // 16 KB of K (and of V) whatever D
 };
 
-__device__ __forceinline__ int swap_bits23(int x) {
-    return (x & ~0xC) | ((x & 4) << 1) | ((x & 8) >> 1);
+// Chunk permutation of a tile row in LDS (see the head of the file).  What it must give:
+// 16 lanes reading the same chunk of 16 consecutive rows (A operand of S^T), and 32 lanes
+// reading 4 consecutive rows x 4 consecutive chunks in 8-byte halves (transposing read of V),
+// each touch all 64 banks once.  Rows are 256 bytes (D = 128: the row does not move the bank)
+// or 128 bytes (D = 64: the row parity picks the bank half, three more row bits permute).
+template <int D> __device__ __forceinline__ int swz(int row);
+template <> __device__ __forceinline__ int swz<128>(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+template <> __device__ __forceinline__ int swz<64>(int row) { return (((row >> 1) & 1) << 2) | ((row >> 2) & 3); }
+
+// One wavefront-wide load of 16 bytes per lane from global memory into LDS: lane i's bytes
+// land at lds_base + 16 i (lds_base wavefront-uniform).  Counted by vmcnt like any load; the
+// compiler does not know that it writes LDS, so whoever reads the bytes waits for vmcnt and
+// passes a barrier first (the tile loop does both once per tile).
+__device__ __forceinline__ void load_to_lds_16(const void* gptr, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :: "v"(gptr), "s"(lds_base) : "m0");
+}
+template <typename P> __device__ __forceinline__ uint32_t lds_address(P* ptr) {
+    return (uint32_t)(size_t)(__attribute__((address_space(3))) void*)ptr;
+}
+
+// Workgroup -> (query block, KV head, sequence).  Workgroups go to the eight XCDs round-robin in
+// launch order and each XCD has an L2 of its own.  When the number of (sequence, KV head) pairs
+// is a multiple of eight the launch is one-dimensional and consecutive workgroups take eight
+// different pairs: all units of a pair, which read the same K/V rows, run on one XCD.
+__host__ __device__ inline bool pairs_fill_xcds(int B, int G) { return (B * G) % 8 == 0; }
+__device__ __forceinline__ void unit_of_workgroup(int B, int G, int nblocks, int& blk, int& g, int& b) {
+    if (pairs_fill_xcds(B, G)) {
+        const int i = blockIdx.x;
+        const int r = i >> 3;
+        const int pair = (r / nblocks) * 8 + (i & 7);
+        blk = r % nblocks;
+        g = pair % G;
+        b = pair / G;
+    } else {
+        blk = blockIdx.x;
+        g = blockIdx.y;
+        b = blockIdx.z;
+    }
 }
 
 __device__ __forceinline__ int rolling_budget(float pct, int tile_start) {
@@ -68,8 +107,8 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
     typedef typename Elem<T>::x4 x4_t;
     typedef typename Elem<T>::x2 x2_t;
     typedef AttnTile<D> G_;
-    constexpr int kKT = G_::kKT, kKStride = G_::kKStride, kVStride = G_::kVStride;
-    constexpr int kKS = G_::kKS, kDB = G_::kDB, kKB = G_::kKB, kS = G_::kS, kChunks = G_::kChunks;
+    constexpr int kKT = G_::kKT, kKS = G_::kKS, kDB = G_::kDB, kKB = G_::kKB, kChunks = G_::kChunks;
+    constexpr int kRPL = G_::kRowsPerLoad, kTileElems = G_::kTileElems;
     constexpr float kScaleLog2 = ScaleLog2<D>::value;
     const int kvh = p.G, nheads = p.G * kGroupSize;
     const T* Qp = (const T*)p.Q;
@@ -80,9 +119,9 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
     const int L = p.L;
     const int Lq = p.Lq;
     const int nqt = (Lq + QT - 1) / QT;
-    const int tq = nqt - 1 - (int)blockIdx.x;   // long (late) query blocks first
-    const int g = blockIdx.y;
-    const int b = blockIdx.z;
+    int blk, g, b;
+    unit_of_workgroup(p.B, p.G, nqt, blk, g, b);
+    const int tq = nqt - 1 - blk;   // long (late) query blocks first
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
     const int lane = tid & 63;
@@ -107,64 +146,80 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
     }
     const int ntiles = sparse ? ng + 1 : (min(q0 + QT, L) + kKT - 1) / kKT;
 
-    const int krow = tid / kChunks;   // tile positions 4*krow + i, 16-byte column kcol
-    const int kcol = tid % kChunks;
-    const T* kbase = PAGED ? Kp + (long long)g * D + kcol * 8
-                           : Kp + (long long)b * p.k_sb + (long long)g * p.k_sh + kcol * 8;
-    const T* vbase = PAGED ? Vp + (long long)g * D + kcol * 8
-                           : Vp + (long long)b * p.k_sb + (long long)g * p.k_sh + kcol * 8;
+    // ---- tile staging: wavefront w fills rows [4w R, 4(w+1) R) of a tile with four loads of R rows
+    // each (R = 4 at D = 128, 8 at D = 64); lane = (row within the load, chunk position) ----
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int lrow = lane / kChunks;
+    const int lchunk = lane % kChunks;
+    const int pos0 = wave * 4 * kRPL + lrow;     // this lane's rows: tile positions pos0 + j R, j = 0..3
+    int coff[4];                                 // element offset of the chunk this lane fetches for row j
+#pragma unroll
+    for (int j = 0; j < 4; ++j) coff[j] = (lchunk ^ swz<D>(pos0 + j * kRPL)) * 8;
+    const T* kbase = PAGED ? Kp + (long long)g * D : Kp + (long long)b * p.k_sb + (long long)g * p.k_sh;
+    const T* vbase = PAGED ? Vp + (long long)g * D : Vp + (long long)b * p.k_sb + (long long)g * p.k_sh;
     const int* bt_row = PAGED ? p.block_table + (long long)b * p.max_pages : nullptr;
     const int page_mask = (1 << p.page_shift) - 1;
     const int max_row = PAGED ? (p.num_pages << p.page_shift) - 1 : 0;
+    const uint32_t lds_k = lds_address(sK) + wave_u * 4096;   // this wavefront's 4 KB of a K buffer
+    const uint32_t lds_v = WITH_V ? lds_address(sV) + wave_u * 4096 : 0;
 
     // key position `pos` of tile `ti` -> key id (contiguous and diagonal tiles)
     auto tile_key = [&](int ti, int pos) {
         return min((sparse ? q0 : ti * kKT) + pos, L - 1);
     };
-    // A thread stages the same four key positions 4*krow .. 4*krow+3 of a tile for K and for V
-    // (V needs four consecutive keys per thread for its transposition; K rows can go anywhere),
-    // so one id and one address offset per position serve both tensors.
-    // ids[]: what the next tile's loads need.  Gathered tiles: key ids (physical rows when
-    // PAGED).  Consecutive keys, PAGED: ids[0] is the block-table entry of the four positions'
-    // common page, fetched a tile ahead so that the loads never wait on the table.  Consecutive
-    // keys, strided: nothing (addresses follow from the tile index).
+    // ids[j]: what the loads of row j of the next tile need, fetched a tile ahead so that the
+    // loads never wait on it.  Gathered tiles: the key id (physical row when PAGED).
+    // Consecutive keys, PAGED: the block-table entry of the key's page.  Consecutive keys,
+    // strided: nothing (addresses follow from the tile index).
     int ids[4];
     int pend_ti = 0;        // tile the ids belong to
-    uint4_t kr[4], vr[4];   // tile data in flight
     const unsigned row_stride = PAGED ? (unsigned)(kvh * D) : (unsigned)p.k_sl;   // host checks < 2^31
     auto fetch_ids = [&](int ti) {
         pend_ti = ti;
         if (sparse && ti < ng) {
-            const int base = ti * kKT + 4 * krow;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) ids[i] = idx_row[min(base + i, n - 1)];   // used (and bounded) a tile later
+            for (int j = 0; j < 4; ++j) ids[j] = idx_row[min(ti * kKT + pos0 + j * kRPL, n - 1)];   // bounded at use
         } else if (PAGED) {
-            ids[0] = bt_row[tile_key(ti, 4 * krow) >> p.page_shift];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) ids[j] = bt_row[tile_key(ti, pos0 + j * kRPL) >> p.page_shift];
         }
     };
-    auto issue_loads = [&]() {
-        long long off[4];
+    // Row addresses of the tile whose ids are held (element offsets from kbase / vbase).  The
+    // loads themselves are issued one at a time between the matrix instructions of the first
+    // product: a wavefront that issued all eight at once would sit in front of the memory
+    // pipeline, which takes 16 cycles per 1 KB load, with nothing running behind it.
+    long long off[4];
+    auto next_offsets = [&]() {
         if (sparse && pend_ti < ng) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {   // a corrupt index must not leave the tensor
-                const int row = max(0, min(ids[i], PAGED ? max_row : L - 1));
-                off[i] = (long long)((unsigned long long)(unsigned)row * row_stride);
+            for (int j = 0; j < 4; ++j) {   // a corrupt index must not leave the tensor
+                const int row = max(0, min(ids[j], PAGED ? max_row : L - 1));
+                off[j] = (long long)((unsigned long long)(unsigned)row * row_stride) + coff[j];
             }
         } else {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int key = tile_key(pend_ti, 4 * krow + i);
-                const int row = PAGED ? (ids[0] << p.page_shift) + (key & page_mask) : key;
-                off[i] = (long long)((unsigned long long)(unsigned)row * row_stride);
+            for (int j = 0; j < 4; ++j) {
+                const int key = tile_key(pend_ti, pos0 + j * kRPL);
+                const int row = PAGED ? (ids[j] << p.page_shift) + (key & page_mask) : key;
+                off[j] = (long long)((unsigned long long)(unsigned)row * row_stride) + coff[j];
             }
         }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) kr[i] = ld_global_16(kbase + off[i]);
-        if (WITH_V) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) vr[i] = ld_global_16(vbase + off[i]);
-        }
     };
+    constexpr int kNumLoads = WITH_V ? 8 : 4;
+    auto issue_load = [&](int i, int buf) {   // i < 4: K row group i; else V row group i - 4
+        if (i < 4) load_to_lds_16(kbase + off[i], lds_k + buf * (kTileElems * 2) + i * 1024);
+        else load_to_lds_16(vbase + off[i - 4], lds_v + buf * (kTileElems * 2) + (i - 4) * 1024);
+    };
+    // LDS read positions (elements, within a tile buffer).  A operand of S^T: row 32 kb + li,
+    // chunk 2 ks + lg.  A operand of O^T (two transposing reads h = 0, 1 of four keys each):
+    // the 16 lanes of a group address rows 16 s + 8 h + 4 lg + (0..3) of a key block, 16 columns
+    // of V from column 32 db + 16 (group & 1) on, and receive one column of the four rows each.
+    const int kx = lg ^ swz<D>(li);
+    const int krd = li * D;
+    const int vcol = lane & 15;
+    const int vrow = 4 * lg + (vcol >> 2);                          // + 32 kb + 16 s + 8 h
+    const int vchunk = 2 * ((lane >> 4) & 1) + ((vcol >> 1) & 1);    // + 4 db
+    const int vrd = vrow * D + 4 * (vcol & 1);
 
     // Softmax state.  m[] is the reference the exponentials are taken against, in log2 units of
     // the scaled scores.  It follows the running maximum lazily: a tile moves it only when one of
@@ -195,7 +250,9 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
     // average under rolling budgets).  Softmax is accumulated online, so the order is free.
     auto tile_at = [&](int s) { return (REUSE && sparse) ? (s == 0 ? ng : s - 1) : s; };
     fetch_ids(tile_at(0));
-    issue_loads();
+    next_offsets();
+#pragma unroll
+    for (int i = 0; i < kNumLoads; ++i) issue_load(i, 0);
     if (ntiles > 1) fetch_ids(tile_at(1));
 
     // ---- Q fragments (B operand of S^T): query li (+32 qb), d chunk 16*ks + 8*lg; requested after
@@ -225,47 +282,52 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
         constexpr int MODE = decltype(mode_c)::value;
         constexpr int nkb = (MODE == kDiag && QT == 32) ? 1 : kKB;
         const int ti = tile_at(sq);
+        const T* bK = sK + (sq & 1) * kTileElems;
+        const T* bV = sV + (sq & 1) * kTileElems;
+        // own loads of this tile landed; after the barrier everybody's have, and everybody is done
+        // reading the other buffer (the tile before), which the next tile's loads may now fill
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        // ---- registers -> LDS ----
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int slot = swap_bits23(4 * krow + i);
-            *reinterpret_cast<uint4_t*>(&sK[slot * kKStride + kcol * 8]) = kr[i];
-        }
-        if (WITH_V) {
-            PackT<T> v0, v1, v2, v3;
-            v0.u = vr[0]; v1.u = vr[1]; v2.u = vr[2]; v3.u = vr[3];
-            const int kq = krow;   // keys 4*kq .. 4*kq+3
-#pragma unroll
-            for (int r = 0; r < 8; ++r) {
-                const int d = kcol * 8 + r;
-                const int sw = (r ^ kcol) & 7;    // = ((d & 7) ^ (d >> 3)) & 7
-                x4_t w = {v0.e[r], v1.e[r], v2.e[r], v3.e[r]};
-                *reinterpret_cast<x4_t*>(&sV[d * kVStride + (((kq >> 1) ^ sw) * 8) + (kq & 1) * 4]) = w;
-            }
-        }
-        __syncthreads();
-        if (sq + 1 < ntiles) {
-            issue_loads();
-            if (sq + 2 < ntiles) fetch_ids(tile_at(sq + 2));
-        }
+        // The next tile's loads go out between the products below, unconditionally: after the last
+        // tile they fetch its rows once more into the idle buffer (1/28 of the traffic on average,
+        // from the cache) rather than put a branch between the matrix instructions.
+        if (sq + 1 < ntiles) next_offsets();
+        const int nbuf = (sq + 1) & 1;
 
-        // ---- S^T = K_tile Q^T ----
+        // ---- S^T = K_tile Q^T.  Step c = (key block c / kKS, contraction step c % kKS); operands are
+        // read from LDS two windows (four steps) ahead of the products that use them, in program
+        // order, because LDS reads do not move across the load statements ----
+        constexpr int kSteps = nkb * kKS;
         float16_t sT[NQB][nkb];
         float16_t zero16;
 #pragma unroll
         for (int v = 0; v < 16; ++v) zero16[v] = 0.f;
+        auto read_a = [&](int c) {
+            return *reinterpret_cast<const x8_t*>(&bK[32 * (c / kKS) * D + krd + ((2 * (c % kKS)) ^ kx) * 8]);
+        };
+        x8_t aw[3][2];
 #pragma unroll
-        for (int kb = 0; kb < nkb; ++kb) {
+        for (int c = 0; c < 4 && c < kSteps; ++c) aw[c >> 1][c & 1] = read_a(c);
 #pragma unroll
-            for (int ks = 0; ks < kKS; ++ks) {
-                x8_t a = *reinterpret_cast<const x8_t*>(&sK[(32 * kb + li) * kKStride + ks * 16 + lg * 8]);
+        for (int w = 0; w < kSteps / 2; ++w) {
+            if (2 * w + 4 < kSteps) {
+                aw[(w + 2) % 3][0] = read_a(2 * w + 4);
+                aw[(w + 2) % 3][1] = read_a(2 * w + 5);
+            }
+            __builtin_amdgcn_sched_barrier(0);   // the scheduler would sink the reads to their use
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int kb = (2 * w + i) / kKS, ks = (2 * w + i) % kKS;
 #pragma unroll
                 for (int qb = 0; qb < NQB; ++qb)   // the first product starts from a constant zero
-                    sT[qb][kb] = Elem<T>::mma_32x32x16(a, qf[qb][ks], ks == 0 ? zero16 : sT[qb][kb]);
+                    sT[qb][kb] = Elem<T>::mma_32x32x16(aw[w % 3][i], qf[qb][ks], ks == 0 ? zero16 : sT[qb][kb]);
             }
+            if (w < kNumLoads) issue_load(w, nbuf);
         }
-        // ---- masks: accumulator v of key block kb is tile position 32kb + 16(v/8) + 8lg + v%8 ----
+#pragma unroll
+        for (int i = kSteps / 2; i < kNumLoads; ++i) issue_load(i, nbuf);
+        if (sq + 2 < ntiles) fetch_ids(tile_at(sq + 2));
+        // ---- masks: accumulator v of key block kb is tile position 32kb + 8(v/4) + 4lg + v%4 ----
         if (MODE != kFull) {
             if (MODE == kMasked && sparse) {   // a selection that ends inside this tile
 #pragma unroll
@@ -274,7 +336,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
                     for (int kb = 0; kb < nkb; ++kb)
 #pragma unroll
                         for (int v = 0; v < 16; ++v) {
-                            const int pos = ti * kKT + 32 * kb + 16 * (v >> 3) + 8 * lg + (v & 7);
+                            const int pos = ti * kKT + 32 * kb + 8 * (v >> 2) + 4 * lg + (v & 3);
                             if (pos >= n) sT[qb][kb][v] = -INFINITY;
                         }
             } else {                           // the causal edge and the end of the sequence
@@ -286,7 +348,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
                     for (int kb = 0; kb < nkb; ++kb)
 #pragma unroll
                         for (int v = 0; v < 16; ++v) {
-                            const int key = kstart + 32 * kb + 16 * (v >> 3) + 8 * lg + (v & 7);
+                            const int key = kstart + 32 * kb + 8 * (v >> 2) + 4 * lg + (v & 3);
                             if (key > q || key >= L) sT[qb][kb][v] = -INFINITY;
                         }
                 }
@@ -346,15 +408,34 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
             }
             l[qb] += sum;   // per-lane partial sum (own key positions)
         }
-        // ---- O^T += V^T P^T ----
+        // ---- O^T += V^T P^T: step s covers the keys of accumulators 8(s&1) .. 8(s&1)+7 of key block
+        // s/2, i.e. rows 16 s + 8 h + 4 lg + (0..3), h = 0, 1, of the tile.  The operands of a block
+        // of 32 output rows are read while the block before it is multiplied ----
         if (WITH_V) {
+            constexpr int kPS = 2 * nkb;
+            auto read_v = [&](int db, int s, int h) {
+                const int row = 16 * s + 8 * h;   // + vrow; only its low four bits enter swz
+                const T* vp = bV + row * D + vrd + ((4 * db + vchunk) ^ swz<D>(row + vrow)) * 8;
+                return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)vp);
+            };
+            short4_t av[2][kPS][2];
+#pragma unroll
+            for (int s = 0; s < kPS; ++s)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) av[0][s][h] = read_v(0, s, h);
 #pragma unroll
             for (int db = 0; db < kDB; ++db) {
-                const int d = 32 * db + li;
-                const int sw = ((d & 7) ^ (d >> 3)) & 7;
+                if (db + 1 < kDB) {
 #pragma unroll
-                for (int s = 0; s < 2 * nkb; ++s) {
-                    x8_t a = *reinterpret_cast<const x8_t*>(&sV[d * kVStride + (((2 * s + lg) ^ sw) * 8)]);
+                    for (int s = 0; s < kPS; ++s)
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) av[(db + 1) & 1][s][h] = read_v(db + 1, s, h);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int s = 0; s < kPS; ++s) {
+                    const short8_t both = __builtin_shufflevector(av[db & 1][s][0], av[db & 1][s][1], 0, 1, 2, 3, 4, 5, 6, 7);
+                    const x8_t a = __builtin_bit_cast(x8_t, both);
 #pragma unroll
                     for (int qb = 0; qb < NQB; ++qb)
                         oT[qb][db] = Elem<T>::mma_32x32x16(a, pf[qb][s], oT[qb][db]);
@@ -374,6 +455,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
         for (; sq < full_end; ++sq) run_tile(sq, std::integral_constant<int, kFull>{});
         for (; sq < ntiles; ++sq) run_tile(sq, std::integral_constant<int, kMasked>{});
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no load may land in LDS after the workgroup has left
 
     // ---- epilogue (rows are local to this call) ----
 #pragma unroll
@@ -401,12 +483,12 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
 
 
 // 32 queries per wavefront: register budget capped so that two workgroups share a
-// compute unit and hide each other's LDS staging and gather latency.
+// compute unit (64 KB of LDS each: two K and two V tile buffers).
 template <bool REUSE, bool WITH_V, bool PAGED, int D, typename T>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2)))
 void prefill_attn_kernel_q32(PrefillParams p) {
-    __shared__ __attribute__((aligned(16))) T sK[AttnTile<D>::kKT * AttnTile<D>::kKStride];
-    __shared__ __attribute__((aligned(16))) T sV[WITH_V ? D * AttnTile<D>::kVStride : 8];
+    __shared__ __attribute__((aligned(1024))) T sK[2 * AttnTile<D>::kTileElems];
+    __shared__ __attribute__((aligned(1024))) T sV[WITH_V ? 2 * AttnTile<D>::kTileElems : 8];
     prefill_attn_body<1, REUSE, WITH_V, PAGED, D, T>(p, sK, sV);
 }
 
@@ -417,7 +499,7 @@ void prefill_attn_kernel_q32(PrefillParams p) {
 template <int D, typename T>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2)))
 void prefill_attn_kernel_q64(PrefillParams p) {
-    __shared__ __attribute__((aligned(16))) T sK[AttnTile<D>::kKT * AttnTile<D>::kKStride];
+    __shared__ __attribute__((aligned(1024))) T sK[2 * AttnTile<D>::kTileElems];
     prefill_attn_body<2, false, false, false, D, T>(p, sK, static_cast<T*>(nullptr));
 }
 
@@ -438,9 +520,9 @@ void prefill_aggregate_kernel(PrefillParams p) {
 
     const int L = p.L;
     const int Lq = p.Lq;
-    const int t = p.T - 1 - (int)blockIdx.x;
-    const int g = blockIdx.y;
-    const int b = blockIdx.z;
+    int blk, g, b;
+    unit_of_workgroup(p.B, p.G, p.T, blk, g, b);
+    const int t = p.T - 1 - blk;
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
     const int lane = tid & 63;
@@ -569,7 +651,9 @@ template <int D, typename T>
 hipError_t launch_attn_t(const PrefillParams& p, bool reuse, bool with_v, int nqb, hipStream_t stream) {
     const int qt = 32 * nqb;
     const bool paged = p.block_table != nullptr;
-    dim3 grid((p.Lq + qt - 1) / qt, p.G, p.B), block(kThreads);
+    const int nqt = (p.Lq + qt - 1) / qt;
+    dim3 grid(nqt, p.G, p.B), block(kThreads);
+    if (pairs_fill_xcds(p.B, p.G)) grid = dim3((unsigned)((long long)nqt * p.G * p.B));
     if (paged) {
         if (reuse)
             hipLaunchKernelGGL((prefill_attn_kernel_q32<true, true, true, D, T>), grid, block, 0, stream, p);
@@ -593,6 +677,7 @@ hipError_t launch_attn_t(const PrefillParams& p, bool reuse, bool with_v, int nq
 template <int D, typename T>
 hipError_t launch_aggregate_t(const PrefillParams& p, hipStream_t stream) {
     dim3 grid(p.T, p.G, p.B), block(kThreads);
+    if (pairs_fill_xcds(p.B, p.G)) grid = dim3((unsigned)((long long)p.T * p.G * p.B));
     if (p.block_table)
         hipLaunchKernelGGL((prefill_aggregate_kernel<true, D, T>), grid, block, 0, stream, p);
     else
