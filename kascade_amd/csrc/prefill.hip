@@ -305,14 +305,15 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
         auto read_a = [&](int c) {
             return *reinterpret_cast<const x8_t*>(&bK[32 * (c / kKS) * D + krd + ((2 * (c % kKS)) ^ kx) * 8]);
         };
-        x8_t aw[3][2];
+        constexpr int kAhead = (kKB <= 2) ? 2 : 1;   // windows read ahead (registers are scarcer at D = 64)
+        x8_t aw[kAhead + 1][2];
 #pragma unroll
-        for (int c = 0; c < 4 && c < kSteps; ++c) aw[c >> 1][c & 1] = read_a(c);
+        for (int c = 0; c < 2 * kAhead && c < kSteps; ++c) aw[c >> 1][c & 1] = read_a(c);
 #pragma unroll
         for (int w = 0; w < kSteps / 2; ++w) {
-            if (2 * w + 4 < kSteps) {
-                aw[(w + 2) % 3][0] = read_a(2 * w + 4);
-                aw[(w + 2) % 3][1] = read_a(2 * w + 5);
+            if (2 * (w + kAhead) < kSteps) {
+                aw[(w + kAhead) % (kAhead + 1)][0] = read_a(2 * (w + kAhead));
+                aw[(w + kAhead) % (kAhead + 1)][1] = read_a(2 * (w + kAhead) + 1);
             }
             __builtin_amdgcn_sched_barrier(0);   // the scheduler would sink the reads to their use
 #pragma unroll
@@ -320,7 +321,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
                 const int kb = (2 * w + i) / kKS, ks = (2 * w + i) % kKS;
 #pragma unroll
                 for (int qb = 0; qb < NQB; ++qb)   // the first product starts from a constant zero
-                    sT[qb][kb] = Elem<T>::mma_32x32x16(aw[w % 3][i], qf[qb][ks], ks == 0 ? zero16 : sT[qb][kb]);
+                    sT[qb][kb] = Elem<T>::mma_32x32x16(aw[w % (kAhead + 1)][i], qf[qb][ks], ks == 0 ? zero16 : sT[qb][kb]);
             }
             if (w < kNumLoads) issue_load(w, nbuf);
         }
@@ -329,7 +330,8 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
         if (sq + 2 < ntiles) fetch_ids(tile_at(sq + 2));
         // ---- masks: accumulator v of key block kb is tile position 32kb + 8(v/4) + 4lg + v%4 ----
         if (MODE != kFull) {
-            if (MODE == kMasked && sparse) {   // a selection that ends inside this tile
+            const bool diag_here = MODE == kDiag || (sparse && ti == ng);
+            if (sparse && !diag_here) {   // a selection that ends inside this tile
 #pragma unroll
                 for (int qb = 0; qb < NQB; ++qb)
 #pragma unroll
@@ -340,7 +342,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
                             if (pos >= n) sT[qb][kb][v] = -INFINITY;
                         }
             } else {                           // the causal edge and the end of the sequence
-                const int kstart = (MODE == kDiag) ? q0 : ti * kKT;
+                const int kstart = diag_here ? q0 : ti * kKT;
 #pragma unroll
                 for (int qb = 0; qb < NQB; ++qb) {
                     const int q = q0 + 32 * qb + li;   // global position
@@ -418,23 +420,28 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
                 const T* vp = bV + row * D + vrd + ((4 * db + vchunk) ^ swz<D>(row + vrow)) * 8;
                 return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)vp);
             };
-            short4_t av[2][kPS][2];
+            // steps in groups of kGrp (a group = 2 kGrp transposing reads, kGrp products per query block)
+            constexpr int kGrp = (kKB <= 2) ? 4 : 2;
+            constexpr int kGroupsPV = kDB * kPS / kGrp;
+            short4_t av[2][kGrp][2];
 #pragma unroll
-            for (int s = 0; s < kPS; ++s)
+            for (int i = 0; i < kGrp; ++i)
 #pragma unroll
-                for (int h = 0; h < 2; ++h) av[0][s][h] = read_v(0, s, h);
+                for (int h = 0; h < 2; ++h) av[0][i][h] = read_v(i / kPS, i % kPS, h);
 #pragma unroll
-            for (int db = 0; db < kDB; ++db) {
-                if (db + 1 < kDB) {
+            for (int gq = 0; gq < kGroupsPV; ++gq) {
+                if (gq + 1 < kGroupsPV) {
 #pragma unroll
-                    for (int s = 0; s < kPS; ++s)
+                    for (int i = 0; i < kGrp; ++i)
 #pragma unroll
-                        for (int h = 0; h < 2; ++h) av[(db + 1) & 1][s][h] = read_v(db + 1, s, h);
+                        for (int h = 0; h < 2; ++h)
+                            av[(gq + 1) & 1][i][h] = read_v((kGrp * (gq + 1) + i) / kPS, (kGrp * (gq + 1) + i) % kPS, h);
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int s = 0; s < kPS; ++s) {
-                    const short8_t both = __builtin_shufflevector(av[db & 1][s][0], av[db & 1][s][1], 0, 1, 2, 3, 4, 5, 6, 7);
+                for (int i = 0; i < kGrp; ++i) {
+                    const int db = (kGrp * gq + i) / kPS, s = (kGrp * gq + i) % kPS;
+                    const short8_t both = __builtin_shufflevector(av[gq & 1][i][0], av[gq & 1][i][1], 0, 1, 2, 3, 4, 5, 6, 7);
                     const x8_t a = __builtin_bit_cast(x8_t, both);
 #pragma unroll
                     for (int qb = 0; qb < NQB; ++qb)
@@ -446,8 +453,9 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
 
     {
         int sq = 0;
-        if (REUSE && sparse) {
-            run_tile(0, std::integral_constant<int, kDiag>{});
+        if (REUSE && sparse) {   // a copy of its own where it halves the tile's products (64-key tiles)
+            if (kKB <= 2) run_tile(0, std::integral_constant<int, kDiag>{});
+            else run_tile(0, std::integral_constant<int, kMasked>{});
             sq = 1;
         }
         // tiles wholly below the unit's first query and inside the sequence / wholly inside the selection
