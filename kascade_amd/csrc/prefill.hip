@@ -515,15 +515,28 @@ void prefill_attn_kernel_q64(PrefillParams p) {
 // of exp2(s*scale - log_sum), for keys before the tile's first (global) position.
 // Two workgroups per compute unit (register budget 256): one wavefront's exponentials run
 // under the other's matrix instructions.
+//
+// A wavefront takes 32 keys of every 128-key tile and nobody else reads them.  Their rows go
+// from global memory straight into the wavefront's own LDS area (whole rows per load: read as
+// B operands directly, a 16-byte piece of 32 different rows per instruction, the same bytes kept
+// the data-return path of the memory pipeline busy 96 % of the kernel) and come back as B
+// operands (lane = key, 8 elements at d = 16 ks + 8 lg) from the chunk-permuted rows.  Two buffers
+// per wavefront, no barrier in the tile loop: the loads of the next tile are issued one per
+// contraction step and waited for at the top of that tile.
 template <bool PAGED, int D, typename T>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2)))
 void prefill_aggregate_kernel(PrefillParams p) {
     typedef typename Elem<T>::x8 x8_t;
     constexpr int kKS = D / 16;
+    constexpr int kChunks = D / 8;
+    constexpr int kRPL = 64 / kChunks;          // rows per load instruction
+    constexpr int kLoads = 32 / kRPL;           // load instructions per wavefront and tile
+    constexpr int kWaveElems = 32 * D;          // a wavefront's 32 rows
     constexpr float kScaleLog2 = ScaleLog2<D>::value;
     const int kvh = p.G, nheads = p.G * kGroupSize;
     const T* Qp = (const T*)p.Q;
     const T* Kp = (const T*)p.K;
+    __shared__ __attribute__((aligned(1024))) T sK[2 * 4 * kWaveElems];
     __shared__ __attribute__((aligned(16))) float s_lse[128];
 
     const int L = p.L;
@@ -564,67 +577,74 @@ void prefill_aggregate_kernel(PrefillParams p) {
             s_lse[tid] = (q < Lq) ? p.log_sum_in[((long long)b * Lq + q) * nheads + g * kGroupSize + (tid >> 5)]
                                   : INFINITY;
         }
-        // A wavefront takes 32 keys of every 128-key tile and nobody else reads them, so its B
-        // operands (lane li = key, 8 halves at d = 16 ks + 8 lg) come straight from global
-        // memory in the layout the matrix instruction wants: no LDS staging, no barriers in the
-        // tile loop.  The registers of operand ks are refilled with the next tile's data as soon
-        // as the products that read them have been issued, which leaves the rest of the tile
-        // (remaining products, exponentials) to cover the load latency.
-        const T* kbase = PAGED ? Kp + (long long)g * D + lg * 8
-                               : Kp + (long long)b * p.k_sb + (long long)g * p.k_sh + lg * 8;
+
+        // ---- staging: load j of a tile covers rows j kRPL + lrow of the wavefront's 32 ----
+        const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+        const int lrow = lane / kChunks;
+        const int lchunk = lane % kChunks;
+        const T* kbase = PAGED ? Kp + (long long)g * D : Kp + (long long)b * p.k_sb + (long long)g * p.k_sh;
+        const unsigned row_stride = PAGED ? (unsigned)(kvh * D) : (unsigned)p.k_sl;
         const int* bt_row = PAGED ? p.block_table + (long long)b * p.max_pages : nullptr;
         const int page_mask = (1 << p.page_shift) - 1;
-        auto key_of = [&](int ti) { return min(ti * kAggKT + 32 * wave + li, L - 1); };
-        auto row_ptr = [&](int ti, int pgv) {
-            const int key = key_of(ti);
-            return PAGED ? kbase + (long long)((pgv << p.page_shift) + (key & page_mask)) * (kvh * D)
-                         : kbase + (long long)key * p.k_sl;
+        const uint32_t lds_w = lds_address(sK) + wave_u * (kWaveElems * 2);   // + buf * 4 * kWaveElems * 2
+        const T* my_k = sK + wave * kWaveElems;
+        // block-table entry of the key this lane stands for (row lane & 31 of the wavefront's 32),
+        // fetched a tile ahead; the lanes of a load pick theirs up with a lane permutation
+        int pg_next = 0;
+        auto fetch_page = [&](int ti) {
+            if (PAGED) pg_next = bt_row[min(ti * kAggKT + 32 * wave + li, L - 1) >> p.page_shift];
         };
-        int pg_next = 0;    // block-table entry of this lane's key in the tile after the current one
-        int pg_after = 0;   // ... and in the one after that (fetched a tile ahead of its use)
-        if (PAGED) {
-            pg_next = bt_row[key_of(0) >> p.page_shift];
-            if (ntiles > 1) pg_after = bt_row[key_of(1) >> p.page_shift];
-        }
-        x8_t kb[kKS];
-        {
-            const T* rp = row_ptr(0, pg_next);
-#pragma unroll
-            for (int ks = 0; ks < kKS; ++ks) {
-                PackT<T> x;
-                x.u = ld_global_16(rp + ks * 16);
-                kb[ks] = x.v8;
-            }
-        }
-        __syncthreads();   // s_lse
-        for (int ti = 0; ti < ntiles; ++ti) {
-            const bool more = ti + 1 < ntiles;
+        int pg_cur = 0;   // entries of the tile whose loads are being issued
+        auto issue_load = [&](int ti, int j, int buf) {
+            const int row = j * kRPL + lrow;
+            const int key = min(ti * kAggKT + 32 * wave + row, L - 1);
+            int src = key;
             if (PAGED) {
-                pg_next = pg_after;
-                if (ti + 2 < ntiles) pg_after = bt_row[key_of(ti + 2) >> p.page_shift];
+                const int pgv = __builtin_amdgcn_ds_bpermute(row << 2, pg_cur);
+                src = (pgv << p.page_shift) + (key & page_mask);
             }
-            const T* rp = row_ptr(more ? ti + 1 : ti, pg_next);
+            const T* gp = kbase + (long long)((unsigned long long)(unsigned)src * row_stride) +
+                          (lchunk ^ swz<D>(row)) * 8;
+            load_to_lds_16(gp, lds_w + buf * (4 * kWaveElems * 2) + j * 1024);
+        };
+        fetch_page(0);
+        pg_cur = pg_next;
+#pragma unroll
+        for (int j = 0; j < kLoads; ++j) issue_load(0, j, 0);
+        if (ntiles > 1) fetch_page(1);
+        const int kx = lg ^ swz<D>(li);
+        __syncthreads();   // s_lse
+
+        for (int ti = 0; ti < ntiles; ++ti) {
+            // this tile's rows have landed (and the next tile's block-table entries arrived)
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            const T* bK = my_k + (ti & 1) * (4 * kWaveElems);
+            const int tn = min(ti + 1, ntiles - 1);   // after the last tile: its rows once more, unused
+            const int nbuf = (ti + 1) & 1;
+            pg_cur = pg_next;
+            if (ti + 2 < ntiles) fetch_page(ti + 2);
 
             float16_t acc[kGroupSize];
             float16_t zero16;   // the first product of a tile starts from a constant zero
 #pragma unroll
             for (int v = 0; v < 16; ++v) zero16[v] = 0.f;
+            auto read_b = [&](int ks) {
+                return *reinterpret_cast<const x8_t*>(&bK[li * D + ((2 * ks) ^ kx) * 8]);
+            };
+            x8_t kb[3];
+            kb[0] = read_b(0);
+            if (kKS > 1) kb[1] = read_b(1);
 #pragma unroll
             for (int ks = 0; ks < kKS; ++ks) {
+                if (ks + 2 < kKS) kb[(ks + 2) % 3] = read_b(ks + 2);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int rb = 0; rb < kGroupSize; ++rb)
-                    acc[rb] = Elem<T>::mma_32x32x16(qa[rb][ks], kb[ks], ks == 0 ? zero16 : acc[rb]);
-                if (more) {
-                    // the refill must stay behind the products that read the old contents, or
-                    // the compiler hoists all eight loads and needs a second set of registers:
-                    // its address is made to depend on the last product of this step
-                    long long off = ks * 16;
-                    asm volatile("" : "+v"(off) : "v"(acc[kGroupSize - 1][0]));
-                    PackT<T> x;
-                    x.u = ld_global_16(rp + off);
-                    kb[ks] = x.v8;
-                }
+                    acc[rb] = Elem<T>::mma_32x32x16(qa[rb][ks], kb[ks % 3], ks == 0 ? zero16 : acc[rb]);
+                if (ks < kLoads) issue_load(tn, ks, nbuf);
             }
+#pragma unroll
+            for (int j = kKS; j < kLoads; ++j) issue_load(tn, j, nbuf);
             // accumulator v of row block rb is query row 8(v/4) + 4lg + v%4, column = key li
             float sum = 0.f;
 #pragma unroll
@@ -636,7 +656,7 @@ void prefill_aggregate_kernel(PrefillParams p) {
                     for (int e = 0; e < 4; ++e)
                         sum += fast_exp2(acc[rb][4 * v4 + e] * kScaleLog2 - ls[e]);
                 }
-            sum += __shfl_xor(sum, 32);
+            sum = sum_with_other_half(sum);
             const int key = ti * kAggKT + 32 * wave + li;
             if (lg == 0 && key < L) {
                 if (key < ts)
@@ -645,6 +665,7 @@ void prefill_aggregate_kernel(PrefillParams p) {
                     out[key] = neg_inf;
             }
         }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no load may land in LDS after the workgroup has left
     }
     if (p.fill_invalid) {
         for (int key = ntiles * kAggKT + tid; key < L; key += kThreads) out[key] = neg_inf;
