@@ -145,16 +145,24 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
         }
     }
     const int ntiles = sparse ? ng + 1 : (min(q0 + QT, L) + kKT - 1) / kKT;
+    const bool idx_vec = REUSE && (p.max_topk & 3) == 0 && (reinterpret_cast<uintptr_t>(p.idx) & 15) == 0;
 
     // ---- tile staging: wavefront w fills rows [4w R, 4(w+1) R) of a tile with four loads of R rows
     // each (R = 4 at D = 128, 8 at D = 64); lane = (row within the load, chunk position) ----
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     const int lrow = lane / kChunks;
     const int lchunk = lane % kChunks;
-    const int pos0 = wave * 4 * kRPL + lrow;     // this lane's rows: tile positions pos0 + j R, j = 0..3
+    // This lane's four rows sit at LDS rows slot0 + j R (j = load) and hold the four consecutive
+    // tile positions pos0 + j: one 16-byte load brings their four indices, one block-table entry
+    // covers their page, and the rows of a tile in LDS are a permutation of its keys -- which only
+    // the masks need to know (both products contract over the same order).
+    const int slot0 = wave * 4 * kRPL + lrow;
+    const int pos0 = 4 * (wave * kRPL + lrow);
     int coff[4];                                 // element offset of the chunk this lane fetches for row j
 #pragma unroll
-    for (int j = 0; j < 4; ++j) coff[j] = (lchunk ^ swz<D>(pos0 + j * kRPL)) * 8;
+    for (int j = 0; j < 4; ++j) coff[j] = (lchunk ^ swz<D>(slot0 + j * kRPL)) * 8;
+    // tile position of LDS row `slot`
+    auto pos_of_slot = [](int slot) { return 4 * ((slot / (4 * kRPL)) * kRPL + slot % kRPL) + (slot / kRPL) % 4; };
     const T* kbase = PAGED ? Kp + (long long)g * D : Kp + (long long)b * p.k_sb + (long long)g * p.k_sh;
     const T* vbase = PAGED ? Vp + (long long)g * D : Vp + (long long)b * p.k_sb + (long long)g * p.k_sh;
     const int* bt_row = PAGED ? p.block_table + (long long)b * p.max_pages : nullptr;
@@ -176,12 +184,17 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
     const unsigned row_stride = PAGED ? (unsigned)(kvh * D) : (unsigned)p.k_sl;   // host checks < 2^31
     auto fetch_ids = [&](int ti) {
         pend_ti = ti;
-        if (sparse && ti < ng) {
+        if (sparse && ti < ng) {   // values are bounded at use
+            if (idx_vec) {   // list length and n are multiples of four: a group lies inside the list or outside
+                const int4_t v = *reinterpret_cast<const int4_t*>(idx_row + min(ti * kKT + pos0, n - 4));
 #pragma unroll
-            for (int j = 0; j < 4; ++j) ids[j] = idx_row[min(ti * kKT + pos0 + j * kRPL, n - 1)];   // bounded at use
-        } else if (PAGED) {
+                for (int j = 0; j < 4; ++j) ids[j] = v[j];
+            } else {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) ids[j] = bt_row[tile_key(ti, pos0 + j * kRPL) >> p.page_shift];
+                for (int j = 0; j < 4; ++j) ids[j] = idx_row[min(ti * kKT + pos0 + j, n - 1)];
+            }
+        } else if (PAGED) {   // four consecutive keys from a multiple of four on: one page
+            ids[0] = bt_row[tile_key(ti, pos0) >> p.page_shift];
         }
     };
     // Row addresses of the tile whose ids are held (element offsets from kbase / vbase).  The
@@ -199,8 +212,8 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
         } else {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const int key = tile_key(pend_ti, pos0 + j * kRPL);
-                const int row = PAGED ? (ids[j] << p.page_shift) + (key & page_mask) : key;
+                const int key = tile_key(pend_ti, pos0 + j);
+                const int row = PAGED ? (ids[0] << p.page_shift) + (key & page_mask) : key;
                 off[j] = (long long)((unsigned long long)(unsigned)row * row_stride) + coff[j];
             }
         }
@@ -328,7 +341,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
 #pragma unroll
         for (int i = kSteps / 2; i < kNumLoads; ++i) issue_load(i, nbuf);
         if (sq + 2 < ntiles) fetch_ids(tile_at(sq + 2));
-        // ---- masks: accumulator v of key block kb is tile position 32kb + 8(v/4) + 4lg + v%4 ----
+        // ---- masks: accumulator v of key block kb is LDS row 32kb + 8(v/4) + 4lg + v%4 of the tile ----
         if (MODE != kFull) {
             const bool diag_here = MODE == kDiag || (sparse && ti == ng);
             if (sparse && !diag_here) {   // a selection that ends inside this tile
@@ -338,7 +351,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
                     for (int kb = 0; kb < nkb; ++kb)
 #pragma unroll
                         for (int v = 0; v < 16; ++v) {
-                            const int pos = ti * kKT + 32 * kb + 8 * (v >> 2) + 4 * lg + (v & 3);
+                            const int pos = ti * kKT + pos_of_slot(32 * kb + 8 * (v >> 2) + 4 * lg + (v & 3));
                             if (pos >= n) sT[qb][kb][v] = -INFINITY;
                         }
             } else {                           // the causal edge and the end of the sequence
@@ -350,7 +363,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
                     for (int kb = 0; kb < nkb; ++kb)
 #pragma unroll
                         for (int v = 0; v < 16; ++v) {
-                            const int key = kstart + 32 * kb + 8 * (v >> 2) + 4 * lg + (v & 3);
+                            const int key = kstart + pos_of_slot(32 * kb + 8 * (v >> 2) + 4 * lg + (v & 3));
                             if (key > q || key >= L) sT[qb][kb][v] = -INFINITY;
                         }
                 }
