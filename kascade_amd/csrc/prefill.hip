@@ -478,25 +478,37 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no load may land in LDS after the workgroup has left
 
-    // ---- epilogue (rows are local to this call) ----
+    // ---- epilogue (rows are local to this call).  A lane holds one query's output spread over its
+    // registers; the rows go through the wavefront's share of the (now idle) K buffers so that they
+    // leave as whole rows: 16-byte stores, four rows per instruction ----
+    static_assert(!WITH_V || NQB == 1, "the output pass is written for 32 queries per wavefront");
+    if (WITH_V) __syncthreads();   // everybody is done with the tile buffers
 #pragma unroll
     for (int qb = 0; qb < NQB; ++qb) {
         const int ql = q0l + 32 * qb + li;
         const float lt = sum_with_other_half(l[qb]);
-        if (ql < Lq) {
-            if (p.log_sum && lg == 0)
-                p.log_sum[((long long)b * Lq + ql) * nheads + head] = fast_log2(lt) + m[qb];
-            if (WITH_V) {
-                const float inv = 1.f / lt;
-                T* op = (T*)p.O + (((long long)b * Lq + ql) * nheads + head) * D;
+        if (p.log_sum && lg == 0 && ql < Lq)
+            p.log_sum[((long long)b * Lq + ql) * nheads + head] = fast_log2(lt) + m[qb];
+        if (WITH_V) {
+            T* so = sK + wave * (32 * D);
+            const float inv = 1.f / lt;
 #pragma unroll
-                for (int db = 0; db < kDB; ++db)
+            for (int db = 0; db < kDB; ++db)
 #pragma unroll
-                    for (int v4 = 0; v4 < 4; ++v4) {
-                        x4_t o = {(T)(oT[qb][db][4 * v4 + 0] * inv), (T)(oT[qb][db][4 * v4 + 1] * inv),
-                                  (T)(oT[qb][db][4 * v4 + 2] * inv), (T)(oT[qb][db][4 * v4 + 3] * inv)};
-                        *reinterpret_cast<x4_t*>(op + 32 * db + 8 * v4 + 4 * lg) = o;
-                    }
+                for (int v4 = 0; v4 < 4; ++v4) {   // d = 32 db + 8 v4 + 4 lg .. +3: chunk 4 db + v4 of row li
+                    x4_t o = {(T)(oT[qb][db][4 * v4 + 0] * inv), (T)(oT[qb][db][4 * v4 + 1] * inv),
+                              (T)(oT[qb][db][4 * v4 + 2] * inv), (T)(oT[qb][db][4 * v4 + 3] * inv)};
+                    *reinterpret_cast<x4_t*>(&so[li * D + (((4 * db + v4) ^ (li & (kChunks - 1))) * 8) + 4 * lg]) = o;
+                }
+            __builtin_amdgcn_wave_barrier();   // the reads below are other lanes' writes (same wavefront: in order)
+#pragma unroll
+            for (int j = 0; j < 32 / kRPL; ++j) {
+                const int r = j * kRPL + lrow;
+                const uint4_t row = *reinterpret_cast<const uint4_t*>(&so[r * D + lchunk * 8]);
+                const int qr = q0l + r;
+                if (qr < Lq)
+                    *reinterpret_cast<uint4_t*>((T*)p.O + (((long long)b * Lq + qr) * nheads + head) * D +
+                                                ((lchunk ^ (r & (kChunks - 1))) * 8)) = row;
             }
         }
     }
