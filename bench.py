@@ -80,7 +80,8 @@ def make_prefill_sets(L, dev):
 
 
 SINGLE_KERNELS = ("membw_copy", "prefill_dense", "prefill_scores", "prefill_aggregate", "prefill_topk", "prefill_reuse",
-                  "decode_dense", "decode_anchor0", "decode_anchor", "decode_topk", "decode_reuse", "rope_append")
+                  "decode_dense", "decode_anchor0", "decode_anchor", "decode_topk", "decode_reuse", "rope_append",
+                  "stack_decode")
 
 
 def run_single_kernel(name, iters, seq_len, dev, head_map, decode_len=65536):
@@ -118,6 +119,28 @@ def run_single_kernel(name, iters, seq_len, dev, head_map, decode_len=65536):
                                       wq, wq, 1e-6, out=out)
         torch.cuda.synchronize()
         print(json.dumps({"kernel": name, "iters": iters}), flush=True)
+        return
+    if name == "stack_decode":
+        # config 4's decode side: 36 layers over a 16384-token paged cache (random contents), the
+        # step captured as one HIP graph and replayed `iters` times with fresh inputs
+        from kascade_amd.stack import KascadeAttentionStack
+        n_layers, anchors, prompt = 36, [0, 2, 8, 13, 14], 16384
+        maps = [list(range(G)) if l in anchors else workloads.random_head_mapping(500 + l) for l in range(n_layers)]
+        st = KascadeAttentionStack(n_layers, anchors, maps, PCT, prompt + max(iters, 1) + 8, batch=1, page_size=16,
+                                   rolling_prefill=True, device=dev, table_seed=2)
+        for l in range(n_layers):
+            st.k_pages[l].normal_()
+            st.v_pages[l].normal_()
+        st.reset(prompt)
+        st.capture_decode()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            st.graph_q.normal_(); st.graph_k.normal_(); st.graph_v.normal_()
+            st.replay_decode()
+        torch.cuda.synchronize()
+        print(json.dumps({"kernel": name, "iters": iters, "layers": n_layers,
+                          "us_per_step_wall": round((time.perf_counter() - t0) / max(iters, 1) * 1e6, 1)}), flush=True)
         return
     if name.startswith("prefill"):
         # the named kernel on config 1, every call on the next of the rotating input sets
