@@ -109,6 +109,23 @@ def test_prefill_reuse(cuda, B, L, p, peaked, rolling):
     assert torch.equal(got_id.cpu(), got.cpu())
 
 
+@pytest.mark.parametrize("width", [130, 200, 321])
+def test_prefill_reuse_list_width_not_a_tile_multiple(cuda, width):
+    """Index rows whose length is no multiple of the key tile (the selection ends inside a tile)
+    and, for odd lengths, no multiple of four either (the rows are then read entry by entry)."""
+    from kascade_amd import kernels
+    L, p = 1500, 10
+    w = _inputs(1, L, seed=7, peaked=True)
+    pooled = orc.pooled_prefill_scores(w.q, w.k, TILE)
+    idx = orc.topk_rows(pooled, 384)[..., :width].contiguous()
+    want = orc.reuse_prefill(w.q_reuse, w.k_reuse, w.v, idx, w.head_mapping, TILE, False, p)
+    hm = torch.tensor(w.head_mapping, dtype=torch.int32, device=cuda)
+    got = kernels.prefill_reuse(w.q_reuse.to(cuda), w.k_reuse.to(cuda), w.v.to(cuda), idx.to(cuda), hm,
+                                float(p), False)
+    torch.cuda.synchronize()
+    assert_close(got, want, f"reuse prefill, list width {width}")
+
+
 def test_prefill_reuse_dense_fallback(cuda):
     """Budget >= tile start for every tile: the result is dense causal attention."""
     from kascade_amd import kernels
