@@ -392,18 +392,19 @@ def main():
     del w, sets
     torch.cuda.empty_cache()
 
-    # ---- longer prompts (the reference publishes 65536 and 131072 on H100: dense FA3 53.77 / 215.76 ms,
-    # Kascade 24.63 / 98.55 ms): the same layer kinds through the strategy; beyond 65536 tokens the
-    # anchors pool and select 512 tiles at a time
+    # ---- longer prompts (the reference publishes 65536, 131072 and 262144 on H100: dense FA3 53.77 /
+    # 215.76 / 864.02 ms, Kascade 24.63 / 98.55 / 408.30 ms): the same layer kinds through the strategy;
+    # beyond 65536 tokens the anchors pool and select 512 tiles at a time
     prefill_long = {}
     if not args.decode_only and not args.skip_long:
-        for Ll in (65536, 131072):
+        for Ll in (65536, 131072, 262144):
             log(f"[bench] prefill L={Ll}")
             a = workloads.prefill_inputs(1, Ll, seed=7, device=dev)
             wl = budgets.topk_width(Ll, PCT)
-            t_d = ev_time(lambda: kernels.prefill_dense(a.q, a.k, a.v), n=2)
-            t_a0 = ev_time(lambda: strat._prefill_recomp_forward(a.q, a.k, a.v, wl, TILE, 0, PCT), n=2)
-            t_a = ev_time(lambda: strat._prefill_recomp_forward(a.q, a.k, a.v, wl, TILE, 2, PCT), n=2)
+            nl = 1 if Ll > 131072 else 2     # a layer takes up to a second at 262144
+            t_d = ev_time(lambda: kernels.prefill_dense(a.q, a.k, a.v), n=nl)
+            t_a0 = ev_time(lambda: strat._prefill_recomp_forward(a.q, a.k, a.v, wl, TILE, 0, PCT), n=nl)
+            t_a = ev_time(lambda: strat._prefill_recomp_forward(a.q, a.k, a.v, wl, TILE, 2, PCT), n=nl)
             t_r = ev_time(lambda: strat._prefill_reuse_forward(a.q_reuse, a.k_reuse, a.v, PCT, 1), n=3)
             kas = (t_a0 + 4 * t_a + 27 * t_r) / 32
             prefill_long[str(Ll)] = {"dense_ms": round(t_d / 1e3, 2), "anchor0_ms": round(t_a0 / 1e3, 2),

@@ -295,9 +295,9 @@ def test_config4_stack_36_layers_prefill_and_256_replayed_decode_steps(cuda):
     assert int(graph.seqlens[0]) == n_tok == graph.length
 
 
-@pytest.mark.parametrize("L", [65536, 131072])
+@pytest.mark.parametrize("L", [65536, 131072, 262144])
 def test_prefill_beyond_32k(cuda, L):
-    """Prompts of 65536 and 131072 tokens (the reference publishes both): an anchor layer > 0
+    """Prompts of 65536, 131072 and 262144 tokens (the reference publishes all three): an anchor layer > 0
     through the strategy -- at 131072 pooled and selected 512 tiles at a time, rows longer than
     65536 entries on the multi-workgroup selection -- and a reuse layer through a head map, against
     the oracle on sampled tiles; every tile's selection against the kernel's own pooled scores on
@@ -308,7 +308,7 @@ def test_prefill_beyond_32k(cuda, L):
     w = workloads.prefill_inputs(1, L, seed=6, device=cuda)
     hm = [list(range(G)), w.head_mapping]
     K = budgets.topk_width(L, P)
-    assert K == {65536: 6656, 131072: 13184}[L]
+    assert K == {65536: 6656, 131072: 13184, 262144: 26240}[L]
     s = EfficientKascadeStrategy([0], None, k=P, tile_size=TILE, rolling_prefill=True, head_mapping=hm, register=False)
     o_anchor = s._prefill_recomp_forward(w.q, w.k, w.v, K, TILE, 1, P)         # anchor > 0: own indices, sparse pass
     idx = s._topk_to_reuse
