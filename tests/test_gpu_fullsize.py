@@ -207,7 +207,7 @@ def test_config4_chunked_prefill_16384_equals_whole_prompt(cuda):
 
 
 def test_config4_stack_36_layers_prefill_and_256_replayed_decode_steps(cuda):
-    """BASELINE config 4 at its real size: 36 layers, anchors {0,2,8,13,14}, a 16384-token prompt
+    """The largest benchmark configuration at its real size: 36 layers, anchors {0,2,8,13,14}, a 16384-token prompt
     in 8 chunks of 2048 over the paged cache, then 256 decode steps, eager on one stack and
     replayed from a captured HIP graph on another.  Every replayed step equals the eager step
     bit for bit; at steps 0, 127 and 255 layer 0, anchor 8 and reuse layers 9 and 20 are checked

@@ -1,5 +1,5 @@
 """Other tensor shapes than the reference's (32 query / 8 KV heads, head_dim 128, fp16): bf16,
-head_dim 64, other KV-head counts -- in particular BASELINE config 0's shape (8 query / 2 KV
+head_dim 64, other KV-head counts -- in particular the shape of the reference's CPU-runnable configuration (8 query / 2 KV
 heads, head_dim 64) -- through the shaped C entry points, against the CPU oracle.
 
 Tolerances.  fp16: the parity tolerances of every other test (outputs atol 2e-3 / rtol 1e-2,
@@ -159,7 +159,7 @@ def test_decode_other_shapes(cuda, H, G, D, dt):
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
 def test_config0_shape_through_the_strategy(cuda, dt):
-    """BASELINE config 0's shape and sizes (batch 1, 8 query / 2 KV heads, head_dim 64, 2048
+    """The reference's CPU-runnable configuration, shape and sizes (batch 1, 8 query / 2 KV heads, head_dim 64, 2048
     tokens, identity head map, anchor layer 0 then a correlated reuse layer) through
     EfficientKascadeStrategy.attention_forward in the HF layout, prefill and one decode step."""
     from kascade_amd.strategy import EfficientKascadeStrategy

@@ -382,7 +382,7 @@ def test_head_mapping_fixtures():
 
 # ------------------------------------------------------------ config 0 (CPU plumbing run)
 def test_config0_cpu_plumbing_run():
-    """BASELINE config 0 in full on the strategy-semantics oracle: batch 1, 8 q-heads / 2 KV heads,
+    """The CPU-runnable configuration of the reference in full on the strategy-semantics oracle: batch 1, 8 q-heads / 2 KV heads,
     head_dim 64, causal prefill of 2048 tokens in fp32, tile 32, top-k 10 %, identity head map,
     N(0,1) inputs from seed 0, reuse layer = anchor + 0.3 N(0,1).  Layer 0 must be dense attention
     (SDPA), the reuse layer the masked softmax over (stored indices U in-tile diagonal) on
