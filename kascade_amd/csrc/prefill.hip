@@ -38,8 +38,8 @@ constexpr int kThreads = 256;
 constexpr int kAggKT = 128;        // keys per tile (aggregate kernel)
 
 // Tile geometry of the attention kernel per head dimension.  A tile is 16 KB of K (and of V)
-// whatever D: 64 keys at D = 128, 128 keys at D = 64, so a thread always stages four consecutive
-// keys of one 16-byte column, both products issue 16 matrix instructions per tile and wavefront,
+// whatever D: 64 keys at D = 128, 128 keys at D = 64, so a wavefront always stages a tile with
+// four 1 KB loads per tensor, both products issue 16 matrix instructions per tile and wavefront,
 // and the score registers a narrower head frees hold the extra keys.
 template <int D> struct AttnTile {
     static constexpr int kKT = 64 * 128 / D;     // keys per tile
