@@ -15,7 +15,7 @@ H, G, D, TILE = 32, 8, 128, 32
 PAGE = 16
 
 
-def _paged_cache(B, L, seed, device):
+def _paged_cache(B, L, seed, device, PAGE=PAGE):
     """Empty cache with a shuffled block table [B, ceil(L/PAGE)] and spare pages."""
     n_pages = B * math.ceil(L / PAGE)
     gen = torch.Generator().manual_seed(seed)
@@ -30,9 +30,10 @@ def _chunks(L, size):
     return [(s, min(size, L - s)) for s in range(0, L, size)]
 
 
-@pytest.mark.parametrize("B,L,chunk,p,rolling", [(1, 1536, 512, 10, True), (2, 1500, 512, 20, True),
-                                                 (1, 1100, 352, 10, False)])
-def test_chunked_kernels_equal_whole_prompt(cuda, B, L, chunk, p, rolling):
+@pytest.mark.parametrize("B,L,chunk,p,rolling,PAGE", [(1, 1536, 512, 10, True, 16), (2, 1500, 512, 20, True, 16),
+                                                      (1, 1100, 352, 10, False, 16), (1, 1300, 416, 10, True, 4),
+                                                      (2, 1200, 512, 10, True, 64), (1, 1000, 320, 20, True, 256)])
+def test_chunked_kernels_equal_whole_prompt(cuda, B, L, chunk, p, rolling, PAGE):
     from kascade_amd import kernels, budgets, workloads
     w = workloads.prefill_inputs(B, L, seed=L + chunk, device="cpu", peaked=True)
     q, k, v = w.q.to(cuda), w.k.to(cuda), w.v.to(cuda)
@@ -50,8 +51,8 @@ def test_chunked_kernels_equal_whole_prompt(cuda, B, L, chunk, p, rolling):
                                    n_sel=torch.tensor(nsel, dtype=torch.int32, device=cuda))
     reuse_all = kernels.prefill_reuse(qr, kr, v, idx_all, hm, float(p), rolling)
 
-    kp, vp, bt = _paged_cache(B, L, seed=3, device=cuda)        # anchor layer's cache
-    kp2, vp2, _ = _paged_cache(B, L, seed=3, device=cuda)       # reuse layer's cache (same table)
+    kp, vp, bt = _paged_cache(B, L, seed=3, device=cuda, PAGE=PAGE)        # anchor layer's cache
+    kp2, vp2, _ = _paged_cache(B, L, seed=3, device=cuda, PAGE=PAGE)       # reuse layer's cache (same table)
     for q_start, Lq in _chunks(L, chunk):
         sl = slice(q_start, q_start + Lq)
         Lk = q_start + Lq
