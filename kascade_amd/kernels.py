@@ -40,15 +40,31 @@ def _shape(Q: torch.Tensor, K: torch.Tensor):
     return Hq, Gk, Dh, Q.dtype
 
 
+_entry = {}     # (name, shaped) -> bound library function: attribute look-ups are per-call cost
+
+
 def _call(lib, name: str, shape, *args):
     """The plain entry point for the reference's shape, its *_shaped_call twin otherwise."""
     _, Gk, Dh, dt = shape
-    if (Gk, Dh, dt) == (G, D, torch.float16):
-        return getattr(lib, f"kascade_{name}_call")(*args)
-    return getattr(lib, f"kascade_{name}_shaped_call")(ctypes.byref(_lib.Shape(Gk, Dh, _ELEM[dt])), *args)
+    if Gk == G and Dh == D and dt is torch.float16:
+        fn = _entry.get((name, False))
+        if fn is None:
+            fn = _entry[(name, False)] = getattr(lib, f"kascade_{name}_call")
+        return fn(*args)
+    fn = _entry.get((name, True))
+    if fn is None:
+        fn = _entry[(name, True)] = getattr(lib, f"kascade_{name}_shaped_call")
+    return fn(ctypes.byref(_lib.Shape(Gk, Dh, _ELEM[dt])), *args)
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
 def _stream() -> int:
+    """Handle of the current stream of the current device.  The raw accessor skips the stream
+    object torch.cuda.current_stream() builds (several microseconds per kernel call)."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -57,12 +73,13 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
 
 
 def _req(t: torch.Tensor, dtype, name: str, contiguous: bool = True):
+    if t.is_cuda and t.dtype is dtype and (not contiguous or t.is_contiguous()):
+        return
     if not t.is_cuda:
         raise KascadeError(f"{name} must be a device tensor")
     if t.dtype != dtype:
         raise KascadeError(f"{name} must be {dtype}, got {t.dtype}")
-    if contiguous and not t.is_contiguous():
-        raise KascadeError(f"{name} must be contiguous")
+    raise KascadeError(f"{name} must be contiguous")
 
 
 def _blhd_strides(t: torch.Tensor, name: str) -> Strides:

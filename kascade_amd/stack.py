@@ -101,15 +101,17 @@ class KascadeAttentionStack:
         # one bookkeeping launch (lengths + 1, anchor budgets), then one attention launch sequence
         # per layer; the first launch of a layer also writes the new token's K/V into the cache
         self.decoder.begin_step(self.seqlens, 1)
+        # one unbind per tensor instead of several index operations per layer (host time)
+        qs, outs = q.unbind(0), out.unbind(0)
+        kns, vns = k_new[:, :, 0].unbind(0), v_new[:, :, 0].unbind(0)
         for l in range(self.num_layers):
-            kn, vn = k_new[l][:, 0], v_new[l][:, 0]
             if self.dense_only:
-                self.decoder.dense(q[l], self.k_pages[l], self.v_pages[l], self.block_table, self.seqlens,
-                                   self.max_seqlen, out=out[l], k_new=kn, v_new=vn)
+                self.decoder.dense(qs[l], self.k_pages[l], self.v_pages[l], self.block_table, self.seqlens,
+                                   self.max_seqlen, out=outs[l], k_new=kns[l], v_new=vns[l])
             else:
-                self.decoder.forward(l, q[l], self.k_pages[l], self.v_pages[l], self.block_table,
-                                     self.seqlens, self.max_seqlen, ragged=True, out=out[l],
-                                     k_new=kn, v_new=vn)
+                self.decoder.forward(l, qs[l], self.k_pages[l], self.v_pages[l], self.block_table,
+                                     self.seqlens, self.max_seqlen, ragged=True, out=outs[l],
+                                     k_new=kns[l], v_new=vns[l])
 
     def decode_step(self, q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor,
                     out: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -275,6 +275,7 @@ class PagedKascadeDecoder:
         self._part = torch.empty(max_batch * H * ns * D, device=dev, dtype=torch.float32)
         self._row_sums = torch.empty(max_batch, H, device=dev, dtype=torch.float32)
         self._scores = torch.empty(max_batch * H * self.stride, device=dev, dtype=torch.float32)
+        self._scratch_views = {}
         self._hm = {None: torch.arange(G, device=dev, dtype=torch.int32)}
         for l, row in enumerate(head_mapping):
             self._hm[l] = torch.tensor(row, device=dev, dtype=torch.int32)
@@ -294,7 +295,11 @@ class PagedKascadeDecoder:
         self._sync_reuse = self._sync if self.ns_reuse <= FUSED_MERGE_MAX_SPLITS else None
 
     def _scratch(self, B, ns):
-        return self._glse[:B * H * ns].view(B, H, ns), self._part[:B * H * ns * D].view(B, H, ns, D)
+        views = self._scratch_views.get((B, ns))
+        if views is None:   # a view costs a microsecond or two of host time per layer call
+            views = self._scratch_views[(B, ns)] = (self._glse[:B * H * ns].view(B, H, ns),
+                                                    self._part[:B * H * ns * D].view(B, H, ns, D))
+        return views
 
     def dense(self, q, k_pages, v_pages, block_table, seqlens, max_len: int, out=None,
               k_new=None, v_new=None):
