@@ -707,7 +707,11 @@ hipError_t launch_attn_t(const PrefillParams& p, bool reuse, bool with_v, int nq
     const bool paged = p.block_table != nullptr;
     const int nqt = (p.Lq + qt - 1) / qt;
     dim3 grid(nqt, p.G, p.B), block(kThreads);
-    if (pairs_fill_xcds(p.B, p.G)) grid = dim3((unsigned)((long long)nqt * p.G * p.B));
+    if (pairs_fill_xcds(p.B, p.G)) {
+        const long long total = (long long)nqt * p.G * p.B;
+        if (total > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+        grid = dim3((unsigned)total);
+    }
     if (paged) {
         if (reuse)
             hipLaunchKernelGGL((prefill_attn_kernel_q32<true, true, true, D, T>), grid, block, 0, stream, p);
@@ -731,7 +735,11 @@ hipError_t launch_attn_t(const PrefillParams& p, bool reuse, bool with_v, int nq
 template <int D, typename T>
 hipError_t launch_aggregate_t(const PrefillParams& p, hipStream_t stream) {
     dim3 grid(p.T, p.G, p.B), block(kThreads);
-    if (pairs_fill_xcds(p.B, p.G)) grid = dim3((unsigned)((long long)p.T * p.G * p.B));
+    if (pairs_fill_xcds(p.B, p.G)) {
+        const long long total = (long long)p.T * p.G * p.B;
+        if (total > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+        grid = dim3((unsigned)total);
+    }
     if (p.block_table)
         hipLaunchKernelGGL((prefill_aggregate_kernel<true, D, T>), grid, block, 0, stream, p);
     else
