@@ -224,7 +224,8 @@ __global__ __launch_bounds__(kThreads) void topk_select_kernel(
 //  * The compaction computes every (chunk, thread) offset with two barriers in all (per-chunk
 //    wavefront scans, then one scan over the chunk x wavefront totals), and stages the selected
 //    indices in LDS in their final order, so that the row's list leaves as full-width stores.
-// Rows must be 16-byte aligned and at most MAXC*8192 entries long.
+// Rows must be 16-byte aligned and at most MAXC*8192 entries long (MAXC = 16: 131072 entries, 64
+// registers of row data per thread, still one workgroup of 1024 threads per CU).
 template <int MAXC>
 __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
     const uint16_t* __restrict__ scores, int* __restrict__ out, long long row_stride,
@@ -235,7 +236,9 @@ __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
     __shared__ uint32_t s_hist[kBins1 * kCopies];
     __shared__ uint32_t s_hist2[32];
     __shared__ uint32_t s_wave[kWaves];
-    __shared__ uint32_t s_tot[MAXC * kWaves];      // pass 3: totals, then exclusive prefixes
+    __shared__ uint32_t s_tot[MAXC * kWaves];      // pass 3: totals per (chunk, wavefront), packed
+    __shared__ uint32_t s_pgt[MAXC * kWaves];      // pass 3: exclusive prefixes of the counts above T
+    __shared__ uint32_t s_peq[MAXC * kWaves];      // ... and of the counts equal to T
     __shared__ uint32_t s_zero[64];                // pass 1: where the zeros' idle atomics go
     __shared__ uint32_t s_sel[4];  // b1, cum_above, T, r
 
@@ -412,20 +415,24 @@ __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
     }
     __syncthreads();
     if (wave == 0) {
-        // exclusive prefix over the MAXC*16 (chunk, wavefront) totals, chunk-major, 64 per step;
-        // an exclusive prefix of either half stays below 65536 (a row has at most 65536 entries)
-        uint32_t carry = 0;
+        // exclusive prefixes over the MAXC*16 (chunk, wavefront) totals, chunk-major, 64 per step.
+        // A wavefront's totals fit the packed halves (at most 512 entries each); the prefixes over
+        // a row of more than 65536 entries do not, so they are kept apart.
+        uint32_t carry_gt = 0, carry_eq = 0;
 #pragma unroll
         for (int i0 = 0; i0 < MAXC * kWaves; i0 += 64) {
             const uint32_t x = s_tot[i0 + lane];
-            uint32_t v = x;
+            const uint32_t xg = x & 0xFFFFu, xe = x >> 16;
+            uint32_t vg = xg, ve = xe;
 #pragma unroll
             for (int o = 1; o < 64; o <<= 1) {
-                const uint32_t t = __shfl_up(v, o);
-                if (lane >= o) v += t;
+                const uint32_t tg = __shfl_up(vg, o), te = __shfl_up(ve, o);
+                if (lane >= o) { vg += tg; ve += te; }
             }
-            s_tot[i0 + lane] = carry + v - x;
-            carry += __shfl(v, 63);
+            s_pgt[i0 + lane] = carry_gt + vg - xg;
+            s_peq[i0 + lane] = carry_eq + ve - xe;
+            carry_gt += __shfl(vg, 63);
+            carry_eq += __shfl(ve, 63);
         }
     }
     __syncthreads();
@@ -434,10 +441,9 @@ __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
         if (c < nchunks) {
-            const uint32_t ex = s_tot[c * kWaves + wave] + exw[c];
             const int nvc = nv_of(c);
-            uint32_t my_gt = ex & 0xFFFFu;
-            uint32_t my_eq = ex >> 16;
+            uint32_t my_gt = s_pgt[c * kWaves + wave] + (exw[c] & 0xFFFFu);
+            uint32_t my_eq = s_peq[c * kWaves + wave] + (exw[c] >> 16);
             const int base = c * kChunk + tid * 8;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
@@ -744,6 +750,8 @@ SplitWs carve_ws(void* workspace, int rows, int max_chunks) {
 
 }  // namespace
 
+int topk_max_register_row() { return 16 * kChunk; }
+
 long long topk_split_workspace_bytes(int rows, long long row_len) {
     if (row_len < kSplitMinLen || rows > kSplitMaxRows) return 0;
     const long long chunks = (row_len + kSplitChunk - 1) / kSplitChunk;
@@ -807,6 +815,9 @@ hipError_t launch_topk(const half_t* scores, int* out_idx, int rows, long long r
                            row_stride, uniform_len, valid_len, n_sel, period, k, fill, ro);
     else if (aligned_rows && uniform_len <= 8 * kChunk)
         hipLaunchKernelGGL(topk_select_reg_kernel<8>, dim3(rows), dim3(kThreads), 0, stream, src, out_idx,
+                           row_stride, uniform_len, valid_len, n_sel, period, k, fill, ro);
+    else if (aligned_rows && uniform_len <= 16 * kChunk)
+        hipLaunchKernelGGL(topk_select_reg_kernel<16>, dim3(rows), dim3(kThreads), 0, stream, src, out_idx,
                            row_stride, uniform_len, valid_len, n_sel, period, k, fill, ro);
     else
         hipLaunchKernelGGL(topk_select_kernel, dim3(rows), dim3(kThreads), 0, stream, src, out_idx,
