@@ -298,8 +298,9 @@ def test_config4_stack_36_layers_prefill_and_256_replayed_decode_steps(cuda):
 @pytest.mark.parametrize("L", [65536, 131072, 262144])
 def test_prefill_beyond_32k(cuda, L):
     """Prompts of 65536, 131072 and 262144 tokens (the reference publishes all three): an anchor layer > 0
-    through the strategy -- at 131072 pooled and selected 512 tiles at a time, rows longer than
-    65536 entries on the multi-workgroup selection -- and a reuse layer through a head map, against
+    through the strategy -- beyond 65536 pooled and selected 512 tiles at a time, rows of up to
+    131072 entries selected from one workgroup's registers, longer ones on the multi-workgroup
+    selection -- and a reuse layer through a head map, against
     the oracle on sampled tiles; every tile's selection against the kernel's own pooled scores on
     one chunk of tiles."""
     from kascade_amd import kernels, budgets, workloads
