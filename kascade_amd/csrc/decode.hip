@@ -410,7 +410,8 @@ void decode_split_kernel(DecodeParams p) {
                 uint16_t* dst = reinterpret_cast<uint16_t*>(row) + r0 + lo;
                 for (int i = tid * 8; i < nrows; i += kThreads * 8) {
                     if (i + 8 <= nrows) {
-                        *reinterpret_cast<uint4_t*>(dst + i) = *reinterpret_cast<const uint4_t*>(&s_code[h][i]);
+                        __builtin_nontemporal_store(*reinterpret_cast<const uint4_t*>(&s_code[h][i]),
+                                                    reinterpret_cast<uint4_t*>(dst + i));
                     } else {
                         for (int e = 0; i + e < nrows; ++e) dst[i + e] = s_code[h][i + e];
                     }
