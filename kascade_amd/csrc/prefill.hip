@@ -506,9 +506,9 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
                 const int r = j * kRPL + lrow;
                 const uint4_t row = *reinterpret_cast<const uint4_t*>(&so[r * D + lchunk * 8]);
                 const int qr = q0l + r;
-                if (qr < Lq)
-                    *reinterpret_cast<uint4_t*>((T*)p.O + (((long long)b * Lq + qr) * nheads + head) * D +
-                                                ((lchunk ^ (r & (kChunks - 1))) * 8)) = row;
+                if (qr < Lq)   // the output is not read again by these kernels: keep it out of the caches
+                    __builtin_nontemporal_store(row, reinterpret_cast<uint4_t*>(
+                        (T*)p.O + (((long long)b * Lq + qr) * nheads + head) * D + ((lchunk ^ (r & (kChunks - 1))) * 8)));
             }
         }
     }
