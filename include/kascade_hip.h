@@ -398,17 +398,29 @@ int kascade_rope_append_paged_call(const kascade_half* q_in, const kascade_strid
                                    kascade_half* K_pages, kascade_half* V_pages,
                                    const int32_t* block_table, int max_pages, int page_size,
                                    int batch, int n_new, void* stream);
+int kascade_rope_append_paged_shaped_call(const kascade_shape* shape, const kascade_half* q_in, const kascade_strides* q_strides,
+                                   const kascade_half* k_in, const kascade_half* v_in,
+                                   const kascade_strides* kv_strides, const float* cos_sin,
+                                   int max_pos, const kascade_half* q_norm_weight,
+                                   const kascade_half* k_norm_weight, float norm_eps,
+                                   const int32_t* start_pos, int pos_offset, kascade_half* q_out,
+                                   kascade_half* K_pages, kascade_half* V_pages,
+                                   const int32_t* block_table, int max_pages, int page_size,
+                                   int batch, int n_new, void* stream);
 
 /* Bookkeeping of a ragged decode step in one small launch (no reference counterpart; the
  * reference's benchmark computes these on the host, recompute_kascade_gqa_decode_with_kvcache.py:
  * 368-377).  Adds `advance` to every cache_seqlens[b] in place (1 when the step's new token is
  * appended by the decode calls themselves, 0 to leave the lengths alone) and writes, per
- * (sequence, KV head) row r = b*8+g of the pooled scores, what kascade_topk_call takes as
+ * (sequence, KV head) row r = b*8+g (b*kv_heads+g for the shaped twin) of the pooled scores, what kascade_topk_call takes as
  * valid_len / n_sel:  valid_len_rows[r] = len_b,
  *                     n_sel_rows[r]     = 128*ceil(floor(topk_percent*len_b/100)/128),
  * with len_b the length after the advance.  Either output may be NULL. */
 int kascade_decode_budgets_call(int32_t* cache_seqlens, int advance, float topk_percent, int batch,
                                 int32_t* valid_len_rows, int32_t* n_sel_rows, void* stream);
+int kascade_decode_budgets_shaped_call(const kascade_shape* shape, int32_t* cache_seqlens, int advance,
+                                       float topk_percent, int batch, int32_t* valid_len_rows,
+                                       int32_t* n_sel_rows, void* stream);
 
 /* ------------------------------------------- chunked prefill over the paged cache */
 
@@ -430,8 +442,20 @@ int kascade_prefill_chunk_dense_call(const kascade_half* Q, const kascade_half* 
                                      kascade_strides q_strides, const int32_t* block_table,
                                      int max_pages, int page_size, int num_pages, int with_output,
                                      void* stream);
+int kascade_prefill_chunk_dense_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K_pages,
+                                     const kascade_half* V_pages, float* log_sum,
+                                     kascade_half* Output, int batch, int q_start, int q_len,
+                                     kascade_strides q_strides, const int32_t* block_table,
+                                     int max_pages, int page_size, int num_pages, int with_output,
+                                     void* stream);
 
 int kascade_prefill_chunk_aggregate_call(const kascade_half* Q, const kascade_half* K_pages,
+                                         const float* log_sum, kascade_half* aggregate_scores,
+                                         int batch, int q_start, int q_len,
+                                         kascade_strides q_strides, const int32_t* block_table,
+                                         int max_pages, int page_size, int num_pages,
+                                         int fill_invalid, void* stream);
+int kascade_prefill_chunk_aggregate_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K_pages,
                                          const float* log_sum, kascade_half* aggregate_scores,
                                          int batch, int q_start, int q_len,
                                          kascade_strides q_strides, const int32_t* block_table,
@@ -442,6 +466,13 @@ int kascade_prefill_chunk_aggregate_call(const kascade_half* Q, const kascade_ha
  * to rows of the paged cache (kascade_translate_indices_call), so that the gather needs no
  * second dependent load. */
 int kascade_prefill_chunk_reuse_call(const kascade_half* Q, const kascade_half* K_pages,
+                                     const kascade_half* V_pages, const int32_t* physical_rows,
+                                     const int32_t* head_mapping, float topk_percent,
+                                     kascade_half* Output, int batch, int q_start, int q_len,
+                                     int max_topk_num, int rolling, kascade_strides q_strides,
+                                     const int32_t* block_table, int max_pages, int page_size,
+                                     int num_pages, void* stream);
+int kascade_prefill_chunk_reuse_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K_pages,
                                      const kascade_half* V_pages, const int32_t* physical_rows,
                                      const int32_t* head_mapping, float topk_percent,
                                      kascade_half* Output, int batch, int q_start, int q_len,

@@ -74,7 +74,9 @@ class Shape(C.Structure):
 
 # every *_shaped_call takes a kascade_shape* followed by the arguments of the plain entry
 for _name in ("decode_reuse_paged", "decode_reuse_rows", "decode_dense_paged", "decode_recompute_paged",
-              "prefill_dense", "prefill_aggregate", "prefill_aggregate_range", "prefill_reuse", "paged_kv_append"):
+              "prefill_dense", "prefill_aggregate", "prefill_aggregate_range", "prefill_reuse", "paged_kv_append",
+              "rope_append_paged", "decode_budgets", "prefill_chunk_dense", "prefill_chunk_aggregate",
+              "prefill_chunk_reuse"):
     _res, _args = SIGNATURES[f"kascade_{_name}_call"]
     SIGNATURES[f"kascade_{_name}_shaped_call"] = (_res, [C.POINTER(Shape)] + list(_args))
 

@@ -30,24 +30,25 @@ class KascadeBlockStack(KascadeAttentionStack):
                  k: float, max_seqlen: int, hidden: int = 4096, batch: int = 1, page_size: int = 16,
                  rolling_prefill: bool = True, device="cuda", table_seed: int = 0, dense: bool = False,
                  weight_seed: int = 0, qk_norm: bool = True, rope_theta: float = 1e6,
-                 norm_eps: float = 1e-6):
+                 norm_eps: float = 1e-6, kv_heads: int = G, head_dim: int = D, dtype=torch.float16):
         super().__init__(num_layers, recompute_layers, head_mapping, k, max_seqlen, batch, page_size,
-                         rolling_prefill, device, table_seed, dense)
+                         rolling_prefill, device, table_seed, dense, kv_heads, head_dim, dtype)
+        H, G, D = self.H, self.G, self.D
         self.hidden, self.norm_eps, self.qk_norm = hidden, norm_eps, qk_norm
         gen = torch.Generator().manual_seed(weight_seed)
         dev = self.device
 
         def w(shape, std, mean=0.0):
-            return (mean + std * torch.randn(shape, generator=gen)).to(torch.float16).to(dev)
+            return (mean + std * torch.randn(shape, generator=gen)).to(dtype).to(dev)
 
         n_qkv = (H + 2 * G) * D
-        # rows of w_qkv: the 32 query heads, then the 8 key heads, then the 8 value heads
+        # rows of w_qkv: the query heads, then the key heads, then the value heads
         self.w_qkv = [w((n_qkv, hidden), hidden ** -0.5) for _ in range(num_layers)]
         self.w_o = [w((hidden, H * D), (H * D) ** -0.5) for _ in range(num_layers)]
         self.ln_w = [w((hidden,), 0.1, 1.0) for _ in range(num_layers)]
         self.q_norm_w = [w((D,), 0.1, 1.0) if qk_norm else None for _ in range(num_layers)]
         self.k_norm_w = [w((D,), 0.1, 1.0) if qk_norm else None for _ in range(num_layers)]
-        self.cos_sin = kernels.rope_table(max_seqlen, rope_theta, device=dev)
+        self.cos_sin = kernels.rope_table(max_seqlen, rope_theta, device=dev, round_to=dtype, head_dim=D)
         self._hgraph = None
 
     # --------------------------------------------------------------- one layer
@@ -55,6 +56,7 @@ class KascadeBlockStack(KascadeAttentionStack):
         """Projection and hand-off of layer l for the tokens in x [B,n,hidden]: returns the
         rotated queries [B,n,H,D]; the new keys and values are in the cache afterwards."""
         B, n, _ = x.shape
+        H, G, D = self.H, self.G, self.D
         h = F.rms_norm(x, (self.hidden,), self.ln_w[l], self.norm_eps)
         qkv = F.linear(h, self.w_qkv[l])                                       # [B,n,(H+2G)*D]
         q_in = qkv[..., :H * D].view(B, n, H, D)
@@ -66,7 +68,7 @@ class KascadeBlockStack(KascadeAttentionStack):
 
     def _residual(self, l: int, x: torch.Tensor, o: torch.Tensor) -> torch.Tensor:
         B, n = x.shape[:2]
-        return x + F.linear(o.reshape(B, n, H * D), self.w_o[l])
+        return x + F.linear(o.reshape(B, n, self.H * self.D), self.w_o[l])
 
     # ------------------------------------------------------------------ prefill
     def prefill_chunk_hidden(self, x: torch.Tensor) -> torch.Tensor:
@@ -119,7 +121,7 @@ class KascadeBlockStack(KascadeAttentionStack):
         ``graph_y``).  The warm-up run appends one token; the lengths are restored afterwards,
         so the first replay overwrites that slot."""
         B, dev = self.batch, self.device
-        self.graph_x = torch.zeros(B, 1, self.hidden, device=dev, dtype=torch.float16)
+        self.graph_x = torch.zeros(B, 1, self.hidden, device=dev, dtype=self.dtype)
         self.graph_y = torch.zeros_like(self.graph_x)
         if self.length + 1 > self.max_seqlen:
             raise KascadeError("no room to capture a decode step")

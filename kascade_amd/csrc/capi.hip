@@ -152,7 +152,7 @@ int set_append(DecodeParams& p, const kascade_half* k_new, const kascade_half* v
 
 extern "C" {
 
-int kascade_abi_version(void) { return 7; }
+int kascade_abi_version(void) { return 8; }
 
 const char* kascade_get_last_error(void) { return g_err; }
 
@@ -747,7 +747,9 @@ int kascade_paged_kv_append_shaped_call(const kascade_shape* shape, kascade_half
     return paged_kv_append_impl(sh, K_pages, V_pages, k_new, v_new, start_pos, block_table, batch, n_new, max_pages, page_size, new_strides, stream);
 }
 
-int kascade_rope_append_paged_call(const kascade_half* q_in, const kascade_strides* q_strides,
+}  // extern "C"
+namespace {
+int rope_append_impl(const Shape& sh, const kascade_half* q_in, const kascade_strides* q_strides,
                                    const kascade_half* k_in, const kascade_half* v_in,
                                    const kascade_strides* kv_strides, const float* cos_sin,
                                    int max_pos, const kascade_half* q_norm_weight,
@@ -765,38 +767,79 @@ int kascade_rope_append_paged_call(const kascade_half* q_in, const kascade_strid
     if (check_paging(block_table, max_pages, page_size, &shift)) return -1;
     RopeAppendParams p{};
     const kascade_strides qs = q_strides ? *q_strides
-        : kascade_strides{(long long)n_new * kHeads * kDim, (long long)kHeads * kDim, kDim};
+        : kascade_strides{(long long)n_new * sh.H() * sh.D, (long long)sh.H() * sh.D, sh.D};
     const kascade_strides ks = kv_strides ? *kv_strides
-        : kascade_strides{(long long)n_new * kGroups * kDim, (long long)kGroups * kDim, kDim};
+        : kascade_strides{(long long)n_new * sh.G * sh.D, (long long)sh.G * sh.D, sh.D};
     if (check_strides(qs, "q_in") || check_strides(ks, "k_in/v_in")) return -1;
     REQUIRE(aligned16(q_in) && aligned16(k_in) && aligned16(v_in) && aligned16(q_out) &&
                 aligned16(K_pages) && aligned16(V_pages) && aligned16(cos_sin) &&
                 aligned16(q_norm_weight) && aligned16(k_norm_weight),
             "rope_append: tensors must be 16-byte aligned");
-    p.q_in = H(q_in); p.k_in = H(k_in); p.v_in = H(v_in);
-    p.cos_sin = cos_sin; p.q_weight = H(q_norm_weight); p.k_weight = H(k_norm_weight);
-    p.start_pos = start_pos; p.q_out = H(q_out); p.Kp = H(K_pages); p.Vp = H(V_pages);
+    p.q_in = E(q_in); p.k_in = E(k_in); p.v_in = E(v_in);
+    p.cos_sin = cos_sin; p.q_weight = E(q_norm_weight); p.k_weight = E(k_norm_weight);
+    p.start_pos = start_pos; p.q_out = E(q_out); p.Kp = E(K_pages); p.Vp = E(V_pages);
     p.block_table = block_table;
     p.q_sb = qs.b; p.q_sl = qs.l; p.q_sh = qs.h;
     p.kv_sb = ks.b; p.kv_sl = ks.l; p.kv_sh = ks.h;
     p.eps = norm_eps; p.pos_offset = pos_offset; p.batch = batch; p.n_new = n_new;
     p.max_pages = max_pages; p.page_shift = shift; p.max_pos = max_pos;
+    p.G = sh.G; p.head_dim = sh.D; p.elem = sh.elem;
     return check_hip(launch_rope_append(p, static_cast<hipStream_t>(stream)), "rope_append");
 }
+}  // namespace
+extern "C" {
 
-int kascade_decode_budgets_call(int32_t* cache_seqlens, int advance, float topk_percent, int batch,
-                                int32_t* valid_len_rows, int32_t* n_sel_rows, void* stream) {
+int kascade_rope_append_paged_call(const kascade_half* q_in, const kascade_strides* q_strides,
+                                   const kascade_half* k_in, const kascade_half* v_in,
+                                   const kascade_strides* kv_strides, const float* cos_sin,
+                                   int max_pos, const kascade_half* q_norm_weight,
+                                   const kascade_half* k_norm_weight, float norm_eps,
+                                   const int32_t* start_pos, int pos_offset, kascade_half* q_out,
+                                   kascade_half* K_pages, kascade_half* V_pages,
+                                   const int32_t* block_table, int max_pages, int page_size,
+                                   int batch, int n_new, void* stream) {
+    return rope_append_impl(kRefShape, q_in, q_strides, k_in, v_in, kv_strides, cos_sin, max_pos, q_norm_weight, k_norm_weight, norm_eps, start_pos, pos_offset, q_out, K_pages, V_pages, block_table, max_pages, page_size, batch, n_new, stream);
+}
+
+int kascade_rope_append_paged_shaped_call(const kascade_shape* shape, const kascade_half* q_in, const kascade_strides* q_strides,
+                                   const kascade_half* k_in, const kascade_half* v_in,
+                                   const kascade_strides* kv_strides, const float* cos_sin,
+                                   int max_pos, const kascade_half* q_norm_weight,
+                                   const kascade_half* k_norm_weight, float norm_eps,
+                                   const int32_t* start_pos, int pos_offset, kascade_half* q_out,
+                                   kascade_half* K_pages, kascade_half* V_pages,
+                                   const int32_t* block_table, int max_pages, int page_size,
+                                   int batch, int n_new, void* stream) {
+    Shape sh;
+    if (get_shape(shape, &sh)) return -1;
+    return rope_append_impl(sh, q_in, q_strides, k_in, v_in, kv_strides, cos_sin, max_pos, q_norm_weight, k_norm_weight, norm_eps, start_pos, pos_offset, q_out, K_pages, V_pages, block_table, max_pages, page_size, batch, n_new, stream);
+}
+
+int kascade_decode_budgets_shaped_call(const kascade_shape* shape, int32_t* cache_seqlens, int advance,
+                                       float topk_percent, int batch, int32_t* valid_len_rows,
+                                       int32_t* n_sel_rows, void* stream) {
+    Shape sh;
+    if (get_shape(shape, &sh)) return -1;
     REQUIRE(cache_seqlens, "decode_budgets: null pointer argument");
     REQUIRE(batch > 0 && batch <= 65535, "decode_budgets: bad batch");
     REQUIRE(topk_percent >= 0.f && topk_percent <= 100.f, "decode_budgets: topk_percent out of range");
-    return check_hip(launch_decode_budgets(cache_seqlens, advance, topk_percent, batch, valid_len_rows,
+    return check_hip(launch_decode_budgets(cache_seqlens, advance, topk_percent, batch, sh.G, valid_len_rows,
                                            n_sel_rows, static_cast<hipStream_t>(stream)),
                      "decode_budgets");
 }
 
+int kascade_decode_budgets_call(int32_t* cache_seqlens, int advance, float topk_percent, int batch,
+                                int32_t* valid_len_rows, int32_t* n_sel_rows, void* stream) {
+    const kascade_shape ref{kRefShape.G, kRefShape.D, KASCADE_F16};
+    return kascade_decode_budgets_shaped_call(&ref, cache_seqlens, advance, topk_percent, batch,
+                                              valid_len_rows, n_sel_rows, stream);
+}
+
 // ---- chunked prefill over the paged cache ----
 
-static int chunk_params(PrefillParams& p, const char* what, const kascade_half* Q, int batch,
+}  // extern "C"
+namespace {
+int chunk_params(PrefillParams& p, const Shape& sh, const kascade_half* Q, int batch,
                         int q_start, int q_len, kascade_strides q_strides,
                         const int32_t* block_table, int max_pages, int page_size, int num_pages) {
     REQUIRE(block_table, "prefill_chunk: block_table is required");
@@ -811,9 +854,8 @@ static int chunk_params(PrefillParams& p, const char* what, const kascade_half* 
             "prefill_chunk: num_pages out of range");
     REQUIRE((long long)max_pages * page_size >= (long long)q_start + q_len,
             "prefill_chunk: block table shorter than q_start + q_len");
-    (void)what;
-    p.G = kRefShape.G; p.head_dim = kRefShape.D; p.elem = kRefShape.elem;
-    p.Q = H(Q);
+    p.G = sh.G; p.head_dim = sh.D; p.elem = sh.elem;
+    p.Q = E(Q);
     p.q_sb = q_strides.b; p.q_sl = q_strides.l; p.q_sh = q_strides.h;
     p.B = batch; p.L = q_start + q_len; p.Lq = q_len; p.q_start = q_start;
     p.T = (q_len + kTile - 1) / kTile;
@@ -822,7 +864,7 @@ static int chunk_params(PrefillParams& p, const char* what, const kascade_half* 
     return 0;
 }
 
-int kascade_prefill_chunk_dense_call(const kascade_half* Q, const kascade_half* K_pages,
+int prefill_chunk_dense_impl(const Shape& sh, const kascade_half* Q, const kascade_half* K_pages,
                                      const kascade_half* V_pages, float* log_sum,
                                      kascade_half* Output, int batch, int q_start, int q_len,
                                      kascade_strides q_strides, const int32_t* block_table,
@@ -834,16 +876,16 @@ int kascade_prefill_chunk_dense_call(const kascade_half* Q, const kascade_half* 
     REQUIRE(aligned16(K_pages) && (!with_output || (aligned16(V_pages) && aligned16(Output))),
             "prefill_chunk_dense: tensors must be 16-byte aligned");
     PrefillParams p{};
-    if (chunk_params(p, "dense", Q, batch, q_start, q_len, q_strides, block_table, max_pages,
+    if (chunk_params(p, sh, Q, batch, q_start, q_len, q_strides, block_table, max_pages,
                      page_size, num_pages))
         return -1;
-    p.K = H(K_pages); p.V = with_output ? H(V_pages) : H(K_pages);
-    p.log_sum = log_sum; p.O = H(Output);
+    p.K = E(K_pages); p.V = with_output ? E(V_pages) : E(K_pages);
+    p.log_sum = log_sum; p.O = E(Output);
     return check_hip(launch_prefill_attn(p, false, with_output != 0, 1,
                                          static_cast<hipStream_t>(stream)), "prefill_chunk_dense");
 }
 
-int kascade_prefill_chunk_aggregate_call(const kascade_half* Q, const kascade_half* K_pages,
+int prefill_chunk_aggregate_impl(const Shape& sh, const kascade_half* Q, const kascade_half* K_pages,
                                          const float* log_sum, kascade_half* aggregate_scores,
                                          int batch, int q_start, int q_len,
                                          kascade_strides q_strides, const int32_t* block_table,
@@ -853,16 +895,16 @@ int kascade_prefill_chunk_aggregate_call(const kascade_half* Q, const kascade_ha
             "prefill_chunk_aggregate: null pointer argument");
     REQUIRE(aligned16(K_pages), "prefill_chunk_aggregate: K must be 16-byte aligned");
     PrefillParams p{};
-    if (chunk_params(p, "aggregate", Q, batch, q_start, q_len, q_strides, block_table, max_pages,
+    if (chunk_params(p, sh, Q, batch, q_start, q_len, q_strides, block_table, max_pages,
                      page_size, num_pages))
         return -1;
-    p.K = H(K_pages); p.V = H(K_pages); p.log_sum_in = log_sum; p.agg = H(aggregate_scores);
+    p.K = E(K_pages); p.V = E(K_pages); p.log_sum_in = log_sum; p.agg = H(aggregate_scores);
     p.fill_invalid = fill_invalid;
     return check_hip(launch_prefill_aggregate(p, static_cast<hipStream_t>(stream)),
                      "prefill_chunk_aggregate");
 }
 
-int kascade_prefill_chunk_reuse_call(const kascade_half* Q, const kascade_half* K_pages,
+int prefill_chunk_reuse_impl(const Shape& sh, const kascade_half* Q, const kascade_half* K_pages,
                                      const kascade_half* V_pages, const int32_t* physical_rows,
                                      const int32_t* head_mapping, float topk_percent,
                                      kascade_half* Output, int batch, int q_start, int q_len,
@@ -876,14 +918,78 @@ int kascade_prefill_chunk_reuse_call(const kascade_half* Q, const kascade_half* 
     REQUIRE(aligned16(K_pages) && aligned16(V_pages) && aligned16(Output),
             "prefill_chunk_reuse: tensors must be 16-byte aligned");
     PrefillParams p{};
-    if (chunk_params(p, "reuse", Q, batch, q_start, q_len, q_strides, block_table, max_pages,
+    if (chunk_params(p, sh, Q, batch, q_start, q_len, q_strides, block_table, max_pages,
                      page_size, num_pages))
         return -1;
-    p.K = H(K_pages); p.V = H(V_pages); p.idx = physical_rows; p.head_map = head_mapping;
-    p.O = H(Output); p.log_sum = nullptr;
+    p.K = E(K_pages); p.V = E(V_pages); p.idx = physical_rows; p.head_map = head_mapping;
+    p.O = E(Output); p.log_sum = nullptr;
     p.max_topk = max_topk_num; p.rolling = rolling; p.topk_percent = topk_percent;
     return check_hip(launch_prefill_attn(p, true, true, 1, static_cast<hipStream_t>(stream)),
                      "prefill_chunk_reuse");
+}
+}  // namespace
+extern "C" {
+
+int kascade_prefill_chunk_dense_call(const kascade_half* Q, const kascade_half* K_pages,
+                                     const kascade_half* V_pages, float* log_sum,
+                                     kascade_half* Output, int batch, int q_start, int q_len,
+                                     kascade_strides q_strides, const int32_t* block_table,
+                                     int max_pages, int page_size, int num_pages, int with_output,
+                                     void* stream) {
+    return prefill_chunk_dense_impl(kRefShape, Q, K_pages, V_pages, log_sum, Output, batch, q_start, q_len, q_strides, block_table, max_pages, page_size, num_pages, with_output, stream);
+}
+
+int kascade_prefill_chunk_dense_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K_pages,
+                                     const kascade_half* V_pages, float* log_sum,
+                                     kascade_half* Output, int batch, int q_start, int q_len,
+                                     kascade_strides q_strides, const int32_t* block_table,
+                                     int max_pages, int page_size, int num_pages, int with_output,
+                                     void* stream) {
+    Shape sh;
+    if (get_shape(shape, &sh)) return -1;
+    return prefill_chunk_dense_impl(sh, Q, K_pages, V_pages, log_sum, Output, batch, q_start, q_len, q_strides, block_table, max_pages, page_size, num_pages, with_output, stream);
+}
+
+int kascade_prefill_chunk_aggregate_call(const kascade_half* Q, const kascade_half* K_pages,
+                                         const float* log_sum, kascade_half* aggregate_scores,
+                                         int batch, int q_start, int q_len,
+                                         kascade_strides q_strides, const int32_t* block_table,
+                                         int max_pages, int page_size, int num_pages,
+                                         int fill_invalid, void* stream) {
+    return prefill_chunk_aggregate_impl(kRefShape, Q, K_pages, log_sum, aggregate_scores, batch, q_start, q_len, q_strides, block_table, max_pages, page_size, num_pages, fill_invalid, stream);
+}
+
+int kascade_prefill_chunk_aggregate_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K_pages,
+                                         const float* log_sum, kascade_half* aggregate_scores,
+                                         int batch, int q_start, int q_len,
+                                         kascade_strides q_strides, const int32_t* block_table,
+                                         int max_pages, int page_size, int num_pages,
+                                         int fill_invalid, void* stream) {
+    Shape sh;
+    if (get_shape(shape, &sh)) return -1;
+    return prefill_chunk_aggregate_impl(sh, Q, K_pages, log_sum, aggregate_scores, batch, q_start, q_len, q_strides, block_table, max_pages, page_size, num_pages, fill_invalid, stream);
+}
+
+int kascade_prefill_chunk_reuse_call(const kascade_half* Q, const kascade_half* K_pages,
+                                     const kascade_half* V_pages, const int32_t* physical_rows,
+                                     const int32_t* head_mapping, float topk_percent,
+                                     kascade_half* Output, int batch, int q_start, int q_len,
+                                     int max_topk_num, int rolling, kascade_strides q_strides,
+                                     const int32_t* block_table, int max_pages, int page_size,
+                                     int num_pages, void* stream) {
+    return prefill_chunk_reuse_impl(kRefShape, Q, K_pages, V_pages, physical_rows, head_mapping, topk_percent, Output, batch, q_start, q_len, max_topk_num, rolling, q_strides, block_table, max_pages, page_size, num_pages, stream);
+}
+
+int kascade_prefill_chunk_reuse_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K_pages,
+                                     const kascade_half* V_pages, const int32_t* physical_rows,
+                                     const int32_t* head_mapping, float topk_percent,
+                                     kascade_half* Output, int batch, int q_start, int q_len,
+                                     int max_topk_num, int rolling, kascade_strides q_strides,
+                                     const int32_t* block_table, int max_pages, int page_size,
+                                     int num_pages, void* stream) {
+    Shape sh;
+    if (get_shape(shape, &sh)) return -1;
+    return prefill_chunk_reuse_impl(sh, Q, K_pages, V_pages, physical_rows, head_mapping, topk_percent, Output, batch, q_start, q_len, max_topk_num, rolling, q_strides, block_table, max_pages, page_size, num_pages, stream);
 }
 
 int kascade_translate_indices_call(const int32_t* token_idx, int32_t* physical_rows,

@@ -37,12 +37,12 @@ __global__ __launch_bounds__(256) void paged_kv_append_kernel(
 // many of them the selection keeps, n(b) = 128*ceil(floor(percent*len_b/100)/128), optionally
 // after adding `advance` to every length in place (the step's new token).
 __global__ __launch_bounds__(256) void decode_budgets_kernel(int* __restrict__ seqlens, int advance,
-                                                             float percent, int batch,
+                                                             float percent, int batch, int groups,
                                                              int* __restrict__ valid_rows,
                                                              int* __restrict__ n_sel_rows) {
     // a single workgroup: the barrier puts the in-place update after every read of a length
-    for (int i = threadIdx.x; i < batch * kGroups; i += blockDim.x) {
-        const int len = seqlens[i / kGroups] + advance;
+    for (int i = threadIdx.x; i < batch * groups; i += blockDim.x) {
+        const int len = seqlens[i / groups] + advance;
         const long long fl = (long long)floor((double)percent * (double)len / 100.0);
         if (valid_rows) valid_rows[i] = len;
         if (n_sel_rows) n_sel_rows[i] = (int)(((fl + 127) / 128) * 128);
@@ -53,85 +53,122 @@ __global__ __launch_bounds__(256) void decode_budgets_kernel(int* __restrict__ s
 }
 
 
-// One workgroup per token, one 16-lane row per head: 32 query heads, 8 key heads, 8 value heads
-// = 48 rows, three per 16-lane group (two query heads; a key head or a value head).  Query and
-// key heads are (optionally) RMS-normalised over the head dimension, then rotated by the token's
-// position in the "rotate half" pairing (i, i + 64): the partner element sits 8 lanes away in the
-// row.  Queries go to a dense [B,n,H,D] tensor; keys and values go straight to their page slots.
+// One workgroup per token, one row of D/8 lanes per head: 4G query heads, G key heads, G value
+// heads = 6G rows, taken 256/(D/8) at a time, three at once (the reference's shape is one trip:
+// two query heads and a key or value head per row of lanes).  Query and key heads are
+// (optionally) RMS-normalised over the head dimension, then rotated by the token's position in
+// the "rotate half" pairing (i, i + D/2): the partner element sits D/16 lanes away in the row.
+// Queries go to a dense [B,n,H,D] tensor; keys and values go straight to their page slots.
 // The position, the page and the angles are the same for the whole workgroup.
+template <int D, typename T>
 __global__ __launch_bounds__(256) void rope_append_kernel(RopeAppendParams p) {
-    const int lane = threadIdx.x & 15;
-    const int grp = threadIdx.x >> 4;                       // 0..15
+    constexpr int kRowLanes = D / 8;                        // 16 or 8
+    constexpr int kRowsPerTrip = 256 / kRowLanes;           // 16 or 32
+    const int lane = threadIdx.x % kRowLanes;
+    const int grp = threadIdx.x / kRowLanes;
     const int t = blockIdx.x % p.n_new;
     const int b = blockIdx.x / p.n_new;
     const int pos = p.start_pos[b] + p.pos_offset + t;
     if (pos < 0) return;
     const bool cache_ok = (pos >> p.page_shift) < p.max_pages;
-    const bool is_v = grp >= kGroups;                       // third row of this group: key or value head
-    const int g_kv = grp & (kGroups - 1);
+    const int G = p.G, Hq = kGroupSize * G, nrows = Hq + 2 * G;
+    const T* q_in = static_cast<const T*>(p.q_in);
+    const T* k_in = static_cast<const T*>(p.k_in);
+    const T* v_in = static_cast<const T*>(p.v_in);
 
-    // all loads first
-    Pack16 x[3], wq, wk;
-    const half_t* qrow = p.q_in + b * p.q_sb + t * p.q_sl;
-    x[0].u = ld_global_16(qrow + grp * p.q_sh + lane * 8);
-    x[1].u = ld_global_16(qrow + (grp + 16) * p.q_sh + lane * 8);
-    x[2].u = ld_global_16((is_v ? p.v_in : p.k_in) + b * p.kv_sb + t * p.kv_sl + g_kv * p.kv_sh + lane * 8);
-    if (p.q_weight) wq.u = ld_global_16(p.q_weight + lane * 8);
-    if (p.k_weight) wk.u = ld_global_16(p.k_weight + lane * 8);
+    PackT<T> wq, wk;
+    if (p.q_weight) wq.u = ld_global_16(static_cast<const T*>(p.q_weight) + lane * 8);
+    if (p.k_weight) wk.u = ld_global_16(static_cast<const T*>(p.k_weight) + lane * 8);
     const int pc = pos < p.max_pos ? pos : p.max_pos - 1;
-    const float* cs = p.cos_sin + (long long)pc * kDim + (lane & 7) * 8;
+    const float* cs = p.cos_sin + (long long)pc * D + (lane % (kRowLanes / 2)) * 8;
     float c[8], sn[8];
     *reinterpret_cast<float4_t*>(c) = *reinterpret_cast<const float4_t*>(cs);
     *reinterpret_cast<float4_t*>(c + 4) = *reinterpret_cast<const float4_t*>(cs + 4);
-    *reinterpret_cast<float4_t*>(sn) = *reinterpret_cast<const float4_t*>(cs + kDim / 2);
-    *reinterpret_cast<float4_t*>(sn + 4) = *reinterpret_cast<const float4_t*>(cs + kDim / 2 + 4);
+    *reinterpret_cast<float4_t*>(sn) = *reinterpret_cast<const float4_t*>(cs + D / 2);
+    *reinterpret_cast<float4_t*>(sn + 4) = *reinterpret_cast<const float4_t*>(cs + D / 2 + 4);
     long long cache_row = 0;
     if (cache_ok) {
         const int pg = p.block_table[(long long)b * p.max_pages + (pos >> p.page_shift)];
         cache_row = ((long long)pg << p.page_shift) + (pos & ((1 << p.page_shift) - 1));
     }
-    const float sign = lane < 8 ? -1.f : 1.f;
+    const float sign = lane < kRowLanes / 2 ? -1.f : 1.f;
 
-    auto rotate = [&](Pack16 v, const half_t* w, const Pack16& wv) {
-        if (w) {
-            float ss = 0.f;
+    // Executed by every lane of the wavefront, whatever its row holds: the exchanges read
+    // neighbouring lanes.
+    auto rotate = [&](PackT<T> v, bool norm, const PackT<T>& wv) {
+        float ss = 0.f;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) ss += (float)v.h[e] * (float)v.h[e];
+        for (int e = 0; e < 8; ++e) ss += (float)v.e[e] * (float)v.e[e];
+        if constexpr (kRowLanes == 16) {
             ss = row16_sum(ss);
-            const float inv = 1.0f / sqrtf(ss * (1.0f / kDim) + p.eps);
+        } else {   // rows of 8 lanes: three exchanges within the half row
+            ss += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ss), 0xB1, 0xF, 0xF, false));
+            ss += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ss), 0x4E, 0xF, 0xF, false));
+            ss += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ss), 0x141, 0xF, 0xF, false));
+        }
+        if (norm) {
+            const float inv = 1.0f / sqrtf(ss * (1.0f / D) + p.eps);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const half_t n = (half_t)((float)v.h[e] * inv);          // normalised, in storage type
-                v.h[e] = (half_t)((float)n * (float)wv.h[e]);            // times the weight, rounded once
+                const T n = (T)((float)v.e[e] * inv);                  // normalised, in storage type
+                v.e[e] = (T)((float)n * (float)wv.e[e]);               // times the weight, rounded once
             }
         }
-        Pack16 y;   // the partner half of the head: lanes 8 apart within the row of 16
+        PackT<T> y;   // the partner half of the head: D/16 lanes away within the row
 #pragma unroll
-        for (int d = 0; d < 4; ++d)
-            y.u[d] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v.u[d], 0x128, 0xF, 0xF, false);  // row_ror:8
+        for (int d = 0; d < 4; ++d) {
+            if constexpr (kRowLanes == 16)
+                y.u[d] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v.u[d], 0x128, 0xF, 0xF, false);  // row_ror:8
+            else
+                y.u[d] = (uint32_t)__builtin_amdgcn_ds_swizzle((int)v.u[d], 0x101F);                      // lane ^ 4
+        }
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v.h[e] = (half_t)((float)v.h[e] * c[e] + sign * ((float)y.h[e] * sn[e]));
+        for (int e = 0; e < 8; ++e) v.e[e] = (T)((float)v.e[e] * c[e] + sign * ((float)y.e[e] * sn[e]));
         return v;
     };
 
-    half_t* qdst = p.q_out + (long long)blockIdx.x * kHeads * kDim + lane * 8;
-    *reinterpret_cast<uint4_t*>(qdst + grp * kDim) = rotate(x[0], p.q_weight, wq).u;
-    *reinterpret_cast<uint4_t*>(qdst + (grp + 16) * kDim) = rotate(x[1], p.q_weight, wq).u;
-    if (cache_ok) {
-        const long long off = (cache_row * kGroups + g_kv) * kDim + lane * 8;
-        if (is_v)      // uniform over the 16 lanes of a row, so the row-wide exchanges above stay whole
-            *reinterpret_cast<uint4_t*>(p.Vp + off) = x[2].u;
-        else
-            *reinterpret_cast<uint4_t*>(p.Kp + off) = rotate(x[2], p.k_weight, wk).u;
+    for (int row0 = 0; row0 < nrows; row0 += 3 * kRowsPerTrip) {   // uniform over the workgroup
+        // all loads first
+        PackT<T> x[3];
+        const T* qrow = q_in + b * p.q_sb + t * p.q_sl;
+        const long long kvoff = b * p.kv_sb + t * p.kv_sl;
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            const int r = row0 + grp + j * kRowsPerTrip;
+            x[j].u = uint4_t{0, 0, 0, 0};
+            if (r < Hq)
+                x[j].u = ld_global_16(qrow + r * p.q_sh + lane * 8);
+            else if (r < Hq + G)
+                x[j].u = ld_global_16(k_in + kvoff + (r - Hq) * p.kv_sh + lane * 8);
+            else if (r < nrows)
+                x[j].u = ld_global_16(v_in + kvoff + (r - Hq - G) * p.kv_sh + lane * 8);
+        }
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            const int r = row0 + grp + j * kRowsPerTrip;
+            const bool is_q = r < Hq, is_k = !is_q && r < Hq + G;
+            const PackT<T> y = rotate(x[j], is_q ? p.q_weight != nullptr : (is_k && p.k_weight != nullptr),
+                                      is_q ? wq : wk);
+            if (is_q) {
+                *reinterpret_cast<uint4_t*>(static_cast<T*>(p.q_out) + ((long long)blockIdx.x * Hq + r) * D + lane * 8) = y.u;
+            } else if (r < nrows && cache_ok) {
+                const int g_kv = is_k ? r - Hq : r - Hq - G;
+                const long long off = (cache_row * G + g_kv) * D + lane * 8;
+                if (is_k)
+                    *reinterpret_cast<uint4_t*>(static_cast<T*>(p.Kp) + off) = y.u;
+                else
+                    *reinterpret_cast<uint4_t*>(static_cast<T*>(p.Vp) + off) = x[j].u;
+            }
+        }
     }
 }
 
 }  // namespace
 
-hipError_t launch_decode_budgets(int* seqlens, int advance, float percent, int batch, int* valid_rows,
-                                 int* n_sel_rows, hipStream_t stream) {
+hipError_t launch_decode_budgets(int* seqlens, int advance, float percent, int batch, int groups,
+                                 int* valid_rows, int* n_sel_rows, hipStream_t stream) {
     hipLaunchKernelGGL(decode_budgets_kernel, dim3(1), dim3(256), 0, stream, seqlens, advance, percent,
-                       batch, valid_rows, n_sel_rows);
+                       batch, groups, valid_rows, n_sel_rows);
     return hipGetLastError();
 }
 
@@ -149,9 +186,18 @@ hipError_t launch_paged_kv_append(half_t* Kp, half_t* Vp, const half_t* k_new, c
 }
 
 hipError_t launch_rope_append(const RopeAppendParams& p, hipStream_t stream) {
-    const long long rows = (long long)p.batch * p.n_new * (kHeads + 2 * kGroups);
-    if (rows == 0) return hipSuccess;
-    hipLaunchKernelGGL(rope_append_kernel, dim3((unsigned)(p.batch * p.n_new)), dim3(256), 0, stream, p);
+    if ((long long)p.batch * p.n_new == 0) return hipSuccess;
+    const dim3 grid((unsigned)(p.batch * p.n_new)), block(256);
+    if (p.head_dim == 128 && p.elem == kElemF16)
+        hipLaunchKernelGGL((rope_append_kernel<128, half_t>), grid, block, 0, stream, p);
+    else if (p.head_dim == 128 && p.elem == kElemBF16)
+        hipLaunchKernelGGL((rope_append_kernel<128, bf16_t>), grid, block, 0, stream, p);
+    else if (p.head_dim == 64 && p.elem == kElemF16)
+        hipLaunchKernelGGL((rope_append_kernel<64, half_t>), grid, block, 0, stream, p);
+    else if (p.head_dim == 64 && p.elem == kElemBF16)
+        hipLaunchKernelGGL((rope_append_kernel<64, bf16_t>), grid, block, 0, stream, p);
+    else
+        return hipErrorInvalidValue;
     return hipGetLastError();
 }
 

@@ -182,7 +182,8 @@ def _new_rows(k_new, v_new, B, shape=(H, G, D, torch.float16)):
     return _ptr(k_new), _ptr(v_new)
 
 
-def decode_budgets(cache_seqlens, topk_percent: float, advance: int = 0, valid_out=None, n_sel_out=None):
+def decode_budgets(cache_seqlens, topk_percent: float, advance: int = 0, valid_out=None, n_sel_out=None,
+                   kv_heads: int = G):
     """One small launch for the bookkeeping of a ragged decode step: adds ``advance`` to the
     lengths in place and returns (valid_len, n_sel) per (sequence, KV head) row as the selection
     takes them.  The reference's benchmark glue does this on the host
@@ -190,17 +191,20 @@ def decode_budgets(cache_seqlens, topk_percent: float, advance: int = 0, valid_o
     lib = _lib.init()
     _req(cache_seqlens, torch.int32, "cache_seqlens")
     B = cache_seqlens.numel()
+    n = B * kv_heads
     if valid_out is None:
-        valid_out = torch.empty(B * G, device=cache_seqlens.device, dtype=torch.int32)
+        valid_out = torch.empty(n, device=cache_seqlens.device, dtype=torch.int32)
     if n_sel_out is None:
-        n_sel_out = torch.empty(B * G, device=cache_seqlens.device, dtype=torch.int32)
+        n_sel_out = torch.empty(n, device=cache_seqlens.device, dtype=torch.int32)
     for t, name in ((valid_out, "valid_out"), (n_sel_out, "n_sel_out")):
         _req(t, torch.int32, name)
-        if t.numel() < B * G:
-            raise KascadeError(f"{name} needs {B * G} entries")
-    _lib.check(lib.kascade_decode_budgets_call(_ptr(cache_seqlens), int(advance), float(topk_percent), B,
-                                               _ptr(valid_out), _ptr(n_sel_out), _stream()))
-    return valid_out[:B * G], n_sel_out[:B * G]
+        if t.numel() < n:
+            raise KascadeError(f"{name} needs {n} entries")
+    # only the KV-head count of the shape matters here
+    _lib.check(_call(lib, "decode_budgets", (GROUP * kv_heads, kv_heads, D, torch.float16),
+                     _ptr(cache_seqlens), int(advance), float(topk_percent), B, _ptr(valid_out), _ptr(n_sel_out),
+                     _stream()))
+    return valid_out[:n], n_sel_out[:n]
 
 
 def _sync_arg(sync, B, groups: int = G):
@@ -603,11 +607,12 @@ def paged_kv_append(K_pages, V_pages, k_new, v_new, start_pos, block_table, page
         B, n_new, block_table.shape[1], page_size, st, _stream()))
 
 
-def rope_table(max_pos: int, theta: float = 1e6, device="cuda", round_to=torch.float16) -> torch.Tensor:
+def rope_table(max_pos: int, theta: float = 1e6, device="cuda", round_to=torch.float16,
+               head_dim: int = D) -> torch.Tensor:
     """[max_pos, D] fp32: cos of position * theta^(-2i/D) for the D/2 pairs, then the sines.  The
     angles are formed in fp32 and the values rounded to ``round_to`` (what the transformers
     rotary module hands an fp16 model; None keeps fp32)."""
-    inv = (1.0 / (theta ** (torch.arange(0, D, 2, dtype=torch.int64).float() / D))).to(device)
+    inv = (1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.int64).float() / head_dim))).to(device)
     ang = torch.arange(max_pos, device=device, dtype=torch.float32)[:, None] * inv
     table = torch.cat((ang.cos(), ang.sin()), dim=1)
     if round_to is not None:
@@ -624,36 +629,38 @@ def rope_append_paged(q_in, k_in, v_in, cos_sin, start_pos, K_pages, V_pages, bl
     queries [B,n,H,D]; the rotated keys and the values land in their page slots, token t of
     sequence b at position start_pos[b] + pos_offset + t."""
     lib = _lib.init()
+    shape = _shape(q_in, k_in)
+    Hq, Gk, Dh, dt = shape
     for t, name in ((q_in, "q_in"), (k_in, "k_in"), (v_in, "v_in")):
-        _req(t, torch.float16, name, False)
+        _req(t, dt, name, False)
     _req(cos_sin, torch.float32, "cos_sin"); _req(start_pos, torch.int32, "start_pos")
-    _req(K_pages, torch.float16, "K_pages"); _req(V_pages, torch.float16, "V_pages")
+    _req(K_pages, dt, "K_pages"); _req(V_pages, dt, "V_pages")
     _req(block_table, torch.int32, "block_table")
     B, n = q_in.shape[0], q_in.shape[1]
-    if tuple(q_in.shape) != (B, n, H, D) or tuple(k_in.shape) != (B, n, G, D) or k_in.shape != v_in.shape:
-        raise KascadeError(f"q_in must be [B,n,{H},{D}] and k_in/v_in [B,n,{G},{D}]")
+    if tuple(q_in.shape) != (B, n, Hq, Dh) or tuple(k_in.shape) != (B, n, Gk, Dh) or k_in.shape != v_in.shape:
+        raise KascadeError(f"q_in must be [B,n,{Hq},{Dh}] and k_in/v_in [B,n,{Gk},{Dh}]")
     if tuple(k_in.stride()) != tuple(v_in.stride()):
         raise KascadeError("k_in and v_in must share strides")
-    if cos_sin.dim() != 2 or cos_sin.shape[1] != D:
-        raise KascadeError(f"cos_sin must be [max_pos,{D}]")
+    if cos_sin.dim() != 2 or cos_sin.shape[1] != Dh:
+        raise KascadeError(f"cos_sin must be [max_pos,{Dh}]")
     if start_pos.numel() != B or block_table.shape[0] != B:
         raise KascadeError("start_pos and block_table must have one row per sequence")
-    if K_pages.dim() != 4 or K_pages.shape[1] != page_size or tuple(K_pages.shape[2:]) != (G, D) \
+    if K_pages.dim() != 4 or K_pages.shape[1] != page_size or tuple(K_pages.shape[2:]) != (Gk, Dh) \
             or K_pages.shape != V_pages.shape:
-        raise KascadeError(f"pages must be [num_pages,{page_size},{G},{D}]")
+        raise KascadeError(f"pages must be [num_pages,{page_size},{Gk},{Dh}]")
     for w, name in ((q_norm_weight, "q_norm_weight"), (k_norm_weight, "k_norm_weight")):
         if w is not None:
-            _req(w, torch.float16, name)
-            if w.numel() != D:
-                raise KascadeError(f"{name} must have {D} elements")
+            _req(w, dt, name)
+            if w.numel() != Dh:
+                raise KascadeError(f"{name} must have {Dh} elements")
     if out is None:
-        out = torch.empty(B, n, H, D, device=q_in.device, dtype=torch.float16)
+        out = torch.empty(B, n, Hq, Dh, device=q_in.device, dtype=dt)
     else:
-        _req(out, torch.float16, "out")
-        if tuple(out.shape) != (B, n, H, D):
+        _req(out, dt, "out")
+        if tuple(out.shape) != (B, n, Hq, Dh):
             raise KascadeError("out must be [B,n,H,D]")
     qs, ks = _blhd_strides(q_in, "q_in"), _blhd_strides(k_in, "k_in")
-    _lib.check(lib.kascade_rope_append_paged_call(
+    _lib.check(_call(lib, "rope_append_paged", shape,
         _ptr(q_in), ctypes.byref(qs), _ptr(k_in), _ptr(v_in), ctypes.byref(ks), _ptr(cos_sin), cos_sin.shape[0],
         _ptr(q_norm_weight), _ptr(k_norm_weight), float(norm_eps), _ptr(start_pos), int(pos_offset),
         _ptr(out), _ptr(K_pages), _ptr(V_pages), _ptr(block_table), block_table.shape[1], page_size,
@@ -663,13 +670,14 @@ def rope_append_paged(q_in, k_in, v_in, cos_sin, start_pos, K_pages, V_pages, bl
 
 # ------------------------------------------- chunked prefill over the paged cache
 def _chunk_args(Q, K_pages, block_table, q_start: int, page_size: int):
-    _req(Q, torch.float16, "Q", False); _req(K_pages, torch.float16, "K_pages")
+    shape = _shape(Q, K_pages)
+    _req(Q, shape[3], "Q", False); _req(K_pages, shape[3], "K_pages")
     _req(block_table, torch.int32, "block_table")
-    if K_pages.dim() != 4 or K_pages.shape[1] != page_size or tuple(K_pages.shape[2:]) != (G, D):
-        raise KascadeError(f"pages must be [num_pages,{page_size},{G},{D}]")
+    if K_pages.dim() != 4 or K_pages.shape[1] != page_size:
+        raise KascadeError(f"pages must be [num_pages,{page_size},G,D]")
     if q_start % TILE:
         raise KascadeError(f"q_start must be a multiple of {TILE}")
-    return Q.shape[0], Q.shape[1], _blhd_strides(Q, "Q")
+    return Q.shape[0], Q.shape[1], _blhd_strides(Q, "Q"), shape
 
 
 def prefill_chunk_dense(Q, K_pages, V_pages, block_table, q_start: int, page_size: int = 16,
@@ -679,12 +687,15 @@ def prefill_chunk_dense(Q, K_pages, V_pages, block_table, q_start: int, page_siz
     ``prefill_recomp1_kernel`` (EfficientKascadeStrategy.py:78, 80).  Returns (log_sum, O);
     O is None without with_output."""
     lib = _lib.init()
-    B, Lq, qs = _chunk_args(Q, K_pages, block_table, q_start, page_size)
-    log_sum = torch.empty(B, Lq, H, device=Q.device, dtype=torch.float32)
-    out = torch.empty(B, Lq, H, D, device=Q.device, dtype=torch.float16) if with_output else None
+    B, Lq, qs, shape = _chunk_args(Q, K_pages, block_table, q_start, page_size)
+    Hq, _, Dh, dt = shape
+    log_sum = torch.empty(B, Lq, Hq, device=Q.device, dtype=torch.float32)
+    out = torch.empty(B, Lq, Hq, Dh, device=Q.device, dtype=dt) if with_output else None
     if with_output:
-        _req(V_pages, torch.float16, "V_pages")
-    _lib.check(lib.kascade_prefill_chunk_dense_call(
+        _req(V_pages, dt, "V_pages")
+        if V_pages.shape != K_pages.shape:
+            raise KascadeError("K_pages and V_pages must share one shape")
+    _lib.check(_call(lib, "prefill_chunk_dense", shape,
         _ptr(Q), _ptr(K_pages), _ptr(V_pages) if with_output else None, _ptr(log_sum), _ptr(out), B,
         q_start, Lq, qs, _ptr(block_table), block_table.shape[1], page_size, K_pages.shape[0],
         1 if with_output else 0, _stream()))
@@ -696,12 +707,13 @@ def prefill_chunk_aggregate(Q, K_pages, log_sum, scores, block_table, q_start: i
     """Chunked ``aggregate_kernel`` (EfficientKascadeStrategy.py:81): scores
     [B,G,ceil(Lq/32),q_start+Lq] fp16, row t valid for keys < q_start + 32 t."""
     lib = _lib.init()
-    B, Lq, qs = _chunk_args(Q, K_pages, block_table, q_start, page_size)
+    B, Lq, qs, shape = _chunk_args(Q, K_pages, block_table, q_start, page_size)
+    Hq, Gk = shape[0], shape[1]
     _req(log_sum, torch.float32, "log_sum"); _req(scores, torch.float16, "scores")
     T = (Lq + TILE - 1) // TILE
-    if tuple(scores.shape) != (B, G, T, q_start + Lq) or tuple(log_sum.shape) != (B, Lq, H):
+    if tuple(scores.shape) != (B, Gk, T, q_start + Lq) or tuple(log_sum.shape) != (B, Lq, Hq):
         raise KascadeError("scores must be [B,G,ceil(Lq/32),q_start+Lq] and log_sum [B,Lq,H]")
-    _lib.check(lib.kascade_prefill_chunk_aggregate_call(
+    _lib.check(_call(lib, "prefill_chunk_aggregate", shape,
         _ptr(Q), _ptr(K_pages), _ptr(log_sum), _ptr(scores), B, q_start, Lq, qs, _ptr(block_table),
         block_table.shape[1], page_size, K_pages.shape[0], 1 if fill_invalid else 0, _stream()))
 
@@ -725,14 +737,17 @@ def prefill_chunk_reuse(Q, K_pages, V_pages, physical_rows, head_mapping, topk_p
     """Chunked ``prefill_reuse_kernel`` (EfficientKascadeStrategy.py:92, 97): physical_rows
     [B,G,ceil(Lq/32),max_topk] comes from ``translate_indices``."""
     lib = _lib.init()
-    B, Lq, qs = _chunk_args(Q, K_pages, block_table, q_start, page_size)
-    _req(V_pages, torch.float16, "V_pages")
+    B, Lq, qs, shape = _chunk_args(Q, K_pages, block_table, q_start, page_size)
+    Hq, Gk, Dh, dt = shape
+    _req(V_pages, dt, "V_pages")
+    if V_pages.shape != K_pages.shape:
+        raise KascadeError("K_pages and V_pages must share one shape")
     _req(physical_rows, torch.int32, "physical_rows"); _req(head_mapping, torch.int32, "head_mapping")
     T = (Lq + TILE - 1) // TILE
-    if tuple(physical_rows.shape[:3]) != (B, G, T):
-        raise KascadeError("physical_rows must be [B,G,ceil(Lq/32),max_topk]")
-    out = torch.empty(B, Lq, H, D, device=Q.device, dtype=torch.float16)
-    _lib.check(lib.kascade_prefill_chunk_reuse_call(
+    if tuple(physical_rows.shape[:3]) != (B, Gk, T) or head_mapping.numel() != Gk:
+        raise KascadeError("physical_rows must be [B,G,ceil(Lq/32),max_topk] and head_mapping [G]")
+    out = torch.empty(B, Lq, Hq, Dh, device=Q.device, dtype=dt)
+    _lib.check(_call(lib, "prefill_chunk_reuse", shape,
         _ptr(Q), _ptr(K_pages), _ptr(V_pages), _ptr(physical_rows), _ptr(head_mapping),
         float(topk_percent), _ptr(out), B, q_start, Lq, physical_rows.shape[-1], 1 if rolling else 0,
         qs, _ptr(block_table), block_table.shape[1], page_size, K_pages.shape[0], _stream()))

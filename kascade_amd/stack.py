@@ -30,8 +30,10 @@ class KascadeAttentionStack:
     def __init__(self, num_layers: int, recompute_layers: Sequence[int], head_mapping: List[List[int]],
                  k: float, max_seqlen: int, batch: int = 1, page_size: int = 16,
                  rolling_prefill: bool = True, device="cuda", table_seed: int = 0,
-                 dense: bool = False):
-        """dense=True runs every layer as dense attention over the same caches (the baseline)."""
+                 dense: bool = False, kv_heads: int = G, head_dim: int = D, dtype=torch.float16):
+        """dense=True runs every layer as dense attention over the same caches (the baseline).
+        kv_heads, head_dim, dtype: the model's shape (4 * kv_heads query heads; head_dim 64 or
+        128; float16 or bfloat16); the default is the reference's."""
         if 0 not in recompute_layers and not dense:
             raise KascadeError("layer 0 must be an anchor layer")
         self.num_layers, self.batch, self.page_size = num_layers, batch, page_size
@@ -39,20 +41,21 @@ class KascadeAttentionStack:
         self.dense_only = dense
         self.device = torch.device(device)
         self.max_seqlen = max_seqlen
+        self.G, self.H, self.D, self.dtype = kv_heads, kernels.GROUP * kv_heads, head_dim, dtype
         pages_per_seq = math.ceil(max_seqlen / page_size)
         n_pages = batch * pages_per_seq
         gen = torch.Generator().manual_seed(table_seed)
         self.block_table = torch.randperm(n_pages, generator=gen).to(torch.int32).view(batch, pages_per_seq) \
             .to(self.device)
-        self.k_pages = [torch.zeros(n_pages, page_size, G, D, device=self.device, dtype=torch.float16)
+        self.k_pages = [torch.zeros(n_pages, page_size, kv_heads, head_dim, device=self.device, dtype=dtype)
                         for _ in range(num_layers)]
         self.v_pages = [torch.zeros_like(p) for p in self.k_pages]
         self.length = 0                                                 # host copy of the common length
         self.seqlens = torch.zeros(batch, device=self.device, dtype=torch.int32)
         self.prefill = PagedKascadePrefill(k, head_mapping, recompute_layers, page_size, rolling_prefill,
-                                           self.device)
+                                           self.device, kv_heads=kv_heads)
         self.decoder = PagedKascadeDecoder(k, head_mapping, recompute_layers, batch, max_seqlen, page_size,
-                                           self.device)
+                                           self.device, kv_heads=kv_heads, head_dim=head_dim)
         self._graph = None
 
     def reset(self, length: int = 0):
@@ -119,7 +122,7 @@ class KascadeAttentionStack:
         if self.length + 1 > self.max_seqlen:
             raise KascadeError("decode step exceeds max_seqlen")
         if out is None:
-            out = torch.empty(self.num_layers, self.batch, H, D, device=self.device, dtype=torch.float16)
+            out = torch.empty(self.num_layers, self.batch, self.H, self.D, device=self.device, dtype=self.dtype)
         self._decode_layers(q, k_new, v_new, out)
         self.length += 1
         return out
@@ -130,10 +133,10 @@ class KascadeAttentionStack:
         capture appends one (zero) token; the lengths are restored afterwards, so that slot is
         simply overwritten by the first replay."""
         n, B, dev = self.num_layers, self.batch, self.device
-        self.graph_q = torch.zeros(n, B, H, D, device=dev, dtype=torch.float16)
-        self.graph_k = torch.zeros(n, B, 1, G, D, device=dev, dtype=torch.float16)
+        self.graph_q = torch.zeros(n, B, self.H, self.D, device=dev, dtype=self.dtype)
+        self.graph_k = torch.zeros(n, B, 1, self.G, self.D, device=dev, dtype=self.dtype)
         self.graph_v = torch.zeros_like(self.graph_k)
-        self.graph_out = torch.zeros(n, B, H, D, device=dev, dtype=torch.float16)
+        self.graph_out = torch.zeros(n, B, self.H, self.D, device=dev, dtype=self.dtype)
         if self.length + 1 > self.max_seqlen:
             raise KascadeError("no room to capture a decode step")
         saved = self.seqlens.clone()

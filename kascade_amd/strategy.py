@@ -245,8 +245,10 @@ class PagedKascadeDecoder:
                  max_batch: int, max_seqlen: int, page_size: int = 16, device="cuda",
                  num_split_dense: Optional[int] = None, num_split_reuse: Optional[int] = None,
                  total_tokens: Optional[int] = None, fused_combine: bool = True,
-                 seqlens_hint: Optional[Sequence[int]] = None):
-        """fused_combine: merge the splits inside the split launch (one launch fewer per layer).
+                 seqlens_hint: Optional[Sequence[int]] = None, kv_heads: int = G, head_dim: int = D):
+        """kv_heads, head_dim: the model's shape (query heads = 4 * kv_heads; the element type is
+        that of the tensors of each call).
+        fused_combine: merge the splits inside the split launch (one launch fewer per layer).
         total_tokens: expected sum of the sequence lengths of a batch (default
         max_batch*max_seqlen); with ragged batches it sizes the splits so that the non-empty
         workgroups, not the grid, cover the device about twice.
@@ -258,6 +260,9 @@ class PagedKascadeDecoder:
         self._head_mapping = head_mapping
         self.device = torch.device(device)
         self.max_batch, self.max_seqlen = max_batch, max_seqlen
+        G, D = kv_heads, head_dim            # this model's, from here on
+        H = kernels.GROUP * G
+        self.G, self.H, self.D = G, H, D
         self.stride = ((max_seqlen + 7) // 8) * 8
         self.max_topk = budgets.decode_budget(max_seqlen, k)
         if seqlens_hint is not None and total_tokens is None:
@@ -265,10 +270,11 @@ class PagedKascadeDecoder:
         total = total_tokens if total_tokens is not None else max_batch * max_seqlen
         dense_rows = list(seqlens_hint) if seqlens_hint is not None else None
         reuse_rows = [budgets.decode_budget(n, k) for n in seqlens_hint] if seqlens_hint is not None else None
-        self.ns_dense = num_split_dense or kernels.default_num_split(G * total, max_seqlen, row_counts=dense_rows)
+        self.ns_dense = num_split_dense or kernels.default_num_split(G * total, max_seqlen, row_counts=dense_rows,
+                                                                         heads=G)
         self.ns_reuse = num_split_reuse or kernels.default_num_split(
             G * budgets.decode_budget(total, k), self.max_topk, cap_rows=kernels.GATHER_ROWS_PER_SPLIT,
-            row_counts=reuse_rows)
+            row_counts=reuse_rows, heads=G)
         ns = max(self.ns_dense, self.ns_reuse)
         dev = self.device
         self._glse = torch.empty(max_batch * H * ns, device=dev, dtype=torch.float32)
@@ -295,6 +301,7 @@ class PagedKascadeDecoder:
         self._sync_reuse = self._sync if self.ns_reuse <= FUSED_MERGE_MAX_SPLITS else None
 
     def _scratch(self, B, ns):
+        H, D = self.H, self.D
         views = self._scratch_views.get((B, ns))
         if views is None:   # a view costs a microsecond or two of host time per layer call
             views = self._scratch_views[(B, ns)] = (self._glse[:B * H * ns].view(B, H, ns),
@@ -314,7 +321,8 @@ class PagedKascadeDecoder:
         (the new token, which the layer calls append themselves when handed ``k_new``/``v_new``)
         and the per-row budgets of the step's anchor layers are computed from the new lengths."""
         self._counts = (self._budget_key(seqlens),
-                        *kernels.decode_budgets(seqlens, float(self.k), advance, self._valid_rows, self._nsel_rows))
+                        *kernels.decode_budgets(seqlens, float(self.k), advance, self._valid_rows, self._nsel_rows,
+                                                kv_heads=self.G))
 
     @staticmethod
     def _budget_key(seqlens):
@@ -326,6 +334,7 @@ class PagedKascadeDecoder:
         keeps indices for reuse layers.  ``k_new``/``v_new`` [B,G,D]: rows of the newest token
         (position seqlens-1), appended to the cache by the anchor launch itself."""
         B = q.shape[0]
+        G, H = self.G, self.H
         stride = ((max_len + 7) // 8) * 8
         glse, part = self._scratch(B, self.ns_dense)
         scores = self._scores[:B * H * stride].view(B, H, stride)
@@ -358,7 +367,7 @@ class PagedKascadeDecoder:
         key = self._budget_key(seqlens)
         if self._counts is None or self._counts[0] != key:
             self._counts = (key, *kernels.decode_budgets(seqlens, float(self.k), 0, self._valid_rows,
-                                                         self._nsel_rows))
+                                                         self._nsel_rows, kv_heads=self.G))
         return self._counts[1], self._counts[2]
 
     def _reuse(self, q, k_pages, v_pages, block_table, seqlens, hm, out=None, k_new=None, v_new=None):
@@ -393,13 +402,14 @@ class PagedKascadePrefill:
     rows a whole-prompt call gives."""
 
     def __init__(self, k: float, head_mapping: List[List[int]], recompute_layers: Sequence[int],
-                 page_size: int = 16, rolling_prefill: bool = True, device="cuda"):
+                 page_size: int = 16, rolling_prefill: bool = True, device="cuda", kv_heads: int = G):
         self.k = k
         self.page_size = page_size
         self.rolling_prefill = rolling_prefill
         self.recompute_layers = list(recompute_layers)
         self.device = torch.device(device)
-        self._hm = {None: torch.arange(G, device=self.device, dtype=torch.int32)}
+        self.G = kv_heads
+        self._hm = {None: torch.arange(kv_heads, device=self.device, dtype=torch.int32)}
         for l, row in enumerate(head_mapping):
             self._hm[l] = torch.tensor(row, device=self.device, dtype=torch.int32)
         self._rows_to_reuse = None      # physical rows [B,G,T,width] of the last anchor
@@ -424,6 +434,7 @@ class PagedKascadePrefill:
         return hit
 
     def _score_buffer(self, B, T, Lk):
+        G = self.G
         n = B * G * T * Lk
         if self._scores is None or self._scores.numel() < n:
             self._scores = torch.empty(n, device=self.device, dtype=torch.float16)
