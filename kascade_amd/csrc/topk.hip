@@ -8,6 +8,8 @@
 // The row is streamed from L2/HBM three times as 16-byte loads.
 #include "topk.h"
 
+#include <type_traits>
+
 #include "prefill.h"   // launch_translate_indices
 
 namespace kascade {
@@ -64,16 +66,53 @@ __device__ __forceinline__ int load_keys(const uint16_t* __restrict__ src, bool 
     return nvalid;
 }
 
+// Inclusive prefix sum over the 64 lanes of a wavefront in six DPP additions: four shifts within
+// the rows of 16 lanes, then the last lane of row 0 / 2 added to row 1 / 3 and lane 31 to the
+// upper half.
+__device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v) {
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xF, 0xF, false);   // row_shr:1
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xF, 0xF, false);   // row_shr:2
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xF, 0xF, false);   // row_shr:4
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xF, 0xF, false);   // row_shr:8
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xA, 0xF, false);   // row_bcast:15 -> rows 1, 3
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xC, 0xF, false);   // row_bcast:31 -> rows 2, 3
+    return v;
+}
+
+// Packed 16-bit operations on the two halves of a word.  Written as instructions: the compiler
+// otherwise turns min(sat(a - b), 1) into two compares, two selects and a byte permute.
+__device__ __forceinline__ uint32_t pk_sub_sat_u16(uint32_t a, uint32_t b) {
+    uint32_t r;
+    asm("v_pk_sub_u16 %0, %1, %2 clamp" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ uint32_t pk_min_u16(uint32_t a, uint32_t b) {
+    uint32_t r;
+    asm("v_pk_min_u16 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+    uint32_t r;
+    asm("v_pk_max_u16 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+// arithmetic shift right by 15 of both halves: 0xFFFF where a half is negative as int16, else 0
+__device__ __forceinline__ uint32_t pk_sign_mask_i16(uint32_t a) {
+    uint32_t r;
+    asm("v_pk_ashrrev_i16 %0, %1, %2" : "=v"(r) : "v"(0x000F000Fu), "v"(a));
+    return r;
+}
+__device__ __forceinline__ uint32_t pk_add_u16(uint32_t a, uint32_t b) {
+    uint32_t r;
+    asm("v_pk_add_u16 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+
 // Exclusive prefix sum over the 1024 threads of the block; *total receives the block sum.
 __device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t* s_wave, uint32_t* total) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    uint32_t inc = v;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        uint32_t t = __shfl_up(inc, o);
-        if (lane >= o) inc += t;
-    }
+    const uint32_t inc = wave_incl_scan(v);
     if (lane == 63) s_wave[wave] = inc;
     __syncthreads();
     uint32_t before = 0, all = 0;
@@ -214,33 +253,44 @@ __global__ __launch_bounds__(kThreads) void topk_select_kernel(
 // once (MAXC 16-byte loads in flight, instead of one per pass and chunk with its latency
 // exposed), turns it into packed order keys once, and the three passes run on registers.  With
 // 16 to 64 entries per thread and eight wavefronts per SIMD the kernel is bound by the
-// instructions spent per entry, so the per-entry work is branch-free and works on the packed
-// pairs where it can.
+// instructions spent per entry, so the per-entry work is kept to a few instructions:
+//  * Real entries carry keys >= 1 (the two lowest negative NaN patterns share key 1) and the
+//    slots past the end of the row key 0, so the threshold key T is >= 1 and no count needs a
+//    validity test: a slot past the end is neither above T nor equal to it.
 //  * The coarse histogram is kept in kCopies copies selected by the lane number, which spreads
 //    the same-address conflicts of the LDS atomics (pooled softmax scores crowd into a few
-//    exponent bins).
-//  * Entries past the end of the row carry key 0 (below every real key but a negative NaN) and
-//    a separate validity count per chunk keeps them out of every count.
+//    exponent bins).  The bin of +0 and the 31 smallest subnormals, where pooled probabilities
+//    underflow to by the thousand, is not counted at all: its count is the row length minus the
+//    sum of the others.
+//  * The fine histogram tests both halves of a word against the threshold bin at once; the counts
+//    above / equal to T are sums of min(sat(key - (T-1)), 2) over packed halves.
 //  * The compaction computes every (chunk, thread) offset with two barriers in all (per-chunk
 //    wavefront scans, then one scan over the chunk x wavefront totals), and stages the selected
 //    indices in LDS in their final order, so that the row's list leaves as full-width stores.
 // Rows must be 16-byte aligned and at most MAXC*8192 entries long (MAXC = 16: 131072 entries, 64
 // registers of row data per thread, still one workgroup of 1024 threads per CU).
 template <int MAXC>
-__global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(MAXC <= 4 ? 8 : 4)))
+void topk_select_reg_kernel(
     const uint16_t* __restrict__ scores, int* __restrict__ out, long long row_stride,
     int uniform_len, const int* __restrict__ valid_len, const int* __restrict__ n_sel, int period,
     int k, int fill, RowsOut ro) {
     constexpr int kCopies = 4;
     constexpr int kStage = kBins1 * kCopies;       // selected indices staged in the histogram's LDS
-    __shared__ uint32_t s_hist[kBins1 * kCopies];
+    constexpr uint32_t kOne = 0x00010001u, kTwo = 0x00020002u;
+    constexpr uint32_t kZeroKey = 0x8000u;         // order key of +0
+    constexpr uint32_t kSkipBin = kZeroKey >> 5;   // coarse bin of +0: counted by subtraction
+    __shared__ __attribute__((aligned(16))) uint32_t s_hist[kBins1 * kCopies];
     __shared__ uint32_t s_hist2[32];
     __shared__ uint32_t s_wave[kWaves];
     __shared__ uint32_t s_tot[MAXC * kWaves];      // pass 3: totals per (chunk, wavefront), packed
     __shared__ uint32_t s_pgt[MAXC * kWaves];      // pass 3: exclusive prefixes of the counts above T
     __shared__ uint32_t s_peq[MAXC * kWaves];      // ... and of the counts equal to T
-    __shared__ uint32_t s_zero[64];                // pass 1: where the zeros' idle atomics go
     __shared__ uint32_t s_sel[4];  // b1, cum_above, T, r
+    // pass 3: the wavefront scans of the per-thread counts; in registers up to 8 chunks, beyond
+    // that the row itself fills the register file
+    constexpr bool kExwInLds = MAXC > 8;
+    __shared__ uint32_t s_exw[kExwInLds ? MAXC * kThreads : 1];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -269,73 +319,87 @@ __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
     // entries of chunk c that lie inside the row (recomputed where needed: an array of them
     // would cost MAXC registers)
     auto nv_of = [&](int c) { return max(0, min(8, len - (c * kChunk + tid * 8))); };
+    // Every thread loads 16 bytes per chunk without a branch around the load, so that the loads
+    // are in flight together: where the chunk's share lies past the end of the row the address
+    // is pulled back inside it and the data replaced below.
+    const int last_full = max(len - 8, 0) & ~7;
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+        data[c] = uint4_t{0, 0, 0, 0};
+        if (len >= 8)   // uniform
+            data[c] = *reinterpret_cast<const uint4_t*>(src + min(c * kChunk + tid * 8, last_full));
+    }
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
         const int base = c * kChunk + tid * 8;
         const int nvc = nv_of(c);
-        uint4_t raw;
+        uint4_t raw = data[c];
         if (nvc == 8) {
-            raw = *reinterpret_cast<const uint4_t*>(src + base);
-        } else {
+            // order_key on both halves at once: negative values flip every bit, others the sign
+            // bit; then at least 1
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                raw[j] = pk_max_u16(raw[j] ^ (pk_sign_mask_i16(raw[j]) | 0x80008000u), kOne);
+        } else {   // the thread at the end of the row, and every thread beyond it
             uint32_t w[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const uint32_t lo = (2 * e < nvc) ? src[base + 2 * e] : 0xFFFFu;       // key 0
-                const uint32_t hi = (2 * e + 1 < nvc) ? src[base + 2 * e + 1] : 0xFFFFu;
+                const uint32_t lo = (2 * e < nvc) ? max(order_key(src[base + 2 * e]), 1u) : 0u;
+                const uint32_t hi = (2 * e + 1 < nvc) ? max(order_key(src[base + 2 * e + 1]), 1u) : 0u;
                 w[e] = lo | (hi << 16);
             }
             raw = uint4_t{w[0], w[1], w[2], w[3]};
         }
-        // order_key on both halves at once: negative values flip every bit, others the sign bit
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint32_t neg = ((raw[j] >> 15) & 0x00010001u) * 0xFFFFu;
-            raw[j] ^= (neg | 0x80008000u);
-        }
         data[c] = raw;
     }
-    auto key_of = [&](int c, int e) {   // e is a compile-time constant at every use
-        const uint32_t w = data[c][e >> 1];
-        return (e & 1) ? (w >> 16) : (w & 0xFFFFu);
-    };
 
     // ---- pass 1: coarse histogram ----
-    for (int i = tid; i < kBins1 * kCopies; i += kThreads) s_hist[i] = 0;
+    {
+        const uint4_t z = {0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < kBins1 * kCopies / (4 * kThreads); ++i)
+            *reinterpret_cast<uint4_t*>(&s_hist[(i * kThreads + tid) * 4]) = z;
+    }
     if (tid < 32) s_hist2[tid] = 0;
     __syncthreads();
-    // Zeros are counted apart: pooled probabilities underflow to +0 by the thousand, and that
-    // many atomics on one address serialise.  Each wavefront counts its zeros with a ballot and
-    // sends those lanes' atomics (adding nothing) to a slot of their own.
     const uint32_t copy = tid & (kCopies - 1);
-    constexpr uint32_t kZeroKey = 0x8000u;         // order key of +0
-    uint32_t zeros = 0;                            // wavefront-uniform
+    auto count1 = [&](uint32_t key) {
+        const uint32_t bin = key >> 5;
+        if (bin != kSkipBin) atomicAdd(&s_hist[bin * kCopies + copy], 1u);
+    };
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
         if (c < nchunks) {
             const int nvc = nv_of(c);
+            if (nvc == 8) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const uint32_t key = key_of(c, e);
-                const bool in = e < nvc;
-                const bool zero = key == kZeroKey;
-                zeros += (uint32_t)__popcll(__ballot(in && zero));
-                atomicAdd(zero ? &s_zero[lane] : &s_hist[(key >> 5) * kCopies + copy], (in && !zero) ? 1u : 0u);
+                for (int j = 0; j < 4; ++j) {
+                    count1(data[c][j] & 0xFFFFu);
+                    count1(data[c][j] >> 16);
+                }
+            } else if (nvc > 0) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (e < nvc) count1((e & 1) ? (data[c][e >> 1] >> 16) : (data[c][e >> 1] & 0xFFFFu));
             }
         }
     }
-    if (lane == 0 && zeros) atomicAdd(&s_hist[(kZeroKey >> 5) * kCopies], zeros);
     __syncthreads();
     {
-        // thread t owns bins 2047-2t and 2046-2t (descending order)
+        // thread t owns bins 2047-2t and 2046-2t (descending order); the uncounted bin is the
+        // lower bin of its owner
         const int rb0 = kBins1 - 1 - 2 * tid;
-        uint32_t c0 = 0, c1 = 0;
-#pragma unroll
-        for (int j = 0; j < kCopies; ++j) {
-            c0 += s_hist[rb0 * kCopies + j];
-            c1 += s_hist[(rb0 - 1) * kCopies + j];
-        }
+        constexpr int kSkipOwner = (kBins1 - 2 - (int)kSkipBin) / 2;
+        static_assert(kBins1 - 2 - 2 * kSkipOwner == (int)kSkipBin, "the uncounted bin must be a lower bin");
+        const uint4_t h0 = *reinterpret_cast<const uint4_t*>(&s_hist[rb0 * kCopies]);
+        const uint4_t h1 = *reinterpret_cast<const uint4_t*>(&s_hist[(rb0 - 1) * kCopies]);
+        const uint32_t c0 = h0[0] + h0[1] + h0[2] + h0[3];
+        uint32_t c1 = h1[0] + h1[1] + h1[2] + h1[3];
         uint32_t total;
-        const uint32_t above0 = block_excl_scan(c0 + c1, s_wave, &total);
+        uint32_t above0 = block_excl_scan(c0 + c1, s_wave, &total);
+        const uint32_t skipped = (uint32_t)len - total;
+        if (tid == kSkipOwner) c1 += skipped;
+        if (tid > kSkipOwner) above0 += skipped;
         const uint32_t above1 = above0 + c0;
         const uint32_t un = (uint32_t)n;
         if (above0 < un && un <= above0 + c0) {
@@ -350,30 +414,49 @@ __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
     const uint32_t b1 = s_sel[0];
     const uint32_t cum_above = s_sel[1];
 
-    // ---- pass 2: fine histogram inside the threshold bin (few entries: a branch is fine) ----
+    // ---- pass 2: fine histogram inside the threshold bin ----
+    if (b1 != kSkipBin) {
+        // few entries match: test both halves of a word at once, then a branch
+        const uint32_t bb = (b1 << 5) | (b1 << 21);
 #pragma unroll
-    for (int c = 0; c < MAXC; ++c) {
-        if (c < nchunks) {
-            const int nvc = nv_of(c);
+        for (int c = 0; c < MAXC; ++c) {
+            if (c < nchunks) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const uint32_t key = key_of(c, e);
-                if ((key >> 5) == b1 && e < nvc && key != kZeroKey) atomicAdd(&s_hist2[key & 31u], 1u);
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t w = data[c][j];
+                    const uint32_t x = (w ^ bb) & 0xFFE0FFE0u;   // a half is 0 iff its key lies in the bin
+                    if (pk_min_u16(x, kOne) != kOne) {
+                        if ((x & 0xFFFFu) == 0) atomicAdd(&s_hist2[w & 31u], 1u);
+                        if ((x >> 16) == 0) atomicAdd(&s_hist2[(w >> 16) & 31u], 1u);
+                    }
+                }
             }
         }
+    } else {
+        // The threshold lies among +0 and the smallest subnormals: that many atomics on one
+        // address would serialise, so each wavefront counts its zeros with a ballot.
+        uint32_t zeros = 0;                        // wavefront-uniform
+#pragma unroll
+        for (int c = 0; c < MAXC; ++c) {
+            if (c < nchunks) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const uint32_t w = data[c][e >> 1];
+                    const uint32_t key = (e & 1) ? (w >> 16) : (w & 0xFFFFu);
+                    const bool zero = key == kZeroKey;
+                    zeros += (uint32_t)__popcll(__ballot(zero));
+                    if ((key >> 5) == b1 && !zero) atomicAdd(&s_hist2[key & 31u], 1u);
+                }
+            }
+        }
+        if (lane == 0 && zeros) atomicAdd(&s_hist2[kZeroKey & 31u], zeros);
     }
-    if (b1 == (kZeroKey >> 5) && lane == 0 && zeros) atomicAdd(&s_hist2[kZeroKey & 31u], zeros);
     __syncthreads();
     if (tid < 64) {
         // suffix sums of the 32 fine bins, top bin first; the threshold is the first bin whose
         // running count reaches n
         const uint32_t c = (lane < 32) ? s_hist2[31 - lane] : 0u;
-        uint32_t v = c;
-#pragma unroll
-        for (int o = 1; o < 32; o <<= 1) {
-            const uint32_t t = __shfl_up(v, o);
-            if (lane >= o) v += t;
-        }
+        const uint32_t v = wave_incl_scan(c);
         const uint32_t above = cum_above + v - c;             // entries in finer bins above this one
         const bool hit = lane < 32 && above < (uint32_t)n && (uint32_t)n <= above + c;
         // bin 0 takes what is left when no finer bin reaches n (cannot happen for a consistent
@@ -381,36 +464,37 @@ __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
         const unsigned long long m = __ballot(hit);
         const int first = m ? __ffsll((long long)m) - 1 : 31;
         if (lane == first) {
-            s_sel[2] = (b1 << 5) | (uint32_t)(31 - first);
+            s_sel[2] = max((b1 << 5) | (uint32_t)(31 - first), 1u);
             s_sel[3] = (uint32_t)n - above;  // entries equal to T to take
         }
     }
     __syncthreads();
     const uint32_t T = s_sel[2];
     const uint32_t r = s_sel[3];
+    const uint32_t tm1 = (T - 1u) | ((T - 1u) << 16);   // T >= 1
 
     // ---- pass 3: ordered compaction (index order = chunk, then thread, then element) ----
+    // code of a half: min(sat(key - (T-1)), 2) = 0 below T, 1 equal to T, 2 above T
     // counts of one (chunk, thread): entries above T in the low half, equal to T in the high half
-    uint32_t exw[MAXC];   // exclusive scan of the counts over the wavefront
+    uint32_t exw[kExwInLds ? 1 : MAXC];   // exclusive scan of the counts over the wavefront
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
         uint32_t cnt = 0;
         if (c < nchunks) {
-            const int nvc = nv_of(c);
+            uint32_t sum = 0, ties = 0;   // per half: sum of the codes (<= 8), number of ones (<= 4)
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const uint32_t key = key_of(c, e);
-                const uint32_t in = (e < nvc) ? 1u : 0u;
-                cnt += ((key > T) ? in : 0u) + ((key == T) ? (in << 16) : 0u);
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t code = pk_min_u16(pk_sub_sat_u16(data[c][j], tm1), kTwo);
+                sum = pk_add_u16(sum, code);
+                ties = pk_add_u16(ties, code & kOne);
             }
+            const uint32_t s2 = (sum & 0xFFFFu) + (sum >> 16);     // ties + 2 * above
+            const uint32_t eq = (ties & 0xFFFFu) + (ties >> 16);
+            cnt = ((s2 - eq) >> 1) | (eq << 16);
         }
-        uint32_t v = cnt;
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-            const uint32_t t = __shfl_up(v, o);
-            if (lane >= o) v += t;
-        }
-        exw[c] = v - cnt;
+        const uint32_t v = wave_incl_scan(cnt);
+        if (kExwInLds) s_exw[c * kThreads + tid] = v - cnt;
+        else exw[c] = v - cnt;
         if (lane == 63) s_tot[c * kWaves + wave] = v;
     }
     __syncthreads();
@@ -423,56 +507,69 @@ __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
         for (int i0 = 0; i0 < MAXC * kWaves; i0 += 64) {
             const uint32_t x = s_tot[i0 + lane];
             const uint32_t xg = x & 0xFFFFu, xe = x >> 16;
-            uint32_t vg = xg, ve = xe;
-#pragma unroll
-            for (int o = 1; o < 64; o <<= 1) {
-                const uint32_t tg = __shfl_up(vg, o), te = __shfl_up(ve, o);
-                if (lane >= o) { vg += tg; ve += te; }
-            }
+            const uint32_t vg = wave_incl_scan(xg), ve = wave_incl_scan(xe);
             s_pgt[i0 + lane] = carry_gt + vg - xg;
             s_peq[i0 + lane] = carry_eq + ve - xe;
-            carry_gt += __shfl(vg, 63);
-            carry_eq += __shfl(ve, 63);
+            carry_gt += (uint32_t)__builtin_amdgcn_readlane((int)vg, 63);
+            carry_eq += (uint32_t)__builtin_amdgcn_readlane((int)ve, 63);
         }
     }
     __syncthreads();
-    const bool staged = n <= kStage;   // uniform
+    // The selected indices are staged in LDS in their final order, kStage positions per round (one
+    // round unless n > kStage), and leave as full-width stores.
     int* stage = reinterpret_cast<int*>(s_hist);
+    for (uint32_t lo = 0; lo < (uint32_t)n; lo += kStage) {
+        auto emit = [&](uint32_t pos, int idx) {
+            if (pos - lo < (uint32_t)kStage) stage[pos - lo] = idx;
+        };
+        // opaque copy: the codes are recomputed per round instead of being kept in registers
+        // across rounds (a second workgroup per CU needs the kernel within 64 registers)
+        uint32_t tm1_r = tm1;
+        asm volatile("" : "+v"(tm1_r));
 #pragma unroll
-    for (int c = 0; c < MAXC; ++c) {
-        if (c < nchunks) {
-            const int nvc = nv_of(c);
-            uint32_t my_gt = s_pgt[c * kWaves + wave] + (exw[c] & 0xFFFFu);
-            uint32_t my_eq = s_peq[c * kWaves + wave] + (exw[c] >> 16);
-            const int base = c * kChunk + tid * 8;
+        for (int c = 0; c < MAXC; ++c) {
+            // with 16 chunks the row fills the registers: keep the chunks' LDS reads from
+            // being moved ahead of the earlier chunks' work
+            if (kExwInLds) __builtin_amdgcn_sched_barrier(0);
+            if (c < nchunks) {
+                const uint32_t ex = kExwInLds ? s_exw[c * kThreads + tid] : exw[c];
+                uint32_t my_eq = s_peq[c * kWaves + wave] + (ex >> 16);
+                // where the next selected entry goes: after the earlier ones above T and the
+                // earlier ties taken
+                uint32_t pos = s_pgt[c * kWaves + wave] + (ex & 0xFFFFu) + min(my_eq, r);
+                const int base = c * kChunk + tid * 8;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const uint32_t key = key_of(c, e);
-                const bool in = e < nvc;
-                const bool is_gt = in && key > T;
-                const bool is_eq = in && key == T;
-                // an entry above T sits after the earlier ones above T and the earlier ties taken;
-                // a tie that is taken (my_eq < r) has min(my_eq, r) = my_eq: one formula for both
-                const int pos = (int)(my_gt + min(my_eq, r));
-                if (is_gt || (is_eq && my_eq < r)) {
-                    if (staged) stage[pos] = base + e;
-                    else put(pos, base + e);
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t code = pk_min_u16(pk_sub_sat_u16(data[c][j], tm1_r), kTwo);
+                    if ((code & kOne) == 0) {           // no tie in this word: the common case
+                        if (code & 0xFFFFu) emit(pos++, base + 2 * j);
+                        if (code >> 16) emit(pos++, base + 2 * j + 1);
+                    } else {
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            const uint32_t ch = h ? (code >> 16) : (code & 0xFFFFu);
+                            if (ch == 2u) {
+                                emit(pos++, base + 2 * j + h);
+                            } else if (ch == 1u) {
+                                if (my_eq < r) emit(pos++, base + 2 * j + h);
+                                ++my_eq;
+                            }
+                        }
+                    }
                 }
-                my_gt += is_gt ? 1u : 0u;
-                my_eq += is_eq ? 1u : 0u;
             }
         }
-    }
-    if (staged) {
         __syncthreads();
+        // this round's slots; the last round also fills the slots from n to k
+        const int hi = (lo + kStage >= (uint32_t)n) ? k : (int)(lo + kStage);
         // k is a multiple of 4 for every budget the library produces; otherwise element stores
         if ((k & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
-            for (int i = tid * 4; i < k; i += kThreads * 4) {
+            for (int i = (int)lo + tid * 4; i < hi; i += kThreads * 4) {
                 int4 v;
-                v.x = (i + 0 < n) ? stage[i + 0] : fill;
-                v.y = (i + 1 < n) ? stage[i + 1] : fill;
-                v.z = (i + 2 < n) ? stage[i + 2] : fill;
-                v.w = (i + 3 < n) ? stage[i + 3] : fill;
+                v.x = (i + 0 < n) ? stage[i + 0 - lo] : fill;
+                v.y = (i + 1 < n) ? stage[i + 1 - lo] : fill;
+                v.z = (i + 2 < n) ? stage[i + 2 - lo] : fill;
+                v.w = (i + 3 < n) ? stage[i + 3 - lo] : fill;
                 *reinterpret_cast<int4*>(dst + i) = v;
                 if (rdst) {   // k % 4 == 0 here; the rows tensor has the layout of the index tensor
                     int4 w;
@@ -488,10 +585,9 @@ __global__ __launch_bounds__(kThreads) void topk_select_reg_kernel(
                 }
             }
         } else {
-            for (int i = tid; i < k; i += kThreads) put(i, (i < n) ? stage[i] : fill);
+            for (int i = (int)lo + tid; i < hi; i += kThreads) put(i, (i < n) ? stage[i - lo] : fill);
         }
-    } else {
-        for (int i = n + tid; i < k; i += kThreads) put(i, fill);
+        __syncthreads();   // the stage is free for the next round
     }
 }
 
