@@ -93,20 +93,20 @@ __global__ __launch_bounds__(256) void rope_append_kernel(RopeAppendParams p) {
     }
     const float sign = lane < kRowLanes / 2 ? -1.f : 1.f;
 
-    // Executed by every lane of the wavefront, whatever its row holds: the exchanges read
-    // neighbouring lanes.
+    // Called per row of lanes (16 or 8): the exchanges stay inside the row, so rows of different
+    // kinds may take different branches.
     auto rotate = [&](PackT<T> v, bool norm, const PackT<T>& wv) {
-        float ss = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) ss += (float)v.e[e] * (float)v.e[e];
-        if constexpr (kRowLanes == 16) {
-            ss = row16_sum(ss);
-        } else {   // rows of 8 lanes: three exchanges within the half row
-            ss += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ss), 0xB1, 0xF, 0xF, false));
-            ss += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ss), 0x4E, 0xF, 0xF, false));
-            ss += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ss), 0x141, 0xF, 0xF, false));
-        }
         if (norm) {
+            float ss = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ss += (float)v.e[e] * (float)v.e[e];
+            if constexpr (kRowLanes == 16) {
+                ss = row16_sum(ss);
+            } else {   // rows of 8 lanes: three exchanges within the half row
+                ss += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ss), 0xB1, 0xF, 0xF, false));
+                ss += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ss), 0x4E, 0xF, 0xF, false));
+                ss += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ss), 0x141, 0xF, 0xF, false));
+            }
             const float inv = 1.0f / sqrtf(ss * (1.0f / D) + p.eps);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
@@ -127,35 +127,31 @@ __global__ __launch_bounds__(256) void rope_append_kernel(RopeAppendParams p) {
         return v;
     };
 
+    const T* qrow = q_in + b * p.q_sb + t * p.q_sl;
+    const long long kvoff = b * p.kv_sb + t * p.kv_sl;
     for (int row0 = 0; row0 < nrows; row0 += 3 * kRowsPerTrip) {   // uniform over the workgroup
-        // all loads first
+        // all loads first, none behind a branch (a row past the last one reads row 0 again)
         PackT<T> x[3];
-        const T* qrow = q_in + b * p.q_sb + t * p.q_sl;
-        const long long kvoff = b * p.kv_sb + t * p.kv_sl;
 #pragma unroll
         for (int j = 0; j < 3; ++j) {
-            const int r = row0 + grp + j * kRowsPerTrip;
-            x[j].u = uint4_t{0, 0, 0, 0};
-            if (r < Hq)
-                x[j].u = ld_global_16(qrow + r * p.q_sh + lane * 8);
-            else if (r < Hq + G)
-                x[j].u = ld_global_16(k_in + kvoff + (r - Hq) * p.kv_sh + lane * 8);
-            else if (r < nrows)
-                x[j].u = ld_global_16(v_in + kvoff + (r - Hq - G) * p.kv_sh + lane * 8);
+            int r = row0 + grp + j * kRowsPerTrip;
+            r = r < nrows ? r : 0;
+            const T* src = r < Hq ? qrow + r * p.q_sh
+                         : r < Hq + G ? k_in + kvoff + (r - Hq) * p.kv_sh
+                                      : v_in + kvoff + (r - Hq - G) * p.kv_sh;
+            x[j].u = ld_global_16(src + lane * 8);
         }
 #pragma unroll
         for (int j = 0; j < 3; ++j) {
-            const int r = row0 + grp + j * kRowsPerTrip;
-            const bool is_q = r < Hq, is_k = !is_q && r < Hq + G;
-            const PackT<T> y = rotate(x[j], is_q ? p.q_weight != nullptr : (is_k && p.k_weight != nullptr),
-                                      is_q ? wq : wk);
-            if (is_q) {
-                *reinterpret_cast<uint4_t*>(static_cast<T*>(p.q_out) + ((long long)blockIdx.x * Hq + r) * D + lane * 8) = y.u;
+            const int r = row0 + grp + j * kRowsPerTrip;   // the same for all lanes of a row
+            if (r < Hq) {
+                *reinterpret_cast<uint4_t*>(static_cast<T*>(p.q_out) + ((long long)blockIdx.x * Hq + r) * D + lane * 8) =
+                    rotate(x[j], p.q_weight != nullptr, wq).u;
             } else if (r < nrows && cache_ok) {
-                const int g_kv = is_k ? r - Hq : r - Hq - G;
-                const long long off = (cache_row * G + g_kv) * D + lane * 8;
+                const bool is_k = r < Hq + G;
+                const long long off = (cache_row * G + (is_k ? r - Hq : r - Hq - G)) * D + lane * 8;
                 if (is_k)
-                    *reinterpret_cast<uint4_t*>(static_cast<T*>(p.Kp) + off) = y.u;
+                    *reinterpret_cast<uint4_t*>(static_cast<T*>(p.Kp) + off) = rotate(x[j], p.k_weight != nullptr, wk).u;
                 else
                     *reinterpret_cast<uint4_t*>(static_cast<T*>(p.Vp) + off) = x[j].u;
             }
