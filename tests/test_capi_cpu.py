@@ -115,6 +115,37 @@ def test_bad_sizes_are_rejected(lib):
     assert "max_topk_num" in _err(lib)
 
 
+def test_shape_descriptors_are_validated(lib):
+    """Every *_shaped_call checks its kascade_shape before anything else."""
+    from kascade_amd._lib import Shape, Strides
+    buf = (C.c_char * 4096)()
+    p = (C.addressof(buf) & ~15) + 16
+    ok = Strides(4096 * 128, 4096, 128)
+    rope = (p, None, p, p, None, p, 64, None, None, 1e-6, p, 0, p, p, p, p, 4, 16, 1, 1, None)
+    chunk_dense = (p, p, p, p, p, 1, 0, 64, ok, p, 4, 16, 8, 1, None)
+    budgets = (p, 1, 10.0, 1, None, None, None)
+    for fn, args in ((lib.kascade_rope_append_paged_shaped_call, rope),
+                     (lib.kascade_prefill_chunk_dense_shaped_call, chunk_dense),
+                     (lib.kascade_decode_budgets_shaped_call, budgets)):
+        assert fn(None, *args) == -1
+        assert "shape" in _err(lib)
+        assert fn(C.byref(Shape(8, 96, 0)), *args) == -1
+        assert "head_dim" in _err(lib)
+        assert fn(C.byref(Shape(0, 128, 0)), *args) == -1
+        assert "kv_heads" in _err(lib)
+        assert fn(C.byref(Shape(8, 128, 2)), *args) == -1
+        assert "dtype" in _err(lib)
+    # a valid shape reaches the argument checks of the call itself
+    sh = C.byref(Shape(2, 64, 1))
+    assert lib.kascade_prefill_chunk_dense_shaped_call(sh, p, p, p, p, p, 1, 16, 64, ok, p, 4, 16, 8, 1, None) == -1
+    assert "multiple of 32" in _err(lib)
+    assert lib.kascade_rope_append_paged_shaped_call(sh, p, None, p, p, None, p, 0, None, None, 1e-6, p, 0, p, p, p, p,
+                                                     4, 16, 1, 1, None) == -1
+    assert "max_pos" in _err(lib)
+    assert lib.kascade_decode_budgets_shaped_call(sh, p, 1, 101.0, 1, None, None, None) == -1
+    assert "topk_percent" in _err(lib)
+
+
 def test_python_wrappers_fail_loudly_without_gpu():
     import torch
     from kascade_amd import kernels
