@@ -49,14 +49,15 @@ typedef struct {
  * heads, head dimension 128, fp16: EfficientKascadeStrategy.py:19-21, README.md:74-75), and the
  * entry points named after them take no shape.  Their `*_shaped_call` twins take this descriptor
  * as first argument and the argument list of the plain entry after it; every size that the
- * comments give as 32 / 8 / 128 reads 4*kv_heads / kv_heads / head_dim there, and kascade_half
- * means an element of `dtype`.  A KV head always serves four query heads.  Pooled scores stay
- * fp16 for both element types.  No counterpart in the reference. */
+ * comments give as 32 / 8 / 128 reads group_size*kv_heads / kv_heads / head_dim there, and
+ * kascade_half means an element of `dtype`.  Pooled scores stay fp16 for both element types.
+ * No counterpart in the reference. */
 enum { KASCADE_F16 = 0, KASCADE_BF16 = 1 };
 typedef struct {
-    int32_t kv_heads; /* >= 1; query heads = 4 * kv_heads */
-    int32_t head_dim; /* 64 or 128 */
-    int32_t dtype;    /* KASCADE_F16 or KASCADE_BF16 */
+    int32_t kv_heads;   /* >= 1 */
+    int32_t head_dim;   /* 64 or 128 */
+    int32_t dtype;      /* KASCADE_F16 or KASCADE_BF16 */
+    int32_t group_size; /* query heads per KV head: 1, 2, 4, 8 or 16; 0 means 4 */
 } kascade_shape;
 
 /* Replaces `init()` of every reference kernel object (e.g. decode reuse .cu:253-258):

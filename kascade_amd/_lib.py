@@ -68,8 +68,9 @@ SIGNATURES = {
 }
 
 class Shape(C.Structure):
-    """kascade_shape: KV heads, head dimension, element type (0 fp16, 1 bf16)."""
-    _fields_ = [("kv_heads", C.c_int32), ("head_dim", C.c_int32), ("dtype", C.c_int32)]
+    """kascade_shape: KV heads, head dimension, element type (0 fp16, 1 bf16), query heads per KV
+    head (0 = 4)."""
+    _fields_ = [("kv_heads", C.c_int32), ("head_dim", C.c_int32), ("dtype", C.c_int32), ("group_size", C.c_int32)]
 
 
 # every *_shaped_call takes a kascade_shape* followed by the arguments of the plain entry

@@ -30,9 +30,10 @@ class KascadeBlockStack(KascadeAttentionStack):
                  k: float, max_seqlen: int, hidden: int = 4096, batch: int = 1, page_size: int = 16,
                  rolling_prefill: bool = True, device="cuda", table_seed: int = 0, dense: bool = False,
                  weight_seed: int = 0, qk_norm: bool = True, rope_theta: float = 1e6,
-                 norm_eps: float = 1e-6, kv_heads: int = G, head_dim: int = D, dtype=torch.float16):
+                 norm_eps: float = 1e-6, kv_heads: int = G, head_dim: int = D, dtype=torch.float16,
+                 group_size: int = kernels.GROUP):
         super().__init__(num_layers, recompute_layers, head_mapping, k, max_seqlen, batch, page_size,
-                         rolling_prefill, device, table_seed, dense, kv_heads, head_dim, dtype)
+                         rolling_prefill, device, table_seed, dense, kv_heads, head_dim, dtype, group_size)
         H, G, D = self.H, self.G, self.D
         self.hidden, self.norm_eps, self.qk_norm = hidden, norm_eps, qk_norm
         gen = torch.Generator().manual_seed(weight_seed)

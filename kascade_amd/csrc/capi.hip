@@ -82,20 +82,25 @@ int check_strides(const kascade_strides& s, const char* name) {
     return 0;
 }
 
-// Shape of the tensors a call works on: KV heads, head dimension, element kind.  Query heads are
-// always kGroupSize per KV head.  The entry points without a shape argument use the reference's.
+// Shape of the tensors a call works on: KV heads, head dimension, element kind, query heads per
+// KV head.  The entry points without a shape argument use the reference's.
 struct Shape {
-    int G, D, elem;
-    int H() const { return G * kGroupSize; }
+    int G, D, elem, gs;
+    int H() const { return G * gs; }
 };
-const Shape kRefShape{kGroups, kDim, kElemF16};
+const Shape kRefShape{kGroups, kDim, kElemF16, kGroupSize};
 
 int get_shape(const kascade_shape* in, Shape* out) {
     REQUIRE(in, "shape: null pointer argument");
     REQUIRE(in->kv_heads >= 1 && in->kv_heads <= 65535, "shape: kv_heads out of range");
     REQUIRE(in->head_dim == 64 || in->head_dim == 128, "shape: head_dim must be 64 or 128, got %d", in->head_dim);
     REQUIRE(in->dtype == KASCADE_F16 || in->dtype == KASCADE_BF16, "shape: dtype must be KASCADE_F16 or KASCADE_BF16");
+    const int gs = in->group_size == 0 ? kGroupSize : in->group_size;
+    REQUIRE(gs == 1 || gs == 2 || gs == 4 || gs == 8 || gs == 16,
+            "shape: group_size (query heads per KV head) must be 1, 2, 4, 8 or 16 (0 = 4), got %d", in->group_size);
+    REQUIRE((long long)in->kv_heads * gs <= 65535, "shape: too many query heads");
     out->G = in->kv_heads; out->D = in->head_dim; out->elem = in->dtype == KASCADE_BF16 ? kElemBF16 : kElemF16;
+    out->gs = gs;
     return 0;
 }
 
@@ -120,7 +125,7 @@ int check_paging(const int32_t* block_table, int max_pages, int page_size, int* 
 // for the contiguous [B,kv_stride_tokens,G,D] cache).
 int set_kv_strides(DecodeParams& p, const Shape& sh, const kascade_strides* strides,
                    const int32_t* block_table, int kv_stride_tokens) {
-    p.G = sh.G; p.head_dim = sh.D; p.elem = sh.elem;
+    p.G = sh.G; p.head_dim = sh.D; p.elem = sh.elem; p.gs = sh.gs;
     if (!strides) {
         p.kv_stride_b = (long long)kv_stride_tokens * sh.G * sh.D;
         p.kv_stride_l = sh.G * sh.D;
@@ -152,7 +157,7 @@ int set_append(DecodeParams& p, const kascade_half* k_new, const kascade_half* v
 
 extern "C" {
 
-int kascade_abi_version(void) { return 8; }
+int kascade_abi_version(void) { return 9; }
 
 const char* kascade_get_last_error(void) { return g_err; }
 
@@ -452,7 +457,7 @@ int decode_recompute_paged_impl(const Shape& sh, const kascade_half* Q, const ka
         return -1;
     return check_hip(launch_decode_aggregate(scores, merge_in_aggregate ? nullptr : row_sums,
                                              merge_in_aggregate ? glse : nullptr, num_split, row_sums,
-                                             cache_seqlens, H(aggregated_scores), batch, sh.G, scores_stride,
+                                             cache_seqlens, H(aggregated_scores), batch, sh.G, sh.gs, scores_stride,
                                              kv_stride_tokens, (int)len_cap, s),
                      "decode_recompute aggregate");
 }
@@ -548,7 +553,7 @@ int prefill_dense_impl(const Shape& sh, const kascade_half* Q, const kascade_hal
             "prefill_dense: tensors must be 16-byte aligned");
     if (check_strides(q_strides, "Q") || check_strides(kv_strides, "K/V")) return -1;
     PrefillParams p{};
-    p.G = sh.G; p.head_dim = sh.D; p.elem = sh.elem;
+    p.G = sh.G; p.head_dim = sh.D; p.elem = sh.elem; p.gs = sh.gs;
     p.Q = H(Q); p.K = H(K); p.V = with_output ? H(V) : H(K); p.log_sum = log_sum; p.O = H(Output);
     p.q_sb = q_strides.b; p.q_sl = q_strides.l; p.q_sh = q_strides.h;
     p.k_sb = kv_strides.b; p.k_sl = kv_strides.l; p.k_sh = kv_strides.h;
@@ -586,7 +591,7 @@ int prefill_aggregate_impl(const Shape& sh, const kascade_half* Q, const kascade
     REQUIRE(aligned16(Q) && aligned16(K), "prefill_aggregate: Q/K must be 16-byte aligned");
     if (check_strides(q_strides, "Q") || check_strides(kv_strides, "K")) return -1;
     PrefillParams p{};
-    p.G = sh.G; p.head_dim = sh.D; p.elem = sh.elem;
+    p.G = sh.G; p.head_dim = sh.D; p.elem = sh.elem; p.gs = sh.gs;
     p.Q = H(Q); p.K = H(K); p.V = H(K); p.log_sum_in = log_sum; p.agg = H(aggregate_scores);
     p.q_sb = q_strides.b; p.q_sl = q_strides.l; p.q_sh = q_strides.h;
     p.k_sb = kv_strides.b; p.k_sl = kv_strides.l; p.k_sh = kv_strides.h;
@@ -627,7 +632,7 @@ int prefill_aggregate_range_impl(const Shape& sh, const kascade_half* Q, const k
     REQUIRE(aligned16(Q) && aligned16(K), "prefill_aggregate_range: Q/K must be 16-byte aligned");
     if (check_strides(q_strides, "Q") || check_strides(kv_strides, "K")) return -1;
     PrefillParams p{};
-    p.G = sh.G; p.head_dim = sh.D; p.elem = sh.elem;
+    p.G = sh.G; p.head_dim = sh.D; p.elem = sh.elem; p.gs = sh.gs;
     p.Q = H(Q); p.K = H(K); p.V = H(K); p.log_sum_in = log_sum; p.agg = H(aggregate_scores);
     p.q_sb = q_strides.b; p.q_sl = q_strides.l; p.q_sh = q_strides.h;
     p.k_sb = kv_strides.b; p.k_sl = kv_strides.l; p.k_sh = kv_strides.h;
@@ -673,7 +678,7 @@ int prefill_reuse_impl(const Shape& sh, const kascade_half* Q, const kascade_hal
             "prefill_reuse: tensors must be 16-byte aligned");
     if (check_strides(q_strides, "Q") || check_strides(kv_strides, "K/V")) return -1;
     PrefillParams p{};
-    p.G = sh.G; p.head_dim = sh.D; p.elem = sh.elem;
+    p.G = sh.G; p.head_dim = sh.D; p.elem = sh.elem; p.gs = sh.gs;
     p.Q = H(Q); p.K = H(K); p.V = H(V); p.idx = topk_indices; p.head_map = head_mapping;
     p.O = H(Output); p.log_sum = nullptr;
     p.q_sb = q_strides.b; p.q_sl = q_strides.l; p.q_sh = q_strides.h;
@@ -783,7 +788,7 @@ int rope_append_impl(const Shape& sh, const kascade_half* q_in, const kascade_st
     p.kv_sb = ks.b; p.kv_sl = ks.l; p.kv_sh = ks.h;
     p.eps = norm_eps; p.pos_offset = pos_offset; p.batch = batch; p.n_new = n_new;
     p.max_pages = max_pages; p.page_shift = shift; p.max_pos = max_pos;
-    p.G = sh.G; p.head_dim = sh.D; p.elem = sh.elem;
+    p.G = sh.G; p.head_dim = sh.D; p.elem = sh.elem; p.gs = sh.gs;
     return check_hip(launch_rope_append(p, static_cast<hipStream_t>(stream)), "rope_append");
 }
 }  // namespace
@@ -830,7 +835,7 @@ int kascade_decode_budgets_shaped_call(const kascade_shape* shape, int32_t* cach
 
 int kascade_decode_budgets_call(int32_t* cache_seqlens, int advance, float topk_percent, int batch,
                                 int32_t* valid_len_rows, int32_t* n_sel_rows, void* stream) {
-    const kascade_shape ref{kRefShape.G, kRefShape.D, KASCADE_F16};
+    const kascade_shape ref{kRefShape.G, kRefShape.D, KASCADE_F16, kRefShape.gs};
     return kascade_decode_budgets_shaped_call(&ref, cache_seqlens, advance, topk_percent, batch,
                                               valid_len_rows, n_sel_rows, stream);
 }
@@ -854,7 +859,7 @@ int chunk_params(PrefillParams& p, const Shape& sh, const kascade_half* Q, int b
             "prefill_chunk: num_pages out of range");
     REQUIRE((long long)max_pages * page_size >= (long long)q_start + q_len,
             "prefill_chunk: block table shorter than q_start + q_len");
-    p.G = sh.G; p.head_dim = sh.D; p.elem = sh.elem;
+    p.G = sh.G; p.head_dim = sh.D; p.elem = sh.elem; p.gs = sh.gs;
     p.Q = E(Q);
     p.q_sb = q_strides.b; p.q_sl = q_strides.l; p.q_sh = q_strides.h;
     p.B = batch; p.L = q_start + q_len; p.Lq = q_len; p.q_start = q_start;

@@ -6,7 +6,7 @@ namespace kascade {
 
 struct DecodeParams {
     // Q, K, V, the new rows and the output hold elements of kind `elem` (fp16 or bf16); G KV heads,
-    // H = 4 G query heads, head dimension head_dim (64 or 128).
+    // H = gs G query heads, head dimension head_dim (64 or 128).
     const void* Q;          // [B,H,D]
     const void* K;          // pages [P,page,G,D], or a strided [B,tokens,G,D] view
     const void* V;
@@ -48,6 +48,7 @@ struct DecodeParams {
     int G;                  // KV heads
     int head_dim;           // 64 or 128
     int elem;               // kElemF16 or kElemBF16
+    int gs;                 // query heads per KV head: 1, 2, 4, 8 or 16
 };
 
 hipError_t launch_decode_split(const DecodeParams& p, bool gather, bool with_v, bool write_scores,
@@ -60,7 +61,7 @@ hipError_t launch_decode_combine(const float* glse, const float* opart, void* ou
 // every sequence length (block-table coverage or cache length, and the score row width).
 hipError_t launch_decode_aggregate(const float* scores, const float* row_sums_in, const float* glse,
                                    int num_split, float* row_sums_out, const int* seqlens,
-                                   half_t* agg, int batch, int groups, int scores_stride, int uniform_len,
-                                   int len_cap, hipStream_t stream);
+                                   half_t* agg, int batch, int groups, int group_size, int scores_stride,
+                                   int uniform_len, int len_cap, hipStream_t stream);
 
 }  // namespace kascade

@@ -61,19 +61,21 @@ __device__ __forceinline__ float2 load_device2(const float* p) {
     return make_float2(x.f[0], x.f[1]);
 }
 
-template <int D>
+template <int D, int HS>
 struct alignas(16) MergeState {  // one per wavefront after the in-wave merge
-    float m[kGroupSize];
-    float l[kGroupSize];
-    float acc[kGroupSize][D];
+    float m[HS];
+    float l[HS];
+    float acc[HS][D];
 };
 
 // PHYS (gather mode over a paged cache): the index lists hold physical cache rows
 // (page * page_size + slot, what translate_indices_kernel writes) instead of token positions, so
 // the block table is not on the path from a list entry to its K/V row.
 // D, T: head dimension (64 or 128) and element type (fp16 or bf16) of Q, K, V and the output; the
-// number of KV heads is a launch parameter, a KV head always serves kGroupSize query heads.
-template <bool GATHER, bool WITH_V, bool WRITE_SCORES, bool PHYS, int D, typename T>
+// number of KV heads and of query heads per KV head (p.gs) are launch parameters.  The query heads
+// of the KV head are columns of the first product, so any number up to 16 rides on the same K/V
+// stream; HS (4, 8 or 16 >= p.gs) sizes what is kept per head in LDS.
+template <bool GATHER, bool WITH_V, bool WRITE_SCORES, bool PHYS, int D, typename T, int HS>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2)))
 void decode_split_kernel(DecodeParams p) {
     typedef typename Elem<T>::x8 x8_t;
@@ -81,24 +83,26 @@ void decode_split_kernel(DecodeParams p) {
     typedef typename Elem<T>::x2 x2_t;
     constexpr float kScaleLog2 = ScaleLog2<D>::value;
     const int kvh = p.G;                 // KV heads
-    const int nheads = p.G * kGroupSize; // query heads
+    const int gs = p.gs;                 // query heads per KV head (<= HS)
+    const int nheads = p.G * gs;         // query heads
     __shared__ int s_row[GATHER ? kSubChunk : 1];
     __shared__ int s_last;
     __shared__ int s_found;   // gather mode: sub-chunk whose index list names the newest token
     // anchor mode: the compact raw scores of kCodePhase * 1024 tokens (see kScoreSteps), written to
     // HBM in one burst per phase; they share their LDS with the merge state, which is only needed
     // after the last burst
-    constexpr int kCodePhase = WITH_V ? 5 : 7;             // what fits beside two workgroups' tiles
+    // what fits beside two workgroups' tiles: 40 / 56 KB of codes
+    constexpr int kCodePhase = HS == 4 ? (WITH_V ? 5 : 7) : HS == 8 ? (WITH_V ? 2 : 3) : 1;
     constexpr int kPhaseRows = WRITE_SCORES ? kCodePhase * 4 * kStripRows : 64;
     union Shared {
-        MergeState<D> merge[4];
+        MergeState<D, HS> merge[4];
         struct {
-            uint16_t code[kGroupSize][kPhaseRows];
-            float ref[kGroupSize][kPhaseRows / 64];
+            uint16_t code[HS][kPhaseRows];
+            float ref[HS][kPhaseRows / 64];
         } sc;
     };
     __shared__ __attribute__((aligned(16))) Shared s_u;
-    MergeState<D>* s_merge = s_u.merge;
+    MergeState<D, HS>* s_merge = s_u.merge;
     auto& s_code = s_u.sc.code;
     auto& s_ref = s_u.sc.ref;
     // per wavefront one tile of 16 K rows (and V rows) on its way into the matrix layouts
@@ -272,8 +276,8 @@ void decode_split_kernel(DecodeParams p) {
 #pragma unroll
     for (int st = 0; st < D / 32; ++st) {
         PackT<T> t;
-        t.u = ld_global_16((const T*)p.Q + ((size_t)b * nheads + g * kGroupSize + (col & 3)) * D + 32 * st + 8 * dq);
-        if (col >= kGroupSize) t.u = uint4_t{0, 0, 0, 0};
+        t.u = ld_global_16((const T*)p.Q + ((size_t)b * nheads + g * gs + min(col, gs - 1)) * D + 32 * st + 8 * dq);
+        if (col >= gs) t.u = uint4_t{0, 0, 0, 0};
         qb[st] = t.v8;
     }
     // Online softmax state of this lane's column.  With V one running maximum per column (the
@@ -377,7 +381,7 @@ void decode_split_kernel(DecodeParams p) {
         mx = fmaxf(mx, __shfl_xor(mx, 16));
         mx = fmaxf(mx, __shfl_xor(mx, 32));
         const float base = (mx == -INFINITY) ? 0.f : mx;
-        if (col < kGroupSize) {
+        if (col < gs) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 uint32_t q[4];
@@ -404,9 +408,8 @@ void decode_split_kernel(DecodeParams p) {
         const int nrows = min(kPhaseRows, cn - lo);
         __syncthreads();
         if (nrows > 0) {
-#pragma unroll
-            for (int h = 0; h < kGroupSize; ++h) {
-                float* row = p.scores + ((size_t)b * nheads + g * kGroupSize + h) * p.scores_stride;
+            for (int h = 0; h < gs; ++h) {
+                float* row = p.scores + ((size_t)b * nheads + g * gs + h) * p.scores_stride;
                 uint16_t* dst = reinterpret_cast<uint16_t*>(row) + r0 + lo;
                 for (int i = tid * 8; i < nrows; i += kThreads * 8) {
                     if (i + 8 <= nrows) {
@@ -599,7 +602,7 @@ void decode_split_kernel(DecodeParams p) {
             mcol = mx;
         }
     }
-    if (col < kGroupSize) {
+    if (col < gs) {
         if (dq == 0) {
             s_merge[wave].m[col] = mcol;
             s_merge[wave].l[col] = lcol;
@@ -611,9 +614,10 @@ void decode_split_kernel(DecodeParams p) {
         }
     }
     __syncthreads();
-    // ---- merge the four wavefronts; thread -> (head, two d's) ----
-    {
-        const int h = tid >> 6;
+    // ---- merge the four wavefronts; thread -> (head, two d's), four heads at a time ----
+#pragma unroll
+    for (int h = tid >> 6; h < HS; h += 4) {
+        if (h >= gs) break;                              // uniform over the wavefront
         const bool has_d = (tid & 63) * 2 < D;           // at D = 64 half of the lanes have no output element
         const int d0 = has_d ? (tid & 63) * 2 : 0;
         float mx = -INFINITY;
@@ -630,7 +634,7 @@ void decode_split_kernel(DecodeParams p) {
                 o1 += s_merge[w].acc[h][d0 + 1] * c;
             }
         }
-        const size_t ph = ((size_t)b * nheads + g * kGroupSize + h) * p.num_split + split;
+        const size_t ph = ((size_t)b * nheads + g * gs + h) * p.num_split + split;
         const float lse_part = (L > 0.f) ? (fast_log2(L) + mref) : -INFINITY;
         const float inv = (L > 0.f) ? 1.f / L : 0.f;
         if (p.counters == nullptr) {
@@ -646,8 +650,8 @@ void decode_split_kernel(DecodeParams p) {
     // the kernels that merge all num_split partial log-sums
     if (split == 0) {
         const int missing = p.num_split - nsplit_b;
-        for (int i = tid; i < kGroupSize * missing; i += kThreads)
-            p.glse[((size_t)b * nheads + g * kGroupSize + i / missing) * p.num_split + nsplit_b + i % missing] = -INFINITY;
+        for (int i = tid; i < gs * missing; i += kThreads)
+            p.glse[((size_t)b * nheads + g * gs + i / missing) * p.num_split + nsplit_b + i % missing] = -INFINITY;
     }
     // ---- fused combine: the last workgroup of (b, g) to arrive merges the splits ----
     // The partial results above are written through to device-coherent memory and the barrier
@@ -670,9 +674,12 @@ void decode_split_kernel(DecodeParams p) {
     if (!s_last) return;
     if (tid == 0)   // ready for the next launch
         __hip_atomic_store(&p.counters[b * kvh + g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    {
-        // wavefront -> head; lanes over the splits for the reductions, then two d's per lane
-        const int head = g * kGroupSize + wave;
+#pragma unroll
+    for (int hh = wave; hh < HS; hh += 4) {
+        if (hh >= gs) break;   // uniform over the wavefront
+        // wavefront -> head (four at a time); lanes over the splits for the reductions, then two
+        // d's per lane
+        const int head = g * gs + hh;
         const int ns = nsplit_b;   // the splits of this sequence that exist
         const size_t base = ((size_t)b * nheads + head) * p.num_split;
         const float* gl = p.glse + base;
@@ -790,63 +797,62 @@ __global__ __launch_bounds__(128) void decode_combine_kernel(const float* __rest
     }
 }
 
-// agg[b,g,j] = fp16( sum_h exp2(s[b,4g+h,j]*scale - lse[b,4g+h]) ), 0 beyond the sequence.
+// agg[b,g,j] = fp16( sum_h exp2(s[b,gs g+h,j]*scale - lse[b,gs g+h]) ), 0 beyond the sequence; the sum
+// runs over the gs query heads of KV head g.
 // grid (ceil(stride/2048), G, B), 256 threads x 8 tokens.
 // The per-head log-sums come either merged (row_sums_in) or as the splits' partial log-sums
-// (glse [B,H,num_split]): then every workgroup merges them itself -- one wavefront per head --
-// and the first workgroup of a (sequence, KV head) also writes them to row_sums_out, which saves
-// the combine launch of an anchor pass that produces no output.
+// (glse [B,H,num_split]): then every workgroup merges them itself -- a wavefront per head, four
+// heads at a time -- and the first workgroup of a (sequence, KV head) also writes them to
+// row_sums_out, which saves the combine launch of an anchor pass that produces no output.
 __global__ __launch_bounds__(256) void decode_aggregate_kernel(const float* __restrict__ scores,
                                                               const float* __restrict__ row_sums_in,
                                                               const float* __restrict__ glse, int num_split,
                                                               float* __restrict__ row_sums_out,
                                                               const int* __restrict__ seqlens,
-                                                              half_t* __restrict__ agg,
+                                                              half_t* __restrict__ agg, int gs,
                                                               int scores_stride, int uniform_len,
                                                               int len_cap) {
-    __shared__ float s_lse[kGroupSize];
+    constexpr int kMaxGroup = 16;
+    __shared__ float s_lse[kMaxGroup];
     const int g = blockIdx.y;
     const int b = blockIdx.z;
-    const int kvh = gridDim.y, nheads = gridDim.y * kGroupSize;
+    const int kvh = gridDim.y, nheads = gridDim.y * gs;
     // the same bound the streaming launch applied to the length: codes beyond it were never written
     const int len = max(0, min(seqlens ? seqlens[b] : uniform_len, len_cap));
     const int j0 = (blockIdx.x * 256 + threadIdx.x) * 8;
-    float lse[kGroupSize];
     if (glse != nullptr) {   // uniform over the launch
         const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-        const float* gl = glse + ((size_t)b * nheads + g * kGroupSize + wave) * num_split;
-        float mx = -INFINITY;
-        for (int sidx = lane; sidx < num_split; sidx += 64) mx = fmaxf(mx, gl[sidx]);
+        for (int h = wave; h < gs; h += 4) {
+            const float* gl = glse + ((size_t)b * nheads + g * gs + h) * num_split;
+            float mx = -INFINITY;
+            for (int sidx = lane; sidx < num_split; sidx += 64) mx = fmaxf(mx, gl[sidx]);
 #pragma unroll
-        for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
-        const float mref = (mx == -INFINITY) ? 0.f : mx;
-        float sum = 0.f;
-        for (int sidx = lane; sidx < num_split; sidx += 64) sum += fast_exp2(gl[sidx] - mref);
+            for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+            const float mref = (mx == -INFINITY) ? 0.f : mx;
+            float sum = 0.f;
+            for (int sidx = lane; sidx < num_split; sidx += 64) sum += fast_exp2(gl[sidx] - mref);
 #pragma unroll
-        for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
-        const float v = (sum > 0.f) ? fast_log2(sum) + mref : -INFINITY;
-        if (lane == 0) {
-            s_lse[wave] = v;
-            if (blockIdx.x == 0 && row_sums_out) row_sums_out[(size_t)b * nheads + g * kGroupSize + wave] = v;
+            for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
+            const float v = (sum > 0.f) ? fast_log2(sum) + mref : -INFINITY;
+            if (lane == 0) {
+                s_lse[h] = v;
+                if (blockIdx.x == 0 && row_sums_out) row_sums_out[(size_t)b * nheads + g * gs + h] = v;
+            }
         }
-        __syncthreads();
-#pragma unroll
-        for (int h = 0; h < kGroupSize; ++h) lse[h] = s_lse[h];
-    } else {
-#pragma unroll
-        for (int h = 0; h < kGroupSize; ++h) lse[h] = row_sums_in[(size_t)b * nheads + g * kGroupSize + h];
+    } else if (threadIdx.x < gs) {
+        s_lse[threadIdx.x] = row_sums_in[(size_t)b * nheads + g * gs + threadIdx.x];
     }
+    __syncthreads();
     if (j0 >= scores_stride) return;
     float sum[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) sum[e] = 0.f;
     const bool full = (j0 + 8 <= scores_stride) && ((scores_stride & 7) == 0);
     if (j0 < len) {   // codes and references beyond the sequence were never written
-#pragma unroll
-        for (int h = 0; h < kGroupSize; ++h) {
-            const float* row = scores + ((size_t)b * nheads + g * kGroupSize + h) * scores_stride;
+        for (int h = 0; h < gs; ++h) {
+            const float* row = scores + ((size_t)b * nheads + g * gs + h) * scores_stride;
             const uint16_t* sp = reinterpret_cast<const uint16_t*>(row) + j0;
-            const float ref = row[scores_stride / 2 + (j0 >> 6)] - lse[h];
+            const float ref = row[scores_stride / 2 + (j0 >> 6)] - s_lse[h];
             uint32_t q[8];
             if (full) {
                 const uint4_t raw = ld_global_16(sp);
@@ -880,22 +886,29 @@ __global__ __launch_bounds__(256) void decode_aggregate_kernel(const float* __re
 
 namespace {
 
-template <int D, typename T>
-hipError_t launch_split_t(const DecodeParams& p, bool gather, bool with_v, bool write_scores, hipStream_t stream) {
+template <int D, typename T, int HS>
+hipError_t launch_split_hs(const DecodeParams& p, bool gather, bool with_v, bool write_scores, hipStream_t stream) {
     dim3 grid(p.G, p.num_split, p.B), block(kThreads);
     if (gather && p.idx_physical) {
-        hipLaunchKernelGGL((decode_split_kernel<true, true, false, true, D, T>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((decode_split_kernel<true, true, false, true, D, T, HS>), grid, block, 0, stream, p);
     } else if (gather) {
-        hipLaunchKernelGGL((decode_split_kernel<true, true, false, false, D, T>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((decode_split_kernel<true, true, false, false, D, T, HS>), grid, block, 0, stream, p);
     } else if (write_scores) {
         if (with_v)
-            hipLaunchKernelGGL((decode_split_kernel<false, true, true, false, D, T>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((decode_split_kernel<false, true, true, false, D, T, HS>), grid, block, 0, stream, p);
         else
-            hipLaunchKernelGGL((decode_split_kernel<false, false, true, false, D, T>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((decode_split_kernel<false, false, true, false, D, T, HS>), grid, block, 0, stream, p);
     } else {
-        hipLaunchKernelGGL((decode_split_kernel<false, true, false, false, D, T>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((decode_split_kernel<false, true, false, false, D, T, HS>), grid, block, 0, stream, p);
     }
     return hipGetLastError();
+}
+
+template <int D, typename T>
+hipError_t launch_split_t(const DecodeParams& p, bool gather, bool with_v, bool write_scores, hipStream_t stream) {
+    if (p.gs <= 4) return launch_split_hs<D, T, 4>(p, gather, with_v, write_scores, stream);
+    if (p.gs <= 8) return launch_split_hs<D, T, 8>(p, gather, with_v, write_scores, stream);
+    return launch_split_hs<D, T, 16>(p, gather, with_v, write_scores, stream);
 }
 
 template <int D, typename T>
@@ -937,11 +950,11 @@ hipError_t launch_decode_combine(const float* glse, const float* opart, void* ou
 
 hipError_t launch_decode_aggregate(const float* scores, const float* row_sums_in, const float* glse,
                                    int num_split, float* row_sums_out, const int* seqlens,
-                                   half_t* agg, int batch, int groups, int scores_stride, int uniform_len,
-                                   int len_cap, hipStream_t stream) {
+                                   half_t* agg, int batch, int groups, int group_size, int scores_stride,
+                                   int uniform_len, int len_cap, hipStream_t stream) {
     dim3 grid((scores_stride + 2047) / 2048, groups, batch), block(256);
     hipLaunchKernelGGL(decode_aggregate_kernel, grid, block, 0, stream, scores, row_sums_in, glse,
-                       num_split, row_sums_out, seqlens, agg, scores_stride, uniform_len, len_cap);
+                       num_split, row_sums_out, seqlens, agg, group_size, scores_stride, uniform_len, len_cap);
     return hipGetLastError();
 }
 

@@ -13,7 +13,7 @@ hipError_t launch_paged_kv_append(half_t* Kp, half_t* Vp, const half_t* k_new, c
 hipError_t launch_decode_budgets(int* seqlens, int advance, float percent, int batch, int groups,
                                  int* valid_rows, int* n_sel_rows, hipStream_t stream);
 
-struct RopeAppendParams {   // element tensors are fp16 or bf16 (elem), H = 4G query heads
+struct RopeAppendParams {   // element tensors are fp16 or bf16 (elem), H = gs G query heads
     const void* q_in;         // [B,n,H,D] through (q_sb, q_sl, q_sh)
     const void* k_in;         // [B,n,G,D] through (kv_sb, kv_sl, kv_sh); v_in shares the strides
     const void* v_in;
@@ -28,7 +28,7 @@ struct RopeAppendParams {   // element tensors are fp16 or bf16 (elem), H = 4G q
     long long q_sb, q_sl, q_sh, kv_sb, kv_sl, kv_sh;
     float eps;
     int pos_offset, batch, n_new, max_pages, page_shift, max_pos;
-    int G, head_dim, elem;
+    int G, head_dim, elem, gs;
 };
 
 hipError_t launch_rope_append(const RopeAppendParams& p, hipStream_t stream);

@@ -53,8 +53,8 @@ __global__ __launch_bounds__(256) void decode_budgets_kernel(int* __restrict__ s
 }
 
 
-// One workgroup per token, one row of D/8 lanes per head: 4G query heads, G key heads, G value
-// heads = 6G rows, taken 256/(D/8) at a time, three at once (the reference's shape is one trip:
+// One workgroup per token, one row of D/8 lanes per head: H query heads, G key heads, G value
+// heads = H + 2G rows, taken 256/(D/8) at a time, three at once (the reference's shape is one trip:
 // two query heads and a key or value head per row of lanes).  Query and key heads are
 // (optionally) RMS-normalised over the head dimension, then rotated by the token's position in
 // the "rotate half" pairing (i, i + D/2): the partner element sits D/16 lanes away in the row.
@@ -71,7 +71,7 @@ __global__ __launch_bounds__(256) void rope_append_kernel(RopeAppendParams p) {
     const int pos = p.start_pos[b] + p.pos_offset + t;
     if (pos < 0) return;
     const bool cache_ok = (pos >> p.page_shift) < p.max_pages;
-    const int G = p.G, Hq = kGroupSize * G, nrows = Hq + 2 * G;
+    const int G = p.G, Hq = p.gs * G, nrows = Hq + 2 * G;
     const T* q_in = static_cast<const T*>(p.q_in);
     const T* k_in = static_cast<const T*>(p.k_in);
     const T* v_in = static_cast<const T*>(p.v_in);

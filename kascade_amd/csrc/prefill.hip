@@ -110,7 +110,8 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
     constexpr int kKT = G_::kKT, kKS = G_::kKS, kDB = G_::kDB, kKB = G_::kKB, kChunks = G_::kChunks;
     constexpr int kRPL = G_::kRowsPerLoad, kTileElems = G_::kTileElems;
     constexpr float kScaleLog2 = ScaleLog2<D>::value;
-    const int kvh = p.G, nheads = p.G * kGroupSize;
+    const HeadSlots hs = head_slots(p.gs);
+    const int kvh = p.G, nheads = p.G * hs.gs;
     const T* Qp = (const T*)p.Q;
     const T* Kp = (const T*)p.K;
     const T* Vp = (const T*)p.V;
@@ -120,7 +121,9 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
     const int Lq = p.Lq;
     const int nqt = (Lq + QT - 1) / QT;
     int blk, g, b;
-    unit_of_workgroup(p.B, p.G, nqt, blk, g, b);
+    unit_of_workgroup(p.B, p.G << hs.vshift, nqt, blk, g, b);   // g: KV head and sub-group
+    const int sub = g & ((1 << hs.vshift) - 1);
+    g >>= hs.vshift;                // the KV head
     const int tq = nqt - 1 - blk;   // long (late) query blocks first
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
@@ -129,7 +132,8 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
     const int lg = lane >> 5;
     const int q0l = tq * QT;            // first query row of this block
     const int q0 = p.q_start + q0l;     // its global position
-    const int head = g * kGroupSize + wave;
+    const int head = g * hs.gs + 4 * sub + (wave & hs.slot_mask);
+    const bool real_head = wave <= hs.slot_mask;   // a repeated head computes along and stores nothing
 
     // ---- key regime of this block ----
     bool sparse = false;
@@ -487,7 +491,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
     for (int qb = 0; qb < NQB; ++qb) {
         const int ql = q0l + 32 * qb + li;
         const float lt = sum_with_other_half(l[qb]);
-        if (p.log_sum && lg == 0 && ql < Lq)
+        if (p.log_sum && lg == 0 && ql < Lq && real_head)
             p.log_sum[((long long)b * Lq + ql) * nheads + head] = fast_log2(lt) + m[qb];
         if (WITH_V) {
             T* so = sK + wave * (32 * D);
@@ -506,7 +510,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
                 const int r = j * kRPL + lrow;
                 const uint4_t row = *reinterpret_cast<const uint4_t*>(&so[r * D + lchunk * 8]);
                 const int qr = q0l + r;
-                if (qr < Lq)   // the output is not read again by these kernels: keep it out of the caches
+                if (qr < Lq && real_head)   // the output is not read again by these kernels: keep it out of the caches
                     __builtin_nontemporal_store(row, reinterpret_cast<uint4_t*>(
                         (T*)p.O + (((long long)b * Lq + qr) * nheads + head) * D + ((lchunk ^ (r & (kChunks - 1))) * 8)));
             }
@@ -558,7 +562,8 @@ void prefill_aggregate_kernel(PrefillParams p) {
     constexpr int kLoads = 32 / kRPL;           // load instructions per wavefront and tile
     constexpr int kWaveElems = 32 * D;          // a wavefront's 32 rows
     constexpr float kScaleLog2 = ScaleLog2<D>::value;
-    const int kvh = p.G, nheads = p.G * kGroupSize;
+    const HeadSlots hs = head_slots(p.gs);
+    const int kvh = p.G, nheads = p.G * hs.gs;
     const T* Qp = (const T*)p.Q;
     const T* Kp = (const T*)p.K;
     __shared__ __attribute__((aligned(1024))) T sK[2 * 4 * kWaveElems];
@@ -581,14 +586,15 @@ void prefill_aggregate_kernel(PrefillParams p) {
 
     const int ntiles = (ts + kAggKT - 1) / kAggKT;
     if (ntiles > 0) {
-        // A operands: row block rb = q-head 4g+rb, row li = query tl+li
+        // A operands: row block rb = head slot rb of this launch's sub-group, row li = query tl+li
+        const int head0 = g * hs.gs + 4 * p.vsub;
         x8_t qa[kGroupSize][kKS];
 #pragma unroll
         for (int rb = 0; rb < kGroupSize; ++rb) {
             const int q = tl + li;
             const bool ok = q < Lq;
             const T* qp = Qp + (long long)b * p.q_sb + (long long)min(q, Lq - 1) * p.q_sl +
-                          (long long)(g * kGroupSize + rb) * p.q_sh + lg * 8;
+                          (long long)(head0 + (rb & hs.slot_mask)) * p.q_sh + lg * 8;
 #pragma unroll
             for (int ks = 0; ks < kKS; ++ks) {
                 PackT<T> x;
@@ -599,7 +605,7 @@ void prefill_aggregate_kernel(PrefillParams p) {
         }
         if (tid < 128) {
             const int q = tl + (tid & 31);
-            s_lse[tid] = (q < Lq) ? p.log_sum_in[((long long)b * Lq + q) * nheads + g * kGroupSize + (tid >> 5)]
+            s_lse[tid] = (q < Lq) ? p.log_sum_in[((long long)b * Lq + q) * nheads + head0 + ((tid >> 5) & hs.slot_mask)]
                                   : INFINITY;
         }
 
@@ -681,11 +687,11 @@ void prefill_aggregate_kernel(PrefillParams p) {
                     for (int e = 0; e < 4; ++e)
                         sum += fast_exp2(acc[rb][4 * v4 + e] * kScaleLog2 - ls[e]);
                 }
-            sum = sum_with_other_half(sum);
+            sum = sum_with_other_half(sum) * hs.pool_scale;
             const int key = ti * kAggKT + 32 * wave + li;
             if (lg == 0 && key < L) {
-                if (key < ts)
-                    out[key] = (half_t)sum;
+                if (key < ts)   // a later sub-group of the KV head adds to what the earlier ones left
+                    out[key] = (half_t)(p.accumulate ? sum + (float)out[key] : sum);
                 else if (p.fill_invalid)
                     out[key] = neg_inf;
             }
@@ -706,9 +712,10 @@ hipError_t launch_attn_t(const PrefillParams& p, bool reuse, bool with_v, int nq
     const int qt = 32 * nqb;
     const bool paged = p.block_table != nullptr;
     const int nqt = (p.Lq + qt - 1) / qt;
-    dim3 grid(nqt, p.G, p.B), block(kThreads);
-    if (pairs_fill_xcds(p.B, p.G)) {
-        const long long total = (long long)nqt * p.G * p.B;
+    const int gv = p.G << head_slots(p.gs).vshift;   // (KV head, sub-group of four query heads) pairs
+    dim3 grid(nqt, gv, p.B), block(kThreads);
+    if (pairs_fill_xcds(p.B, gv)) {
+        const long long total = (long long)nqt * gv * p.B;
         if (total > 0x7fffffffLL) return hipErrorInvalidConfiguration;
         grid = dim3((unsigned)total);
     }
@@ -759,10 +766,22 @@ hipError_t launch_prefill_attn(const PrefillParams& p, bool reuse, bool with_v, 
                                : launch_attn_t<64, half_t>(p, reuse, with_v, nqb, stream);
 }
 
-hipError_t launch_prefill_aggregate(const PrefillParams& p, hipStream_t stream) {
-    if (p.head_dim == 128)
-        return p.elem == kElemBF16 ? launch_aggregate_t<128, bf16_t>(p, stream) : launch_aggregate_t<128, half_t>(p, stream);
-    return p.elem == kElemBF16 ? launch_aggregate_t<64, bf16_t>(p, stream) : launch_aggregate_t<64, half_t>(p, stream);
+hipError_t launch_prefill_aggregate(const PrefillParams& p0, hipStream_t stream) {
+    // one launch per sub-group of four query heads; the launches after the first add to the
+    // pooled scores (launches on a stream run in order)
+    PrefillParams p = p0;
+    const int subs = 1 << head_slots(p.gs).vshift;
+    for (int v = 0; v < subs; ++v) {
+        p.vsub = v;
+        p.accumulate = v > 0;
+        hipError_t e;
+        if (p.head_dim == 128)
+            e = p.elem == kElemBF16 ? launch_aggregate_t<128, bf16_t>(p, stream) : launch_aggregate_t<128, half_t>(p, stream);
+        else
+            e = p.elem == kElemBF16 ? launch_aggregate_t<64, bf16_t>(p, stream) : launch_aggregate_t<64, half_t>(p, stream);
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
 }
 
 // idx[i] (token position) -> physical row of the paged cache, in place or to another buffer.

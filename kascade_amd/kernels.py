@@ -23,20 +23,21 @@ from ._lib import Strides, KascadeError
 from . import budgets
 
 H, G, D, TILE = 32, 8, 128, 32      # the reference's shape (EfficientKascadeStrategy.py:19-21)
-GROUP = 4                             # query heads per KV head, for every shape
+GROUP = 4                             # query heads per KV head of the reference's shape
+GROUPS_OK = (1, 2, 4, 8, 16)          # ... and what the kernels take
 _ELEM = {torch.float16: 0, torch.bfloat16: 1}
 
 
 def _shape(Q: torch.Tensor, K: torch.Tensor):
     """(query heads, KV heads, head_dim, dtype) of a call, from Q [..., H, D] and K [..., G, D]:
-    fp16 or bf16, head_dim 64 or 128, four query heads per KV head."""
+    fp16 or bf16, head_dim 64 or 128, 1, 2, 4, 8 or 16 query heads per KV head."""
     Hq, Dh, Gk = Q.shape[-2], Q.shape[-1], K.shape[-2]
     if Q.dtype not in _ELEM or K.dtype != Q.dtype:
         raise KascadeError(f"Q and K must both be float16 or bfloat16, got {Q.dtype} / {K.dtype}")
     if Dh not in (64, 128) or K.shape[-1] != Dh:
         raise KascadeError(f"head_dim must be 64 or 128 for Q and K, got {Dh} / {K.shape[-1]}")
-    if Gk < 1 or Hq != GROUP * Gk:
-        raise KascadeError(f"need {GROUP} query heads per KV head, got {Hq} query / {Gk} KV heads")
+    if Gk < 1 or Hq % Gk or Hq // Gk not in GROUPS_OK:
+        raise KascadeError(f"need 1, 2, 4, 8 or 16 query heads per KV head, got {Hq} query / {Gk} KV heads")
     return Hq, Gk, Dh, Q.dtype
 
 
@@ -45,8 +46,8 @@ _entry = {}     # (name, shaped) -> bound library function: attribute look-ups a
 
 def _call(lib, name: str, shape, *args):
     """The plain entry point for the reference's shape, its *_shaped_call twin otherwise."""
-    _, Gk, Dh, dt = shape
-    if Gk == G and Dh == D and dt is torch.float16:
+    Hq, Gk, Dh, dt = shape
+    if Gk == G and Dh == D and dt is torch.float16 and Hq == H:
         fn = _entry.get((name, False))
         if fn is None:
             fn = _entry[(name, False)] = getattr(lib, f"kascade_{name}_call")
@@ -54,7 +55,7 @@ def _call(lib, name: str, shape, *args):
     fn = _entry.get((name, True))
     if fn is None:
         fn = _entry[(name, True)] = getattr(lib, f"kascade_{name}_shaped_call")
-    return fn(ctypes.byref(_lib.Shape(Gk, Dh, _ELEM[dt])), *args)
+    return fn(ctypes.byref(_lib.Shape(Gk, Dh, _ELEM[dt], Hq // Gk)), *args)
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)

@@ -30,10 +30,12 @@ class KascadeAttentionStack:
     def __init__(self, num_layers: int, recompute_layers: Sequence[int], head_mapping: List[List[int]],
                  k: float, max_seqlen: int, batch: int = 1, page_size: int = 16,
                  rolling_prefill: bool = True, device="cuda", table_seed: int = 0,
-                 dense: bool = False, kv_heads: int = G, head_dim: int = D, dtype=torch.float16):
+                 dense: bool = False, kv_heads: int = G, head_dim: int = D, dtype=torch.float16,
+                 group_size: int = kernels.GROUP):
         """dense=True runs every layer as dense attention over the same caches (the baseline).
-        kv_heads, head_dim, dtype: the model's shape (4 * kv_heads query heads; head_dim 64 or
-        128; float16 or bfloat16); the default is the reference's."""
+        kv_heads, head_dim, dtype, group_size: the model's shape (group_size * kv_heads query
+        heads, group_size 1, 2, 4, 8 or 16; head_dim 64 or 128; float16 or bfloat16); the default
+        is the reference's."""
         if 0 not in recompute_layers and not dense:
             raise KascadeError("layer 0 must be an anchor layer")
         self.num_layers, self.batch, self.page_size = num_layers, batch, page_size
@@ -41,7 +43,7 @@ class KascadeAttentionStack:
         self.dense_only = dense
         self.device = torch.device(device)
         self.max_seqlen = max_seqlen
-        self.G, self.H, self.D, self.dtype = kv_heads, kernels.GROUP * kv_heads, head_dim, dtype
+        self.G, self.H, self.D, self.dtype = kv_heads, group_size * kv_heads, head_dim, dtype
         pages_per_seq = math.ceil(max_seqlen / page_size)
         n_pages = batch * pages_per_seq
         gen = torch.Generator().manual_seed(table_seed)
@@ -55,7 +57,8 @@ class KascadeAttentionStack:
         self.prefill = PagedKascadePrefill(k, head_mapping, recompute_layers, page_size, rolling_prefill,
                                            self.device, kv_heads=kv_heads)
         self.decoder = PagedKascadeDecoder(k, head_mapping, recompute_layers, batch, max_seqlen, page_size,
-                                           self.device, kv_heads=kv_heads, head_dim=head_dim)
+                                           self.device, kv_heads=kv_heads, head_dim=head_dim,
+                                           group_size=group_size)
         self._graph = None
 
     def reset(self, length: int = 0):

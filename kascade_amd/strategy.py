@@ -186,11 +186,12 @@ class EfficientKascadeStrategy:
             return ALL_ATTENTION_FUNCTIONS["sdpa"](module, query, key, value, attention_mask,
                                                    scaling=scaling, dropout=dropout, **kwargs)
         # the reference's kernels exist for fp16, 32 query / 8 KV heads, head_dim 128 only
-        # (EfficientKascadeStrategy.py:19-21); here any model with four query heads per KV head,
-        # head_dim 64 or 128, in fp16 or bf16
-        if query.shape[1] != 4 * key.shape[1] or query.shape[-1] not in (64, 128) \
-                or query.dtype not in (torch.float16, torch.bfloat16):
-            raise KascadeError("efficient_kascade needs fp16 or bf16, four query heads per KV head, head_dim 64 or 128")
+        # (EfficientKascadeStrategy.py:19-21); here any model with 1, 2, 4, 8 or 16 query heads per
+        # KV head, head_dim 64 or 128, in fp16 or bf16
+        if query.shape[1] % key.shape[1] or query.shape[1] // key.shape[1] not in kernels.GROUPS_OK \
+                or query.shape[-1] not in (64, 128) or query.dtype not in (torch.float16, torch.bfloat16):
+            raise KascadeError("efficient_kascade needs fp16 or bf16, 1, 2, 4, 8 or 16 query heads per KV head, "
+                               "head_dim 64 or 128")
         is_decode = (query.shape[2] == 1)
         Lk = key.shape[-2]
         rounded_k = budgets.topk_width(Lk, self.k)
@@ -245,9 +246,10 @@ class PagedKascadeDecoder:
                  max_batch: int, max_seqlen: int, page_size: int = 16, device="cuda",
                  num_split_dense: Optional[int] = None, num_split_reuse: Optional[int] = None,
                  total_tokens: Optional[int] = None, fused_combine: bool = True,
-                 seqlens_hint: Optional[Sequence[int]] = None, kv_heads: int = G, head_dim: int = D):
-        """kv_heads, head_dim: the model's shape (query heads = 4 * kv_heads; the element type is
-        that of the tensors of each call).
+                 seqlens_hint: Optional[Sequence[int]] = None, kv_heads: int = G, head_dim: int = D,
+                 group_size: int = kernels.GROUP):
+        """kv_heads, head_dim, group_size: the model's shape (query heads = group_size * kv_heads;
+        the element type is that of the tensors of each call).
         fused_combine: merge the splits inside the split launch (one launch fewer per layer).
         total_tokens: expected sum of the sequence lengths of a batch (default
         max_batch*max_seqlen); with ragged batches it sizes the splits so that the non-empty
@@ -261,7 +263,7 @@ class PagedKascadeDecoder:
         self.device = torch.device(device)
         self.max_batch, self.max_seqlen = max_batch, max_seqlen
         G, D = kv_heads, head_dim            # this model's, from here on
-        H = kernels.GROUP * G
+        H = group_size * G
         self.G, self.H, self.D = G, H, D
         self.stride = ((max_seqlen + 7) // 8) * 8
         self.max_topk = budgets.decode_budget(max_seqlen, k)

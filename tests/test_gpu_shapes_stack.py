@@ -1,4 +1,5 @@
-"""Other tensor shapes than the reference's through the rest of the path: the projection ->
+"""Other tensor shapes than the reference's (KV-head count, head_dim 64, bf16, 1 / 2 / 8 / 16
+query heads per KV head) through the rest of the path: the projection ->
 attention hand-off kernel, the chunked prefill over the paged cache, the attention stack (chunked
 prefill + eager / graph-replayed decode) and the decoder blocks over it.
 
@@ -21,6 +22,8 @@ SHAPES = [  # (query heads, KV heads, head_dim, dtype)
     (8, 2, 64, torch.float16), (8, 2, 64, torch.bfloat16), (32, 8, 128, torch.bfloat16),
     (12, 3, 128, torch.float16), (4, 1, 64, torch.bfloat16), (64, 16, 64, torch.float16),
     (160, 40, 128, torch.bfloat16),     # 240 rows per token: more than one trip of the hand-off kernel
+    # other numbers of query heads per KV head: 8, 1, 2, 16
+    (32, 4, 128, torch.bfloat16), (8, 8, 128, torch.float16), (8, 4, 64, torch.bfloat16), (32, 2, 64, torch.float16),
 ]
 
 
@@ -108,7 +111,7 @@ def test_decode_budgets_other_kv_head_counts(cuda):
 
 
 # ------------------------------------------------------------------ chunked prefill
-@pytest.mark.parametrize("H,G,D,dt", SHAPES[:6])
+@pytest.mark.parametrize("H,G,D,dt", SHAPES[:6] + SHAPES[7:])
 def test_chunked_kernels_equal_whole_prompt_other_shapes(cuda, H, G, D, dt):
     """Every chunk's rows equal the rows of the whole-prompt calls (which test_gpu_shapes.py checks
     against the oracle), bit for bit, for dense / log-sum / pooled scores / reuse."""
@@ -166,7 +169,9 @@ def _maps(G):
 
 
 @pytest.mark.parametrize("H,G,D,dt", [(8, 2, 64, torch.float16), (8, 2, 64, torch.bfloat16),
-                                      (32, 8, 128, torch.bfloat16), (12, 3, 128, torch.float16)])
+                                      (32, 8, 128, torch.bfloat16), (12, 3, 128, torch.float16),
+                                      (32, 4, 128, torch.bfloat16), (4, 2, 64, torch.float16),
+                                      (3, 3, 128, torch.float16), (32, 2, 64, torch.bfloat16)])
 def test_attention_stack_other_shapes(cuda, H, G, D, dt):
     """Chunked prefill equals the whole-prompt strategy calls bit for bit; decode steps: replayed
     graph equals eager launches bit for bit, layer 0 equals dense decode and the reuse layers the
@@ -189,7 +194,7 @@ def test_attention_stack_other_shapes(cuda, H, G, D, dt):
     def make():
         return KascadeAttentionStack(N_LAYERS, ANCHORS, maps, P, PROMPT + 32, batch=1, page_size=16,
                                      rolling_prefill=True, device=cuda, table_seed=1, kv_heads=G, head_dim=D,
-                                     dtype=dt)
+                                     dtype=dt, group_size=H // G)
 
     def prefill(st):
         outs = [[] for _ in range(N_LAYERS)]
@@ -246,7 +251,8 @@ def test_attention_stack_other_shapes(cuda, H, G, D, dt):
 
 # ------------------------------------------------------------------ decoder blocks
 @pytest.mark.parametrize("H,G,D,dt", [(8, 2, 64, torch.float16), (8, 2, 64, torch.bfloat16),
-                                      (32, 8, 128, torch.bfloat16)])
+                                      (32, 8, 128, torch.bfloat16), (16, 2, 128, torch.float16),
+                                      (4, 2, 64, torch.bfloat16)])
 def test_blocks_other_shapes(cuda, H, G, D, dt):
     """Dense blocks against the fp32 oracle; 100 % selection equals dense; graph replay equals eager."""
     from kascade_amd.blocks import KascadeBlockStack
@@ -258,7 +264,7 @@ def test_blocks_other_shapes(cuda, H, G, D, dt):
     def make(k, max_len, dense):
         return KascadeBlockStack(layers, anchors, maps, k, max_len, hidden=hidden, batch=1, page_size=16,
                                  rolling_prefill=True, device=cuda, table_seed=3, dense=dense, weight_seed=7,
-                                 qk_norm=True, kv_heads=G, head_dim=D, dtype=dt)
+                                 qk_norm=True, kv_heads=G, head_dim=D, dtype=dt, group_size=H // G)
 
     def run(st, x, prompt, chunk, steps):
         outs = []
