@@ -57,7 +57,7 @@ typedef struct {
     int32_t kv_heads;   /* >= 1 */
     int32_t head_dim;   /* 64 or 128 */
     int32_t dtype;      /* KASCADE_F16 or KASCADE_BF16 */
-    int32_t group_size; /* query heads per KV head: 1, 2, 4, 8 or 16; 0 means 4 */
+    int32_t group_size; /* query heads per KV head: 1 to 16; 0 means 4 */
 } kascade_shape;
 
 /* Replaces `init()` of every reference kernel object (e.g. decode reuse .cu:253-258):

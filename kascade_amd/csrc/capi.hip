@@ -96,8 +96,8 @@ int get_shape(const kascade_shape* in, Shape* out) {
     REQUIRE(in->head_dim == 64 || in->head_dim == 128, "shape: head_dim must be 64 or 128, got %d", in->head_dim);
     REQUIRE(in->dtype == KASCADE_F16 || in->dtype == KASCADE_BF16, "shape: dtype must be KASCADE_F16 or KASCADE_BF16");
     const int gs = in->group_size == 0 ? kGroupSize : in->group_size;
-    REQUIRE(gs == 1 || gs == 2 || gs == 4 || gs == 8 || gs == 16,
-            "shape: group_size (query heads per KV head) must be 1, 2, 4, 8 or 16 (0 = 4), got %d", in->group_size);
+    REQUIRE(gs >= 1 && gs <= 16,
+            "shape: group_size (query heads per KV head) must be 1 to 16 (0 = 4), got %d", in->group_size);
     REQUIRE((long long)in->kv_heads * gs <= 65535, "shape: too many query heads");
     out->G = in->kv_heads; out->D = in->head_dim; out->elem = in->dtype == KASCADE_BF16 ? kElemBF16 : kElemF16;
     out->gs = gs;

@@ -48,7 +48,7 @@ struct DecodeParams {
     int G;                  // KV heads
     int head_dim;           // 64 or 128
     int elem;               // kElemF16 or kElemBF16
-    int gs;                 // query heads per KV head: 1, 2, 4, 8 or 16
+    int gs;                 // query heads per KV head: 1 to 16
 };
 
 hipError_t launch_decode_split(const DecodeParams& p, bool gather, bool with_v, bool write_scores,

@@ -9,11 +9,11 @@ struct PrefillParams {
     // [0, L), L = q_start + Lq.  A whole-prompt call has q_start = 0 and Lq = L.
     // Q, K, V and O hold elements of kind `elem` (fp16 or bf16); G KV heads, H = gs G query heads,
     // head dimension head_dim (64 or 128).  A workgroup always works on four head slots of one
-    // KV head.  gs >= 4: the KV head's query heads are taken four at a time, gs/4 "sub-groups" --
+    // KV head: the KV head's gs query heads are taken four at a time, ceil(gs/4) "sub-groups" --
     // the attention kernels launch one workgroup per (KV head, sub-group), the pooling kernel is
-    // launched once per sub-group (vsub) and adds to the pooled scores of the earlier ones.
-    // gs < 4: the slots beyond gs repeat the KV head's query heads; their outputs are dropped and
-    // the pooled sums, which count every head 4/gs times, are scaled back.
+    // launched once per sub-group (vsub) and adds to the pooled scores of the earlier ones.  A
+    // slot beyond the KV head's last query head computes along on that head's data and leaves
+    // nothing behind: no output, no log-sum, nothing in the pooled sums.
     const void* Q;            // [B,Lq,H,D] through (q_sb, q_sl, q_sh)
     const void* K;            // [B,L,G,D] through (k_sb, k_sl, k_sh); V shares the strides.
     const void* V;            //   Paged: [num_pages, page, G, D] contiguous, strides unused
@@ -36,23 +36,17 @@ struct PrefillParams {
     int G;                    // KV heads
     int head_dim;             // 64 or 128
     int elem;                 // kElemF16 or kElemBF16
-    int gs;                   // query heads per KV head: 1, 2, 4, 8 or 16 (0 = 4)
+    int gs;                   // query heads per KV head: 1 to 16 (0 = 4)
     int vsub, accumulate;     // pooling kernel: sub-group of this launch; add to what agg holds
 };
 
-// Derived from gs: log2 of the sub-groups per KV head, and the mask that folds a slot onto a head.
+// Query heads per KV head and the sub-groups of four head slots they take.
 struct HeadSlots {
-    int gs, vshift, slot_mask;
-    float pool_scale;
+    int gs, subs;
 };
 __host__ __device__ inline HeadSlots head_slots(int gs) {
     if (gs <= 0) gs = 4;
-    HeadSlots h;
-    h.gs = gs;
-    h.vshift = gs >= 16 ? 2 : gs >= 8 ? 1 : 0;
-    h.slot_mask = gs >= 4 ? 3 : gs - 1;
-    h.pool_scale = gs >= 4 ? 1.f : (float)gs * 0.25f;
-    return h;
+    return HeadSlots{gs, (gs + 3) / 4};
 }
 
 hipError_t launch_prefill_attn(const PrefillParams& p, bool reuse, bool with_v, int nqb,

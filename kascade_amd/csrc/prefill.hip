@@ -121,9 +121,12 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
     const int Lq = p.Lq;
     const int nqt = (Lq + QT - 1) / QT;
     int blk, g, b;
-    unit_of_workgroup(p.B, p.G << hs.vshift, nqt, blk, g, b);   // g: KV head and sub-group
-    const int sub = g & ((1 << hs.vshift) - 1);
-    g >>= hs.vshift;                // the KV head
+    unit_of_workgroup(p.B, p.G * hs.subs, nqt, blk, g, b);   // g: KV head and sub-group
+    int sub = 0;
+    if (hs.subs > 1) {
+        sub = g % hs.subs;
+        g /= hs.subs;               // the KV head
+    }
     const int tq = nqt - 1 - blk;   // long (late) query blocks first
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
@@ -132,8 +135,8 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
     const int lg = lane >> 5;
     const int q0l = tq * QT;            // first query row of this block
     const int q0 = p.q_start + q0l;     // its global position
-    const int head = g * hs.gs + 4 * sub + (wave & hs.slot_mask);
-    const bool real_head = wave <= hs.slot_mask;   // a repeated head computes along and stores nothing
+    const int head = g * hs.gs + min(4 * sub + wave, hs.gs - 1);
+    const bool real_head = 4 * sub + wave < hs.gs;   // a slot beyond the last head computes along and stores nothing
 
     // ---- key regime of this block ----
     bool sparse = false;
@@ -594,7 +597,7 @@ void prefill_aggregate_kernel(PrefillParams p) {
             const int q = tl + li;
             const bool ok = q < Lq;
             const T* qp = Qp + (long long)b * p.q_sb + (long long)min(q, Lq - 1) * p.q_sl +
-                          (long long)(head0 + (rb & hs.slot_mask)) * p.q_sh + lg * 8;
+                          (long long)min(head0 + rb, g * hs.gs + hs.gs - 1) * p.q_sh + lg * 8;
 #pragma unroll
             for (int ks = 0; ks < kKS; ++ks) {
                 PackT<T> x;
@@ -605,8 +608,9 @@ void prefill_aggregate_kernel(PrefillParams p) {
         }
         if (tid < 128) {
             const int q = tl + (tid & 31);
-            s_lse[tid] = (q < Lq) ? p.log_sum_in[((long long)b * Lq + q) * nheads + head0 + ((tid >> 5) & hs.slot_mask)]
-                                  : INFINITY;
+            // a query row past the chunk, or a slot past the KV head's last query head, adds exp2(-inf) = 0
+            const bool counts = q < Lq && 4 * p.vsub + (tid >> 5) < hs.gs;
+            s_lse[tid] = counts ? p.log_sum_in[((long long)b * Lq + q) * nheads + head0 + (tid >> 5)] : INFINITY;
         }
 
         // ---- staging: load j of a tile covers rows j kRPL + lrow of the wavefront's 32 ----
@@ -687,7 +691,7 @@ void prefill_aggregate_kernel(PrefillParams p) {
                     for (int e = 0; e < 4; ++e)
                         sum += fast_exp2(acc[rb][4 * v4 + e] * kScaleLog2 - ls[e]);
                 }
-            sum = sum_with_other_half(sum) * hs.pool_scale;
+            sum = sum_with_other_half(sum);
             const int key = ti * kAggKT + 32 * wave + li;
             if (lg == 0 && key < L) {
                 if (key < ts)   // a later sub-group of the KV head adds to what the earlier ones left
@@ -712,7 +716,7 @@ hipError_t launch_attn_t(const PrefillParams& p, bool reuse, bool with_v, int nq
     const int qt = 32 * nqb;
     const bool paged = p.block_table != nullptr;
     const int nqt = (p.Lq + qt - 1) / qt;
-    const int gv = p.G << head_slots(p.gs).vshift;   // (KV head, sub-group of four query heads) pairs
+    const int gv = p.G * head_slots(p.gs).subs;   // (KV head, sub-group of four query heads) pairs
     dim3 grid(nqt, gv, p.B), block(kThreads);
     if (pairs_fill_xcds(p.B, gv)) {
         const long long total = (long long)nqt * gv * p.B;
@@ -770,7 +774,7 @@ hipError_t launch_prefill_aggregate(const PrefillParams& p0, hipStream_t stream)
     // one launch per sub-group of four query heads; the launches after the first add to the
     // pooled scores (launches on a stream run in order)
     PrefillParams p = p0;
-    const int subs = 1 << head_slots(p.gs).vshift;
+    const int subs = head_slots(p.gs).subs;
     for (int v = 0; v < subs; ++v) {
         p.vsub = v;
         p.accumulate = v > 0;

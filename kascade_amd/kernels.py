@@ -24,20 +24,20 @@ from . import budgets
 
 H, G, D, TILE = 32, 8, 128, 32      # the reference's shape (EfficientKascadeStrategy.py:19-21)
 GROUP = 4                             # query heads per KV head of the reference's shape
-GROUPS_OK = (1, 2, 4, 8, 16)          # ... and what the kernels take
+GROUPS_OK = tuple(range(1, 17))       # ... and what the kernels take
 _ELEM = {torch.float16: 0, torch.bfloat16: 1}
 
 
 def _shape(Q: torch.Tensor, K: torch.Tensor):
     """(query heads, KV heads, head_dim, dtype) of a call, from Q [..., H, D] and K [..., G, D]:
-    fp16 or bf16, head_dim 64 or 128, 1, 2, 4, 8 or 16 query heads per KV head."""
+    fp16 or bf16, head_dim 64 or 128, 1 to 16 query heads per KV head."""
     Hq, Dh, Gk = Q.shape[-2], Q.shape[-1], K.shape[-2]
     if Q.dtype not in _ELEM or K.dtype != Q.dtype:
         raise KascadeError(f"Q and K must both be float16 or bfloat16, got {Q.dtype} / {K.dtype}")
     if Dh not in (64, 128) or K.shape[-1] != Dh:
         raise KascadeError(f"head_dim must be 64 or 128 for Q and K, got {Dh} / {K.shape[-1]}")
     if Gk < 1 or Hq % Gk or Hq // Gk not in GROUPS_OK:
-        raise KascadeError(f"need 1, 2, 4, 8 or 16 query heads per KV head, got {Hq} query / {Gk} KV heads")
+        raise KascadeError(f"need 1 to 16 query heads per KV head, got {Hq} query / {Gk} KV heads")
     return Hq, Gk, Dh, Q.dtype
 
 

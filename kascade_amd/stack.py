@@ -34,7 +34,7 @@ class KascadeAttentionStack:
                  group_size: int = kernels.GROUP):
         """dense=True runs every layer as dense attention over the same caches (the baseline).
         kv_heads, head_dim, dtype, group_size: the model's shape (group_size * kv_heads query
-        heads, group_size 1, 2, 4, 8 or 16; head_dim 64 or 128; float16 or bfloat16); the default
+        heads, group_size 1 to 16; head_dim 64 or 128; float16 or bfloat16); the default
         is the reference's."""
         if 0 not in recompute_layers and not dense:
             raise KascadeError("layer 0 must be an anchor layer")

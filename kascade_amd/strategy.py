@@ -186,11 +186,11 @@ class EfficientKascadeStrategy:
             return ALL_ATTENTION_FUNCTIONS["sdpa"](module, query, key, value, attention_mask,
                                                    scaling=scaling, dropout=dropout, **kwargs)
         # the reference's kernels exist for fp16, 32 query / 8 KV heads, head_dim 128 only
-        # (EfficientKascadeStrategy.py:19-21); here any model with 1, 2, 4, 8 or 16 query heads per
-        # KV head, head_dim 64 or 128, in fp16 or bf16
+        # (EfficientKascadeStrategy.py:19-21); here any model with 1 to 16 query heads per KV head,
+        # head_dim 64 or 128, in fp16 or bf16
         if query.shape[1] % key.shape[1] or query.shape[1] // key.shape[1] not in kernels.GROUPS_OK \
                 or query.shape[-1] not in (64, 128) or query.dtype not in (torch.float16, torch.bfloat16):
-            raise KascadeError("efficient_kascade needs fp16 or bf16, 1, 2, 4, 8 or 16 query heads per KV head, "
+            raise KascadeError("efficient_kascade needs fp16 or bf16, 1 to 16 query heads per KV head, "
                                "head_dim 64 or 128")
         is_decode = (query.shape[2] == 1)
         Lk = key.shape[-2]

@@ -1,5 +1,5 @@
 """Other tensor shapes than the reference's (32 query / 8 KV heads, head_dim 128, fp16): bf16,
-head_dim 64, other KV-head counts, 1 / 2 / 8 / 16 query heads per KV head -- in particular the shape of the reference's CPU-runnable configuration (8 query / 2 KV
+head_dim 64, other KV-head counts, 1 to 16 query heads per KV head -- in particular the shape of the reference's CPU-runnable configuration (8 query / 2 KV
 heads, head_dim 64) -- through the shaped C entry points, against the CPU oracle.
 
 Tolerances.  fp16: the parity tolerances of every other test (outputs atol 2e-3 / rtol 1e-2,
@@ -26,6 +26,9 @@ SHAPES = [  # (query heads, KV heads, head_dim, dtype)
     # other numbers of query heads per KV head: 8, 8, 1, 2, 16, 2
     (16, 2, 64, torch.float16), (32, 4, 128, torch.bfloat16), (8, 8, 128, torch.float16),
     (8, 4, 64, torch.bfloat16), (32, 2, 128, torch.float16), (6, 3, 64, torch.float16),
+    # ... and numbers that do not fill their last group of four head slots: 3, 5, 7, 12, 6
+    (6, 2, 64, torch.float16), (20, 4, 128, torch.bfloat16), (28, 4, 128, torch.float16),
+    (12, 1, 64, torch.bfloat16), (12, 2, 128, torch.float16),
 ]
 
 

@@ -1,4 +1,4 @@
-"""Other tensor shapes than the reference's (KV-head count, head_dim 64, bf16, 1 / 2 / 8 / 16
+"""Other tensor shapes than the reference's (KV-head count, head_dim 64, bf16, 1 to 16
 query heads per KV head) through the rest of the path: the projection ->
 attention hand-off kernel, the chunked prefill over the paged cache, the attention stack (chunked
 prefill + eager / graph-replayed decode) and the decoder blocks over it.
@@ -24,6 +24,7 @@ SHAPES = [  # (query heads, KV heads, head_dim, dtype)
     (160, 40, 128, torch.bfloat16),     # 240 rows per token: more than one trip of the hand-off kernel
     # other numbers of query heads per KV head: 8, 1, 2, 16
     (32, 4, 128, torch.bfloat16), (8, 8, 128, torch.float16), (8, 4, 64, torch.bfloat16), (32, 2, 64, torch.float16),
+    (28, 4, 128, torch.bfloat16), (6, 2, 64, torch.float16),     # 7 and 3
 ]
 
 
@@ -171,7 +172,8 @@ def _maps(G):
 @pytest.mark.parametrize("H,G,D,dt", [(8, 2, 64, torch.float16), (8, 2, 64, torch.bfloat16),
                                       (32, 8, 128, torch.bfloat16), (12, 3, 128, torch.float16),
                                       (32, 4, 128, torch.bfloat16), (4, 2, 64, torch.float16),
-                                      (3, 3, 128, torch.float16), (32, 2, 64, torch.bfloat16)])
+                                      (3, 3, 128, torch.float16), (32, 2, 64, torch.bfloat16),
+                                      (28, 4, 128, torch.float16), (10, 2, 64, torch.bfloat16)])
 def test_attention_stack_other_shapes(cuda, H, G, D, dt):
     """Chunked prefill equals the whole-prompt strategy calls bit for bit; decode steps: replayed
     graph equals eager launches bit for bit, layer 0 equals dense decode and the reuse layers the
