@@ -207,6 +207,7 @@ def main():
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-stack", action="store_true", help="skip the 36-layer chunked-prefill + decode stack")
     ap.add_argument("--skip-ceilings", action="store_true", help="skip the library copy / gather / GEMM rates")
+    ap.add_argument("--skip-shapes", action="store_true", help="skip the timings at other head shapes")
     ap.add_argument("--decode-only", action="store_true", help="skip the per-kernel prefill section")
     ap.add_argument("--kernel", choices=sorted(SINGLE_KERNELS), default=None,
                     help="profiling mode: run only this kernel --iters times on its benchmark workload")
@@ -617,6 +618,67 @@ def main():
         torch.cuda.empty_cache()
 
     # ---------------------------------------------- what this device delivers to library kernels
+    # ------------------------------------------------------------------ other head shapes
+    # The layer mixes of configs[1] (32768-token prefill) and configs[2] (batch 16 x 65536 paged
+    # decode) at shapes the reference's kernels do not take: 64 query heads on 8 KV heads
+    # (Llama-3-70B / Qwen3-32B class), the reference's shape in bf16, 28 / 4 heads (Qwen2.5-7B).
+    # Gaussian inputs; selections are the anchors' own.
+    shapes = {}
+    if not args.skip_shapes and not args.decode_only and L == 32768:
+        torch.cuda.empty_cache()
+        n_anchor, n_reuse = len(ANCHORS) - 1, N_LAYERS - len(ANCHORS)
+        for Hs, Gs, Ds, dts, tag in ((64, 8, 128, torch.float16, "H64_G8_D128_f16"),
+                                     (32, 8, 128, torch.bfloat16, "H32_G8_D128_bf16"),
+                                     (28, 4, 128, torch.bfloat16, "H28_G4_D128_bf16")):
+            gen = torch.Generator(device=dev)
+            gen.manual_seed(Hs)
+            rnd = lambda *sh: torch.randn(*sh, device=dev, generator=gen).to(dts)
+            res = {}
+            # prefill
+            q, k, v = rnd(1, L, Hs, Ds), rnd(1, L, Gs, Ds), rnd(1, L, Gs, Ds)
+            hm = torch.arange(Gs, dtype=torch.int32, device=dev)
+            valid, nsel = budgets.prefill_tile_budgets(L, TILE, PCT, True, width)
+            valid_t = torch.tensor(valid, dtype=torch.int32, device=dev)
+            nsel_t = torch.tensor(nsel, dtype=torch.int32, device=dev)
+            sc = torch.empty(1, Gs, T, L, device=dev, dtype=torch.float16)
+            t_dense = ev_time(lambda: kernels.prefill_dense(q, k, v), n=3)
+            ls, _ = kernels.prefill_recompute0(q, k, v)
+
+            def select():
+                kernels.prefill_aggregate(q, k, ls, sc, fill_invalid=False)
+                return kernels.topk_indices(sc, width, valid_len=valid_t, n_sel=nsel_t)
+            idx = select()
+            t_sel = ev_time(select, n=3)
+            t_p0 = ev_time(lambda: kernels.prefill_recompute0(q, k, v), n=3)
+            t_p1 = ev_time(lambda: kernels.prefill_recompute1(q, k), n=3)
+            t_reuse = ev_time(lambda: kernels.prefill_reuse(q, k, v, idx, hm, float(PCT), True), n=5)
+            mix = ((t_p0 + t_sel) + n_anchor * (t_p1 + t_sel + t_reuse) + n_reuse * t_reuse) / N_LAYERS
+            res["prefill_32768"] = {"dense_ms": round(t_dense / 1e3, 3), "kascade_ms_per_layer": round(mix / 1e3, 3),
+                                    "speedup_vs_dense": round(t_dense / mix, 3), "reuse_ms": round(t_reuse / 1e3, 3)}
+            del q, k, v, sc, ls, idx
+            # decode
+            Bd, Ld, page = 16, 65536, 16
+            P = Bd * Ld // page
+            kp, vp = rnd(P, page, Gs, Ds), rnd(P, page, Gs, Ds)
+            bt = torch.randperm(P, device=dev).to(torch.int32).view(Bd, -1)
+            lens = torch.full((Bd,), Ld, dtype=torch.int32, device=dev)
+            qd = rnd(Bd, Hs, Ds)
+            dec = PagedKascadeDecoder(PCT, [list(range(Gs))] * 2, [0], Bd, Ld, page, dev, kv_heads=Gs, head_dim=Ds,
+                                      group_size=Hs // Gs)
+            out_d = torch.empty(Bd, Hs, Ds, device=dev, dtype=dts)
+            t_dd = ev_time(lambda: dec.dense(qd, kp, vp, bt, lens, Ld, out=out_d), n=5)
+            t_a0 = ev_time(lambda: dec.anchor(0, qd, kp, vp, bt, lens, Ld, ragged=True, out=out_d), n=5)
+            t_a1 = ev_time(lambda: dec.anchor(1, qd, kp, vp, bt, lens, Ld, ragged=True, out=out_d), n=5)
+            t_r = ev_time(lambda: dec.reuse(1, qd, kp, vp, bt, lens, out=out_d), n=5, reps=5)
+            mixd = (t_a0 + n_anchor * t_a1 + n_reuse * t_r) / N_LAYERS
+            res["decode_B16_L65536"] = {"dense_us": round(t_dd, 1), "anchor0_us": round(t_a0, 1), "anchor_us": round(t_a1, 1),
+                                        "reuse_us": round(t_r, 1), "kascade_us_per_layer": round(mixd, 1),
+                                        "speedup_vs_dense": round(t_dd / mixd, 3)}
+            del kp, vp, bt, dec, qd, out_d
+            torch.cuda.empty_cache()
+            shapes[tag] = res
+            log(f"[bench] shape {tag}: {res}")
+
     # Context for the roofline fractions (which are priced against the published peaks): library
     # routines on the same box in the same run -- a 1 GiB device copy, a streaming reduction, a
     # gather of random 256-byte rows (the reuse decode access pattern) and an fp16 GEMM on random
@@ -760,6 +822,7 @@ def main():
                    "seq_len": L, "layers_per_step": N_LAYERS,
                    "baseline_note": "vs_baseline = value / 6.42 ms, the reference's published H100 figure"},
         "roofline": roofline, "roofline_decode": roofline_decode or None, "cpu_baseline": cpu, "prefill": prefill, "prefill_long": prefill_long, "decode": decode, "stack": stack_res,
+        "other_shapes": shapes,
         "library_ceilings": ceilings,
         "kernels": kern,
     }
