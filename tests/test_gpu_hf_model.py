@@ -17,7 +17,7 @@ ANCHORS = [0, 2]
 HEAD_MAPS = [list(range(G)), [5, 0, 0, 3, 7, 1, 6, 2], list(range(G)), [1, 2, 3, 4, 5, 6, 7, 0]]
 
 
-def _tiny_model(cuda, family="llama"):
+def _tiny_model(cuda, family="llama", H=H, G=G, D=D, dtype=torch.float16):
     """Random-init decoder from a local config: Llama-shaped, or Qwen3-shaped (RMS-normalised
     query and key heads before the rotary embedding)."""
     kw = dict(hidden_size=256, intermediate_size=512, num_hidden_layers=len(HEAD_MAPS),
@@ -40,7 +40,7 @@ def _tiny_model(cuda, family="llama"):
             else:
                 layer.self_attn.q_norm.weight.mul_(2.5)
                 layer.self_attn.k_norm.weight.mul_(2.0)
-    return model.half().to(cuda)
+    return model.to(dtype).to(cuda)
 
 
 def _bld(x):   # HF layout [B,h,L,D] -> [B,L,h,D] on the CPU
@@ -132,3 +132,42 @@ def test_full_budget_equals_sdpa_model(cuda, family):
     scale = float(logits["sdpa"].std())
     assert scale > 0.05
     assert_close(logits[s.name], logits["sdpa"], "logits at k=100 vs SDPA", atol=2e-2 * scale, rtol=2e-2)
+
+
+@pytest.mark.parametrize("family,Hs,Gs,Ds,dt", [("qwen3", 14, 2, 64, torch.float16), ("qwen3", 14, 2, 64, torch.bfloat16),
+                                               ("llama", 16, 2, 128, torch.float16), ("llama", 8, 8, 64, torch.bfloat16)])
+def test_full_budget_equals_sdpa_model_other_shapes(cuda, family, Hs, Gs, Ds, dt):
+    """The same comparison for models of other shapes: 7, 8 and 1 query heads per KV head, head
+    dimension 64, bf16 weights.  fp16 at the tolerance of the test above.  Two bf16 implementations
+    of one model round at different places and drift apart over four layers; the yardstick is the
+    library itself: the distance between its own "eager" and "sdpa" attention on the same bf16
+    weights, and the registered function must stay within three times that of "sdpa"."""
+    from kascade_amd.strategy import EfficientKascadeStrategy
+    L, B = 500, 2
+    model = _tiny_model(cuda, family, Hs, Gs, Ds, dt)
+    gen = torch.Generator().manual_seed(4)
+    maps = [list(range(Gs)) if l in ANCHORS else torch.randint(0, Gs, (Gs,), generator=gen).tolist()
+            for l in range(len(HEAD_MAPS))]
+    s = EfficientKascadeStrategy(ANCHORS, None, k=100, tile_size=TILE, rolling_prefill=True,
+                                 head_mapping=maps, register=True)
+    ids = torch.randint(2, 256, (B, L), generator=gen).to(cuda)
+    nxt = [torch.randint(2, 256, (B, 1), generator=gen).to(cuda) for _ in range(2)]
+    logits = {}
+    for impl in ("sdpa", "eager", s.name):
+        model.config._attn_implementation = impl
+        with torch.no_grad():
+            r = model(ids, use_cache=True)
+            got = [r.logits[:, -1].float().cpu()]
+            for t in nxt:
+                r = model(t, past_key_values=r.past_key_values, use_cache=True)
+                got.append(r.logits[:, -1].float().cpu())
+        logits[impl] = torch.stack(got)
+    scale = float(logits["sdpa"].std())
+    assert scale > 0.05
+    if dt == torch.float16:
+        assert_close(logits[s.name], logits["sdpa"], "logits at k=100 vs SDPA", atol=2e-2 * scale, rtol=2e-2)
+    else:
+        yard = float((logits["eager"] - logits["sdpa"]).abs().max())
+        err = float((logits[s.name] - logits["sdpa"]).abs().max())
+        assert err <= 3 * yard, f"bf16 logits: {err:.3e} from SDPA, the library's own two paths differ by {yard:.3e}"
+        assert err <= 0.25 * scale, f"bf16 logits: {err:.3e} from SDPA at a logit spread of {scale:.3e}"
