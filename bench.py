@@ -177,7 +177,7 @@ def run_single_kernel(name, iters, seq_len, dev, head_map, decode_len=65536):
         caches = [workloads.paged_decode_inputs(seqlens, seed=10 + i, device=dev, reuse_keys=False)
                   for i in range(3)]
         c0 = caches[0]
-        dec = PagedKascadeDecoder(PCT, head_map, ANCHORS, 16, Ld, device=dev)
+        dec = PagedKascadeDecoder(PCT, head_map, ANCHORS, 16, Ld, device=dev, seqlens_hint=[Ld] * 16)
         dec.anchor(0, c0.q, c0.k_pages, c0.v_pages, c0.block_table, c0.seqlens, Ld, ragged=False)
         agg = torch.rand(16, G, Ld, device=dev).half()
         for i in range(iters):
@@ -664,7 +664,7 @@ def main():
             lens = torch.full((Bd,), Ld, dtype=torch.int32, device=dev)
             qd = rnd(Bd, Hs, Ds)
             dec = PagedKascadeDecoder(PCT, [list(range(Gs))] * 2, [0], Bd, Ld, page, dev, kv_heads=Gs, head_dim=Ds,
-                                      group_size=Hs // Gs)
+                                      group_size=Hs // Gs, seqlens_hint=[Ld] * Bd)
             out_d = torch.empty(Bd, Hs, Ds, device=dev, dtype=dts)
             t_dd = ev_time(lambda: dec.dense(qd, kp, vp, bt, lens, Ld, out=out_d), n=5)
             t_a0 = ev_time(lambda: dec.anchor(0, qd, kp, vp, bt, lens, Ld, ragged=True, out=out_d), n=5)
