@@ -482,7 +482,7 @@ def main():
                 "reuse_frac_hbm": round(reuse_bytes / t_r / 1e3 / HBM_PEAK_GBS, 4),
                 "dense_GBps": round(dense_bytes / t_dense / 1e3, 1),
                 "dense_frac_hbm": round(dense_bytes / t_dense / 1e3 / HBM_PEAK_GBS, 4),
-                "num_split_dense": dec.ns_dense, "num_split_reuse": dec.ns_reuse,
+                "num_split_dense": dec.ns_dense, "num_split_anchor": dec.ns_anchor, "num_split_reuse": dec.ns_reuse,
             }
             log(f"[bench] decode {name}: {decode[name]}")
             del caches, c0, dec

@@ -35,6 +35,7 @@ from ._lib import KascadeError
 
 H, G, D, TILE = 32, 8, 128, 32
 FUSED_MERGE_MAX_SPLITS = 32
+ANCHOR_ROWS_PER_SPLIT = 8192
 
 
 def get_head_mapping(model_name: str, recompute_layers: Sequence[int],
@@ -281,7 +282,15 @@ class PagedKascadeDecoder:
         self.ns_reuse = num_split_reuse or kernels.default_num_split(
             G * budgets.decode_budget(total, k), self.max_topk, wgs_per_cu=1 if uniform else 2,
             cap_rows=kernels.GATHER_ROWS_PER_SPLIT, row_counts=reuse_rows, heads=G)
-        ns = max(self.ns_dense, self.ns_reuse)
+        # The anchor passes (which also write their score codes) run 2 % faster with twice the
+        # splits where two workgroups per compute unit leave a split more than 8192 rows
+        # (16 x 65536: 795 / 508 us with 8 splits against 815 / 521 with 4); dense decode does not
+        # care, and beyond 32 splits the merge inside the launch would be lost.
+        self.ns_anchor = self.ns_dense
+        if (not num_split_dense and -(-max_seqlen // self.ns_dense) > ANCHOR_ROWS_PER_SPLIT
+                and 2 * self.ns_dense <= FUSED_MERGE_MAX_SPLITS):
+            self.ns_anchor = 2 * self.ns_dense
+        ns = max(self.ns_dense, self.ns_reuse, self.ns_anchor)
         dev = self.device
         self._glse = torch.empty(max_batch * H * ns, device=dev, dtype=torch.float32)
         self._part = torch.empty(max_batch * H * ns * D, device=dev, dtype=torch.float32)
@@ -304,6 +313,7 @@ class PagedKascadeDecoder:
         # memory: a win up to about 32 splits; beyond that the combine launch, which spreads the
         # merge over 32 workgroups per sequence, is faster
         self._sync_dense = self._sync if self.ns_dense <= FUSED_MERGE_MAX_SPLITS else None
+        self._sync_anchor = self._sync if self.ns_anchor <= FUSED_MERGE_MAX_SPLITS else None
         self._sync_reuse = self._sync if self.ns_reuse <= FUSED_MERGE_MAX_SPLITS else None
 
     def _scratch(self, B, ns):
@@ -342,11 +352,11 @@ class PagedKascadeDecoder:
         B = q.shape[0]
         G, H = self.G, self.H
         stride = ((max_len + 7) // 8) * 8
-        glse, part = self._scratch(B, self.ns_dense)
+        glse, part = self._scratch(B, self.ns_anchor)
         scores = self._scores[:B * H * stride].view(B, H, stride)
         o, agg = kernels.decode_recompute(q, k_pages, v_pages, glse, part, self._row_sums[:B], scores, layer,
                                           cache_seqlens=seqlens, block_table=block_table,
-                                          page_size=self.page_size, kv_len=max_len, out=out, sync=self._sync_dense,
+                                          page_size=self.page_size, kv_len=max_len, out=out, sync=self._sync_anchor,
                                           k_new=k_new, v_new=v_new)
         if ragged:
             width = budgets.decode_budget(max_len, self.k)
