@@ -145,6 +145,8 @@ class EfficientKascadeStrategy:
 
     def _prefill_reuse_forward(self, Q, K, V, topk_percent, layer):
         """Reuse prefill (EfficientKascadeStrategy.py:95-98)."""
+        if self._topk_to_reuse is None:
+            raise KascadeError("reuse layer called before any anchor layer")
         return kernels.prefill_reuse(Q, K, V, self._topk_to_reuse, self._hm(layer, Q.device, K.shape[2]), topk_percent,
                                      self.rolling_prefill)
 
@@ -173,6 +175,8 @@ class EfficientKascadeStrategy:
 
     def _decode_reuse_forward(self, Q, K, V, layer):
         """Reuse decode (EfficientKascadeStrategy.py:117-123)."""
+        if self._topk_to_reuse is None:
+            raise KascadeError("reuse layer called before any anchor layer")
         B, G = Q.shape[0], K.shape[2]
         topk = self._topk_to_reuse.shape[-1]
         ns = kernels.default_num_split(B * G * topk, topk, cap_rows=kernels.GATHER_ROWS_PER_SPLIT, heads=G)

@@ -161,6 +161,29 @@ def test_config3_ragged_long_decode(cuda):
     assert_close(o0[b:b + 1], want0, "ragged dense decode, shortest sequence")
     want1 = orc.reuse_decode(c.q_reuse[b:b + 1].cpu(), kc, vc, idx[b:b + 1].cpu(), c.head_mapping, [counts[b]])
     assert_close(o1[b:b + 1], want1, "ragged reuse decode, shortest sequence")
+    # oracle on the longest sequence (524288 tokens: its rows go through the multi-workgroup
+    # selection), one KV head at a time: dense output, the selected set against the oracle's
+    # pooled probabilities, and the reuse output of the KV head that reads this head's list
+    b, n = 3, seqlens[3]
+    rows = (c.block_table[b].long().view(-1, 1) * c.page_size + torch.arange(c.page_size, device=cuda)).view(-1)[:n]
+    for g in (2, 7):
+        kc = c.k_pages.view(-1, G, D)[rows, g].view(1, n, 1, D).cpu()
+        vc = c.v_pages.view(-1, G, D)[rows, g].view(1, n, 1, D).cpu()
+        heads = slice(4 * g, 4 * g + 4)
+        want0, _ = orc.dense_decode(c.q[b:b + 1, heads].cpu(), kc, vc)
+        assert_close(o0[b:b + 1, heads], want0, f"ragged dense decode, longest sequence, KV head {g}")
+        agg_want = orc.pooled_decode_scores(c.q[b:b + 1, heads].cpu(), kc)
+        src = c.head_mapping[g]                          # the list this KV head's reuse pass reads
+        if src == g:
+            ok, _, msg = orc.topk_agreement(agg_want[0, 0], idx[b, g, :counts[b]].cpu(), counts[b], n, ulps=1.0)
+            assert ok, f"longest sequence, KV head {g}: {msg}"
+        ks = c.k_pages.view(-1, G, D)[rows, src].view(1, n, 1, D).cpu()
+        ok, _, msg = orc.topk_agreement(orc.pooled_decode_scores(c.q[b:b + 1, 4 * src:4 * src + 4].cpu(), ks)[0, 0],
+                                        idx[b, src, :counts[b]].cpu(), counts[b], n, ulps=1.0)
+        assert ok, f"longest sequence, KV head {src}: {msg}"
+        want1 = orc.reuse_decode(c.q_reuse[b:b + 1, heads].cpu(), kc, vc, idx[b:b + 1, src:src + 1].cpu(), [0],
+                                 [counts[b]])
+        assert_close(o1[b:b + 1, heads], want1, f"ragged reuse decode, longest sequence, KV head {g}")
     # pooled probabilities: mass 4 per (sequence, KV head), zero beyond each length; the multi-workgroup
     # selection is exact on them for every row
     glse, part = dec._scratch(B, dec.ns_dense)

@@ -84,6 +84,40 @@ def test_strategy_decode_layers(cuda):
     assert_close(o2[:, 0], orc.reuse_decode(q[:, :, 0], kc, vc, idx2, list(range(G))), "decode anchor>0")
 
 
+@pytest.mark.parametrize("Lk", [100, 128, 129])
+def test_short_context_boundary(cuda, Lk):
+    """Up to 128 keys the call is SDPA on the caller's tensors and mask
+    (EfficientKascadeStrategy.py:137-140); from 129 on it is the kernels.  Both sides of the
+    boundary against the oracle, prefill then one decode step."""
+    from kascade_amd.strategy import EfficientKascadeStrategy
+    g = torch.Generator().manual_seed(Lk)
+    B, p = 2, 10
+    q = torch.randn(B, H, Lk, D, generator=g).half()
+    k = torch.randn(B, G, Lk, D, generator=g).half()
+    v = torch.randn(B, G, Lk, D, generator=g).half()
+    hm = [list(range(G)), [1, 0, 3, 2, 5, 4, 7, 6]]
+    s = EfficientKascadeStrategy([0], None, k=p, tile_size=TILE, head_mapping=hm, register=False)
+    kc, vc = k.permute(0, 2, 1, 3).contiguous(), v.permute(0, 2, 1, 3).contiguous()
+    mask = orc.causal_additive_mask(Lk, Lk, torch.float16).expand(B, 1, Lk, Lk).to(cuda)
+    want, _ = orc.dense_prefill(q.permute(0, 2, 1, 3), kc, vc)
+    for layer in (0, 1):
+        o, none = s.attention_forward(_Module(layer), q.to(cuda), k.to(cuda), v.to(cuda), mask, D ** -0.5)
+        assert none is None and tuple(o.shape) == (B, Lk, H, D)
+        if Lk <= 128 or layer == 0:
+            assert_close(o, want, f"Lk={Lk} prefill layer {layer}")
+        else:   # a budget of 128 of 129 keys: every tile is in the dense regime of the reuse kernel
+            assert_close(o, want, f"Lk={Lk} reuse prefill in the dense regime")
+    assert (s._topk_to_reuse is None) == (Lk <= 128)
+    qd = q[:, :, -1:].contiguous()
+    od, _ = s.attention_forward(_Module(0), qd.to(cuda), k.to(cuda), v.to(cuda), None, D ** -0.5)
+    wd, _ = orc.dense_decode(qd[:, :, 0], kc, vc)
+    assert_close(od[:, 0], wd, f"Lk={Lk} decode layer 0")
+    if Lk > 128:
+        o1, _ = s.attention_forward(_Module(1), qd.to(cuda), k.to(cuda), v.to(cuda), None, D ** -0.5)
+        assert_close(o1[:, 0], orc.reuse_decode(qd[:, :, 0], kc, vc, s._topk_to_reuse.cpu(), hm[1]),
+                     f"Lk={Lk} decode reuse layer")
+
+
 def test_full_kernel_observables(cuda):
     """(O, indices, scores) of the anchor glue functions, as the reference's correctness mode compares them."""
     from kascade_amd import kernels, workloads

@@ -79,6 +79,41 @@ def test_strategy_registers_with_hf():
     assert w is None and torch.allclose(out, ref, atol=1e-5)
 
 
+@pytest.mark.parametrize("Lk", [100, 128])
+def test_short_context_falls_back_to_sdpa(Lk):
+    """EfficientKascadeStrategy.py:137-140: up to 128 keys the call is SDPA with the caller's mask,
+    prefill and decode alike, and the strategy's stored indices are not touched."""
+    from kascade_amd.strategy import EfficientKascadeStrategy
+    hm = [list(range(8))] * 2
+    s = EfficientKascadeStrategy([0], None, k=10, tile_size=32, head_mapping=hm, register=False)
+
+    class M(torch.nn.Module):
+        layer_idx = 1
+        num_key_value_groups = 4
+    g = torch.Generator().manual_seed(Lk)
+    k = torch.randn(2, 8, Lk, 128, generator=g)
+    v = torch.randn(2, 8, Lk, 128, generator=g)
+    for Lq in (Lk, 1):
+        q = torch.randn(2, 32, Lq, 128, generator=g)
+        mask = orc.causal_additive_mask(Lk, Lk, torch.float32)[:, :, Lk - Lq:]
+        out, w = s.attention_forward(M(), q, k, v, mask.expand(2, 1, Lq, Lk), 128 ** -0.5)
+        want, _ = orc.dense_prefill(torch.cat([torch.zeros(2, Lk - Lq, 32, 128), q.transpose(1, 2)], 1),
+                                    k.transpose(1, 2), v.transpose(1, 2))
+        assert w is None and tuple(out.shape) == (2, Lq, 32, 128)
+        assert torch.allclose(out, want[:, Lk - Lq:], atol=2e-5)
+    assert s._topk_to_reuse is None
+    # one key more goes to the kernels, which need the HIP library and a GPU: no silent fallback
+    from kascade_amd._lib import KascadeError
+    k1 = torch.randn(2, 8, Lk + 29, 128, generator=g).half()
+    q1 = torch.randn(2, 32, 1, 128, generator=g).half()
+    with pytest.raises(KascadeError, match="before any anchor"):
+        s.attention_forward(M(), q1, k1, k1, None, 128 ** -0.5)
+    if not torch.cuda.is_available():
+        M.layer_idx = 0
+        with pytest.raises((KascadeError, RuntimeError)):
+            s.attention_forward(M(), q1, k1, k1, None, 128 ** -0.5)
+
+
 def test_default_num_split_heuristic(monkeypatch):
     from kascade_amd import kernels, _lib
 

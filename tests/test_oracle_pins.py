@@ -366,6 +366,109 @@ def test_strategy_oracle_decode_step():
     assert torch.allclose(o1[:, 0], want, atol=1e-5)
 
 
+def _pooled_by_loops(q, k, tile, scaling):
+    """Pooled tile probabilities straight from the definition (KascadeStrategy.py:72-82), in
+    float64 with plain loops: every query row's causal softmax, summed over the query heads of a
+    KV head and over the rows of a tile; zero from the tile's first position on.  q [H,L,D],
+    k [G,L,D] -> [G,T,L]."""
+    H, L, _ = q.shape
+    G = k.shape[0]
+    rep = H // G
+    T = -(-L // tile)
+    qn, kn = q.double().numpy(), k.double().numpy()
+    pooled = np.zeros((G, T, L))
+    for i in range(L):
+        for h in range(H):
+            s = kn[h // rep, :i + 1] @ qn[h, i] * scaling
+            e = np.exp(s - s.max())
+            pooled[h // rep, i // tile, :i + 1] += e / e.sum()
+    for t in range(T):
+        pooled[:, t, t * tile:] = 0.0
+    return pooled
+
+
+def _check_stored_rows(stored, pooled, L, tile, p, rolling):
+    """stored [G,L,k] (one row per query) against pooled [G,T,L] from the loops."""
+    G, _, kw = stored.shape
+    assert kw == orc.k_strat(L, p, tile)
+    short = 0
+    for t in range(-(-L // tile)):
+        n = orc.n_strat(t * tile, p, kw) if (rolling and L > 128) else kw
+        short += n < kw
+        for g in range(G):
+            rows = stored[g, t * tile:(t + 1) * tile]
+            assert bool((rows == rows[:1]).all()), "rows of a tile share one list"
+            row = rows[0].tolist()
+            assert all(x == L - 1 for x in row[n:]), (t, g, "slots beyond the rolling budget hold Lk-1")
+            got = row[:n]
+            valid = t * tile                        # keys with a non-zero pooled value
+            order = np.argsort(-pooled[g, t], kind="stable")
+            if valid >= n:                          # the n largest pooled values, largest first
+                assert got == order[:n].tolist(), (t, g)
+            else:                                   # every valid key, then arbitrary zero-valued positions
+                assert got[:valid] == order[:valid].tolist(), (t, g)
+                assert len(set(got)) == len(got) and all(0 <= x < L for x in got)
+    return short
+
+
+@pytest.mark.parametrize("rolling", [False, True])
+def test_strategy_oracle_stored_indices_by_brute_force(rolling):
+    """The state the strategy keeps between layers (pool -> x tile mask -> topk -> rolling fill,
+    KascadeStrategy.py:72-92) against an independent computation by loops.  L = 640 at 40 %
+    gives k_strat = 224 and rolling budgets of 128 .. 224, so most tiles consume a proper prefix."""
+    L, tile, p, D = 640, 32, 40, 16
+    q, k, v = _strategy_case(L, seed=3)
+    mask = orc.causal_additive_mask(L, L, torch.float32)
+    st = orc.StrategyOracle([0], [[0, 1], [0, 1]], k=p, tile_size=tile, rolling_prefill=rolling, block_size=256)
+    st.attention_forward(0, q, k, v, mask, D ** -0.5)
+    pooled = _pooled_by_loops(q[0], k[0], tile, D ** -0.5)
+    short = _check_stored_rows(st._topk_to_reuse[0], pooled, L, tile, p, rolling)
+    assert (short > 0) == rolling
+
+
+def test_strategy_oracle_second_anchor_layer():
+    """An anchor layer above layer 0 (KascadeStrategy.py:72-108): it stores its own selection and
+    attends to that selection plus the in-tile diagonal, with the dense softmax weights
+    renormalised over this set.  Output and stored indices by loops."""
+    L, tile, p, D = 384, 32, 40, 16
+    q, k, v = _strategy_case(L, seed=4)
+    gen = torch.Generator().manual_seed(9)
+    q1 = q + 0.5 * torch.randn(q.shape, generator=gen)
+    k1 = k + 0.5 * torch.randn(k.shape, generator=gen)
+    mask = orc.causal_additive_mask(L, L, torch.float32)
+    st = orc.StrategyOracle([0, 1], [[0, 1], [0, 1], [1, 0]], k=p, tile_size=tile, rolling_prefill=True,
+                            block_size=160)
+    st.attention_forward(0, q, k, v, mask, D ** -0.5)
+    first = st._topk_to_reuse.clone()
+    o1 = st.attention_forward(1, q1, k1, v, mask, D ** -0.5)
+    assert not torch.equal(first, st._topk_to_reuse)          # the second anchor replaced the state
+    pooled = _pooled_by_loops(q1[0], k1[0], tile, D ** -0.5)
+    _check_stored_rows(st._topk_to_reuse[0], pooled, L, tile, p, True)
+    idx = st._topk_to_reuse
+    sparse_rows = 0
+    for i in list(range(0, L, 29)) + [L - 1]:
+        for h in range(8):
+            g = h // 4
+            s = (k1[0, g, :i + 1].double() @ q1[0, h, i].double()) * D ** -0.5
+            pr = torch.softmax(s, 0)                           # dense causal weights of the row
+            keep = {int(x) for x in idx[0, g, i] if int(x) <= i} | set(range((i // tile) * tile, i + 1))
+            sparse_rows += len(keep) < i + 1
+            ks = sorted(keep)
+            w = pr[ks] / pr[ks].sum()
+            want = (w[:, None] * v[0, g, ks].double()).sum(0)
+            assert torch.allclose(o1[0, i, h].double(), want, atol=1e-5), (i, h)
+    assert sparse_rows > 0
+    # a reuse layer above it reads the second anchor's lists through its head map
+    o2 = st.attention_forward(2, q1, k1, v, mask, D ** -0.5)
+    for i in (200, 383):
+        for h in (1, 6):
+            g = h // 4
+            keys = {int(x) for x in idx[0, [1, 0][g], i]} | set(range((i // tile) * tile, i + 1))
+            ks = sorted(j for j in keys if j <= i)
+            s = (k1[0, g, ks] @ q1[0, h, i]) * D ** -0.5
+            assert torch.allclose(o2[0, i, h], torch.softmax(s, 0) @ v[0, g, ks], atol=1e-5), (i, h)
+
+
 # ------------------------------------------------------------ data fixtures
 def test_head_mapping_fixtures():
     root = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "kascade_amd", "head_mappings")
