@@ -361,18 +361,20 @@ int kascade_prefill_reuse_shaped_call(const kascade_shape* shape, const kascade_
  * start_pos[b] .. start_pos[b]+n_new-1.  The reference has no counterpart (it
  * re-materialises the whole cache every step: EfficientKascadeStrategy.py:149-150);
  * this is the step right before the decode path.
- *   k_new, v_new [B,n_new,G,D] with strides new_strides (b, l, h=g). */
+ *   k_new, v_new [B,n_new,G,D] with strides new_strides (b, l, h=g).
+ *   n_new_rows   NULL, or [B] i32: sequence b brings only its first n_new_rows[b] (<= n_new) rows.
+ *   Positions beyond what the block table covers are skipped. */
 int kascade_paged_kv_append_call(kascade_half* K_pages, kascade_half* V_pages,
                                  const kascade_half* k_new, const kascade_half* v_new,
                                  const int32_t* start_pos, const int32_t* block_table, int batch,
                                  int n_new, int max_pages, int page_size,
-                                 kascade_strides new_strides, void* stream);
+                                 kascade_strides new_strides, const int32_t* n_new_rows, void* stream);
 /* kascade_paged_kv_append_call for any kascade_shape. */
 int kascade_paged_kv_append_shaped_call(const kascade_shape* shape, kascade_half* K_pages, kascade_half* V_pages,
                                  const kascade_half* k_new, const kascade_half* v_new,
                                  const int32_t* start_pos, const int32_t* block_table, int batch,
                                  int n_new, int max_pages, int page_size,
-                                 kascade_strides new_strides, void* stream);
+                                 kascade_strides new_strides, const int32_t* n_new_rows, void* stream);
 
 /* The hand-off from a decoder layer's projections to the attention path in one launch: RMS
  * normalisation of every query and key head (optional), rotary position embedding of queries
@@ -416,7 +418,8 @@ int kascade_rope_append_paged_shaped_call(const kascade_shape* shape, const kasc
  * (sequence, KV head) row r = b*8+g (b*kv_heads+g for the shaped twin) of the pooled scores, what kascade_topk_call takes as
  * valid_len / n_sel:  valid_len_rows[r] = len_b,
  *                     n_sel_rows[r]     = 128*ceil(floor(topk_percent*len_b/100)/128),
- * with len_b the length after the advance.  Either output may be NULL. */
+ * with len_b the length after the advance.  Either output may be NULL.  A sequence of length 0
+ * is an empty slot of the batch: it is not advanced (and the decode calls append nothing to it). */
 int kascade_decode_budgets_call(int32_t* cache_seqlens, int advance, float topk_percent, int batch,
                                 int32_t* valid_len_rows, int32_t* n_sel_rows, void* stream);
 int kascade_decode_budgets_shaped_call(const kascade_shape* shape, int32_t* cache_seqlens, int advance,
@@ -436,18 +439,32 @@ int kascade_decode_budgets_shaped_call(const kascade_shape* shape, int32_t* cach
  *   - outputs indexed by the chunk's own rows: log_sum [B,q_len,H], Output [B,q_len,H,D],
  *     aggregate_scores [B,G,ceil(q_len/32),q_start+q_len].
  * With q_start = 0 and q_len = L they compute what the whole-prompt calls compute; a prompt
- * processed in 32-aligned chunks gives bit-identical rows.  No counterpart in the reference. */
+ * processed in 32-aligned chunks gives bit-identical rows.  No counterpart in the reference.
+ *
+ * A batch whose sequences stand at different positions passes two more arrays (both NULL: every
+ * sequence starts at q_start and owns all q_len rows):
+ *   q_start_rows [B] i32: first global position of sequence b's rows, a multiple of 32 and at most
+ *                q_start, which then is the largest of them (it sizes aggregate_scores and is what
+ *                the block table must cover);
+ *   q_len_rows   [B] i32 or NULL: how many of the q_len rows of Q belong to sequence b (0: none).
+ * Rows beyond a sequence's own are left alone: no Output, no log_sum; their tiles' pooled scores
+ * are not written (-inf with fill_invalid).  Sequence b then attends to cache positions
+ * [0, q_start_rows[b] + q_len_rows[b]) and gets exactly the rows it gets in a call of its own;
+ * without the rolling budget a sparse tile uses min(max_topk_num, the row width of a prompt of the
+ * sequence's own length) entries of its list. */
 int kascade_prefill_chunk_dense_call(const kascade_half* Q, const kascade_half* K_pages,
                                      const kascade_half* V_pages, float* log_sum,
                                      kascade_half* Output, int batch, int q_start, int q_len,
                                      kascade_strides q_strides, const int32_t* block_table,
-                                     int max_pages, int page_size, int num_pages, int with_output,
+                                     int max_pages, int page_size, int num_pages, int with_output, const int32_t* q_start_rows,
+                                     const int32_t* q_len_rows,
                                      void* stream);
 int kascade_prefill_chunk_dense_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K_pages,
                                      const kascade_half* V_pages, float* log_sum,
                                      kascade_half* Output, int batch, int q_start, int q_len,
                                      kascade_strides q_strides, const int32_t* block_table,
-                                     int max_pages, int page_size, int num_pages, int with_output,
+                                     int max_pages, int page_size, int num_pages, int with_output, const int32_t* q_start_rows,
+                                     const int32_t* q_len_rows,
                                      void* stream);
 
 int kascade_prefill_chunk_aggregate_call(const kascade_half* Q, const kascade_half* K_pages,
@@ -455,13 +472,15 @@ int kascade_prefill_chunk_aggregate_call(const kascade_half* Q, const kascade_ha
                                          int batch, int q_start, int q_len,
                                          kascade_strides q_strides, const int32_t* block_table,
                                          int max_pages, int page_size, int num_pages,
-                                         int fill_invalid, void* stream);
+                                         int fill_invalid, const int32_t* q_start_rows,
+                                     const int32_t* q_len_rows, void* stream);
 int kascade_prefill_chunk_aggregate_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K_pages,
                                          const float* log_sum, kascade_half* aggregate_scores,
                                          int batch, int q_start, int q_len,
                                          kascade_strides q_strides, const int32_t* block_table,
                                          int max_pages, int page_size, int num_pages,
-                                         int fill_invalid, void* stream);
+                                         int fill_invalid, const int32_t* q_start_rows,
+                                     const int32_t* q_len_rows, void* stream);
 
 /* physical_rows [B,G,ceil(q_len/32),max_topk_num]: the tile's top-k tokens already translated
  * to rows of the paged cache (kascade_translate_indices_call), so that the gather needs no
@@ -472,14 +491,16 @@ int kascade_prefill_chunk_reuse_call(const kascade_half* Q, const kascade_half* 
                                      kascade_half* Output, int batch, int q_start, int q_len,
                                      int max_topk_num, int rolling, kascade_strides q_strides,
                                      const int32_t* block_table, int max_pages, int page_size,
-                                     int num_pages, void* stream);
+                                     int num_pages, const int32_t* q_start_rows,
+                                     const int32_t* q_len_rows, void* stream);
 int kascade_prefill_chunk_reuse_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K_pages,
                                      const kascade_half* V_pages, const int32_t* physical_rows,
                                      const int32_t* head_mapping, float topk_percent,
                                      kascade_half* Output, int batch, int q_start, int q_len,
                                      int max_topk_num, int rolling, kascade_strides q_strides,
                                      const int32_t* block_table, int max_pages, int page_size,
-                                     int num_pages, void* stream);
+                                     int num_pages, const int32_t* q_start_rows,
+                                     const int32_t* q_len_rows, void* stream);
 
 /* physical_rows[b,i] = block_table[b, t / page_size] * page_size + t % page_size with
  * t = clamp(token_idx[b,i], 0, kv_len-1), i < per_sequence.  physical_rows may alias token_idx.

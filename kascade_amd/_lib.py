@@ -52,16 +52,16 @@ SIGNATURES = {
     "kascade_prefill_aggregate_range_call": (_I, [_P, _P, _P, _P, _I, _I, _I, Strides, Strides, _I, _P]),
     "kascade_prefill_reuse_call": (_I, [_P, _P, _P, _P, _P, _F, _P, _I, _I, _I, _I, Strides, Strides,
                                         _P]),
-    "kascade_paged_kv_append_call": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, Strides, _P]),
+    "kascade_paged_kv_append_call": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, Strides, _P, _P]),
     "kascade_rope_append_paged_call": (_I, [_P, _SP, _P, _P, _SP, _P, _I, _P, _P, _F, _P, _I, _P, _P, _P,
                                             _P, _I, _I, _I, _I, _P]),
     "kascade_decode_budgets_call": (_I, [_P, _I, _F, _I, _P, _P, _P]),
     "kascade_prefill_chunk_dense_call": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, Strides, _P, _I, _I, _I,
-                                              _I, _P]),
+                                              _I, _P, _P, _P]),
     "kascade_prefill_chunk_aggregate_call": (_I, [_P, _P, _P, _P, _I, _I, _I, Strides, _P, _I, _I, _I,
-                                                  _I, _P]),
+                                                  _I, _P, _P, _P]),
     "kascade_prefill_chunk_reuse_call": (_I, [_P, _P, _P, _P, _P, _F, _P, _I, _I, _I, _I, _I, Strides,
-                                              _P, _I, _I, _I, _P]),
+                                              _P, _I, _I, _I, _P, _P, _P]),
     "kascade_translate_indices_call": (_I, [_P, _P, _P, _I, C.c_int64, _I, _I, _I, _P]),
     "kascade_diag_stream_read_call": (_I, [_P, _L, _P, _P]),
     "kascade_diag_gather_rows_call": (_I, [_P, _P, _P, _L, _L, _P, _P]),

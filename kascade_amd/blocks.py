@@ -76,6 +76,8 @@ class KascadeBlockStack(KascadeAttentionStack):
         """One chunk of hidden states [B,Lq,hidden] through all layers; the chunk starts at the
         current length, a multiple of 32.  Returns the hidden states after the last layer."""
         B, Lq, _ = x.shape
+        if len(set(self.cache.lengths)) != 1:
+            raise KascadeError("the block stack prefills a batch of one common length")
         q_start = self.length
         if q_start % TILE:
             raise KascadeError("a prefill chunk must start at a multiple of 32 tokens")
@@ -88,8 +90,8 @@ class KascadeBlockStack(KascadeAttentionStack):
             else:
                 o = self.prefill.forward(l, q, self.k_pages[l], self.v_pages[l], self.block_table, q_start)
             x = self._residual(l, x, o)
-        self.length += Lq
         self.seqlens += Lq
+        self.cache.note_advance(Lq, range(self.batch))
         return x
 
     # ------------------------------------------------------------------- decode
@@ -109,12 +111,11 @@ class KascadeBlockStack(KascadeAttentionStack):
 
     def decode_step_hidden(self, x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """x [B,1,hidden] -> hidden states after the last layer (eager launches)."""
-        if self.length + 1 > self.max_seqlen:
-            raise KascadeError("decode step exceeds max_seqlen")
+        self._before_step()
         if out is None:
             out = torch.empty_like(x)
         self._decode_hidden_layers(x, out)
-        self.length += 1
+        self.cache.note_advance(1)
         return out
 
     def capture_decode_hidden(self):
@@ -141,8 +142,7 @@ class KascadeBlockStack(KascadeAttentionStack):
     def replay_decode_hidden(self) -> torch.Tensor:
         if self._hgraph is None:
             raise KascadeError("capture_decode_hidden() first")
-        if self.length + 1 > self.max_seqlen:
-            raise KascadeError("decode step exceeds max_seqlen")
+        self._before_step()
         self._hgraph.replay()
-        self.length += 1
+        self.cache.note_advance(1)
         return self.graph_y

@@ -157,7 +157,7 @@ int set_append(DecodeParams& p, const kascade_half* k_new, const kascade_half* v
 
 extern "C" {
 
-int kascade_abi_version(void) { return 9; }
+int kascade_abi_version(void) { return 10; }
 
 const char* kascade_get_last_error(void) { return g_err; }
 
@@ -715,7 +715,7 @@ int paged_kv_append_impl(const Shape& sh, kascade_half* K_pages, kascade_half* V
                                  const kascade_half* k_new, const kascade_half* v_new,
                                  const int32_t* start_pos, const int32_t* block_table, int batch,
                                  int n_new, int max_pages, int page_size,
-                                 kascade_strides new_strides, void* stream) {
+                                 kascade_strides new_strides, const int32_t* n_new_rows, void* stream) {
     REQUIRE(K_pages && V_pages && k_new && v_new && start_pos && block_table,
             "paged_kv_append: null pointer argument");
     REQUIRE(batch > 0 && n_new >= 0, "paged_kv_append: bad batch/n_new");
@@ -726,7 +726,7 @@ int paged_kv_append_impl(const Shape& sh, kascade_half* K_pages, kascade_half* V
     REQUIRE(aligned16(K_pages) && aligned16(V_pages) && aligned16(k_new) && aligned16(v_new),
             "paged_kv_append: tensors must be 16-byte aligned");
     return check_hip(launch_paged_kv_append(H(K_pages), H(V_pages), H(k_new), H(v_new), start_pos,
-                                            block_table, batch, n_new, max_pages, shift,
+                                            block_table, batch, n_new, n_new_rows, max_pages, shift,
                                             new_strides.b, new_strides.l, new_strides.h, sh.G, sh.D,
                                             static_cast<hipStream_t>(stream)),
                      "paged_kv_append");
@@ -738,18 +738,18 @@ int kascade_paged_kv_append_call(kascade_half* K_pages, kascade_half* V_pages,
                                  const kascade_half* k_new, const kascade_half* v_new,
                                  const int32_t* start_pos, const int32_t* block_table, int batch,
                                  int n_new, int max_pages, int page_size,
-                                 kascade_strides new_strides, void* stream) {
-    return paged_kv_append_impl(kRefShape, K_pages, V_pages, k_new, v_new, start_pos, block_table, batch, n_new, max_pages, page_size, new_strides, stream);
+                                 kascade_strides new_strides, const int32_t* n_new_rows, void* stream) {
+    return paged_kv_append_impl(kRefShape, K_pages, V_pages, k_new, v_new, start_pos, block_table, batch, n_new, max_pages, page_size, new_strides, n_new_rows, stream);
 }
 
 int kascade_paged_kv_append_shaped_call(const kascade_shape* shape, kascade_half* K_pages, kascade_half* V_pages,
                                  const kascade_half* k_new, const kascade_half* v_new,
                                  const int32_t* start_pos, const int32_t* block_table, int batch,
                                  int n_new, int max_pages, int page_size,
-                                 kascade_strides new_strides, void* stream) {
+                                 kascade_strides new_strides, const int32_t* n_new_rows, void* stream) {
     Shape sh;
     if (get_shape(shape, &sh)) return -1;
-    return paged_kv_append_impl(sh, K_pages, V_pages, k_new, v_new, start_pos, block_table, batch, n_new, max_pages, page_size, new_strides, stream);
+    return paged_kv_append_impl(sh, K_pages, V_pages, k_new, v_new, start_pos, block_table, batch, n_new, max_pages, page_size, new_strides, n_new_rows, stream);
 }
 
 }  // extern "C"
@@ -846,7 +846,8 @@ int kascade_decode_budgets_call(int32_t* cache_seqlens, int advance, float topk_
 namespace {
 int chunk_params(PrefillParams& p, const Shape& sh, const kascade_half* Q, int batch,
                         int q_start, int q_len, kascade_strides q_strides,
-                        const int32_t* block_table, int max_pages, int page_size, int num_pages) {
+                        const int32_t* block_table, int max_pages, int page_size, int num_pages,
+                        const int32_t* q_start_rows, const int32_t* q_len_rows) {
     REQUIRE(block_table, "prefill_chunk: block_table is required");
     REQUIRE(batch > 0 && batch <= 65535 && q_len > 0, "prefill_chunk: bad batch/q_len");
     REQUIRE(q_start >= 0 && q_start % kTile == 0, "prefill_chunk: q_start must be a multiple of 32");
@@ -866,6 +867,8 @@ int chunk_params(PrefillParams& p, const Shape& sh, const kascade_half* Q, int b
     p.T = (q_len + kTile - 1) / kTile;
     p.block_table = block_table; p.max_pages = max_pages; p.page_shift = shift;
     p.num_pages = num_pages;
+    REQUIRE(q_start_rows || !q_len_rows, "prefill_chunk: q_len_rows comes with q_start_rows");
+    p.q_start_rows = q_start_rows; p.q_len_rows = q_len_rows;
     return 0;
 }
 
@@ -873,7 +876,8 @@ int prefill_chunk_dense_impl(const Shape& sh, const kascade_half* Q, const kasca
                                      const kascade_half* V_pages, float* log_sum,
                                      kascade_half* Output, int batch, int q_start, int q_len,
                                      kascade_strides q_strides, const int32_t* block_table,
-                                     int max_pages, int page_size, int num_pages, int with_output,
+                                     int max_pages, int page_size, int num_pages, int with_output, const int32_t* q_start_rows,
+                                     const int32_t* q_len_rows,
                                      void* stream) {
     REQUIRE(Q && K_pages, "prefill_chunk_dense: null pointer argument");
     REQUIRE(!with_output || (V_pages && Output), "prefill_chunk_dense: with_output needs V and Output");
@@ -882,7 +886,7 @@ int prefill_chunk_dense_impl(const Shape& sh, const kascade_half* Q, const kasca
             "prefill_chunk_dense: tensors must be 16-byte aligned");
     PrefillParams p{};
     if (chunk_params(p, sh, Q, batch, q_start, q_len, q_strides, block_table, max_pages,
-                     page_size, num_pages))
+                     page_size, num_pages, q_start_rows, q_len_rows))
         return -1;
     p.K = E(K_pages); p.V = with_output ? E(V_pages) : E(K_pages);
     p.log_sum = log_sum; p.O = E(Output);
@@ -895,13 +899,14 @@ int prefill_chunk_aggregate_impl(const Shape& sh, const kascade_half* Q, const k
                                          int batch, int q_start, int q_len,
                                          kascade_strides q_strides, const int32_t* block_table,
                                          int max_pages, int page_size, int num_pages,
-                                         int fill_invalid, void* stream) {
+                                         int fill_invalid, const int32_t* q_start_rows,
+                                     const int32_t* q_len_rows, void* stream) {
     REQUIRE(Q && K_pages && log_sum && aggregate_scores,
             "prefill_chunk_aggregate: null pointer argument");
     REQUIRE(aligned16(K_pages), "prefill_chunk_aggregate: K must be 16-byte aligned");
     PrefillParams p{};
     if (chunk_params(p, sh, Q, batch, q_start, q_len, q_strides, block_table, max_pages,
-                     page_size, num_pages))
+                     page_size, num_pages, q_start_rows, q_len_rows))
         return -1;
     p.K = E(K_pages); p.V = E(K_pages); p.log_sum_in = log_sum; p.agg = H(aggregate_scores);
     p.fill_invalid = fill_invalid;
@@ -915,7 +920,8 @@ int prefill_chunk_reuse_impl(const Shape& sh, const kascade_half* Q, const kasca
                                      kascade_half* Output, int batch, int q_start, int q_len,
                                      int max_topk_num, int rolling, kascade_strides q_strides,
                                      const int32_t* block_table, int max_pages, int page_size,
-                                     int num_pages, void* stream) {
+                                     int num_pages, const int32_t* q_start_rows,
+                                     const int32_t* q_len_rows, void* stream) {
     REQUIRE(Q && K_pages && V_pages && physical_rows && head_mapping && Output,
             "prefill_chunk_reuse: null pointer argument");
     REQUIRE(max_topk_num > 0, "prefill_chunk_reuse: max_topk_num must be > 0");
@@ -924,7 +930,7 @@ int prefill_chunk_reuse_impl(const Shape& sh, const kascade_half* Q, const kasca
             "prefill_chunk_reuse: tensors must be 16-byte aligned");
     PrefillParams p{};
     if (chunk_params(p, sh, Q, batch, q_start, q_len, q_strides, block_table, max_pages,
-                     page_size, num_pages))
+                     page_size, num_pages, q_start_rows, q_len_rows))
         return -1;
     p.K = E(K_pages); p.V = E(V_pages); p.idx = physical_rows; p.head_map = head_mapping;
     p.O = E(Output); p.log_sum = nullptr;
@@ -939,20 +945,22 @@ int kascade_prefill_chunk_dense_call(const kascade_half* Q, const kascade_half* 
                                      const kascade_half* V_pages, float* log_sum,
                                      kascade_half* Output, int batch, int q_start, int q_len,
                                      kascade_strides q_strides, const int32_t* block_table,
-                                     int max_pages, int page_size, int num_pages, int with_output,
+                                     int max_pages, int page_size, int num_pages, int with_output, const int32_t* q_start_rows,
+                                     const int32_t* q_len_rows,
                                      void* stream) {
-    return prefill_chunk_dense_impl(kRefShape, Q, K_pages, V_pages, log_sum, Output, batch, q_start, q_len, q_strides, block_table, max_pages, page_size, num_pages, with_output, stream);
+    return prefill_chunk_dense_impl(kRefShape, Q, K_pages, V_pages, log_sum, Output, batch, q_start, q_len, q_strides, block_table, max_pages, page_size, num_pages, with_output, q_start_rows, q_len_rows, stream);
 }
 
 int kascade_prefill_chunk_dense_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K_pages,
                                      const kascade_half* V_pages, float* log_sum,
                                      kascade_half* Output, int batch, int q_start, int q_len,
                                      kascade_strides q_strides, const int32_t* block_table,
-                                     int max_pages, int page_size, int num_pages, int with_output,
+                                     int max_pages, int page_size, int num_pages, int with_output, const int32_t* q_start_rows,
+                                     const int32_t* q_len_rows,
                                      void* stream) {
     Shape sh;
     if (get_shape(shape, &sh)) return -1;
-    return prefill_chunk_dense_impl(sh, Q, K_pages, V_pages, log_sum, Output, batch, q_start, q_len, q_strides, block_table, max_pages, page_size, num_pages, with_output, stream);
+    return prefill_chunk_dense_impl(sh, Q, K_pages, V_pages, log_sum, Output, batch, q_start, q_len, q_strides, block_table, max_pages, page_size, num_pages, with_output, q_start_rows, q_len_rows, stream);
 }
 
 int kascade_prefill_chunk_aggregate_call(const kascade_half* Q, const kascade_half* K_pages,
@@ -960,8 +968,9 @@ int kascade_prefill_chunk_aggregate_call(const kascade_half* Q, const kascade_ha
                                          int batch, int q_start, int q_len,
                                          kascade_strides q_strides, const int32_t* block_table,
                                          int max_pages, int page_size, int num_pages,
-                                         int fill_invalid, void* stream) {
-    return prefill_chunk_aggregate_impl(kRefShape, Q, K_pages, log_sum, aggregate_scores, batch, q_start, q_len, q_strides, block_table, max_pages, page_size, num_pages, fill_invalid, stream);
+                                         int fill_invalid, const int32_t* q_start_rows,
+                                     const int32_t* q_len_rows, void* stream) {
+    return prefill_chunk_aggregate_impl(kRefShape, Q, K_pages, log_sum, aggregate_scores, batch, q_start, q_len, q_strides, block_table, max_pages, page_size, num_pages, fill_invalid, q_start_rows, q_len_rows, stream);
 }
 
 int kascade_prefill_chunk_aggregate_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K_pages,
@@ -969,10 +978,11 @@ int kascade_prefill_chunk_aggregate_shaped_call(const kascade_shape* shape, cons
                                          int batch, int q_start, int q_len,
                                          kascade_strides q_strides, const int32_t* block_table,
                                          int max_pages, int page_size, int num_pages,
-                                         int fill_invalid, void* stream) {
+                                         int fill_invalid, const int32_t* q_start_rows,
+                                     const int32_t* q_len_rows, void* stream) {
     Shape sh;
     if (get_shape(shape, &sh)) return -1;
-    return prefill_chunk_aggregate_impl(sh, Q, K_pages, log_sum, aggregate_scores, batch, q_start, q_len, q_strides, block_table, max_pages, page_size, num_pages, fill_invalid, stream);
+    return prefill_chunk_aggregate_impl(sh, Q, K_pages, log_sum, aggregate_scores, batch, q_start, q_len, q_strides, block_table, max_pages, page_size, num_pages, fill_invalid, q_start_rows, q_len_rows, stream);
 }
 
 int kascade_prefill_chunk_reuse_call(const kascade_half* Q, const kascade_half* K_pages,
@@ -981,8 +991,9 @@ int kascade_prefill_chunk_reuse_call(const kascade_half* Q, const kascade_half* 
                                      kascade_half* Output, int batch, int q_start, int q_len,
                                      int max_topk_num, int rolling, kascade_strides q_strides,
                                      const int32_t* block_table, int max_pages, int page_size,
-                                     int num_pages, void* stream) {
-    return prefill_chunk_reuse_impl(kRefShape, Q, K_pages, V_pages, physical_rows, head_mapping, topk_percent, Output, batch, q_start, q_len, max_topk_num, rolling, q_strides, block_table, max_pages, page_size, num_pages, stream);
+                                     int num_pages, const int32_t* q_start_rows,
+                                     const int32_t* q_len_rows, void* stream) {
+    return prefill_chunk_reuse_impl(kRefShape, Q, K_pages, V_pages, physical_rows, head_mapping, topk_percent, Output, batch, q_start, q_len, max_topk_num, rolling, q_strides, block_table, max_pages, page_size, num_pages, q_start_rows, q_len_rows, stream);
 }
 
 int kascade_prefill_chunk_reuse_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K_pages,
@@ -991,10 +1002,11 @@ int kascade_prefill_chunk_reuse_shaped_call(const kascade_shape* shape, const ka
                                      kascade_half* Output, int batch, int q_start, int q_len,
                                      int max_topk_num, int rolling, kascade_strides q_strides,
                                      const int32_t* block_table, int max_pages, int page_size,
-                                     int num_pages, void* stream) {
+                                     int num_pages, const int32_t* q_start_rows,
+                                     const int32_t* q_len_rows, void* stream) {
     Shape sh;
     if (get_shape(shape, &sh)) return -1;
-    return prefill_chunk_reuse_impl(sh, Q, K_pages, V_pages, physical_rows, head_mapping, topk_percent, Output, batch, q_start, q_len, max_topk_num, rolling, q_strides, block_table, max_pages, page_size, num_pages, stream);
+    return prefill_chunk_reuse_impl(sh, Q, K_pages, V_pages, physical_rows, head_mapping, topk_percent, Output, batch, q_start, q_len, max_topk_num, rolling, q_strides, block_table, max_pages, page_size, num_pages, q_start_rows, q_len_rows, stream);
 }
 
 int kascade_translate_indices_call(const int32_t* token_idx, int32_t* physical_rows,

@@ -96,8 +96,8 @@ void decode_split_kernel(DecodeParams p) {
     constexpr int kPhaseRows = WRITE_SCORES ? kCodePhase * 4 * kStripRows : 64;
     union Shared {
         MergeState<D, HS> merge[4];
-        struct {
-            uint16_t code[HS][kPhaseRows];
+        struct {   // head rows 32 bytes apart in the banks: the 4 x 4 lanes of a granule write hit 16 bank pairs
+            uint16_t code[HS][kPhaseRows + 16];
             float ref[HS][kPhaseRows / 64];
         } sc;
     };
@@ -290,7 +290,8 @@ void decode_split_kernel(DecodeParams p) {
     for (int blk = 0; blk < (WITH_V ? kOBlocks : 1); ++blk) oacc[blk] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     const int* idx_row = nullptr;
-    if (GATHER) idx_row = p.idx + ((size_t)b * kvh + p.head_map[g]) * p.topk;
+    // a map built for another KV-head count must not leave the index tensor
+    if (GATHER) idx_row = p.idx + ((size_t)b * kvh + max(0, min(p.head_map[g], kvh - 1))) * p.topk;
     const int page_mask = (1 << p.page_shift) - 1;
     const unsigned stride_l = p.kv_stride_l;
     T* kt = &s_kt[wave][0];

@@ -6,7 +6,7 @@ namespace kascade {
 
 hipError_t launch_paged_kv_append(half_t* Kp, half_t* Vp, const half_t* k_new, const half_t* v_new,
                                   const int* start_pos, const int* block_table, int batch,
-                                  int n_new, int max_pages, int page_shift, long long sb,
+                                  int n_new, const int* n_new_rows, int max_pages, int page_shift, long long sb,
                                   long long sl, long long sh, int groups, int head_dim,
                                   hipStream_t stream);
 

@@ -10,8 +10,8 @@ namespace {
 __global__ __launch_bounds__(256) void paged_kv_append_kernel(
     half_t* __restrict__ Kp, half_t* __restrict__ Vp, const half_t* __restrict__ k_new,
     const half_t* __restrict__ v_new, const int* __restrict__ start_pos,
-    const int* __restrict__ block_table, int batch, int n_new, int max_pages, int page_shift,
-    long long sb, long long sl, long long sh, int groups, int head_dim) {
+    const int* __restrict__ block_table, int batch, int n_new, const int* __restrict__ n_new_rows,
+    int max_pages, int page_shift, long long sb, long long sl, long long sh, int groups, int head_dim) {
     const int chunks = head_dim / 8;
     const long long total = (long long)batch * n_new * groups * chunks;
     const long long c = (long long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -21,6 +21,7 @@ __global__ __launch_bounds__(256) void paged_kv_append_kernel(
     const long long bt = c / (chunks * groups);
     const int t = (int)(bt % n_new);
     const int b = (int)(bt / n_new);
+    if (n_new_rows && t >= n_new_rows[b]) return;   // this sequence brings fewer rows than the batch's widest
     const int tok = start_pos[b] + t;
     // a position before the sequence or beyond what the block table covers has no slot: skipped,
     // like rope_append_kernel does (reading the table there would land in another sequence's row)
@@ -42,14 +43,16 @@ __global__ __launch_bounds__(256) void decode_budgets_kernel(int* __restrict__ s
                                                              int* __restrict__ n_sel_rows) {
     // a single workgroup: the barrier puts the in-place update after every read of a length
     for (int i = threadIdx.x; i < batch * groups; i += blockDim.x) {
-        const int len = seqlens[i / groups] + advance;
+        const int cur = seqlens[i / groups];
+        const int len = cur > 0 ? cur + advance : cur;   // length 0: an empty slot of the batch, left alone
         const long long fl = (long long)floor((double)percent * (double)len / 100.0);
         if (valid_rows) valid_rows[i] = len;
         if (n_sel_rows) n_sel_rows[i] = (int)(((fl + 127) / 128) * 128);
     }
     __syncthreads();
     if (advance != 0)
-        for (int b = threadIdx.x; b < batch; b += blockDim.x) seqlens[b] += advance;
+        for (int b = threadIdx.x; b < batch; b += blockDim.x)
+            if (seqlens[b] > 0) seqlens[b] += advance;
 }
 
 
@@ -170,14 +173,14 @@ hipError_t launch_decode_budgets(int* seqlens, int advance, float percent, int b
 
 hipError_t launch_paged_kv_append(half_t* Kp, half_t* Vp, const half_t* k_new, const half_t* v_new,
                                   const int* start_pos, const int* block_table, int batch,
-                                  int n_new, int max_pages, int page_shift, long long sb,
+                                  int n_new, const int* n_new_rows, int max_pages, int page_shift, long long sb,
                                   long long sl, long long sh, int groups, int head_dim,
                                   hipStream_t stream) {
     const long long total = (long long)batch * n_new * groups * (head_dim / 8);
     if (total == 0) return hipSuccess;
     dim3 grid((unsigned)((total + 255) / 256)), block(256);
     hipLaunchKernelGGL(paged_kv_append_kernel, grid, block, 0, stream, Kp, Vp, k_new, v_new,
-                       start_pos, block_table, batch, n_new, max_pages, page_shift, sb, sl, sh, groups, head_dim);
+                       start_pos, block_table, batch, n_new, n_new_rows, max_pages, page_shift, sb, sl, sh, groups, head_dim);
     return hipGetLastError();
 }
 

@@ -24,6 +24,12 @@ struct PrefillParams {
     void* O;                  // [B,Lq,H,D] contiguous
     half_t* agg;              // [B,G,T,L] (aggregate)
     const int* block_table;   // [B,max_pages] or null (strided K/V)
+    // Chunked prefill of a batch whose sequences stand at different positions (both null: every
+    // sequence starts at q_start and has Lq rows).  q_start_rows[b]: first global position of
+    // sequence b's rows (a multiple of 32, at most q_start); q_len_rows[b]: how many of the Lq rows
+    // of Q belong to it (null: all).  Rows beyond are left alone: no output, no log-sum, no scores.
+    const int* q_start_rows;
+    const int* q_len_rows;
     long long q_sb, q_sl, q_sh;
     long long k_sb, k_sl, k_sh;
     int B, L, T;              // T = ceil(Lq / 32) query tiles of this call

@@ -98,6 +98,25 @@ __device__ __forceinline__ int rolling_budget(float pct, int tile_start) {
     return (int)(((fl + 127) / 128) * 128);
 }
 
+// Index-row width the host gives a prompt of L keys: min(128 ceil(min(max(128, floor(pct L / 100)), L) / 128), L).
+__device__ __forceinline__ int topk_width_of(float pct, int L) {
+    long long k = (long long)floor((double)pct * (double)L / 100.0);
+    if (k < 128) k = 128;
+    if (k > L) k = L;
+    k = ((k + 127) / 128) * 128;
+    return (int)(k > L ? L : k);
+}
+
+// Where sequence b's rows of a chunked call stand: first global position and number of rows.
+__device__ __forceinline__ void chunk_of_sequence(const PrefillParams& p, int b, int& q_start, int& rows) {
+    q_start = p.q_start;
+    rows = p.Lq;
+    if (p.q_start_rows) {
+        q_start = max(0, min(p.q_start_rows[b], p.q_start)) & ~(kTile - 1);
+        if (p.q_len_rows) rows = max(0, min(p.q_len_rows[b], p.Lq));
+    }
+}
+
 // Queries are rows [0, Lq) of Q at global positions q_start + row (q_start a multiple of 32);
 // keys are positions [0, L) with L = q_start + Lq.  PAGED: K/V are pages [P, page, G, D]
 // addressed through the block table, and gathered index rows hold physical row numbers.
@@ -117,11 +136,13 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
     const T* Vp = (const T*)p.V;
 
     constexpr int QT = 32 * NQB;
-    const int L = p.L;
-    const int Lq = p.Lq;
+    const int Lq = p.Lq;            // rows of Q and of the outputs per sequence
     const int nqt = (Lq + QT - 1) / QT;
     int blk, g, b;
     unit_of_workgroup(p.B, p.G * hs.subs, nqt, blk, g, b);   // g: KV head and sub-group
+    int q_start, Lqv;               // this sequence's first position and how many of the rows are its own
+    chunk_of_sequence(p, b, q_start, Lqv);
+    const int L = q_start + Lqv;    // keys of this sequence
     int sub = 0;
     if (hs.subs > 1) {
         sub = g % hs.subs;
@@ -134,7 +155,8 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
     const int li = lane & 31;
     const int lg = lane >> 5;
     const int q0l = tq * QT;            // first query row of this block
-    const int q0 = p.q_start + q0l;     // its global position
+    if (q0l >= Lqv) return;             // a block past this sequence's rows (uniform over the workgroup)
+    const int q0 = q_start + q0l;       // its global position
     const int head = g * hs.gs + min(4 * sub + wave, hs.gs - 1);
     const bool real_head = 4 * sub + wave < hs.gs;   // a slot beyond the last head computes along and stores nothing
 
@@ -143,12 +165,16 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
     int n = 0, ng = 0;
     const int* idx_row = nullptr;
     if (REUSE) {
-        n = (p.rolling && L > 128) ? rolling_budget(p.topk_percent, q0) : p.max_topk;
-        n = min(n, p.max_topk);
+        // a sequence of a mixed batch keeps the budget it has on its own (the rows are as wide as
+        // the longest sequence needs)
+        const int width = p.q_start_rows ? min(p.max_topk, topk_width_of(p.topk_percent, L)) : p.max_topk;
+        n = (p.rolling && L > 128) ? rolling_budget(p.topk_percent, q0) : width;
+        n = min(n, width);
         if (q0 > n) {
             sparse = true;
             ng = (n + kKT - 1) / kKT;
-            idx_row = p.idx + (((long long)b * kvh + p.head_map[g]) * p.T + tq) * p.max_topk;
+            const int src = max(0, min(p.head_map[g], kvh - 1));   // a map built for another head count must not leave the tensor
+            idx_row = p.idx + (((long long)b * kvh + src) * p.T + tq) * p.max_topk;
         }
     }
     const int ntiles = sparse ? ng + 1 : (min(q0 + QT, L) + kKT - 1) / kKT;
@@ -281,8 +307,8 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
 #pragma unroll
     for (int qb = 0; qb < NQB; ++qb) {
         const int ql = q0l + 32 * qb + li;
-        const bool ok = ql < Lq;
-        const T* qp = Qp + (long long)b * p.q_sb + (long long)min(ql, Lq - 1) * p.q_sl +
+        const bool ok = ql < Lqv;
+        const T* qp = Qp + (long long)b * p.q_sb + (long long)min(ql, Lqv - 1) * p.q_sl +
                       (long long)head * p.q_sh + lg * 8;
 #pragma unroll
         for (int ks = 0; ks < kKS; ++ks) {
@@ -494,7 +520,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
     for (int qb = 0; qb < NQB; ++qb) {
         const int ql = q0l + 32 * qb + li;
         const float lt = sum_with_other_half(l[qb]);
-        if (p.log_sum && lg == 0 && ql < Lq && real_head)
+        if (p.log_sum && lg == 0 && ql < Lqv && real_head)
             p.log_sum[((long long)b * Lq + ql) * nheads + head] = fast_log2(lt) + m[qb];
         if (WITH_V) {
             T* so = sK + wave * (32 * D);
@@ -513,7 +539,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
                 const int r = j * kRPL + lrow;
                 const uint4_t row = *reinterpret_cast<const uint4_t*>(&so[r * D + lchunk * 8]);
                 const int qr = q0l + r;
-                if (qr < Lq && real_head)   // the output is not read again by these kernels: keep it out of the caches
+                if (qr < Lqv && real_head)   // the output is not read again by these kernels: keep it out of the caches
                     __builtin_nontemporal_store(row, reinterpret_cast<uint4_t*>(
                         (T*)p.O + (((long long)b * Lq + qr) * nheads + head) * D + ((lchunk ^ (r & (kChunks - 1))) * 8)));
             }
@@ -572,10 +598,13 @@ void prefill_aggregate_kernel(PrefillParams p) {
     __shared__ __attribute__((aligned(1024))) T sK[2 * 4 * kWaveElems];
     __shared__ __attribute__((aligned(16))) float s_lse[128];
 
-    const int L = p.L;
+    const int Ls = p.L;                  // width of a row of pooled scores
     const int Lq = p.Lq;
     int blk, g, b;
     unit_of_workgroup(p.B, p.G, p.T, blk, g, b);
+    int q_start, Lqv;                    // this sequence's first position and how many of the rows are its own
+    chunk_of_sequence(p, b, q_start, Lqv);
+    const int L = q_start + Lqv;         // keys of this sequence
     const int t = p.T - 1 - blk;
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
@@ -583,11 +612,11 @@ void prefill_aggregate_kernel(PrefillParams p) {
     const int li = lane & 31;
     const int lg = lane >> 5;
     const int tl = t * kTile;            // first query row of the tile
-    const int ts = p.q_start + tl;       // its global position
-    half_t* out = p.agg + (((long long)b * kvh + g) * p.T + t) * L;
+    const int ts = q_start + tl;         // its global position
+    half_t* out = p.agg + (((long long)b * kvh + g) * p.T + t) * Ls;
     const half_t neg_inf = (half_t)(-INFINITY);
 
-    const int ntiles = (ts + kAggKT - 1) / kAggKT;
+    const int ntiles = tl < Lqv ? (ts + kAggKT - 1) / kAggKT : 0;   // a tile past the sequence's rows pools nothing
     if (ntiles > 0) {
         // A operands: row block rb = head slot rb of this launch's sub-group, row li = query tl+li
         const int head0 = g * hs.gs + 4 * p.vsub;
@@ -595,8 +624,8 @@ void prefill_aggregate_kernel(PrefillParams p) {
 #pragma unroll
         for (int rb = 0; rb < kGroupSize; ++rb) {
             const int q = tl + li;
-            const bool ok = q < Lq;
-            const T* qp = Qp + (long long)b * p.q_sb + (long long)min(q, Lq - 1) * p.q_sl +
+            const bool ok = q < Lqv;
+            const T* qp = Qp + (long long)b * p.q_sb + (long long)min(q, Lqv - 1) * p.q_sl +
                           (long long)min(head0 + rb, g * hs.gs + hs.gs - 1) * p.q_sh + lg * 8;
 #pragma unroll
             for (int ks = 0; ks < kKS; ++ks) {
@@ -609,7 +638,7 @@ void prefill_aggregate_kernel(PrefillParams p) {
         if (tid < 128) {
             const int q = tl + (tid & 31);
             // a query row past the chunk, or a slot past the KV head's last query head, adds exp2(-inf) = 0
-            const bool counts = q < Lq && 4 * p.vsub + (tid >> 5) < hs.gs;
+            const bool counts = q < Lqv && 4 * p.vsub + (tid >> 5) < hs.gs;
             s_lse[tid] = counts ? p.log_sum_in[((long long)b * Lq + q) * nheads + head0 + (tid >> 5)] : INFINITY;
         }
 
@@ -693,7 +722,7 @@ void prefill_aggregate_kernel(PrefillParams p) {
                 }
             sum = sum_with_other_half(sum);
             const int key = ti * kAggKT + 32 * wave + li;
-            if (lg == 0 && key < L) {
+            if (lg == 0 && key < Ls) {
                 if (key < ts)   // a later sub-group of the KV head adds to what the earlier ones left
                     out[key] = (half_t)(p.accumulate ? sum + (float)out[key] : sum);
                 else if (p.fill_invalid)
@@ -703,7 +732,7 @@ void prefill_aggregate_kernel(PrefillParams p) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no load may land in LDS after the workgroup has left
     }
     if (p.fill_invalid) {
-        for (int key = ntiles * kAggKT + tid; key < L; key += kThreads) out[key] = neg_inf;
+        for (int key = ntiles * kAggKT + tid; key < Ls; key += kThreads) out[key] = neg_inf;
     }
 }
 

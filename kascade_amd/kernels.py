@@ -587,8 +587,10 @@ def prefill_reuse(Q, K, V, topk_idx, head_mapping, topk_percent, rolling: bool) 
 
 
 # ------------------------------------------------------------- KV append
-def paged_kv_append(K_pages, V_pages, k_new, v_new, start_pos, block_table, page_size: int = 16):
-    """Write k_new/v_new [B,n_new,G,D] into the paged cache at positions start_pos[b]+t."""
+def paged_kv_append(K_pages, V_pages, k_new, v_new, start_pos, block_table, page_size: int = 16,
+                    n_new_rows=None):
+    """Write k_new/v_new [B,n_new,G,D] into the paged cache at positions start_pos[b]+t.
+    n_new_rows [B] int32: sequence b brings only its first n_new_rows[b] rows."""
     lib = _lib.init()
     dt = K_pages.dtype
     if dt not in _ELEM:
@@ -603,9 +605,15 @@ def paged_kv_append(K_pages, V_pages, k_new, v_new, start_pos, block_table, page
         raise KascadeError("pages [num_pages,page,G,D] and new rows [B,n,G,D] must agree, D 64 or 128")
     B, n_new = k_new.shape[0], k_new.shape[1]
     st = _blhd_strides(k_new, "k_new")
+    if start_pos.numel() != B or block_table.shape[0] != B:
+        raise KascadeError("start_pos and block_table must have one row per sequence")
+    if n_new_rows is not None:
+        _req(n_new_rows, torch.int32, "n_new_rows")
+        if n_new_rows.numel() != B:
+            raise KascadeError("n_new_rows must have one entry per sequence")
     _lib.check(_call(lib, "paged_kv_append", (GROUP * Gk, Gk, Dh, dt),
         _ptr(K_pages), _ptr(V_pages), _ptr(k_new), _ptr(v_new), _ptr(start_pos), _ptr(block_table),
-        B, n_new, block_table.shape[1], page_size, st, _stream()))
+        B, n_new, block_table.shape[1], page_size, st, _ptr(n_new_rows), _stream()))
 
 
 def rope_table(max_pos: int, theta: float = 1e6, device="cuda", round_to=torch.float16,
@@ -670,7 +678,7 @@ def rope_append_paged(q_in, k_in, v_in, cos_sin, start_pos, K_pages, V_pages, bl
 
 
 # ------------------------------------------- chunked prefill over the paged cache
-def _chunk_args(Q, K_pages, block_table, q_start: int, page_size: int):
+def _chunk_args(Q, K_pages, block_table, q_start: int, page_size: int, q_starts=None, q_lens=None):
     shape = _shape(Q, K_pages)
     _req(Q, shape[3], "Q", False); _req(K_pages, shape[3], "K_pages")
     _req(block_table, torch.int32, "block_table")
@@ -678,17 +686,30 @@ def _chunk_args(Q, K_pages, block_table, q_start: int, page_size: int):
         raise KascadeError(f"pages must be [num_pages,{page_size},G,D]")
     if q_start % TILE:
         raise KascadeError(f"q_start must be a multiple of {TILE}")
+    if block_table.shape[0] != Q.shape[0]:
+        raise KascadeError("block_table must have one row per sequence")
+    for t, name in ((q_starts, "q_starts"), (q_lens, "q_lens")):
+        if t is not None:
+            _req(t, torch.int32, name)
+            if t.numel() != Q.shape[0]:
+                raise KascadeError(f"{name} must have one entry per sequence")
+    if q_lens is not None and q_starts is None:
+        raise KascadeError("q_lens comes with q_starts")
     return Q.shape[0], Q.shape[1], _blhd_strides(Q, "Q"), shape
 
 
 def prefill_chunk_dense(Q, K_pages, V_pages, block_table, q_start: int, page_size: int = 16,
-                        with_output: bool = True) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+                        with_output: bool = True, q_starts=None, q_lens=None
+                        ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """Dense causal attention of a chunk's queries (global positions q_start..q_start+Lq-1) over
     cache positions [0, q_start+Lq): the chunked form of ``prefill_recomp0_kernel`` /
     ``prefill_recomp1_kernel`` (EfficientKascadeStrategy.py:78, 80).  Returns (log_sum, O);
-    O is None without with_output."""
+    O is None without with_output.
+    q_starts / q_lens [B] int32 (device): a batch whose sequences stand at different positions --
+    sequence b's rows start at q_starts[b] (a multiple of 32, at most q_start) and the first
+    q_lens[b] rows of Q are its own; rows beyond are not written."""
     lib = _lib.init()
-    B, Lq, qs, shape = _chunk_args(Q, K_pages, block_table, q_start, page_size)
+    B, Lq, qs, shape = _chunk_args(Q, K_pages, block_table, q_start, page_size, q_starts, q_lens)
     Hq, _, Dh, dt = shape
     log_sum = torch.empty(B, Lq, Hq, device=Q.device, dtype=torch.float32)
     out = torch.empty(B, Lq, Hq, Dh, device=Q.device, dtype=dt) if with_output else None
@@ -699,16 +720,16 @@ def prefill_chunk_dense(Q, K_pages, V_pages, block_table, q_start: int, page_siz
     _lib.check(_call(lib, "prefill_chunk_dense", shape,
         _ptr(Q), _ptr(K_pages), _ptr(V_pages) if with_output else None, _ptr(log_sum), _ptr(out), B,
         q_start, Lq, qs, _ptr(block_table), block_table.shape[1], page_size, K_pages.shape[0],
-        1 if with_output else 0, _stream()))
+        1 if with_output else 0, _ptr(q_starts), _ptr(q_lens), _stream()))
     return log_sum, out
 
 
 def prefill_chunk_aggregate(Q, K_pages, log_sum, scores, block_table, q_start: int,
-                            page_size: int = 16, fill_invalid: bool = False) -> None:
+                            page_size: int = 16, fill_invalid: bool = False, q_starts=None, q_lens=None) -> None:
     """Chunked ``aggregate_kernel`` (EfficientKascadeStrategy.py:81): scores
     [B,G,ceil(Lq/32),q_start+Lq] fp16, row t valid for keys < q_start + 32 t."""
     lib = _lib.init()
-    B, Lq, qs, shape = _chunk_args(Q, K_pages, block_table, q_start, page_size)
+    B, Lq, qs, shape = _chunk_args(Q, K_pages, block_table, q_start, page_size, q_starts, q_lens)
     Hq, Gk = shape[0], shape[1]
     _req(log_sum, torch.float32, "log_sum"); _req(scores, torch.float16, "scores")
     T = (Lq + TILE - 1) // TILE
@@ -716,7 +737,8 @@ def prefill_chunk_aggregate(Q, K_pages, log_sum, scores, block_table, q_start: i
         raise KascadeError("scores must be [B,G,ceil(Lq/32),q_start+Lq] and log_sum [B,Lq,H]")
     _lib.check(_call(lib, "prefill_chunk_aggregate", shape,
         _ptr(Q), _ptr(K_pages), _ptr(log_sum), _ptr(scores), B, q_start, Lq, qs, _ptr(block_table),
-        block_table.shape[1], page_size, K_pages.shape[0], 1 if fill_invalid else 0, _stream()))
+        block_table.shape[1], page_size, K_pages.shape[0], 1 if fill_invalid else 0, _ptr(q_starts),
+        _ptr(q_lens), _stream()))
 
 
 def translate_indices(token_idx, block_table, kv_len: int, page_size: int = 16, out=None):
@@ -734,11 +756,12 @@ def translate_indices(token_idx, block_table, kv_len: int, page_size: int = 16, 
 
 
 def prefill_chunk_reuse(Q, K_pages, V_pages, physical_rows, head_mapping, topk_percent,
-                        rolling: bool, block_table, q_start: int, page_size: int = 16) -> torch.Tensor:
+                        rolling: bool, block_table, q_start: int, page_size: int = 16,
+                        q_starts=None, q_lens=None) -> torch.Tensor:
     """Chunked ``prefill_reuse_kernel`` (EfficientKascadeStrategy.py:92, 97): physical_rows
     [B,G,ceil(Lq/32),max_topk] comes from ``translate_indices``."""
     lib = _lib.init()
-    B, Lq, qs, shape = _chunk_args(Q, K_pages, block_table, q_start, page_size)
+    B, Lq, qs, shape = _chunk_args(Q, K_pages, block_table, q_start, page_size, q_starts, q_lens)
     Hq, Gk, Dh, dt = shape
     _req(V_pages, dt, "V_pages")
     if V_pages.shape != K_pages.shape:
@@ -751,7 +774,8 @@ def prefill_chunk_reuse(Q, K_pages, V_pages, physical_rows, head_mapping, topk_p
     _lib.check(_call(lib, "prefill_chunk_reuse", shape,
         _ptr(Q), _ptr(K_pages), _ptr(V_pages), _ptr(physical_rows), _ptr(head_mapping),
         float(topk_percent), _ptr(out), B, q_start, Lq, physical_rows.shape[-1], 1 if rolling else 0,
-        qs, _ptr(block_table), block_table.shape[1], page_size, K_pages.shape[0], _stream()))
+        qs, _ptr(block_table), block_table.shape[1], page_size, K_pages.shape[0], _ptr(q_starts),
+        _ptr(q_lens), _stream()))
     return out
 
 

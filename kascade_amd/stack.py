@@ -4,13 +4,16 @@ strategy (EfficientKascadeStrategy.py:126-161 decides per call between the four 
 the same decision is made per layer of a chunk or of a decode step).
 
 Only attention runs here: the caller supplies each layer's Q and the new K/V rows (in a model
-they come from the layer's projections).  Every layer has its own pages; all layers share the
-sequence's block table, so an anchor layer's selection, translated once to cache rows, serves
-the reuse layers that follow it.
+they come from the layer's projections).  Every layer has its own pages; all layers share one
+block table (``paging.PagedKVCache``), so an anchor layer's selection, translated once to cache
+rows, serves the reuse layers that follow it.  The batch is a fixed number of slots; a slot of
+length 0 is empty, sequences join (``admit`` + prefill chunks at their own offsets) and leave
+(``release``) while the others keep decoding.
 
 A decode step is a fixed launch sequence whose only varying inputs live in device memory (the
-new rows and the sequence lengths), so it can be captured once into a HIP graph and replayed:
-at short contexts the step is launch-bound and the graph removes the host from the loop.
+new rows, the sequence lengths and the block table), so it can be captured once into a HIP graph
+and replayed: at short contexts the step is launch-bound and the graph removes the host from the
+loop.
 """
 from __future__ import annotations
 
@@ -21,6 +24,7 @@ import torch
 
 from . import kernels
 from ._lib import KascadeError
+from .paging import PagedKVCache
 from .strategy import PagedKascadeDecoder, PagedKascadePrefill
 
 H, G, D, TILE = 32, 8, 128, 32
@@ -31,11 +35,14 @@ class KascadeAttentionStack:
                  k: float, max_seqlen: int, batch: int = 1, page_size: int = 16,
                  rolling_prefill: bool = True, device="cuda", table_seed: int = 0,
                  dense: bool = False, kv_heads: int = G, head_dim: int = D, dtype=torch.float16,
-                 group_size: int = kernels.GROUP):
+                 group_size: int = kernels.GROUP, num_pages: Optional[int] = None, reserve: bool = True):
         """dense=True runs every layer as dense attention over the same caches (the baseline).
         kv_heads, head_dim, dtype, group_size: the model's shape (group_size * kv_heads query
         heads, group_size 1 to 16; head_dim 64 or 128; float16 or bfloat16); the default
-        is the reference's."""
+        is the reference's.
+        num_pages: size of the page pool (default: every slot can reach max_seqlen).
+        reserve: every slot starts admitted with pages for max_seqlen tokens (a fixed batch);
+        with reserve=False slots start empty and take pages as their sequences grow."""
         if 0 not in recompute_layers and not dense:
             raise KascadeError("layer 0 must be an anchor layer")
         self.num_layers, self.batch, self.page_size = num_layers, batch, page_size
@@ -45,15 +52,13 @@ class KascadeAttentionStack:
         self.max_seqlen = max_seqlen
         self.G, self.H, self.D, self.dtype = kv_heads, group_size * kv_heads, head_dim, dtype
         pages_per_seq = math.ceil(max_seqlen / page_size)
-        n_pages = batch * pages_per_seq
-        gen = torch.Generator().manual_seed(table_seed)
-        self.block_table = torch.randperm(n_pages, generator=gen).to(torch.int32).view(batch, pages_per_seq) \
-            .to(self.device)
-        self.k_pages = [torch.zeros(n_pages, page_size, kv_heads, head_dim, device=self.device, dtype=dtype)
-                        for _ in range(num_layers)]
-        self.v_pages = [torch.zeros_like(p) for p in self.k_pages]
-        self.length = 0                                                 # host copy of the common length
-        self.seqlens = torch.zeros(batch, device=self.device, dtype=torch.int32)
+        self.cache = PagedKVCache(num_layers, num_pages or batch * pages_per_seq, batch, pages_per_seq, page_size,
+                                  kv_heads, head_dim, dtype, self.device, shuffle_seed=table_seed)
+        self.k_pages, self.v_pages = self.cache.k_pages, self.cache.v_pages
+        self.block_table, self.seqlens = self.cache.block_table, self.cache.seqlens
+        if reserve:
+            for b in range(batch):
+                self.cache.admit(max_seqlen, slot=b)
         self.prefill = PagedKascadePrefill(k, head_mapping, recompute_layers, page_size, rolling_prefill,
                                            self.device, kv_heads=kv_heads)
         self.decoder = PagedKascadeDecoder(k, head_mapping, recompute_layers, batch, max_seqlen, page_size,
@@ -61,44 +66,89 @@ class KascadeAttentionStack:
                                            group_size=group_size)
         self._graph = None
 
+    @property
+    def lengths(self) -> List[int]:
+        """Host view of the per-slot lengths."""
+        return self.cache.lengths
+
+    @property
+    def length(self) -> int:
+        """The longest sequence of the batch (the common length of a uniform batch)."""
+        return max(self.cache.lengths)
+
+    # ------------------------------------------------------------------ sequences
+    def admit(self, reserve_tokens: int = 0, slot: Optional[int] = None) -> int:
+        """A new sequence takes a free slot (length 0 until its first prefill chunk)."""
+        return self.cache.admit(reserve_tokens, slot)
+
+    def release(self, slot: int) -> None:
+        """The slot's sequence leaves the batch; its pages return to the pool."""
+        self.cache.release(slot)
+
     def reset(self, length: int = 0):
         """Forget everything cached beyond ``length`` tokens (the pages keep their contents)."""
-        self.length = length
-        self.seqlens.fill_(length)
+        for b in self.cache.active_slots():
+            self.cache.set_length(b, length)
 
     def set_lengths(self, lengths: Sequence[int]):
         """Per-sequence lengths for decoding a batch whose caches were filled sequence by
         sequence (``kernels.paged_kv_append`` into ``k_pages`` / ``v_pages`` through
-        ``block_table``).  Chunked prefill through ``prefill_chunk`` needs a common length."""
+        ``block_table``)."""
         if len(lengths) != self.batch or max(lengths) > self.max_seqlen or min(lengths) < 0:
             raise KascadeError("set_lengths: one length per sequence, each within max_seqlen")
-        self.length = int(max(lengths))
-        self.seqlens.copy_(torch.tensor(list(lengths), dtype=torch.int32))
+        for b, n in enumerate(lengths):
+            self.cache.set_length(b, int(n))
 
     # ------------------------------------------------------------------ prefill
+    def _chunk_geometry(self, Lq: int, q_lens: Optional[Sequence[int]]):
+        """Start and row count per slot of a chunk, as PagedKascadePrefill takes them, with room
+        reserved in the cache.  A uniform batch (every slot at one length, all rows) stays uniform."""
+        cur = self.cache.lengths
+        active = self.cache.active_slots()
+        lens = [Lq if b in active else 0 for b in range(self.batch)] if q_lens is None else [int(n) for n in q_lens]
+        if len(lens) != self.batch or any(n < 0 or n > Lq for n in lens):
+            raise KascadeError("q_lens: one row count per slot, each within the rows of q")
+        for b, n in enumerate(lens):
+            if n == 0:
+                continue
+            if b not in active:
+                raise KascadeError(f"slot {b} holds no sequence")
+            if cur[b] % TILE:
+                raise KascadeError("a prefill chunk must start at a multiple of 32 tokens")
+            if cur[b] + n > self.max_seqlen:
+                raise KascadeError("chunk exceeds max_seqlen")
+            self.cache.reserve(b, cur[b] + n)
+        starts = [cur[b] if lens[b] else 0 for b in range(self.batch)]
+        if len(set(starts)) == 1 and all(n == Lq for n in lens):
+            return starts[0], None, lens
+        return starts, lens, lens
+
     def prefill_chunk(self, q: Sequence[torch.Tensor], k_new: Sequence[torch.Tensor],
-                      v_new: Sequence[torch.Tensor]) -> List[torch.Tensor]:
-        """One chunk through all layers.  q[l] [B,Lq,H,D], k_new[l]/v_new[l] [B,Lq,G,D]; the chunk
-        starts at the current length, which must be a multiple of 32.  Returns O[l] [B,Lq,H,D]."""
+                      v_new: Sequence[torch.Tensor], q_lens: Optional[Sequence[int]] = None) -> List[torch.Tensor]:
+        """One chunk through all layers.  q[l] [B,Lq,H,D], k_new[l]/v_new[l] [B,Lq,G,D]; every
+        slot's rows start at that slot's current length, which must be a multiple of 32.
+        q_lens: how many of the Lq rows belong to each slot (default: all rows of every slot that
+        holds a sequence; 0 = the slot sits this chunk out).  Returns O[l] [B,Lq,H,D]; rows that
+        belong to no sequence are not written."""
         Lq = q[0].shape[1]
-        q_start = self.length
-        if self.batch > 1 and int(self.seqlens.min()) != q_start:
-            raise KascadeError("chunked prefill of a batch needs sequences of one common length")
-        if q_start % TILE:
-            raise KascadeError("a prefill chunk must start at a multiple of 32 tokens")
-        if q_start + Lq > self.max_seqlen:
-            raise KascadeError("chunk exceeds max_seqlen")
+        q_start, ragged_lens, lens = self._chunk_geometry(Lq, q_lens)
+        n_rows = None if ragged_lens is None else self.prefill._geometry(q_start, ragged_lens, Lq)[2]
         outs = []
         for l in range(self.num_layers):
             kernels.paged_kv_append(self.k_pages[l], self.v_pages[l], k_new[l], v_new[l], self.seqlens,
-                                    self.block_table, self.page_size)
+                                    self.block_table, self.page_size, n_new_rows=n_rows)
             if self.dense_only:
-                outs.append(self.prefill.dense(q[l], self.k_pages[l], self.v_pages[l], self.block_table, q_start))
+                outs.append(self.prefill.dense(q[l], self.k_pages[l], self.v_pages[l], self.block_table, q_start,
+                                               ragged_lens))
             else:
                 outs.append(self.prefill.forward(l, q[l], self.k_pages[l], self.v_pages[l], self.block_table,
-                                                 q_start))
-        self.length += Lq
-        self.seqlens += Lq
+                                                 q_start, ragged_lens))
+        if n_rows is None:
+            self.seqlens += Lq
+        else:
+            self.seqlens += n_rows
+        for b, n in enumerate(lens):
+            self.cache.lengths[b] += n
         return outs
 
     # ------------------------------------------------------------------- decode
@@ -122,13 +172,18 @@ class KascadeAttentionStack:
     def decode_step(self, q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor,
                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """q [layers,B,H,D], k_new/v_new [layers,B,1,G,D] -> O [layers,B,H,D] (eager launches)."""
-        if self.length + 1 > self.max_seqlen:
-            raise KascadeError("decode step exceeds max_seqlen")
+        self._before_step()
         if out is None:
             out = torch.empty(self.num_layers, self.batch, self.H, self.D, device=self.device, dtype=self.dtype)
         self._decode_layers(q, k_new, v_new, out)
-        self.length += 1
+        self.cache.note_advance(1)
         return out
+
+    def _before_step(self):
+        """Every non-empty slot has a page for its next token (slots of length 0 sit the step out)."""
+        if self.length + 1 > self.max_seqlen:
+            raise KascadeError("decode step exceeds max_seqlen")
+        self.cache.ensure_room(1)
 
     def capture_decode(self):
         """Capture one decode step into a HIP graph over static input/output buffers
@@ -158,8 +213,7 @@ class KascadeAttentionStack:
         """Replay the captured step on the inputs currently in the static buffers."""
         if self._graph is None:
             raise KascadeError("capture_decode() first")
-        if self.length + 1 > self.max_seqlen:
-            raise KascadeError("decode step exceeds max_seqlen")
+        self._before_step()
         self._graph.replay()
-        self.length += 1
+        self.cache.note_advance(1)
         return self.graph_out

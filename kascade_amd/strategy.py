@@ -54,6 +54,16 @@ def get_head_mapping(model_name: str, recompute_layers: Sequence[int],
     raise ValueError(f"Head mapping file not found for model {model_name} with layers {list(recompute_layers)}.")
 
 
+def _head_map_tensor(row, groups: int, layer, device) -> torch.Tensor:
+    """One layer's head map as a device tensor: one entry per KV head, each naming a KV head."""
+    row = [int(x) for x in row]
+    if len(row) != groups:
+        raise KascadeError(f"head mapping of layer {layer} has {len(row)} entries for {groups} KV heads")
+    if any(x < 0 or x >= groups for x in row):
+        raise KascadeError(f"head mapping of layer {layer} names a KV head outside 0..{groups - 1}")
+    return torch.tensor(row, device=device, dtype=torch.int32)
+
+
 class EfficientKascadeStrategy:
     """Drop-in for the reference's EfficientKascadeStrategy (name ``efficient_kascade``)."""
 
@@ -91,9 +101,7 @@ class EfficientKascadeStrategy:
         key = (layer, str(device), groups)
         if key not in self._hm_cache:
             row = list(range(groups)) if layer is None else self._head_mapping[layer]
-            if len(row) != groups:
-                raise KascadeError(f"head mapping of layer {layer} has {len(row)} entries for {groups} KV heads")
-            self._hm_cache[key] = torch.tensor(row, device=device, dtype=torch.int32)
+            self._hm_cache[key] = _head_map_tensor(row, groups, layer, device)
         return self._hm_cache[key]
 
     def _tile_budgets(self, L, width, device):
@@ -303,7 +311,7 @@ class PagedKascadeDecoder:
         self._scratch_views = {}
         self._hm = {None: torch.arange(G, device=dev, dtype=torch.int32)}
         for l, row in enumerate(head_mapping):
-            self._hm[l] = torch.tensor(row, device=dev, dtype=torch.int32)
+            self._hm[l] = _head_map_tensor(row, G, l, dev)
         self._topk_to_reuse = None      # the last anchor's selection as token positions
         self._rows_to_reuse = None      # ... translated to cache rows, what the reuse launches gather from
         widest = max(self.max_topk, budgets.topk_width(max_seqlen, k), budgets.CHUNK)
@@ -431,10 +439,11 @@ class PagedKascadePrefill:
         self.G = kv_heads
         self._hm = {None: torch.arange(kv_heads, device=self.device, dtype=torch.int32)}
         for l, row in enumerate(head_mapping):
-            self._hm[l] = torch.tensor(row, device=self.device, dtype=torch.int32)
+            self._hm[l] = _head_map_tensor(row, kv_heads, l, self.device)
         self._rows_to_reuse = None      # physical rows [B,G,T,width] of the last anchor
         self._topk_to_reuse = None      # the same selection as token positions
         self._budget_cache = {}
+        self._geom_cache = {}
         self._scores = None
 
     def _tile_budgets(self, q_start: int, Lq: int, width: int):
@@ -453,6 +462,55 @@ class PagedKascadePrefill:
             self._budget_cache[key] = hit
         return hit
 
+    def _geometry(self, q_start, q_lens, Lq: int):
+        """Where the rows of a call stand.  q_start: one int for the whole batch, or one per
+        sequence (the scheduler's view: host ints, multiples of 32); q_lens: how many of the Lq
+        rows belong to each sequence (default all).  Returns (largest start, device starts,
+        device lengths, host starts, host lengths); the device tensors are None for a uniform batch."""
+        if isinstance(q_start, int) and q_lens is None:
+            return q_start, None, None, None, None
+        starts = [int(q_start)] * len(q_lens) if isinstance(q_start, int) else [int(x) for x in q_start]
+        lens = [Lq] * len(starts) if q_lens is None else [int(x) for x in q_lens]
+        if len(lens) != len(starts) or any(x % TILE or x < 0 for x in starts) or any(n < 0 or n > Lq for n in lens):
+            raise KascadeError("per-sequence chunk starts must be multiples of 32 and lengths within the rows of Q")
+        key = (tuple(starts), tuple(lens))
+        hit = self._geom_cache.get(key)
+        if hit is None:
+            if len(self._geom_cache) > 64:
+                self._geom_cache.clear()
+            hit = (torch.tensor(starts, dtype=torch.int32, device=self.device),
+                   torch.tensor(lens, dtype=torch.int32, device=self.device))
+            self._geom_cache[key] = hit
+        return max(starts), hit[0], hit[1], starts, lens
+
+    def _ragged_budgets(self, starts, lens, Lq: int, width: int):
+        """(valid_len, n_sel) per (sequence, KV head, tile) row of the pooled scores of a mixed
+        batch: every sequence gets the budgets of a call of its own."""
+        key = (tuple(starts), tuple(lens), Lq, width)
+        hit = self._budget_cache.get(key)
+        if hit is None:
+            T = (Lq + TILE - 1) // TILE
+            valid, nsel = [], []
+            for s, n in zip(starts, lens):
+                Lk = s + n
+                own = min(width, budgets.topk_width(Lk, self.k)) if Lk > 0 else 0
+                v_row, n_row = [], []
+                for t in range(T):
+                    if TILE * t >= n:                      # a tile past the sequence's rows selects nothing
+                        v_row.append(0); n_row.append(0)
+                        continue
+                    v_row.append(s + TILE * t)
+                    roll = self.rolling_prefill and Lk > budgets.CHUNK
+                    n_row.append(min(budgets.rolling_budget(s + TILE * t, self.k), own) if roll else own)
+                valid += v_row * self.G
+                nsel += n_row * self.G
+            if len(self._budget_cache) > 64:
+                self._budget_cache.clear()
+            hit = (torch.tensor(valid, dtype=torch.int32, device=self.device),
+                   torch.tensor(nsel, dtype=torch.int32, device=self.device))
+            self._budget_cache[key] = hit
+        return hit
+
     def _score_buffer(self, B, T, Lk):
         G = self.G
         n = B * G * T * Lk
@@ -460,36 +518,47 @@ class PagedKascadePrefill:
             self._scores = torch.empty(n, device=self.device, dtype=torch.float16)
         return self._scores[:n].view(B, G, T, Lk)
 
-    def anchor(self, layer, q, k_pages, v_pages, block_table, q_start: int):
+    def anchor(self, layer, q, k_pages, v_pages, block_table, q_start, q_lens=None):
         B, Lq = q.shape[:2]
-        Lk = q_start + Lq
+        qs_max, qs_dev, ql_dev, starts, lens = self._geometry(q_start, q_lens, Lq)
+        Lk = qs_max + Lq
         T = (Lq + TILE - 1) // TILE
         width = budgets.topk_width(Lk, self.k)
-        log_sum, o = kernels.prefill_chunk_dense(q, k_pages, v_pages, block_table, q_start,
-                                                 self.page_size, with_output=(layer == 0))
+        log_sum, o = kernels.prefill_chunk_dense(q, k_pages, v_pages, block_table, qs_max,
+                                                 self.page_size, with_output=(layer == 0),
+                                                 q_starts=qs_dev, q_lens=ql_dev)
         scores = self._score_buffer(B, T, Lk)
-        kernels.prefill_chunk_aggregate(q, k_pages, log_sum, scores, block_table, q_start, self.page_size)
-        valid, nsel = self._tile_budgets(q_start, Lq, width)
+        kernels.prefill_chunk_aggregate(q, k_pages, log_sum, scores, block_table, qs_max, self.page_size,
+                                        q_starts=qs_dev, q_lens=ql_dev)
+        if qs_dev is None:
+            valid, nsel = self._tile_budgets(qs_max, Lq, width)
+        else:
+            valid, nsel = self._ragged_budgets(starts, lens, Lq, width)
         self._topk_to_reuse, self._rows_to_reuse = kernels.topk_indices(
             scores, width, valid_len=valid, n_sel=nsel, block_table=block_table, page_size=self.page_size)
         if layer != 0:
-            o = self._reuse(q, k_pages, v_pages, block_table, q_start, self._hm[None])
+            o = self._reuse(q, k_pages, v_pages, block_table, qs_max, self._hm[None], qs_dev, ql_dev)
         return o
 
-    def _reuse(self, q, k_pages, v_pages, block_table, q_start, hm):
+    def _reuse(self, q, k_pages, v_pages, block_table, q_start, hm, q_starts=None, q_lens=None):
         return kernels.prefill_chunk_reuse(q, k_pages, v_pages, self._rows_to_reuse, hm, float(self.k),
-                                           self.rolling_prefill, block_table, q_start, self.page_size)
+                                           self.rolling_prefill, block_table, q_start, self.page_size,
+                                           q_starts=q_starts, q_lens=q_lens)
 
-    def reuse(self, layer, q, k_pages, v_pages, block_table, q_start: int):
+    def reuse(self, layer, q, k_pages, v_pages, block_table, q_start, q_lens=None):
         if self._rows_to_reuse is None:
             raise KascadeError("reuse layer called before any anchor layer")
-        return self._reuse(q, k_pages, v_pages, block_table, q_start, self._hm[layer])
+        qs_max, qs_dev, ql_dev, _, _ = self._geometry(q_start, q_lens, q.shape[1])
+        return self._reuse(q, k_pages, v_pages, block_table, qs_max, self._hm[layer], qs_dev, ql_dev)
 
-    def dense(self, q, k_pages, v_pages, block_table, q_start: int):
-        return kernels.prefill_chunk_dense(q, k_pages, v_pages, block_table, q_start, self.page_size)[1]
+    def dense(self, q, k_pages, v_pages, block_table, q_start, q_lens=None):
+        qs_max, qs_dev, ql_dev, _, _ = self._geometry(q_start, q_lens, q.shape[1])
+        return kernels.prefill_chunk_dense(q, k_pages, v_pages, block_table, qs_max, self.page_size,
+                                           q_starts=qs_dev, q_lens=ql_dev)[1]
 
-    def forward(self, layer, q, k_pages, v_pages, block_table, q_start: int):
-        """q [B,Lq,H,D] at global positions q_start.. (K/V of the chunk already in the cache)."""
+    def forward(self, layer, q, k_pages, v_pages, block_table, q_start, q_lens=None):
+        """q [B,Lq,H,D] at global positions q_start.. (K/V of the chunk already in the cache).
+        q_start: one int, or one per sequence; q_lens: rows of q that belong to each sequence."""
         if layer in self.recompute_layers:
-            return self.anchor(layer, q, k_pages, v_pages, block_table, q_start)
-        return self.reuse(layer, q, k_pages, v_pages, block_table, q_start)
+            return self.anchor(layer, q, k_pages, v_pages, block_table, q_start, q_lens)
+        return self.reuse(layer, q, k_pages, v_pages, block_table, q_start, q_lens)

@@ -64,7 +64,7 @@ def test_null_pointers_are_rejected(lib):
     assert lib.kascade_prefill_dense_call(None, None, None, None, None, 1, 64, s, s, 1, None) == -1
     assert lib.kascade_prefill_aggregate_call(None, None, None, None, 1, 64, s, s, 0, None) == -1
     assert lib.kascade_prefill_reuse_call(None, None, None, None, None, 10.0, None, 1, 64, 128, 1, s, s, None) == -1
-    assert lib.kascade_paged_kv_append_call(None, None, None, None, None, None, 1, 1, 1, 16, s, None) == -1
+    assert lib.kascade_paged_kv_append_call(None, None, None, None, None, None, 1, 1, 1, 16, s, None, None) == -1
     assert lib.kascade_rope_append_paged_call(None, None, None, None, None, None, 64, None, None, 1e-6, None, 0,
                                               None, None, None, None, 4, 16, 1, 1, None) == -1
     assert "null pointer" in _err(lib)
@@ -122,7 +122,7 @@ def test_shape_descriptors_are_validated(lib):
     p = (C.addressof(buf) & ~15) + 16
     ok = Strides(4096 * 128, 4096, 128)
     rope = (p, None, p, p, None, p, 64, None, None, 1e-6, p, 0, p, p, p, p, 4, 16, 1, 1, None)
-    chunk_dense = (p, p, p, p, p, 1, 0, 64, ok, p, 4, 16, 8, 1, None)
+    chunk_dense = (p, p, p, p, p, 1, 0, 64, ok, p, 4, 16, 8, 1, None, None, None)
     budgets = (p, 1, 10.0, 1, None, None, None)
     for fn, args in ((lib.kascade_rope_append_paged_shaped_call, rope),
                      (lib.kascade_prefill_chunk_dense_shaped_call, chunk_dense),
@@ -137,8 +137,10 @@ def test_shape_descriptors_are_validated(lib):
         assert "dtype" in _err(lib)
     # a valid shape reaches the argument checks of the call itself
     sh = C.byref(Shape(2, 64, 1))
-    assert lib.kascade_prefill_chunk_dense_shaped_call(sh, p, p, p, p, p, 1, 16, 64, ok, p, 4, 16, 8, 1, None) == -1
+    assert lib.kascade_prefill_chunk_dense_shaped_call(sh, p, p, p, p, p, 1, 16, 64, ok, p, 4, 16, 8, 1, None, None, None) == -1
     assert "multiple of 32" in _err(lib)
+    assert lib.kascade_prefill_chunk_dense_shaped_call(sh, p, p, p, p, p, 1, 32, 64, ok, p, 8, 16, 8, 1, None, p, None) == -1
+    assert "q_len_rows comes with q_start_rows" in _err(lib)
     assert lib.kascade_rope_append_paged_shaped_call(sh, p, None, p, p, None, p, 0, None, None, 1e-6, p, 0, p, p, p, p,
                                                      4, 16, 1, 1, None) == -1
     assert "max_pos" in _err(lib)

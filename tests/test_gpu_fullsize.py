@@ -291,7 +291,7 @@ def test_config4_stack_36_layers_prefill_and_256_replayed_decode_steps(cuda):
                             eager.max_seqlen, ragged=True, out=want[l], k_new=kn[l][:, 0], v_new=vn[l][:, 0])
                 if l in anchors:
                     picks[l] = dec._topk_to_reuse.clone()
-            eager.length += 1
+            eager.cache.note_advance(1)
         graph.graph_q.copy_(q); graph.graph_k.copy_(kn); graph.graph_v.copy_(vn)
         got = graph.replay_decode()
         assert torch.equal(got, want), f"step {step}: graph replay differs from eager launches"
