@@ -115,7 +115,12 @@ int kascade_decode_reuse_call(const kascade_half* Q, const kascade_half* K, cons
  *   k_new,v_new NULL, or [B,G,D] f16: the K and V rows of each sequence's newest token, i.e. of
  *               position cache_seqlens[b]-1 (kv_stride_tokens-1 without cache_seqlens).  The
  *               launch writes them into that slot of the cache (through K and V) and attends
- *               to them, so a decode step needs no separate kascade_paged_kv_append_call. */
+ *               to them, so a decode step needs no separate kascade_paged_kv_append_call.
+ *   log_sum     NULL, or [B,H] f32: log2 of the sum of 2^(q.k*scale) over the rows each head
+ *               attended to (the merged log-sum of the splits, which the reference's combine
+ *               step forms and drops, reuse_kascade_gqa_decode.py:160-177).  Next to the dense
+ *               log-sum of the same layer it says how much attention mass an index list covers,
+ *               which is what the layer / head calibration measures. */
 int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K,
                                     const kascade_half* V, const int32_t* cache_seqlens,
                                     const int32_t* topk_indices, const int32_t* head_mapping,
@@ -124,7 +129,7 @@ int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K
                                     int topk, int num_split, const int32_t* block_table,
                                     int max_pages, int page_size, const kascade_strides* kv_strides,
                                     const kascade_half* k_new, const kascade_half* v_new,
-                                    int32_t* sync_counters, void* stream);
+                                    int32_t* sync_counters, float* log_sum, void* stream);
 /* kascade_decode_reuse_paged_call for any kascade_shape. */
 int kascade_decode_reuse_paged_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K,
                                     const kascade_half* V, const int32_t* cache_seqlens,
@@ -134,7 +139,7 @@ int kascade_decode_reuse_paged_shaped_call(const kascade_shape* shape, const kas
                                     int topk, int num_split, const int32_t* block_table,
                                     int max_pages, int page_size, const kascade_strides* kv_strides,
                                     const kascade_half* k_new, const kascade_half* v_new,
-                                    int32_t* sync_counters, void* stream);
+                                    int32_t* sync_counters, float* log_sum, void* stream);
 
 /* Reuse-layer decode over a paged cache whose index lists were translated to cache rows once, at
  * the anchor (kascade_translate_indices_call): cache_rows [B,G,topk] holds page * page_size + slot
@@ -153,7 +158,7 @@ int kascade_decode_reuse_rows_call(const kascade_half* Q, const kascade_half* K_
                                    kascade_half* Output, int batch, int topk, int num_split,
                                    const int32_t* block_table, int max_pages, int page_size,
                                    int num_pages, const kascade_half* k_new,
-                                   const kascade_half* v_new, int32_t* sync_counters, void* stream);
+                                   const kascade_half* v_new, int32_t* sync_counters, float* log_sum, void* stream);
 /* kascade_decode_reuse_rows_call for any kascade_shape. */
 int kascade_decode_reuse_rows_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K_pages,
                                    const kascade_half* V_pages, const int32_t* cache_seqlens,
@@ -162,7 +167,7 @@ int kascade_decode_reuse_rows_shaped_call(const kascade_shape* shape, const kasc
                                    kascade_half* Output, int batch, int topk, int num_split,
                                    const int32_t* block_table, int max_pages, int page_size,
                                    int num_pages, const kascade_half* k_new,
-                                   const kascade_half* v_new, int32_t* sync_counters, void* stream);
+                                   const kascade_half* v_new, int32_t* sync_counters, float* log_sum, void* stream);
 
 /* kascade_decode_reuse_paged_call for callers that cannot allocate device memory and have no
  * scratch of their own to pass: code under HIP graph capture, tight serving loops, harnesses
@@ -342,18 +347,21 @@ int kascade_prefill_aggregate_range_shaped_call(const kascade_shape* shape, cons
  * the reference bakes into two separate objects.
  *   topk_indices [B,G,ceil(L/32),max_topk_num] i32, head_mapping [G] i32.
  *   rolling != 0 and seq_len > 128: tile t uses its first
- *   128*ceil(max(floor(topk_percent*32t/100),128)/128) indices, else max_topk_num. */
+ *   128*ceil(max(floor(topk_percent*32t/100),128)/128) indices, else max_topk_num.
+ *   log_sum NULL, or [B,L,H] f32: per (token, head) log2 of the sum of 2^(q.k*scale) over the keys
+ *   the row attended to (its tile's list and its own tile up to itself); see
+ *   kascade_decode_reuse_paged_call. */
 int kascade_prefill_reuse_call(const kascade_half* Q, const kascade_half* K, const kascade_half* V,
                                const int32_t* topk_indices, const int32_t* head_mapping,
                                float topk_percent, kascade_half* Output, int batch, int seq_len,
                                int max_topk_num, int rolling, kascade_strides q_strides,
-                               kascade_strides kv_strides, void* stream);
+                               kascade_strides kv_strides, float* log_sum, void* stream);
 /* kascade_prefill_reuse_call for any kascade_shape. */
 int kascade_prefill_reuse_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K, const kascade_half* V,
                                const int32_t* topk_indices, const int32_t* head_mapping,
                                float topk_percent, kascade_half* Output, int batch, int seq_len,
                                int max_topk_num, int rolling, kascade_strides q_strides,
-                               kascade_strides kv_strides, void* stream);
+                               kascade_strides kv_strides, float* log_sum, void* stream);
 
 /* --------------------------------------------------------------- KV append */
 
@@ -492,7 +500,7 @@ int kascade_prefill_chunk_reuse_call(const kascade_half* Q, const kascade_half* 
                                      int max_topk_num, int rolling, kascade_strides q_strides,
                                      const int32_t* block_table, int max_pages, int page_size,
                                      int num_pages, const int32_t* q_start_rows,
-                                     const int32_t* q_len_rows, void* stream);
+                                     const int32_t* q_len_rows, float* log_sum, void* stream);
 int kascade_prefill_chunk_reuse_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K_pages,
                                      const kascade_half* V_pages, const int32_t* physical_rows,
                                      const int32_t* head_mapping, float topk_percent,
@@ -500,7 +508,7 @@ int kascade_prefill_chunk_reuse_shaped_call(const kascade_shape* shape, const ka
                                      int max_topk_num, int rolling, kascade_strides q_strides,
                                      const int32_t* block_table, int max_pages, int page_size,
                                      int num_pages, const int32_t* q_start_rows,
-                                     const int32_t* q_len_rows, void* stream);
+                                     const int32_t* q_len_rows, float* log_sum, void* stream);
 
 /* physical_rows[b,i] = block_table[b, t / page_size] * page_size + t % page_size with
  * t = clamp(token_idx[b,i], 0, kv_len-1), i < per_sequence.  physical_rows may alias token_idx.
@@ -509,18 +517,48 @@ int kascade_translate_indices_call(const int32_t* token_idx, int32_t* physical_r
                                    const int32_t* block_table, int batch, int64_t per_sequence,
                                    int max_pages, int page_size, int kv_len, void* stream);
 
-/* ------------------------------------------------------------- diagnostics */
+/* ------------------------------------ the reference's argument lists, verbatim */
 
-/* Read-only kernels with no arithmetic, for measuring what the device delivers to the two access
- * patterns of the decode path (no counterpart in the reference; used by the benchmark only).
- * Nothing is written except, never in practice, 16 bytes at `sink`.
- *   stream_read: reads `bytes` bytes of src, 16 bytes per lane, four loads in flight per lane.
- *   gather_rows: for each of the n_rows entries of row_ids reads the 256 bytes at
- *                rows_a + row_ids[i]*row_stride_bytes (and the same row of rows_b when non-NULL),
- *                16 lanes per row; every id must address a row inside the arrays. */
-int kascade_diag_stream_read_call(const void* src, int64_t bytes, void* sink, void* stream);
-int kascade_diag_gather_rows_call(const void* rows_a, const void* rows_b, const int32_t* row_ids,
-                                  int64_t n_rows, int64_t row_stride_bytes, void* sink, void* stream);
+/* The five kernel objects the reference ships as generated sources each export
+ * `call(<pointers>, <dims>, stream)`.  The entry points below take exactly those argument lists,
+ * in that order and with those types, so a loader that binds the reference's `call` can bind
+ * these instead; each forwards to the entry point above that does the work, with what the
+ * reference fixes implicitly: contiguous [B,L,heads,128] tensors, 8 splits (the shape of the
+ * reference's glse [B,32,8] and Output_partial [B,32,8,128] scratch: attention_utils.py:36-59,
+ * EfficientKascadeStrategy.py:103-104, 119-120), a combine launch, no -inf fill by the kernel
+ * (the reference pre-fills aggregate_scores on the host, EfficientKascadeStrategy.py:75-76). */
+
+/* `call` of flash_decoding/kascade_decode_cu_kernels/
+ * dynamic_alllen_reuse_cp_async_dim128_gsize4_heads32_groups8.cu:260 */
+int kascade_ref_decode_reuse_call(kascade_half* Q, kascade_half* K, kascade_half* V,
+                                  int* topk_indices, int* head_mapping, float* glse,
+                                  float* Output_partial, kascade_half* Output, int batch,
+                                  int kv_seqlen, int topk, void* stream);
+
+/* `call` of ..._groups8_with_kvcache.cu:249 (K, V [B,max_cache_seqlen,8,128]) */
+int kascade_ref_decode_reuse_kvcache_call(kascade_half* Q, kascade_half* K, kascade_half* V,
+                                          int* cache_seqlens, int* topk_indices, int* head_mapping,
+                                          float topk_percent, float* glse, float* Output_partial,
+                                          kascade_half* Output, int batch, int max_cache_seqlen,
+                                          int topk, void* stream);
+
+/* `call` of flash_attention/kascade_prefill_cu_kernels/
+ * dynamic_alllen_aggregate_cp_async_ts32_dim128_gsize4_heads32_groups8.cu:138 */
+int kascade_ref_prefill_aggregate_call(kascade_half* Q, kascade_half* K, float* log_sum,
+                                       kascade_half* aggregate_scores, int batch, int seq_len,
+                                       void* stream);
+
+/* `call` of ...reuse_cp_async_ts32_dim128_gsize4_heads32_groups8_rolling.cu:268 */
+int kascade_ref_prefill_reuse_rolling_call(kascade_half* Q, kascade_half* K, kascade_half* V,
+                                           int* topk_indices, int* head_mapping,
+                                           float topk_percent, kascade_half* Output, int batch,
+                                           int seq_len, int max_topk_num, void* stream);
+
+/* `call` of ...reuse_cp_async_ts32_dim128_gsize4_heads32_groups8.cu:260 (every tile uses topk_num) */
+int kascade_ref_prefill_reuse_call(kascade_half* Q, kascade_half* K, kascade_half* V,
+                                   int* topk_indices, int* head_mapping, float topk_percent,
+                                   kascade_half* Output, int batch, int seq_len, int topk_num,
+                                   void* stream);
 
 #ifdef __cplusplus
 }

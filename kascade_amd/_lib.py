@@ -1,4 +1,5 @@
-"""ctypes binding of libkascade_hip.so (the C ABI declared in include/kascade_hip.h).
+"""ctypes binding of libkascade_hip.so (the C ABI declared in include/kascade_hip.h; the
+benchmark's two measurement helpers in include/kascade_hip_diag.h).
 
 Loading fails loudly: there is no fallback implementation.  ``load()`` returns
 the library with argument types set; ``check(rc)`` turns a -1 return code into
@@ -27,7 +28,7 @@ _F = C.c_float
 _L = C.c_int64
 _SP = C.POINTER(Strides)   # optional kascade_strides*
 
-# name -> (restype, argtypes); must list every symbol of include/kascade_hip.h
+# name -> (restype, argtypes); must list every symbol of include/kascade_hip.h and include/kascade_hip_diag.h
 SIGNATURES = {
     "kascade_init": (_I, []),
     "kascade_get_last_error": (C.c_char_p, []),
@@ -35,9 +36,9 @@ SIGNATURES = {
     "kascade_device_cu_count": (_I, []),
     "kascade_decode_reuse_call": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _P]),
     "kascade_decode_reuse_paged_call": (_I, [_P, _P, _P, _P, _P, _P, _F, _P, _P, _P, _I, _I, _I, _I,
-                                             _P, _I, _I, _SP, _P, _P, _P, _P]),
+                                             _P, _I, _I, _SP, _P, _P, _P, _P, _P]),
     "kascade_decode_reuse_rows_call": (_I, [_P, _P, _P, _P, _P, _P, _F, _P, _P, _P, _I, _I, _I, _P, _I, _I, _I,
-                                            _P, _P, _P, _P]),
+                                            _P, _P, _P, _P, _P]),
     "kascade_decode_reuse_paged_noalloc_call": (_I, [_P, _P, _P, _P, _P, _P, _F, _P, _I, _I, _I, _I,
                                                      _P, _I, _I, _SP, _P, _P, _P]),
     "kascade_decode_dense_paged_call": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _I, _I, _SP,
@@ -51,7 +52,7 @@ SIGNATURES = {
     "kascade_prefill_aggregate_call": (_I, [_P, _P, _P, _P, _I, _I, Strides, Strides, _I, _P]),
     "kascade_prefill_aggregate_range_call": (_I, [_P, _P, _P, _P, _I, _I, _I, Strides, Strides, _I, _P]),
     "kascade_prefill_reuse_call": (_I, [_P, _P, _P, _P, _P, _F, _P, _I, _I, _I, _I, Strides, Strides,
-                                        _P]),
+                                        _P, _P]),
     "kascade_paged_kv_append_call": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, Strides, _P, _P]),
     "kascade_rope_append_paged_call": (_I, [_P, _SP, _P, _P, _SP, _P, _I, _P, _P, _F, _P, _I, _P, _P, _P,
                                             _P, _I, _I, _I, _I, _P]),
@@ -61,8 +62,13 @@ SIGNATURES = {
     "kascade_prefill_chunk_aggregate_call": (_I, [_P, _P, _P, _P, _I, _I, _I, Strides, _P, _I, _I, _I,
                                                   _I, _P, _P, _P]),
     "kascade_prefill_chunk_reuse_call": (_I, [_P, _P, _P, _P, _P, _F, _P, _I, _I, _I, _I, _I, Strides,
-                                              _P, _I, _I, _I, _P, _P, _P]),
+                                              _P, _I, _I, _I, _P, _P, _P, _P]),
     "kascade_translate_indices_call": (_I, [_P, _P, _P, _I, C.c_int64, _I, _I, _I, _P]),
+    "kascade_ref_decode_reuse_call": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P]),
+    "kascade_ref_decode_reuse_kvcache_call": (_I, [_P, _P, _P, _P, _P, _P, _F, _P, _P, _P, _I, _I, _I, _P]),
+    "kascade_ref_prefill_aggregate_call": (_I, [_P, _P, _P, _P, _I, _I, _P]),
+    "kascade_ref_prefill_reuse_rolling_call": (_I, [_P, _P, _P, _P, _P, _F, _P, _I, _I, _I, _P]),
+    "kascade_ref_prefill_reuse_call": (_I, [_P, _P, _P, _P, _P, _F, _P, _I, _I, _I, _P]),
     "kascade_diag_stream_read_call": (_I, [_P, _L, _P, _P]),
     "kascade_diag_gather_rows_call": (_I, [_P, _P, _P, _L, _L, _P, _P]),
 }

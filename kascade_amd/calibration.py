@@ -13,8 +13,14 @@ the selection logic of the reference's statistics runner (src/runners/stats_runn
   find_head_mappings   :341-351   per layer and head, the anchor head that covers it best
   select_layers        :183-197   the loop over anchor counts that writes the .npy files
 
-Statistics collection itself (running a model with attention weights exposed) is outside the
-attention path and is not rebuilt; the functions take the accumulated tensors.
+The reference gathers its statistics from dense [heads, tiles, keys] pooled attention weights
+held in memory (PostSoftmaxPooledPrefillTopkStrategy.py:61-86), which cannot exist at the lengths
+the sparse path is for.  ``covered_mass`` / ``tile_similarity`` / ``layer_statistics`` compute the
+same ratios on the device from what the attention kernels already form: the log-sum of a row over
+the keys it attended to (its tile's index list and its own tile) next to its dense log-sum is the
+attention mass the list covers, and the statistic is a ratio of such masses pooled per tile.
+Running a model to obtain each layer's Q and K is outside the attention path; the functions take
+those tensors.
 """
 from __future__ import annotations
 
@@ -141,3 +147,120 @@ def select_layers(sim_avg, importance, counts: Iterable[int] = (3, 4, 5, 6, 7, 8
             base = model_name.split("/")[-1]
             np.save(os.path.join(out_dir, f"{base}_layers_{'_'.join(map(str, pivots))}.npy"), maps)
     return out
+
+
+# ---------------------------------------------------------------- statistics on the device
+TILE = 32
+
+
+def covered_mass(q: torch.Tensor, k: torch.Tensor, log_sum_full: torch.Tensor, idx: torch.Tensor,
+                 head_map: Sequence[int], topk_percent: float, rolling: bool) -> torch.Tensor:
+    """mass[b, g, t] = sum over the 32 queries of tile t and the query heads of KV head g of the
+    share of the row's dense attention that falls on (idx[b, head_map[g], t, :n(t)] U the row's own
+    tile up to itself): the numerator / denominator of stats_runner.py:155-168 with its
+    ``last_tile_attn`` term included.  q [B,L,H,D], k [B,L,G,D] (device), log_sum_full [B,L,H] from
+    the dense pass of the same layer, idx [B,G,T,K] int32.  One launch of the reuse prefill
+    kernel, whose log-sum output is the log2 of the attended mass before normalisation."""
+    from . import kernels
+    B, L, Hq, _ = q.shape
+    G = k.shape[2]
+    hm = torch.tensor(list(head_map), dtype=torch.int32, device=q.device)
+    _, lse = kernels.prefill_reuse(q, k, k, idx, hm, float(topk_percent), rolling, return_log_sum=True)
+    share = torch.exp2(lse - log_sum_full)                                   # [B,L,H], <= 1
+    T = (L + TILE - 1) // TILE
+    pad = T * TILE - L
+    if pad:
+        share = torch.cat([share, share.new_zeros(B, pad, Hq)], dim=1)
+    return share.view(B, T, TILE, G, Hq // G).sum(dim=(2, 4)).permute(0, 2, 1)   # [B,G,T]
+
+
+def own_tile_mass(q: torch.Tensor, k: torch.Tensor, log_sum_full: torch.Tensor,
+                  scores: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """tail[b, g, t]: the attention the queries of tile t (all query heads of KV head g) put on
+    their own tile, the reference's ``last_tile_attn``
+    (PostSoftmaxPooledPrefillTopkStrategy.py:75-79) -- every row's probabilities sum to one, so it
+    is the number of rows minus the tile's pooled scores over the keys before the tile.
+    ``scores``: the layer's pooled tile scores [B,G,T,L] when the caller already has them."""
+    from . import kernels
+    B, L, Hq, _ = q.shape
+    G = k.shape[2]
+    T = (L + TILE - 1) // TILE
+    if scores is None:
+        scores = torch.empty(B, G, T, L, device=q.device, dtype=torch.float16)
+        kernels.prefill_aggregate(q, k, log_sum_full, scores)
+    before = torch.arange(L, device=q.device)[None, :] < (torch.arange(T, device=q.device) * TILE)[:, None]
+    pooled = torch.where(before, scores.float(), scores.new_zeros((), dtype=torch.float32)).sum(-1)      # [B,G,T]
+    rows = torch.full((T,), TILE, device=q.device, dtype=torch.float32)
+    rows[-1] = L - (T - 1) * TILE
+    return rows * (Hq // G) - pooled
+
+
+def tile_similarity(q_b: torch.Tensor, k_b: torch.Tensor, idx_a: torch.Tensor, idx_b: torch.Tensor,
+                    topk_percent: float, rolling: bool = False, reduce: str = "amin",
+                    log_sum_full: Optional[torch.Tensor] = None, tail_b: Optional[torch.Tensor] = None,
+                    reference_tail: bool = True) -> torch.Tensor:
+    """sim[hb, ha] of stats_runner.py:155-168 for one pair of layers, on the device: how well the
+    index lists of layer A's KV head ha cover the attention of layer B's KV head hb, relative to
+    layer B's own lists, reduced over the query tiles of batch element 0 ("amin" for anchor
+    selection, "mean" for the plots).  q_b, k_b: layer B's queries and keys; idx_a, idx_b
+    [B,G,T,K] int32 from the selections of the two layers.  G + 1 launches of the reuse kernel
+    (every rotation of the head map pairs each hb with one ha).
+
+    reference_tail: the reference adds, to numerator and denominator of entry (hb, ha), the
+    own-tile attention of head **ha** of layer B (its [B,heads,tiles] tensor broadcasts against
+    the ha axis of [B,hb,ha,tiles], stats_runner.py:166); the kernel's masses carry that of head hb,
+    which is what the ratio means.  True reproduces the reference's numbers (the head maps it
+    would write); False keeps head hb's.  The diagonal is the same either way."""
+    from . import kernels
+    if reduce not in ("amin", "mean"):
+        raise ValueError("reduce must be 'amin' or 'mean'")
+    G = k_b.shape[2]
+    if log_sum_full is None:
+        log_sum_full = kernels.prefill_recompute1(q_b, k_b)
+    if reference_tail and tail_b is None:
+        tail_b = own_tile_mass(q_b, k_b, log_sum_full)
+    own = covered_mass(q_b, k_b, log_sum_full, idx_b, range(G), topk_percent, rolling)      # [B,G,T]
+    sim = torch.empty(G, G, device=q_b.device, dtype=torch.float32)
+    for s in range(G):
+        hm = [(g + s) % G for g in range(G)]
+        num, den = covered_mass(q_b, k_b, log_sum_full, idx_a, hm, topk_percent, rolling), own
+        if reference_tail:      # swap head hb's own-tile term for head ha's
+            shift = tail_b[:, hm] - tail_b
+            num, den = num + shift, den + shift
+        ratio = num / den
+        red = ratio.amin(-1) if reduce == "amin" else ratio.mean(-1)
+        sim[torch.arange(G), torch.tensor(hm)] = red[0]
+    return sim
+
+
+def layer_statistics(layers: Sequence[Tuple[torch.Tensor, torch.Tensor]], topk_percent: float,
+                     rolling: bool = False, reduce: str = "amin", reference_tail: bool = True) -> torch.Tensor:
+    """[N,N,G,G] similarity statistics of one prompt (the upper triangle A <= B, as
+    stats_runner.py:127-131 accumulates them; the rest is zero) from every layer's prefill queries
+    and keys: layers[l] = (q [1,L,H,D], k [1,L,G,D]) on the device.  Each layer's own lists come
+    from the anchor pipeline (dense log-sum pass, pooled tile scores, selection)."""
+    from . import budgets, kernels
+    n = len(layers)
+    q0, k0 = layers[0]
+    B, L, _, _ = q0.shape
+    G = k0.shape[2]
+    T = (L + TILE - 1) // TILE
+    K = budgets.topk_width(L, topk_percent)
+    valid, nsel = budgets.prefill_tile_budgets(L, TILE, topk_percent, rolling, K)
+    valid = torch.tensor(valid, dtype=torch.int32, device=q0.device)
+    nsel = torch.tensor(nsel, dtype=torch.int32, device=q0.device)
+    scores = torch.empty(B, G, T, L, device=q0.device, dtype=torch.float16)
+    lses, idxs, tails = [], [], []
+    for q, k in layers:
+        ls = kernels.prefill_recompute1(q, k)
+        kernels.prefill_aggregate(q, k, ls, scores)
+        lses.append(ls)
+        idxs.append(kernels.topk_indices(scores, K, valid_len=valid, n_sel=nsel))
+        tails.append(own_tile_mass(q, k, ls, scores) if reference_tail else None)
+    sim = torch.zeros(n, n, G, G, device=q0.device, dtype=torch.float32)
+    for b in range(n):
+        q, k = layers[b]
+        for a in range(b + 1):
+            sim[a, b] = tile_similarity(q, k, idxs[a], idxs[b], topk_percent, rolling, reduce, lses[b], tails[b],
+                                        reference_tail)
+    return sim

@@ -3,10 +3,13 @@
 // caller's.  Validation failures are reported before anything is launched, so
 // they can be exercised on a machine without a GPU.
 #include "../../include/kascade_hip.h"
+#include "../../include/kascade_hip_diag.h"
 
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
+
+#include <mutex>
 
 #include "decode.h"
 #include "diag.h"
@@ -31,6 +34,7 @@ constexpr size_t kNoAllocFloats = (size_t)kNoAllocUnits * kHeads * (1 + kDim);  
 static __device__ __align__(256) float scratch[kNoAllocFloats];
 constexpr int kMaxDevices = 64;
 float* g_noalloc_ptr[kMaxDevices] = {};
+std::mutex g_noalloc_mutex;   // host threads that meet in the first call on a device
 
 int fail(const char* fmt, ...) {
     va_list ap;
@@ -61,6 +65,7 @@ int noalloc_scratch(float** out) {
     int dev = 0;
     if (check_hip(hipGetDevice(&dev), "hipGetDevice")) return -1;
     REQUIRE(dev >= 0 && dev < kMaxDevices, "device ordinal %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_noalloc_mutex);
     if (!g_noalloc_ptr[dev]) {
         void* ptr = nullptr;
         if (check_hip(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)"))
@@ -102,6 +107,14 @@ int get_shape(const kascade_shape* in, Shape* out) {
     out->G = in->kv_heads; out->D = in->head_dim; out->elem = in->dtype == KASCADE_BF16 ? kElemBF16 : kElemF16;
     out->gs = gs;
     return 0;
+}
+
+// what the reference's scratch shapes fix for its decode kernels (attention_utils.py:36-59)
+constexpr int kRefNumSplit = 8;
+
+// element strides of a contiguous [B,seq_len,heads,128] tensor
+kascade_strides contiguous_strides(int seq_len, int heads) {
+    return kascade_strides{(int64_t)seq_len * heads * kDim, (int64_t)heads * kDim, (int64_t)kDim};
 }
 
 int rows_per_split(long long max_rows, int num_split) {
@@ -183,7 +196,7 @@ int kascade_decode_reuse_call(const kascade_half* Q, const kascade_half* K, cons
     return kascade_decode_reuse_paged_call(Q, K, V, nullptr, topk_indices, head_mapping, 0.f, glse,
                                            Output_partial, Output, batch, kv_seqlen, topk,
                                            num_split, nullptr, 0, 1, nullptr, nullptr, nullptr, sync_counters,
-                                           stream);
+                                           nullptr, stream);
 }
 
 }  // extern "C"
@@ -196,7 +209,7 @@ int decode_reuse_paged_impl(const Shape& sh, const kascade_half* Q, const kascad
                                     int topk, int num_split, const int32_t* block_table,
                                     int max_pages, int page_size, const kascade_strides* kv_strides,
                                     const kascade_half* k_new, const kascade_half* v_new,
-                                    int32_t* sync_counters, void* stream) {
+                                    int32_t* sync_counters, float* log_sum, void* stream) {
     REQUIRE(Q && K && V && topk_indices && head_mapping && glse && Output_partial && Output,
             "decode_reuse: null pointer argument");
     REQUIRE(batch > 0 && topk > 0 && num_split > 0, "decode_reuse: batch, topk, num_split must be > 0");
@@ -216,11 +229,11 @@ int decode_reuse_paged_impl(const Shape& sh, const kascade_half* Q, const kascad
     p.topk = topk; p.topk_percent = topk_percent; p.scores_stride = 0; p.num_split = num_split;
     p.rows_per_split = rows_per_split(topk, num_split);
     p.B = batch;
-    p.counters = sync_counters; p.out = H(Output);
+    p.counters = sync_counters; p.out = H(Output); p.row_sums = log_sum;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (check_hip(launch_decode_split(p, true, true, false, s), "decode_reuse split")) return -1;
     if (sync_counters) return 0;   // the split kernel's last workgroups have combined
-    return check_hip(launch_decode_combine(glse, Output_partial, E(Output), nullptr, batch, sh.H(), num_split, true, sh.D, sh.elem, s), "decode_reuse combine");
+    return check_hip(launch_decode_combine(glse, Output_partial, E(Output), log_sum, batch, sh.H(), num_split, true, sh.D, sh.elem, s), "decode_reuse combine");
 }
 }  // namespace
 extern "C" {
@@ -233,8 +246,8 @@ int kascade_decode_reuse_paged_call(const kascade_half* Q, const kascade_half* K
                                     int topk, int num_split, const int32_t* block_table,
                                     int max_pages, int page_size, const kascade_strides* kv_strides,
                                     const kascade_half* k_new, const kascade_half* v_new,
-                                    int32_t* sync_counters, void* stream) {
-    return decode_reuse_paged_impl(kRefShape, Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_percent, glse, Output_partial, Output, batch, kv_stride_tokens, topk, num_split, block_table, max_pages, page_size, kv_strides, k_new, v_new, sync_counters, stream);
+                                    int32_t* sync_counters, float* log_sum, void* stream) {
+    return decode_reuse_paged_impl(kRefShape, Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_percent, glse, Output_partial, Output, batch, kv_stride_tokens, topk, num_split, block_table, max_pages, page_size, kv_strides, k_new, v_new, sync_counters, log_sum, stream);
 }
 
 int kascade_decode_reuse_paged_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K,
@@ -245,10 +258,10 @@ int kascade_decode_reuse_paged_shaped_call(const kascade_shape* shape, const kas
                                     int topk, int num_split, const int32_t* block_table,
                                     int max_pages, int page_size, const kascade_strides* kv_strides,
                                     const kascade_half* k_new, const kascade_half* v_new,
-                                    int32_t* sync_counters, void* stream) {
+                                    int32_t* sync_counters, float* log_sum, void* stream) {
     Shape sh;
     if (get_shape(shape, &sh)) return -1;
-    return decode_reuse_paged_impl(sh, Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_percent, glse, Output_partial, Output, batch, kv_stride_tokens, topk, num_split, block_table, max_pages, page_size, kv_strides, k_new, v_new, sync_counters, stream);
+    return decode_reuse_paged_impl(sh, Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_percent, glse, Output_partial, Output, batch, kv_stride_tokens, topk, num_split, block_table, max_pages, page_size, kv_strides, k_new, v_new, sync_counters, log_sum, stream);
 }
 
 }  // extern "C"
@@ -260,7 +273,7 @@ int decode_reuse_rows_impl(const Shape& sh, const kascade_half* Q, const kascade
                                    kascade_half* Output, int batch, int topk, int num_split,
                                    const int32_t* block_table, int max_pages, int page_size,
                                    int num_pages, const kascade_half* k_new,
-                                   const kascade_half* v_new, int32_t* sync_counters, void* stream) {
+                                   const kascade_half* v_new, int32_t* sync_counters, float* log_sum, void* stream) {
     REQUIRE(Q && K_pages && V_pages && cache_rows && head_mapping && glse && Output_partial && Output &&
                 block_table, "decode_reuse_rows: null pointer argument");
     REQUIRE(batch > 0 && topk > 0 && num_split > 0, "decode_reuse_rows: batch, topk, num_split must be > 0");
@@ -284,11 +297,11 @@ int decode_reuse_rows_impl(const Shape& sh, const kascade_half* Q, const kascade
     p.topk = topk; p.topk_percent = topk_percent; p.scores_stride = 0; p.num_split = num_split;
     p.rows_per_split = rows_per_split(topk, num_split);
     p.B = batch;
-    p.counters = sync_counters; p.out = H(Output);
+    p.counters = sync_counters; p.out = H(Output); p.row_sums = log_sum;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (check_hip(launch_decode_split(p, true, true, false, s), "decode_reuse_rows split")) return -1;
     if (sync_counters) return 0;
-    return check_hip(launch_decode_combine(glse, Output_partial, E(Output), nullptr, batch, sh.H(), num_split, true, sh.D, sh.elem, s), "decode_reuse_rows combine");
+    return check_hip(launch_decode_combine(glse, Output_partial, E(Output), log_sum, batch, sh.H(), num_split, true, sh.D, sh.elem, s), "decode_reuse_rows combine");
 }
 }  // namespace
 extern "C" {
@@ -300,8 +313,8 @@ int kascade_decode_reuse_rows_call(const kascade_half* Q, const kascade_half* K_
                                    kascade_half* Output, int batch, int topk, int num_split,
                                    const int32_t* block_table, int max_pages, int page_size,
                                    int num_pages, const kascade_half* k_new,
-                                   const kascade_half* v_new, int32_t* sync_counters, void* stream) {
-    return decode_reuse_rows_impl(kRefShape, Q, K_pages, V_pages, cache_seqlens, cache_rows, head_mapping, topk_percent, glse, Output_partial, Output, batch, topk, num_split, block_table, max_pages, page_size, num_pages, k_new, v_new, sync_counters, stream);
+                                   const kascade_half* v_new, int32_t* sync_counters, float* log_sum, void* stream) {
+    return decode_reuse_rows_impl(kRefShape, Q, K_pages, V_pages, cache_seqlens, cache_rows, head_mapping, topk_percent, glse, Output_partial, Output, batch, topk, num_split, block_table, max_pages, page_size, num_pages, k_new, v_new, sync_counters, log_sum, stream);
 }
 
 int kascade_decode_reuse_rows_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K_pages,
@@ -311,10 +324,10 @@ int kascade_decode_reuse_rows_shaped_call(const kascade_shape* shape, const kasc
                                    kascade_half* Output, int batch, int topk, int num_split,
                                    const int32_t* block_table, int max_pages, int page_size,
                                    int num_pages, const kascade_half* k_new,
-                                   const kascade_half* v_new, int32_t* sync_counters, void* stream) {
+                                   const kascade_half* v_new, int32_t* sync_counters, float* log_sum, void* stream) {
     Shape sh;
     if (get_shape(shape, &sh)) return -1;
-    return decode_reuse_rows_impl(sh, Q, K_pages, V_pages, cache_seqlens, cache_rows, head_mapping, topk_percent, glse, Output_partial, Output, batch, topk, num_split, block_table, max_pages, page_size, num_pages, k_new, v_new, sync_counters, stream);
+    return decode_reuse_rows_impl(sh, Q, K_pages, V_pages, cache_seqlens, cache_rows, head_mapping, topk_percent, glse, Output_partial, Output, batch, topk, num_split, block_table, max_pages, page_size, num_pages, k_new, v_new, sync_counters, log_sum, stream);
 }
 
 int kascade_decode_reuse_paged_noalloc_call(const kascade_half* Q, const kascade_half* K,
@@ -338,7 +351,7 @@ int kascade_decode_reuse_paged_noalloc_call(const kascade_half* Q, const kascade
     return decode_reuse_paged_impl(kRefShape, Q, K, V, cache_seqlens, topk_indices, head_mapping,
                                            topk_percent, glse, opart, Output, batch,
                                            kv_stride_tokens, topk, num_split, block_table, max_pages,
-                                           page_size, kv_strides, k_new, v_new, nullptr, stream);
+                                           page_size, kv_strides, k_new, v_new, nullptr, nullptr, stream);
 }
 
 }  // extern "C"
@@ -668,7 +681,7 @@ int prefill_reuse_impl(const Shape& sh, const kascade_half* Q, const kascade_hal
                                const int32_t* topk_indices, const int32_t* head_mapping,
                                float topk_percent, kascade_half* Output, int batch, int seq_len,
                                int max_topk_num, int rolling, kascade_strides q_strides,
-                               kascade_strides kv_strides, void* stream) {
+                               kascade_strides kv_strides, float* log_sum, void* stream) {
     REQUIRE(Q && K && V && topk_indices && head_mapping && Output,
             "prefill_reuse: null pointer argument");
     REQUIRE(batch > 0 && seq_len > 0 && batch <= 65535, "prefill_reuse: bad batch/seq_len");
@@ -680,7 +693,7 @@ int prefill_reuse_impl(const Shape& sh, const kascade_half* Q, const kascade_hal
     PrefillParams p{};
     p.G = sh.G; p.head_dim = sh.D; p.elem = sh.elem; p.gs = sh.gs;
     p.Q = H(Q); p.K = H(K); p.V = H(V); p.idx = topk_indices; p.head_map = head_mapping;
-    p.O = H(Output); p.log_sum = nullptr;
+    p.O = H(Output); p.log_sum = log_sum;
     p.q_sb = q_strides.b; p.q_sl = q_strides.l; p.q_sh = q_strides.h;
     p.k_sb = kv_strides.b; p.k_sl = kv_strides.l; p.k_sh = kv_strides.h;
     p.B = batch; p.L = seq_len; p.Lq = seq_len; p.T = (seq_len + kTile - 1) / kTile;
@@ -695,18 +708,18 @@ int kascade_prefill_reuse_call(const kascade_half* Q, const kascade_half* K, con
                                const int32_t* topk_indices, const int32_t* head_mapping,
                                float topk_percent, kascade_half* Output, int batch, int seq_len,
                                int max_topk_num, int rolling, kascade_strides q_strides,
-                               kascade_strides kv_strides, void* stream) {
-    return prefill_reuse_impl(kRefShape, Q, K, V, topk_indices, head_mapping, topk_percent, Output, batch, seq_len, max_topk_num, rolling, q_strides, kv_strides, stream);
+                               kascade_strides kv_strides, float* log_sum, void* stream) {
+    return prefill_reuse_impl(kRefShape, Q, K, V, topk_indices, head_mapping, topk_percent, Output, batch, seq_len, max_topk_num, rolling, q_strides, kv_strides, log_sum, stream);
 }
 
 int kascade_prefill_reuse_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K, const kascade_half* V,
                                const int32_t* topk_indices, const int32_t* head_mapping,
                                float topk_percent, kascade_half* Output, int batch, int seq_len,
                                int max_topk_num, int rolling, kascade_strides q_strides,
-                               kascade_strides kv_strides, void* stream) {
+                               kascade_strides kv_strides, float* log_sum, void* stream) {
     Shape sh;
     if (get_shape(shape, &sh)) return -1;
-    return prefill_reuse_impl(sh, Q, K, V, topk_indices, head_mapping, topk_percent, Output, batch, seq_len, max_topk_num, rolling, q_strides, kv_strides, stream);
+    return prefill_reuse_impl(sh, Q, K, V, topk_indices, head_mapping, topk_percent, Output, batch, seq_len, max_topk_num, rolling, q_strides, kv_strides, log_sum, stream);
 }
 
 }  // extern "C"
@@ -921,7 +934,7 @@ int prefill_chunk_reuse_impl(const Shape& sh, const kascade_half* Q, const kasca
                                      int max_topk_num, int rolling, kascade_strides q_strides,
                                      const int32_t* block_table, int max_pages, int page_size,
                                      int num_pages, const int32_t* q_start_rows,
-                                     const int32_t* q_len_rows, void* stream) {
+                                     const int32_t* q_len_rows, float* log_sum, void* stream) {
     REQUIRE(Q && K_pages && V_pages && physical_rows && head_mapping && Output,
             "prefill_chunk_reuse: null pointer argument");
     REQUIRE(max_topk_num > 0, "prefill_chunk_reuse: max_topk_num must be > 0");
@@ -933,7 +946,7 @@ int prefill_chunk_reuse_impl(const Shape& sh, const kascade_half* Q, const kasca
                      page_size, num_pages, q_start_rows, q_len_rows))
         return -1;
     p.K = E(K_pages); p.V = E(V_pages); p.idx = physical_rows; p.head_map = head_mapping;
-    p.O = E(Output); p.log_sum = nullptr;
+    p.O = E(Output); p.log_sum = log_sum;
     p.max_topk = max_topk_num; p.rolling = rolling; p.topk_percent = topk_percent;
     return check_hip(launch_prefill_attn(p, true, true, 1, static_cast<hipStream_t>(stream)),
                      "prefill_chunk_reuse");
@@ -992,8 +1005,8 @@ int kascade_prefill_chunk_reuse_call(const kascade_half* Q, const kascade_half* 
                                      int max_topk_num, int rolling, kascade_strides q_strides,
                                      const int32_t* block_table, int max_pages, int page_size,
                                      int num_pages, const int32_t* q_start_rows,
-                                     const int32_t* q_len_rows, void* stream) {
-    return prefill_chunk_reuse_impl(kRefShape, Q, K_pages, V_pages, physical_rows, head_mapping, topk_percent, Output, batch, q_start, q_len, max_topk_num, rolling, q_strides, block_table, max_pages, page_size, num_pages, q_start_rows, q_len_rows, stream);
+                                     const int32_t* q_len_rows, float* log_sum, void* stream) {
+    return prefill_chunk_reuse_impl(kRefShape, Q, K_pages, V_pages, physical_rows, head_mapping, topk_percent, Output, batch, q_start, q_len, max_topk_num, rolling, q_strides, block_table, max_pages, page_size, num_pages, q_start_rows, q_len_rows, log_sum, stream);
 }
 
 int kascade_prefill_chunk_reuse_shaped_call(const kascade_shape* shape, const kascade_half* Q, const kascade_half* K_pages,
@@ -1003,10 +1016,10 @@ int kascade_prefill_chunk_reuse_shaped_call(const kascade_shape* shape, const ka
                                      int max_topk_num, int rolling, kascade_strides q_strides,
                                      const int32_t* block_table, int max_pages, int page_size,
                                      int num_pages, const int32_t* q_start_rows,
-                                     const int32_t* q_len_rows, void* stream) {
+                                     const int32_t* q_len_rows, float* log_sum, void* stream) {
     Shape sh;
     if (get_shape(shape, &sh)) return -1;
-    return prefill_chunk_reuse_impl(sh, Q, K_pages, V_pages, physical_rows, head_mapping, topk_percent, Output, batch, q_start, q_len, max_topk_num, rolling, q_strides, block_table, max_pages, page_size, num_pages, q_start_rows, q_len_rows, stream);
+    return prefill_chunk_reuse_impl(sh, Q, K_pages, V_pages, physical_rows, head_mapping, topk_percent, Output, batch, q_start, q_len, max_topk_num, rolling, q_strides, block_table, max_pages, page_size, num_pages, q_start_rows, q_len_rows, log_sum, stream);
 }
 
 int kascade_translate_indices_call(const int32_t* token_idx, int32_t* physical_rows,
@@ -1023,6 +1036,53 @@ int kascade_translate_indices_call(const int32_t* token_idx, int32_t* physical_r
                                               per_sequence, max_pages, shift, kv_len,
                                               static_cast<hipStream_t>(stream)),
                      "translate_indices");
+}
+
+// ---- the reference's argument lists, verbatim ----
+
+int kascade_ref_decode_reuse_call(kascade_half* Q, kascade_half* K, kascade_half* V,
+                                  int* topk_indices, int* head_mapping, float* glse,
+                                  float* Output_partial, kascade_half* Output, int batch,
+                                  int kv_seqlen, int topk, void* stream) {
+    return kascade_decode_reuse_call(Q, K, V, topk_indices, head_mapping, glse, Output_partial, Output,
+                                     batch, kv_seqlen, topk, kRefNumSplit, nullptr, stream);
+}
+
+int kascade_ref_decode_reuse_kvcache_call(kascade_half* Q, kascade_half* K, kascade_half* V,
+                                          int* cache_seqlens, int* topk_indices, int* head_mapping,
+                                          float topk_percent, float* glse, float* Output_partial,
+                                          kascade_half* Output, int batch, int max_cache_seqlen,
+                                          int topk, void* stream) {
+    return kascade_decode_reuse_paged_call(Q, K, V, cache_seqlens, topk_indices, head_mapping,
+                                           topk_percent, glse, Output_partial, Output, batch,
+                                           max_cache_seqlen, topk, kRefNumSplit, nullptr, 0, 1, nullptr,
+                                           nullptr, nullptr, nullptr, nullptr, stream);
+}
+
+int kascade_ref_prefill_aggregate_call(kascade_half* Q, kascade_half* K, float* log_sum,
+                                       kascade_half* aggregate_scores, int batch, int seq_len,
+                                       void* stream) {
+    return kascade_prefill_aggregate_call(Q, K, log_sum, aggregate_scores, batch, seq_len,
+                                          contiguous_strides(seq_len, kHeads), contiguous_strides(seq_len, kGroups),
+                                          0, stream);
+}
+
+int kascade_ref_prefill_reuse_rolling_call(kascade_half* Q, kascade_half* K, kascade_half* V,
+                                           int* topk_indices, int* head_mapping,
+                                           float topk_percent, kascade_half* Output, int batch,
+                                           int seq_len, int max_topk_num, void* stream) {
+    return kascade_prefill_reuse_call(Q, K, V, topk_indices, head_mapping, topk_percent, Output, batch,
+                                      seq_len, max_topk_num, 1, contiguous_strides(seq_len, kHeads),
+                                      contiguous_strides(seq_len, kGroups), nullptr, stream);
+}
+
+int kascade_ref_prefill_reuse_call(kascade_half* Q, kascade_half* K, kascade_half* V,
+                                   int* topk_indices, int* head_mapping, float topk_percent,
+                                   kascade_half* Output, int batch, int seq_len, int topk_num,
+                                   void* stream) {
+    return kascade_prefill_reuse_call(Q, K, V, topk_indices, head_mapping, topk_percent, Output, batch,
+                                      seq_len, topk_num, 0, contiguous_strides(seq_len, kHeads),
+                                      contiguous_strides(seq_len, kGroups), nullptr, stream);
 }
 
 // ---- diagnostics ----

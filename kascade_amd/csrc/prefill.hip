@@ -120,7 +120,9 @@ __device__ __forceinline__ void chunk_of_sequence(const PrefillParams& p, int b,
 // Queries are rows [0, Lq) of Q at global positions q_start + row (q_start a multiple of 32);
 // keys are positions [0, L) with L = q_start + Lq.  PAGED: K/V are pages [P, page, G, D]
 // addressed through the block table, and gathered index rows hold physical row numbers.
-template <int NQB, bool REUSE, bool WITH_V, bool PAGED, int D, typename T>
+// EXACT_SUM: the softmax denominators are summed in fp32 from the unrounded exponentials (the
+// passes whose log-sum is an output); otherwise reuse units sum them as they enter the second product.
+template <int NQB, bool REUSE, bool WITH_V, bool PAGED, int D, typename T, bool EXACT_SUM = false>
 __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK, T* sV) {
     typedef typename Elem<T>::x8 x8_t;
     typedef typename Elem<T>::x4 x4_t;
@@ -276,7 +278,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
     constexpr float kRefSlack = 8.f;
     // Reuse units sum the exponentials as they enter the second product (rounded to the element
     // type, two per instruction); the passes whose log-sum feeds the selection sum them in fp32.
-    constexpr bool kPairSum = REUSE && WITH_V;
+    constexpr bool kPairSum = REUSE && WITH_V && !EXACT_SUM;
     float m[NQB], l[NQB];
     float16_t oT[NQB][kDB];
 #pragma unroll
@@ -550,12 +552,12 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
 
 // 32 queries per wavefront: register budget capped so that two workgroups share a
 // compute unit (64 KB of LDS each: two K and two V tile buffers).
-template <bool REUSE, bool WITH_V, bool PAGED, int D, typename T>
+template <bool REUSE, bool WITH_V, bool PAGED, int D, typename T, bool EXACT_SUM = false>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2)))
 void prefill_attn_kernel_q32(PrefillParams p) {
     __shared__ __attribute__((aligned(1024))) T sK[2 * AttnTile<D>::kTileElems];
     __shared__ __attribute__((aligned(1024))) T sV[WITH_V ? 2 * AttnTile<D>::kTileElems : 8];
-    prefill_attn_body<1, REUSE, WITH_V, PAGED, D, T>(p, sK, sV);
+    prefill_attn_body<1, REUSE, WITH_V, PAGED, D, T, EXACT_SUM>(p, sK, sV);
 }
 
 // 64 queries per wavefront for the K-only log-sum pass, whose state fits 256 registers: two
@@ -752,7 +754,12 @@ hipError_t launch_attn_t(const PrefillParams& p, bool reuse, bool with_v, int nq
         if (total > 0x7fffffffLL) return hipErrorInvalidConfiguration;
         grid = dim3((unsigned)total);
     }
-    if (paged) {
+    if (reuse && p.log_sum) {   // a reuse pass that also reports its log-sums: fp32 sums
+        if (paged)
+            hipLaunchKernelGGL((prefill_attn_kernel_q32<true, true, true, D, T, true>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((prefill_attn_kernel_q32<true, true, false, D, T, true>), grid, block, 0, stream, p);
+    } else if (paged) {
         if (reuse)
             hipLaunchKernelGGL((prefill_attn_kernel_q32<true, true, true, D, T>), grid, block, 0, stream, p);
         else if (with_v)

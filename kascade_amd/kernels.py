@@ -208,6 +208,28 @@ def decode_budgets(cache_seqlens, topk_percent: float, advance: int = 0, valid_o
     return valid_out[:n], n_sel_out[:n]
 
 
+def _decode_shapes(Q, shape, idx=None, head_mapping=None, glse=None, Output_partial=None,
+                   block_table=None, cache_seqlens=None) -> None:
+    """Tensor metadata of a decode call against the shape the kernels will index with: a scratch or
+    index tensor sized for another head count would be read or written out of bounds on the device."""
+    Hq, Gk, Dh, _ = shape
+    B = Q.shape[0]
+    if tuple(Q.shape) != (B, Hq, Dh):
+        raise KascadeError(f"Q must be [B,{Hq},{Dh}]")
+    if idx is not None and (idx.dim() != 3 or tuple(idx.shape[:2]) != (B, Gk)):
+        raise KascadeError(f"index lists must be [{B},{Gk},topk]")
+    if head_mapping is not None and head_mapping.numel() != Gk:
+        raise KascadeError(f"head_mapping must have {Gk} entries")
+    if glse is not None:
+        ns = glse.shape[2] if glse.dim() == 3 else -1
+        if tuple(glse.shape) != (B, Hq, ns) or Output_partial is None or tuple(Output_partial.shape) != (B, Hq, ns, Dh):
+            raise KascadeError(f"glse must be [{B},{Hq},S] and Output_partial [{B},{Hq},S,{Dh}]")
+    if block_table is not None and (block_table.dim() != 2 or block_table.shape[0] != B):
+        raise KascadeError(f"block_table must be [{B},max_pages]")
+    if cache_seqlens is not None and cache_seqlens.numel() != B:
+        raise KascadeError(f"cache_seqlens must have {B} entries")
+
+
 def _sync_arg(sync, B, groups: int = G):
     """Optional [B*G] int32 counter array for the fused combine (zero-initialised by the caller)."""
     if sync is None:
@@ -218,10 +240,20 @@ def _sync_arg(sync, B, groups: int = G):
     return _ptr(sync)
 
 
-def decode_reuse(Q, K, V, topk_indices, head_mapping, glse, Output_partial, sync=None) -> torch.Tensor:
+def _log_sum_arg(log_sum, B, Hq):
+    """Optional [B,H] fp32 output: the merged log-sum of the rows every head attended to."""
+    if log_sum is None:
+        return None
+    _req(log_sum, torch.float32, "log_sum")
+    if tuple(log_sum.shape) != (B, Hq):
+        raise KascadeError(f"log_sum must be [{B},{Hq}]")
+    return _ptr(log_sum)
+
+
+def decode_reuse(Q, K, V, topk_indices, head_mapping, glse, Output_partial, sync=None, log_sum=None) -> torch.Tensor:
     """``decode_reuse_kernel(Q, K, V, topk_indices, head_mapping, glse, Output_partial) -> O``
     (out_idx=[7]; EfficientKascadeStrategy.py:30-38, 113, 122).  Contiguous cache
-    K,V [B,L,G,D]; the split count is glse.shape[2]."""
+    K,V [B,L,G,D]; the split count is glse.shape[2].  log_sum: optional [B,H] fp32 output."""
     lib = _lib.init()
     B = Q.shape[0]
     L = K.shape[1]
@@ -235,7 +267,7 @@ def decode_reuse(Q, K, V, topk_indices, head_mapping, glse, Output_partial, sync
     if tuple(glse.shape) != (B, Hq, ns) or tuple(Output_partial.shape) != (B, Hq, ns, Dh):
         raise KascadeError("glse must be [B,H,S] and Output_partial [B,H,S,D]")
     out = torch.empty(B, Hq, Dh, device=Q.device, dtype=dt)
-    if kv_strides is None and shape == (H, G, D, torch.float16):
+    if kv_strides is None and shape == (H, G, D, torch.float16) and log_sum is None:
         _lib.check(lib.kascade_decode_reuse_call(
             _ptr(Q), _ptr(K), _ptr(V), _ptr(topk_indices), _ptr(head_mapping), _ptr(glse),
             _ptr(Output_partial), _ptr(out), B, L, topk_indices.shape[-1], ns, _sync_arg(sync, B), _stream()))
@@ -243,13 +275,13 @@ def decode_reuse(Q, K, V, topk_indices, head_mapping, glse, Output_partial, sync
         _lib.check(_call(lib, "decode_reuse_paged", shape,
             _ptr(Q), _ptr(K), _ptr(V), None, _ptr(topk_indices), _ptr(head_mapping), 0.0, _ptr(glse),
             _ptr(Output_partial), _ptr(out), B, L, topk_indices.shape[-1], ns, None, 0, 1, kv_strides,
-            None, None, _sync_arg(sync, B, Gk), _stream()))
+            None, None, _sync_arg(sync, B, Gk), _log_sum_arg(log_sum, B, Hq), _stream()))
     return out
 
 
 def decode_reuse_paged(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_percent, glse,
                        Output_partial, block_table=None, page_size: int = 16, out=None,
-                       sync=None, k_new=None, v_new=None) -> torch.Tensor:
+                       sync=None, k_new=None, v_new=None, log_sum=None) -> torch.Tensor:
     """``reuse kvcache kernel(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_percent,
     glse, Output_partial) -> O`` (out_idx=[9]; reuse_kascade_gqa_decode_with_kvcache.py:160-173)
     with an optional block table.  Without one K,V are the padded [B,maxL,G,D] cache;
@@ -263,6 +295,7 @@ def decode_reuse_paged(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_
     _req(glse, torch.float32, "glse"); _req(Output_partial, torch.float32, "Output_partial")
     if cache_seqlens is not None:
         _req(cache_seqlens, torch.int32, "cache_seqlens")
+    _decode_shapes(Q, shape, topk_indices, head_mapping, glse, Output_partial, block_table, cache_seqlens)
     ns = glse.shape[2]
     if block_table is not None:
         _req(block_table, torch.int32, "block_table")
@@ -274,13 +307,14 @@ def decode_reuse_paged(Q, K, V, cache_seqlens, topk_indices, head_mapping, topk_
         _ptr(Q), _ptr(K), _ptr(V), _ptr(cache_seqlens), _ptr(topk_indices), _ptr(head_mapping),
         float(topk_percent), _ptr(glse), _ptr(Output_partial), _ptr(out), B, stride_tokens,
         topk_indices.shape[-1], ns, _ptr(block_table), max_pages, page_size, kv_strides,
-        *_new_rows(k_new, v_new, B, shape), _sync_arg(sync, B, shape[1]), _stream()))
+        *_new_rows(k_new, v_new, B, shape), _sync_arg(sync, B, shape[1]), _log_sum_arg(log_sum, B, shape[0]),
+        _stream()))
     return out
 
 
 def decode_reuse_rows(Q, K_pages, V_pages, cache_seqlens, cache_rows, head_mapping, topk_percent, glse,
                       Output_partial, block_table, page_size: int = 16, out=None, sync=None,
-                      k_new=None, v_new=None) -> torch.Tensor:
+                      k_new=None, v_new=None, log_sum=None) -> torch.Tensor:
     """Reuse decode over a paged cache from index lists already translated to cache rows
     (``translate_indices`` of the anchor's selection): one dependent load fewer per row than
     ``decode_reuse_paged``.  cache_rows [B,G,topk] int32."""
@@ -296,13 +330,14 @@ def decode_reuse_rows(Q, K_pages, V_pages, cache_seqlens, cache_rows, head_mappi
         _req(cache_seqlens, torch.int32, "cache_seqlens")
     if K_pages.dim() != 4 or K_pages.shape[1] != page_size or K_pages.shape != V_pages.shape:
         raise KascadeError(f"pages must be [num_pages,{page_size},{Gk},{Dh}]")
+    _decode_shapes(Q, shape, cache_rows, head_mapping, glse, Output_partial, block_table, cache_seqlens)
     ns = glse.shape[2]
     out = _out_buffer(out, B, Q.device, shape)
     _lib.check(_call(lib, "decode_reuse_rows", shape,
         _ptr(Q), _ptr(K_pages), _ptr(V_pages), _ptr(cache_seqlens), _ptr(cache_rows), _ptr(head_mapping),
         float(topk_percent), _ptr(glse), _ptr(Output_partial), _ptr(out), B, cache_rows.shape[-1], ns,
         _ptr(block_table), block_table.shape[1], page_size, K_pages.shape[0], *_new_rows(k_new, v_new, B, shape),
-        _sync_arg(sync, B, Gk), _stream()))
+        _sync_arg(sync, B, Gk), _log_sum_arg(log_sum, B, Hq), _stream()))
     return out
 
 
@@ -317,11 +352,15 @@ def decode_reuse_paged_noalloc(Q, K, V, cache_seqlens, topk_indices, head_mappin
     the caller's, and nothing is allocated on the way -- not by this wrapper either."""
     lib = _lib.init()
     B = Q.shape[0]
+    shape = _shape(Q, K)
+    if shape != (H, G, D, torch.float16):
+        raise KascadeError(f"the no-allocation entry exists for {H} query / {G} KV heads, head_dim {D}, float16 only")
     _req(Q, torch.float16, "Q")
     kv_strides = _decode_kv(K, V, block_table)
     _req(topk_indices, torch.int32, "topk_indices"); _req(head_mapping, torch.int32, "head_mapping")
     if cache_seqlens is not None:
         _req(cache_seqlens, torch.int32, "cache_seqlens")
+    _decode_shapes(Q, shape, topk_indices, head_mapping, None, None, block_table, cache_seqlens)
     if block_table is not None:
         _req(block_table, torch.int32, "block_table")
         stride_tokens, max_pages = 0, block_table.shape[1]
@@ -346,6 +385,7 @@ def decode_dense_paged(Q, K, V, cache_seqlens, glse, Output_partial, block_table
     _req(Q, shape[3], "Q")
     kv_strides = _decode_kv(K, V, block_table, shape)
     _req(glse, torch.float32, "glse"); _req(Output_partial, torch.float32, "Output_partial")
+    _decode_shapes(Q, shape, None, None, glse, Output_partial, block_table, cache_seqlens)
     ns = glse.shape[2]
     if block_table is not None:
         _req(block_table, torch.int32, "block_table")
@@ -378,6 +418,12 @@ def decode_recompute(Q, K, V, glse, Output_partial, row_sums, scores, layer: int
     _req(glse, torch.float32, "glse"); _req(row_sums, torch.float32, "row_sums")
     _req(scores, torch.float32, "scores")
     with_out = 1 if layer == 0 else 0
+    _decode_shapes(Q, shape, None, None, glse, Output_partial if with_out else None, block_table, cache_seqlens) \
+        if with_out else _decode_shapes(Q, shape, None, None, None, None, block_table, cache_seqlens)
+    Hq = shape[0]
+    if glse.dim() != 3 or tuple(glse.shape[:2]) != (B, Hq) or tuple(row_sums.shape) != (B, Hq) \
+            or scores.dim() != 3 or tuple(scores.shape[:2]) != (B, Hq):
+        raise KascadeError(f"glse must be [{B},{Hq},S], row_sums [{B},{Hq}] and scores [{B},{Hq},stride]")
     ns = glse.shape[2]
     stride = scores.shape[2]
     if block_table is not None:
@@ -563,10 +609,11 @@ def prefill_aggregate_range(Q, K, log_sum, scores, q_start: int, q_len: int, fil
                      q_start, q_len, qs, ks, 1 if fill_invalid else 0, _stream()))
 
 
-def prefill_reuse(Q, K, V, topk_idx, head_mapping, topk_percent, rolling: bool) -> torch.Tensor:
+def prefill_reuse(Q, K, V, topk_idx, head_mapping, topk_percent, rolling: bool, return_log_sum: bool = False):
     """``prefill_reuse_kernel(Q, K, V, topk_indices, head_mapping, topk_percent) -> O``
     (out_idx=[6]; EfficientKascadeStrategy.py:61-70, 92, 97); ``rolling`` selects between the
-    reference's two compiled objects."""
+    reference's two compiled objects.  With return_log_sum also the [B,L,H] fp32 log2-domain
+    log-sum over the keys every row attended to: returns (O, log_sum)."""
     lib = _lib.init()
     shape = _shape(Q, K)
     Hq, Gk, Dh, dt = shape
@@ -580,10 +627,11 @@ def prefill_reuse(Q, K, V, topk_idx, head_mapping, topk_percent, rolling: bool) 
     if tuple(V.stride()) != tuple(K.stride()) or V.shape != K.shape:
         raise KascadeError("K and V must share shape and strides")
     out = torch.empty(B, L, Hq, Dh, device=Q.device, dtype=dt)
+    log_sum = torch.empty(B, L, Hq, device=Q.device, dtype=torch.float32) if return_log_sum else None
     _lib.check(_call(lib, "prefill_reuse", shape,
         _ptr(Q), _ptr(K), _ptr(V), _ptr(topk_idx), _ptr(head_mapping), float(topk_percent), _ptr(out),
-        B, L, topk_idx.shape[-1], 1 if rolling else 0, qs, ks, _stream()))
-    return out
+        B, L, topk_idx.shape[-1], 1 if rolling else 0, qs, ks, _ptr(log_sum), _stream()))
+    return (out, log_sum) if return_log_sum else out
 
 
 # ------------------------------------------------------------- KV append
@@ -757,7 +805,7 @@ def translate_indices(token_idx, block_table, kv_len: int, page_size: int = 16, 
 
 def prefill_chunk_reuse(Q, K_pages, V_pages, physical_rows, head_mapping, topk_percent,
                         rolling: bool, block_table, q_start: int, page_size: int = 16,
-                        q_starts=None, q_lens=None) -> torch.Tensor:
+                        q_starts=None, q_lens=None, return_log_sum: bool = False):
     """Chunked ``prefill_reuse_kernel`` (EfficientKascadeStrategy.py:92, 97): physical_rows
     [B,G,ceil(Lq/32),max_topk] comes from ``translate_indices``."""
     lib = _lib.init()
@@ -771,12 +819,13 @@ def prefill_chunk_reuse(Q, K_pages, V_pages, physical_rows, head_mapping, topk_p
     if tuple(physical_rows.shape[:3]) != (B, Gk, T) or head_mapping.numel() != Gk:
         raise KascadeError("physical_rows must be [B,G,ceil(Lq/32),max_topk] and head_mapping [G]")
     out = torch.empty(B, Lq, Hq, Dh, device=Q.device, dtype=dt)
+    log_sum = torch.empty(B, Lq, Hq, device=Q.device, dtype=torch.float32) if return_log_sum else None
     _lib.check(_call(lib, "prefill_chunk_reuse", shape,
         _ptr(Q), _ptr(K_pages), _ptr(V_pages), _ptr(physical_rows), _ptr(head_mapping),
         float(topk_percent), _ptr(out), B, q_start, Lq, physical_rows.shape[-1], 1 if rolling else 0,
         qs, _ptr(block_table), block_table.shape[1], page_size, K_pages.shape[0], _ptr(q_starts),
-        _ptr(q_lens), _stream()))
-    return out
+        _ptr(q_lens), _ptr(log_sum), _stream()))
+    return (out, log_sum) if return_log_sum else out
 
 
 # ------------------------------------------------- benchmark / correctness glue

@@ -20,9 +20,12 @@ def lib():
 
 
 def _declared_functions():
-    text = open(HEADER).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(kascade_[a-z0-9_]+)\s*\(", text)))
+    import glob
+    names = set()
+    for path in glob.glob(os.path.join(ROOT, "include", "*.h")):
+        text = re.sub(r"/\*.*?\*/", "", open(path).read(), flags=re.S)
+        names |= set(re.findall(r"\b(kascade_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
 
 
 def test_header_symbols_are_exported_and_bound(lib):
@@ -30,7 +33,7 @@ def test_header_symbols_are_exported_and_bound(lib):
     names = _declared_functions()
     assert len(names) >= 14
     for n in names:
-        assert hasattr(lib, n), f"{n} declared in include/kascade_hip.h but not exported"
+        assert hasattr(lib, n), f"{n} declared under include/ but not exported"
         assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
     assert sorted(_lib.SIGNATURES) == names
 
@@ -63,7 +66,7 @@ def test_null_pointers_are_rejected(lib):
     assert lib.kascade_topk_call(None, None, 1, 10, 10, None, None, 1, 4, 0, None, None) == -1
     assert lib.kascade_prefill_dense_call(None, None, None, None, None, 1, 64, s, s, 1, None) == -1
     assert lib.kascade_prefill_aggregate_call(None, None, None, None, 1, 64, s, s, 0, None) == -1
-    assert lib.kascade_prefill_reuse_call(None, None, None, None, None, 10.0, None, 1, 64, 128, 1, s, s, None) == -1
+    assert lib.kascade_prefill_reuse_call(None, None, None, None, None, 10.0, None, 1, 64, 128, 1, s, s, None, None) == -1
     assert lib.kascade_paged_kv_append_call(None, None, None, None, None, None, 1, 1, 1, 16, s, None, None) == -1
     assert lib.kascade_rope_append_paged_call(None, None, None, None, None, None, 64, None, None, 1e-6, None, 0,
                                               None, None, None, None, 4, 16, 1, 1, None) == -1
@@ -75,9 +78,9 @@ def test_bad_sizes_are_rejected(lib):
     buf = (C.c_char * 4096)()
     p = C.addressof(buf) & ~15          # fake, 16-byte aligned, never dereferenced: validation fails first
     p += 16
-    assert lib.kascade_decode_reuse_paged_call(p, p, p, None, p, p, 0.0, p, p, p, 0, 128, 128, 8, None, 0, 16, None, None, None, None, None) == -1
+    assert lib.kascade_decode_reuse_paged_call(p, p, p, None, p, p, 0.0, p, p, p, 0, 128, 128, 8, None, 0, 16, None, None, None, None, None, None) == -1
     assert "batch" in _err(lib)
-    assert lib.kascade_decode_reuse_paged_call(p, p, p, None, p, p, 10.0, p, p, p, 1, 128, 128, 8, None, 0, 16, None, None, None, None, None) == -1
+    assert lib.kascade_decode_reuse_paged_call(p, p, p, None, p, p, 10.0, p, p, p, 1, 128, 128, 8, None, 0, 16, None, None, None, None, None, None) == -1
     assert "cache_seqlens" in _err(lib)
     assert lib.kascade_decode_dense_paged_call(p, p, p, None, p, p, p, 1, 128, 8, p, 4, 12, None, None, None, None, None) == -1
     assert "power of two" in _err(lib)
@@ -109,9 +112,9 @@ def test_bad_sizes_are_rejected(lib):
     ok = Strides(4096 * 128, 4096, 128)
     assert lib.kascade_prefill_dense_call(p, p, p, p, p, 1, 64, bad, ok, 1, None) == -1
     assert "strides" in _err(lib)
-    assert lib.kascade_prefill_reuse_call(p, p, p, p, p, 0.0, p, 1, 64, 128, 1, ok, ok, None) == -1
+    assert lib.kascade_prefill_reuse_call(p, p, p, p, p, 0.0, p, 1, 64, 128, 1, ok, ok, None, None) == -1
     assert "rolling" in _err(lib)
-    assert lib.kascade_prefill_reuse_call(p, p, p, p, p, 10.0, p, 1, 64, 0, 0, ok, ok, None) == -1
+    assert lib.kascade_prefill_reuse_call(p, p, p, p, p, 10.0, p, 1, 64, 0, 0, ok, ok, None, None) == -1
     assert "max_topk_num" in _err(lib)
 
 

@@ -31,11 +31,16 @@ def test_no_alloc_entry_matches_caller_scratch_entry(cuda):
         part = torch.empty(B, H, ns, D, device=cuda, dtype=torch.float32)
         want = kernels.decode_reuse_paged(q, kp, vp, lens, idx, hm, 0.0, glse, part, block_table=bt, page_size=page)
         out = torch.full((B, H, D), float("nan"), device=cuda, dtype=torch.float16)
+        # one untimed call first: whatever the runtime sets up on a kernel's first launch is not the call's doing
+        kernels.decode_reuse_paged_noalloc(q, kp, vp, lens, idx, hm, 0.0, ns, out, block_table=bt, page_size=page)
+        out.fill_(float("nan"))
         torch.cuda.synchronize()
-        before = torch.cuda.memory_stats()["allocation.all.allocated"]      # allocations made so far
+        before = torch.cuda.memory_stats()["allocation.all.allocated"]      # torch's allocator: the Python wrapper
+        free_before = torch.cuda.mem_get_info()[0]                          # the device: the library itself
         got = kernels.decode_reuse_paged_noalloc(q, kp, vp, lens, idx, hm, 0.0, ns, out, block_table=bt, page_size=page)
         torch.cuda.synchronize()
-        assert torch.cuda.memory_stats()["allocation.all.allocated"] == before, "the call allocated device memory"
+        assert torch.cuda.memory_stats()["allocation.all.allocated"] == before, "the wrapper allocated device memory"
+        assert torch.cuda.mem_get_info()[0] == free_before, "free device memory changed across the call"
         assert got.data_ptr() == out.data_ptr()
         assert torch.isfinite(got).all() and torch.equal(got, want), f"{seqlens}: differs from the caller-scratch entry"
     # per-sequence budgets (topk_percent > 0) take the same path
