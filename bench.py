@@ -803,11 +803,59 @@ def main():
             cpu_decode["sample"] = (f"oracle on {Bs} of the 16 sequences of configs[2] (65536-token contexts, "
                                     f"contiguous cache), one decode step per layer kind, scaled by 16/{Bs}")
             log(f"[bench] cpu decode: {cpu_decode}")
+        # config 0 in full: the one configuration that is the reference's own CPU path (strategy
+        # semantics, fp32): batch 1, 8 query / 2 KV heads, head_dim 64, causal prefill of 2048 tokens,
+        # one anchor layer then one reuse layer
+        g0 = torch.Generator().manual_seed(0)
+        q0 = torch.randn(1, 8, 2048, 64, generator=g0); k0 = torch.randn(1, 2, 2048, 64, generator=g0)
+        v0 = torch.randn(1, 2, 2048, 64, generator=g0)
+        q1 = q0 + 0.3 * torch.randn(q0.shape, generator=g0); k1 = k0 + 0.3 * torch.randn(k0.shape, generator=g0)
+        mask0 = orc.causal_additive_mask(2048, 2048, torch.float32)
+        t_cfg0 = []
+        for _ in range(3):
+            st0 = orc.StrategyOracle([0], [[0, 1], [0, 1]], k=PCT, tile_size=TILE, rolling_prefill=False)
+            t0 = time.perf_counter()
+            st0.attention_forward(0, q0, k0, v0, mask0, 64 ** -0.5)
+            ta0 = time.perf_counter()
+            st0.attention_forward(1, q1, k1, v0, mask0, 64 ** -0.5)
+            t_cfg0.append((ta0 - t0, time.perf_counter() - ta0))
+        t_cfg0.sort(key=lambda x: x[0] + x[1])
+        cpu_cfg0 = {"anchor0_ms": round(t_cfg0[1][0] * 1e3, 1), "reuse_ms": round(t_cfg0[1][1] * 1e3, 1),
+                    "sample": "configs[0] in full: StrategyOracle (the reference's unoptimised PyTorch path restated), "
+                              "fp32, 2048 tokens, 8/2 heads, head_dim 64, anchor layer then reuse layer; median of 3"}
+        log(f"[bench] cpu config 0: {cpu_cfg0}")
+        del q0, k0, v0, q1, k1, mask0
+        # config 3: one decode step of the three layer kinds on its shortest sequence (131072 tokens),
+        # scaled by the batch's token count
+        cpu_cfg3 = None
+        if not args.skip_decode:
+            L3, total3 = 131072, 131072 + 196608 + 262144 + 524288
+            dk = workloads.peaked_keys(L3, seed=90, device="cpu")[None]
+            dv = workloads.gaussian((1, L3, G, D), seed=91, device="cpu")
+            dq = workloads.gaussian((1, H, D), seed=92, device="cpu")
+            t0 = time.perf_counter()
+            orc.dense_decode(dq, dk, dv)
+            t_dd = time.perf_counter() - t0
+            t0 = time.perf_counter()
+            idx_d = orc.topk_rows(orc.pooled_decode_scores(dq, dk), budgets.decode_budget(L3, PCT))
+            t_da = time.perf_counter() - t0
+            t0 = time.perf_counter()
+            orc.reuse_decode(dq, dk, dv, idx_d, list(head_map[1]))
+            t_dr = time.perf_counter() - t0
+            scale = total3 / L3 * 1e6
+            per = {"dense_us": t_dd * scale, "anchor0_us": (t_dd + t_da) * scale,
+                   "anchor_us": (t_da + t_dr) * scale, "reuse_us": t_dr * scale}
+            per["kascade_us_per_layer"] = (per["anchor0_us"] + 4 * per["anchor_us"] + 27 * per["reuse_us"]) / N_LAYERS
+            cpu_cfg3 = {k: round(v, 0) for k, v in per.items()}
+            cpu_cfg3["sample"] = ("oracle on the 131072-token sequence of configs[3] (contiguous cache), one decode "
+                                  f"step per layer kind, scaled by the batch's tokens ({total3}/{L3})")
+            log(f"[bench] cpu decode config 3: {cpu_cfg3}")
+            del dk, dv, dq
         cpu = {"value": round(cpu_ms, 1), "unit": "ms", "cores": nthreads, "kind": "port",
                "sample": f"oracle (dense-matrix PyTorch, fp32) on {nblk} blocks of {rows} query rows centred in "
                          f"each quarter of the {Lc}-token prompt, extrapolated by rows; layer mix 1/4/27",
                "per_layer_ms": {k: round(v * 1e3, 1) for k, v in est.items()},
-               "decode_cfg2": cpu_decode}
+               "decode_cfg2": cpu_decode, "cfg0": cpu_cfg0, "decode_cfg3": cpu_cfg3}
 
     out = {
         "metric": "kascade prefill attn ms/layer @32K (value) & decode attn us/layer @64K/128K/ragged (decode), "
