@@ -144,3 +144,71 @@ def test_sequences_join_and_leave(cuda):
         for l in (0, N_LAYERS - 1):
             kc = orc.paged_to_contiguous(st.k_pages[l].cpu(), st.block_table.cpu()[slot:slot + 1], [n])
             assert torch.equal(kc[0], data[1][l][:n]), f"{name} layer {l} cache"
+
+
+@pytest.mark.parametrize("Hq,Gk,Dh,dt", [(16, 2, 64, torch.bfloat16), (12, 3, 128, torch.float16)])
+def test_mixed_batch_other_shapes(cuda, Hq, Gk, Dh, dt):
+    """Per-sequence chunk offsets and empty slots at other shapes (8 and 4 query heads per KV head,
+    head_dim 64 and 128, bf16 and fp16): every sequence of a mixed batch gets, bit for bit, what
+    it gets alone."""
+    from kascade_amd.stack import KascadeAttentionStack
+    layers, anchors, p, max_len, slots = 3, [0, 1], 25, 512, 2
+    maps = [list(range(Gk)), list(range(Gk)), [(g + 1) % Gk for g in range(Gk)]]
+
+    def stack():
+        return KascadeAttentionStack(layers, anchors, maps, p, max_len, batch=slots, page_size=16, rolling_prefill=True,
+                                     device=cuda, table_seed=5, kv_heads=Gk, head_dim=Dh, dtype=dt,
+                                     group_size=Hq // Gk, reserve=False)
+
+    def data(seed, n):
+        g = torch.Generator().manual_seed(seed)
+        return ([(torch.randn(n, Hq, Dh, generator=g) + 0.5).to(dt) for _ in range(layers)],
+                [(torch.randn(n, Gk, Dh, generator=g) * 1.5).to(dt) for _ in range(layers)],
+                [torch.randn(n, Gk, Dh, generator=g).to(dt) for _ in range(layers)])
+
+    def run(st, seqs, plan):
+        """plan: list of ('p', {slot: rows}) / ('d',) steps; returns per-slot outputs."""
+        pos = {b: 0 for b in seqs}
+        got = {b: [] for b in seqs}
+        for step in plan:
+            if step[0] == 'p':
+                rows = step[1]
+                Lq = max(rows.values())
+                q = [torch.zeros(slots, Lq, Hq, Dh, dtype=dt) for _ in range(layers)]
+                k = [torch.zeros(slots, Lq, Gk, Dh, dtype=dt) for _ in range(layers)]
+                v = [torch.zeros(slots, Lq, Gk, Dh, dtype=dt) for _ in range(layers)]
+                lens = [0] * slots
+                for b, n in rows.items():
+                    lens[b] = n
+                    for l in range(layers):
+                        q[l][b, :n], k[l][b, :n], v[l][b, :n] = (x[l][pos[b]:pos[b] + n] for x in seqs[b])
+                out = st.prefill_chunk([x.to(cuda) for x in q], [x.to(cuda) for x in k], [x.to(cuda) for x in v], q_lens=lens)
+                for b, n in rows.items():
+                    got[b].append(torch.stack([o[b, :n] for o in out]).cpu())
+                    pos[b] += n
+            else:
+                q = torch.zeros(layers, slots, Hq, Dh, dtype=dt)
+                k = torch.zeros(layers, slots, 1, Gk, Dh, dtype=dt)
+                v = torch.zeros(layers, slots, 1, Gk, Dh, dtype=dt)
+                for b in seqs:
+                    if pos[b]:
+                        for l in range(layers):
+                            q[l, b], k[l, b, 0], v[l, b, 0] = (x[l][pos[b]] for x in seqs[b])
+                out = st.decode_step(q.to(cuda), k.to(cuda), v.to(cuda)).cpu()
+                for b in seqs:
+                    if pos[b]:
+                        got[b].append(out[:, b].clone())
+                        pos[b] += 1
+        return got
+
+    a, b = data(1, 300), data(2, 200)
+    st = stack(); st.admit(0, 0); st.admit(0, 1)
+    both = run(st, {0: a, 1: b}, [('p', {0: 160}), ('p', {0: 128, 1: 192}), ('d',), ('d',)])
+    st0 = stack(); st0.admit(0, 0)
+    alone_a = run(st0, {0: a}, [('p', {0: 160}), ('p', {0: 128}), ('d',), ('d',)])
+    st1 = stack(); st1.admit(0, 1)
+    alone_b = run(st1, {1: b}, [('p', {1: 192}), ('d',), ('d',)])
+    for x, y in zip(both[0], alone_a[0]):
+        assert torch.isfinite(x.float()).all() and torch.equal(x, y)
+    for x, y in zip(both[1], alone_b[1]):
+        assert torch.isfinite(x.float()).all() and torch.equal(x, y)
