@@ -31,12 +31,38 @@
 #include <algorithm>
 #include <type_traits>
 
+// Wave priority around the phases of a tile.  Two wavefronts share a SIMD; which of them the
+// scheduler serves first when both have an instruction ready decides how well one's softmax hides
+// under the other's matrix instructions.  Modes: 0 none; 1 the wavefront in its softmax goes first;
+// 2 the one in its products; 4 the one in its second product only; 5 the one in its first product
+// only.  Measured at 32K tokens against mode 0 (same box, two rounds): kernels with a second
+// product mode 2 -1.1 % (reuse) / -1.4 % (dense), mode 1 +1.2 %, mode 4 +1 %, mode 5 -0.5 %; the
+// K-only log-sum pass mode 1 -2.6 %, mode 2 -0.8 %, mode 5 -0.5 %; the pooling kernel mode 2 -1.9 %,
+// mode 1 -1.7 %.
+#ifndef KASCADE_PRIO_V
+#define KASCADE_PRIO_V 2
+#endif
+#ifndef KASCADE_PRIO_K
+#define KASCADE_PRIO_K 1
+#endif
+#ifndef KASCADE_PRIO_AGG
+#define KASCADE_PRIO_AGG 2
+#endif
+
 namespace kascade {
 
 namespace {
 
 constexpr int kThreads = 256;
 constexpr int kAggKT = 128;        // keys per tile (aggregate kernel)
+
+// phase: 0 = first product begins, 1 = softmax begins, 2 = second product begins (or the tile ends)
+template <int MODE> __device__ __forceinline__ void tile_phase(int phase) {
+    if (MODE == 1) { if (phase == 1) __builtin_amdgcn_s_setprio(1); else if (phase == 2) __builtin_amdgcn_s_setprio(0); }
+    if (MODE == 2) { if (phase == 1) __builtin_amdgcn_s_setprio(0); else if (phase == 2) __builtin_amdgcn_s_setprio(1); }
+    if (MODE == 4) { if (phase == 0) __builtin_amdgcn_s_setprio(0); else if (phase == 2) __builtin_amdgcn_s_setprio(1); }
+    if (MODE == 5) { if (phase == 0) __builtin_amdgcn_s_setprio(1); else if (phase == 1) __builtin_amdgcn_s_setprio(0); }
+}
 
 // Queries are rows [0, Lq) of Q at global positions q_start + row (q_start a multiple of 32);
 // keys are positions [0, L) with L = q_start + Lq.  PAGED: K/V are pages [P, page, G, D]
@@ -196,6 +222,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
     // (representable in fp16 and bf16, sums and products are kept in fp32) and the rescaling of the
     // accumulators -- 64 products per lane -- runs on the first tiles of a unit and then almost
     // never.  The quotient is the same: numerator and denominator carry the same factor.
+    constexpr int kPrio = WITH_V ? KASCADE_PRIO_V : KASCADE_PRIO_K;
     constexpr float kRefSlack = 8.f;
     // Reuse units sum the exponentials as they enter the second product (rounded to the element
     // type, two per instruction); the passes whose log-sum feeds the selection sum them in fp32.
@@ -263,6 +290,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
         if (sq + 1 < ntiles) next_offsets();
         const int nbuf = (sq + 1) & 1;
 
+        tile_phase<kPrio>(0);
         // ---- S^T = K_tile Q^T.  Step c = (key block c / kKS, contraction step c % kKS); operands are
         // read from LDS two windows (four steps) ahead of the products that use them, in program
         // order, because LDS reads do not move across the load statements ----
@@ -326,6 +354,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
             }
         }
         // ---- online softmax (one query column per lane pair: lanes li and li + 32) ----
+        tile_phase<kPrio>(1);
         x8_t pf[NQB][2 * nkb];
 #pragma unroll
         for (int qb = 0; qb < NQB; ++qb) {
@@ -379,6 +408,7 @@ __device__ __forceinline__ void prefill_attn_body(const PrefillParams& p, T* sK,
             }
             l[qb] += sum;   // per-lane partial sum (own key positions)
         }
+        tile_phase<kPrio>(2);
         // ---- O^T += V^T P^T: step s covers the keys of accumulators 8(s&1) .. 8(s&1)+7 of key block
         // s/2, i.e. rows 16 s + 8 h + 4 lg + (0..3), h = 0, 1, of the tile.  The operands of a block
         // of 32 output rows are read while the block before it is multiplied ----
@@ -633,6 +663,7 @@ void prefill_aggregate_kernel(PrefillParams p) {
 #pragma unroll
             for (int j = kKS; j < kLoads; ++j) issue_load(tn, j, nbuf);
             // accumulator v of row block rb is query row 8(v/4) + 4lg + v%4, column = key li
+            tile_phase<KASCADE_PRIO_AGG>(1);
             float sum = 0.f;
 #pragma unroll
             for (int rb = 0; rb < kGroupSize; ++rb)
@@ -644,6 +675,7 @@ void prefill_aggregate_kernel(PrefillParams p) {
                         sum += fast_exp2(acc[rb][4 * v4 + e] * kScaleLog2 - ls[e]);
                 }
             sum = sum_with_other_half(sum);
+            tile_phase<KASCADE_PRIO_AGG>(2);
             const int key = ti * kAggKT + 32 * wave + li;
             if (lg == 0 && key < Ls) {
                 if (key < ts)   // a later sub-group of the KV head adds to what the earlier ones left
