@@ -264,3 +264,31 @@ def layer_statistics(layers: Sequence[Tuple[torch.Tensor, torch.Tensor]], topk_p
             sim[a, b] = tile_similarity(q, k, idxs[a], idxs[b], topk_percent, rolling, reduce, lses[b], tails[b],
                                         reference_tail)
     return sim
+
+
+def decode_similarity(q_b: torch.Tensor, k_b: torch.Tensor, idx_a: torch.Tensor, idx_b: torch.Tensor,
+                      log_sum_full: torch.Tensor, num_split: int = 4) -> torch.Tensor:
+    """The same statistic for a decode step (the reference accumulates decode steps too, with no
+    own-tile term: stats_runner.py:42-61, 155-168): sim[hb, ha] = attention mass of layer B's KV
+    head hb (summed over its query heads) on the rows idx_a[b, ha] over its mass on its own rows
+    idx_b[b, hb], for sequence 0.  q_b [B,H,D]; k_b [B,L,G,D] contiguous cache of layer B; idx_*
+    [B,G,k] int32; log_sum_full [B,H]: layer B's dense log2-domain log-sum (``row_sums`` of the
+    anchor decode pass).  G + 1 launches of the reuse decode kernel, read through ``log_sum``."""
+    from . import kernels
+    B, Hq, Dh = q_b.shape
+    G = k_b.shape[2]
+    glse = torch.empty(B, Hq, num_split, device=q_b.device, dtype=torch.float32)
+    part = torch.empty(B, Hq, num_split, Dh, device=q_b.device, dtype=torch.float32)
+    ls = torch.empty(B, Hq, device=q_b.device, dtype=torch.float32)
+
+    def mass(idx, hm):
+        kernels.decode_reuse(q_b, k_b, k_b, idx, torch.tensor(hm, dtype=torch.int32, device=q_b.device), glse, part,
+                             log_sum=ls)
+        return torch.exp2(ls - log_sum_full).view(B, G, Hq // G).sum(-1)          # [B,G]
+
+    own = mass(idx_b, list(range(G)))
+    sim = torch.empty(G, G, device=q_b.device, dtype=torch.float32)
+    for s_ in range(G):
+        hm = [(g + s_) % G for g in range(G)]
+        sim[torch.arange(G), torch.tensor(hm)] = (mass(idx_a, hm) / own)[0]
+    return sim

@@ -152,3 +152,34 @@ def test_decode_reuse_log_sum_output(cuda):
     _, dense_lse = orc.dense_decode(w.q, kc, orc.paged_to_contiguous(w.v_pages, w.block_table, seqlens), seqlens)
     share = torch.exp2(ls.cpu() - dense_lse * 1.4426950408889634)     # the oracle's is a natural log
     assert float(share.max()) <= 1.0 + 1e-4 and float(share.min()) > 0.0
+
+
+def test_decode_similarity_matches_dense_definition(cuda):
+    """One decode step: the device statistic against stats_runner.py:155-168 evaluated on the dense
+    pooled attention row of every KV head (calibration.similarity_layer with no own-tile term)."""
+    from kascade_amd import kernels, workloads
+    from oracle import kascade_oracle as orc
+    L, topk = 3000, 384
+    w = workloads.paged_decode_inputs([L], seed=12, device="cpu")
+    kc = orc.paged_to_contiguous(w.k_pages, w.block_table, [L])                    # [1,L,G,D]
+    q = w.q
+    pooled = orc.pooled_decode_scores(q, kc).float()                               # [1,G,L] (fp16-rounded)
+    sc = torch.einsum("hd,lhd->hl", q[0].float(), kc[0].float().repeat_interleave(H // G, dim=1)) * D ** -0.5
+    dense = torch.softmax(sc, -1).view(G, H // G, L).sum(1)[None, :, None]         # [1,G,1,L] exact
+    gen = torch.Generator().manual_seed(4)
+    idx_b = torch.topk(pooled, topk, dim=-1).indices.sort(-1).values.to(torch.int32)   # layer B's own lists
+    idx_a = torch.empty_like(idx_b)                                                  # layer A's: half of B's, half others
+    for g in range(G):
+        keep = idx_b[0, g][torch.randperm(topk, generator=gen)[:topk // 2]]
+        free = torch.ones(L, dtype=torch.bool)
+        free[keep.long()] = False
+        others = torch.nonzero(free)[:, 0][torch.randperm(L - topk // 2, generator=gen)[:topk - topk // 2]]
+        idx_a[0, g] = torch.cat([keep, others.to(torch.int32)]).sort().values         # distinct: a gather counts duplicates twice
+    want = cal.similarity_layer(idx_a[:, :, None].long(), idx_b[:, :, None].long(), dense, None, "amin")
+    _, lse_nat = orc.dense_decode(q, kc, kc)
+    got = cal.decode_similarity(q.to(cuda), kc.to(cuda), idx_a.to(cuda), idx_b.to(cuda),
+                                (lse_nat * 1.4426950408889634).to(cuda)).cpu()
+    assert torch.allclose(got, want, atol=1e-3), float((got - want).abs().max())
+    assert torch.allclose(torch.diagonal(cal.decode_similarity(q.to(cuda), kc.to(cuda), idx_b.to(cuda), idx_b.to(cuda),
+                                                                 (lse_nat * 1.4426950408889634).to(cuda)).cpu()),
+                          torch.ones(G), atol=1e-5)
