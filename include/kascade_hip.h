@@ -286,6 +286,22 @@ int kascade_topk_rows_call(const kascade_half* scores, int32_t* out_idx, int row
                            const int32_t* block_table, int max_pages, int page_size,
                            int rows_per_sequence, void* stream);
 
+/* The selection in the form torch.topk(scores[..., :uniform_len], k).indices has
+ * (EfficientKascadeStrategy.py:82, 90, 111): full-width rows ordered by descending score, for a
+ * consumer that slices its own prefix of a row.
+ *   out_idx [rows, k] i32: the k largest entries among the first valid_len[r % period] of row r
+ *   (valid_len == NULL: uniform_len), largest first, equal scores by ascending position.  A row
+ *   with fewer than k valid entries lists all of them in that order, then the positions
+ *   valid_len, valid_len + 1, ... (where the reference's tensor holds -inf; torch.topk leaves
+ *   the choice among those open).  0 < k <= uniform_len.
+ *   workspace: device scratch of kascade_topk_sorted_workspace_bytes(rows, uniform_len, k) bytes
+ *   (NULL when that is 0: lists of up to 4096 entries over rows short enough for one workgroup).
+ * Runs kascade_topk_call and then a stable two-pass radix sort of each row's list. */
+int64_t kascade_topk_sorted_workspace_bytes(int rows, int64_t row_len, int k);
+int kascade_topk_sorted_call(const kascade_half* scores, int32_t* out_idx, int rows, int64_t row_stride,
+                             int uniform_len, const int32_t* valid_len, int period, int k,
+                             void* workspace, void* stream);
+
 /* ----------------------------------------------------------------- prefill */
 
 /* Anchor layer 0: dense causal GQA flash attention that also emits the log2

@@ -47,6 +47,8 @@ SIGNATURES = {
                                                  _I, _I, _P, _I, _I, _SP, _P, _P, _P, _P]),
     "kascade_topk_workspace_bytes": (_L, [_I, _L]),
     "kascade_topk_call": (_I, [_P, _P, _I, _L, _I, _P, _P, _I, _I, _I, _P, _P]),
+    "kascade_topk_sorted_workspace_bytes": (_L, [_I, _L, _I]),
+    "kascade_topk_sorted_call": (_I, [_P, _P, _I, _L, _I, _P, _I, _I, _P, _P]),
     "kascade_topk_rows_call": (_I, [_P, _P, _I, _L, _I, _P, _P, _I, _I, _I, _P, _P, _P, _I, _I, _I, _P]),
     "kascade_prefill_dense_call": (_I, [_P, _P, _P, _P, _P, _I, _I, Strides, Strides, _I, _P]),
     "kascade_prefill_aggregate_call": (_I, [_P, _P, _P, _P, _I, _I, Strides, Strides, _I, _P]),

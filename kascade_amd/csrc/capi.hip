@@ -552,6 +552,36 @@ int kascade_topk_rows_call(const kascade_half* scores, int32_t* out_idx, int row
                                  period, k, fill_value, &tr, s), "topk");
 }
 
+namespace {
+inline long long sorted_list_bytes(int rows, int k) {
+    return (topk_sort_workspace_bytes(rows, k) + 255) / 256 * 256;
+}
+}  // namespace
+
+int64_t kascade_topk_sorted_workspace_bytes(int rows, int64_t row_len, int k) {
+    if (rows < 0 || k < 0) return 0;
+    return sorted_list_bytes(rows, k) + topk_split_workspace_bytes(rows, row_len);
+}
+
+int kascade_topk_sorted_call(const kascade_half* scores, int32_t* out_idx, int rows, int64_t row_stride,
+                             int uniform_len, const int32_t* valid_len, int period, int k,
+                             void* workspace, void* stream) {
+    REQUIRE(k > 0 && k <= uniform_len, "topk_sorted: 0 < k <= uniform_len required (as torch.topk)");
+    REQUIRE(rows >= 0, "topk_sorted: rows >= 0 required");
+    REQUIRE(workspace || kascade_topk_sorted_workspace_bytes(rows, uniform_len, k) == 0,
+            "topk_sorted: workspace of kascade_topk_sorted_workspace_bytes() bytes required");
+    char* ws = static_cast<char*>(workspace);
+    void* split_ws = topk_split_workspace_bytes(rows, uniform_len) > 0 ? ws + sorted_list_bytes(rows, k) : nullptr;
+    // the k largest of every row in position order (all valid positions, then the first positions
+    // past the row's end, when a row holds fewer than k), then the reordering by score
+    if (kascade_topk_call(scores, out_idx, rows, row_stride, uniform_len, valid_len, nullptr, period, k, 0,
+                          split_ws, stream))
+        return -1;
+    if (period <= 0) period = 1;
+    return check_hip(launch_topk_sort_rows(H(scores), out_idx, ws, rows, row_stride, uniform_len, valid_len,
+                                           period, k, static_cast<hipStream_t>(stream)), "topk_sorted");
+}
+
 }  // extern "C"
 namespace {
 int prefill_dense_impl(const Shape& sh, const kascade_half* Q, const kascade_half* K, const kascade_half* V,

@@ -27,4 +27,12 @@ hipError_t launch_topk_split(const half_t* scores, int* out_idx, int rows, long 
                              int period, int k, int fill, void* workspace, const TopkRows* tr,
                              hipStream_t stream);
 
+// Reorders the first min(k, valid length) entries of every row of idx [rows, k] by descending score
+// (equal scores: ascending position); workspace: topk_sort_workspace_bytes(rows, k) bytes (0 for
+// short lists, which are sorted in LDS).
+long long topk_sort_workspace_bytes(int rows, int k);
+hipError_t launch_topk_sort_rows(const half_t* scores, int* idx, void* workspace, int rows,
+                                 long long row_stride, int uniform_len, const int* valid_len,
+                                 int period, int k, hipStream_t stream);
+
 }  // namespace kascade

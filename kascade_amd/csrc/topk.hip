@@ -844,6 +844,138 @@ SplitWs carve_ws(void* workspace, int rows, int max_chunks) {
     return ws;
 }
 
+
+// ---------------------------------------------------------------- rows ordered by score
+// Reorders the first n entries of every row's position list by descending score, equal scores by
+// ascending position: the order of torch.topk(...).indices.  A radix sort on the 16-bit order key
+// in two stable passes (low byte, then high byte), one workgroup per row.  The keys are gathered
+// once (the only dependent loads), then keys and positions move together between two buffers: in
+// LDS for lists of up to kSortLdsEntries entries, in the caller's workspace for longer ones.  A
+// wavefront owns a contiguous share of the list and walks it 64 entries at a time, the next
+// step's entries already in flight; the lanes that hold the same digit find each other with
+// eight ballots, so every entry's place follows from counters per (wavefront, digit) in LDS: no
+// atomics, nothing depends on timing, and the input order (ascending position) survives among
+// equal scores.
+constexpr int kSortLdsEntries = 4096;
+
+// lanes of the wavefront that are valid and hold the same 8-bit digit as this lane
+__device__ __forceinline__ uint64_t digit_peers(uint32_t d, bool valid) {
+    uint64_t peers = __ballot(valid);
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+        const bool bit = (d >> b) & 1u;
+        const uint64_t set = __ballot(bit);
+        peers &= bit ? set : ~set;
+    }
+    return valid ? peers : 0ull;
+}
+
+template <int WAVES, int LDS_N>
+__global__ __launch_bounds__(WAVES * 64) void topk_sort_rows_kernel(
+    const uint16_t* __restrict__ scores, int* __restrict__ idx, int* __restrict__ ws_pos,
+    uint16_t* __restrict__ ws_keys, long long row_stride, int uniform_len,
+    const int* __restrict__ valid_len, int period, int k) {
+    constexpr int kT = WAVES * 64;
+    static_assert(kT >= 256, "one thread per digit in the offset step");
+    __shared__ uint32_t s_cnt[WAVES][256];
+    __shared__ uint32_t s_wsum[4];
+    __shared__ int s_pos[LDS_N > 0 ? 2 * LDS_N : 1];
+    __shared__ uint16_t s_key[LDS_N > 0 ? 2 * LDS_N : 2];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const long long row = blockIdx.x;
+    const int len = valid_len ? min(valid_len[(int)(row % period)], uniform_len) : uniform_len;
+    const int n = max(0, min(k, len));   // entries beyond n name positions past the row's end: they stay
+    if (n <= 1) return;
+    const uint16_t* src = scores + row * row_stride;
+    int* first = idx + row * (long long)k;
+    int *pos_a, *pos_b;
+    uint16_t *key_a, *key_b;
+    if constexpr (LDS_N > 0) {
+        pos_a = s_pos; pos_b = s_pos + LDS_N; key_a = s_key; key_b = s_key + LDS_N;
+    } else {
+        pos_a = first; pos_b = ws_pos + row * (long long)k;
+        key_a = ws_keys + row * 2ll * k; key_b = key_a + k;
+    }
+    for (int i = tid; i < n; i += kT) {
+        const int pos = first[i];
+        if constexpr (LDS_N > 0) pos_a[i] = pos;
+        key_a[i] = (uint16_t)order_key(src[pos]);
+    }
+    __syncthreads();
+
+    const int seg = (n + kT - 1) / kT * 64;
+    const int s0 = min(n, wave * seg), s1 = min(n, s0 + seg);
+    const uint64_t below = (1ull << lane) - 1ull;
+    volatile uint32_t* mine = s_cnt[wave];
+
+    for (int pass = 0; pass < 2; ++pass) {
+        const int* from_pos = pass ? pos_b : pos_a;
+        const uint16_t* from_key = pass ? key_b : key_a;
+        int* to_pos = pass ? first : pos_b;
+        const int shift = 8 * pass;
+        for (int i = tid; i < WAVES * 256; i += kT) (&s_cnt[0][0])[i] = 0;
+        __syncthreads();
+        // how many entries of each digit this wavefront's share holds
+        {
+            bool valid = s0 + lane < s1;
+            uint32_t key = valid ? from_key[s0 + lane] : 0u;
+            for (int base = s0; base < s1; base += 64) {
+                const bool nvalid = base + 64 + lane < s1;
+                const uint32_t nkey = nvalid ? from_key[base + 64 + lane] : 0u;
+                const uint32_t d = (key >> shift) & 255u;
+                const uint64_t peers = digit_peers(d, valid);
+                if (valid && (peers & below) == 0) mine[d] += (uint32_t)__popcll(peers);
+                valid = nvalid; key = nkey;
+            }
+        }
+        __syncthreads();
+        // thread t < 256 owns digit 255 - t: the entries with a larger digit come first, then the
+        // earlier shares' entries of the same digit
+        {
+            const int d = 255 - (tid & 255);
+            uint32_t c[WAVES], total = 0;
+            if (tid < 256) {
+#pragma unroll
+                for (int w = 0; w < WAVES; ++w) { c[w] = s_cnt[w][d]; total += c[w]; }
+            }
+            const uint32_t inc = wave_incl_scan(total);
+            if (tid < 256 && lane == 63) s_wsum[wave] = inc;
+            __syncthreads();
+            if (tid < 256) {
+                uint32_t start = inc - total;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) if (w < wave) start += s_wsum[w];
+#pragma unroll
+                for (int w = 0; w < WAVES; ++w) { s_cnt[w][d] = start; start += c[w]; }
+            }
+        }
+        __syncthreads();
+        // place: the counter of a digit is read by all its lanes, then advanced by the first of them
+        {
+            bool valid = s0 + lane < s1;
+            int pos = valid ? from_pos[s0 + lane] : 0;
+            uint32_t key = valid ? from_key[s0 + lane] : 0u;
+            for (int base = s0; base < s1; base += 64) {
+                const bool nvalid = base + 64 + lane < s1;
+                const int npos = nvalid ? from_pos[base + 64 + lane] : 0;
+                const uint32_t nkey = nvalid ? from_key[base + 64 + lane] : 0u;
+                const uint32_t d = (key >> shift) & 255u;
+                const uint64_t peers = digit_peers(d, valid);
+                const uint32_t rank = (uint32_t)__popcll(peers & below);
+                const uint32_t at = valid ? mine[d] : 0u;
+                if (valid && rank == 0) mine[d] = at + (uint32_t)__popcll(peers);
+                if (valid) {
+                    to_pos[at + rank] = pos;
+                    if (pass == 0) key_b[at + rank] = (uint16_t)key;
+                }
+                valid = nvalid; pos = npos; key = nkey;
+            }
+        }
+        __syncthreads();   // the second pass reads what other wavefronts placed
+    }
+}
+
 }  // namespace
 
 int topk_max_register_row() { return 16 * kChunk; }
@@ -918,6 +1050,27 @@ hipError_t launch_topk(const half_t* scores, int* out_idx, int rows, long long r
     else
         hipLaunchKernelGGL(topk_select_kernel, dim3(rows), dim3(kThreads), 0, stream, src, out_idx,
                            row_stride, uniform_len, valid_len, n_sel, period, k, fill, ro);
+    return hipGetLastError();
+}
+
+long long topk_sort_workspace_bytes(int rows, int k) {
+    return k <= kSortLdsEntries ? 0 : 8ll * rows * k;   // positions (4 bytes) and two key buffers (2 + 2)
+}
+
+hipError_t launch_topk_sort_rows(const half_t* scores, int* idx, void* workspace, int rows,
+                                 long long row_stride, int uniform_len, const int* valid_len,
+                                 int period, int k, hipStream_t stream) {
+    if (rows == 0) return hipSuccess;
+    const uint16_t* src = reinterpret_cast<const uint16_t*>(scores);
+    if (k <= kSortLdsEntries) {
+        hipLaunchKernelGGL((topk_sort_rows_kernel<4, kSortLdsEntries>), dim3(rows), dim3(256), 0, stream, src, idx,
+                           (int*)nullptr, (uint16_t*)nullptr, row_stride, uniform_len, valid_len, period, k);
+    } else {
+        int* ws_pos = static_cast<int*>(workspace);
+        uint16_t* ws_keys = reinterpret_cast<uint16_t*>(ws_pos + (long long)rows * k);
+        hipLaunchKernelGGL((topk_sort_rows_kernel<16, 0>), dim3(rows), dim3(1024), 0, stream, src, idx, ws_pos,
+                           ws_keys, row_stride, uniform_len, valid_len, period, k);
+    }
     return hipGetLastError();
 }
 

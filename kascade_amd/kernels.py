@@ -520,6 +520,29 @@ def topk_indices(scores: torch.Tensor, k: int, valid_len=None, n_sel=None,
     return out, rows_out
 
 
+def topk_sorted(scores: torch.Tensor, k: int, valid_len=None, uniform_len: Optional[int] = None) -> torch.Tensor:
+    """``torch.topk(scores[..., :uniform_len], k, dim=-1).indices.to(int32)`` in the reference's own
+    form (EfficientKascadeStrategy.py:82, 90, 111): full-width rows, largest score first, equal
+    scores by ascending position; a row with fewer than k valid entries (valid_len, an int32
+    device tensor indexed by row % len) continues with the positions past its end.  For a
+    consumer that slices its own prefix of a row; the kernels here take ``topk_indices``."""
+    lib = _lib.init()
+    _req(scores, torch.float16, "scores")
+    Lrow = scores.shape[-1]
+    lead = scores.shape[:-1]
+    rows = int(math.prod(lead)) if len(lead) else 1
+    ulen = Lrow if uniform_len is None else uniform_len
+    period = 1
+    if valid_len is not None:
+        _req(valid_len, torch.int32, "valid_len"); period = valid_len.numel()
+    out = torch.empty(*lead, k, device=scores.device, dtype=torch.int32)
+    ws = torch.empty(max(1, lib.kascade_topk_sorted_workspace_bytes(rows, ulen, k)), dtype=torch.uint8,
+                     device=scores.device)
+    _lib.check(lib.kascade_topk_sorted_call(_ptr(scores), _ptr(out), rows, Lrow, ulen, _ptr(valid_len), period, k,
+                                            _ptr(ws), _stream()))
+    return out
+
+
 # --------------------------------------------------------------- prefill
 def prefill_recompute0(Q, K, V) -> Tuple[torch.Tensor, torch.Tensor]:
     """``prefill_recomp0_kernel(Q, K, V) -> (log_sum, O)`` (out_idx=[3,4];

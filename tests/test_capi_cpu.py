@@ -54,6 +54,18 @@ def _err(lib):
     return lib.kascade_get_last_error().decode()
 
 
+def test_sorted_topk_workspace_and_argument_checks(lib):
+    import ctypes
+    assert lib.kascade_topk_sorted_workspace_bytes(8192, 32768, 3328) == 0     # lists of up to 4096 entries: LDS
+    assert (lib.kascade_topk_sorted_workspace_bytes(32, 524288, 52480)
+            == (8 * 32 * 52480 + 255) // 256 * 256 + lib.kascade_topk_workspace_bytes(32, 524288))
+    p = ctypes.c_void_p(256)
+    assert lib.kascade_topk_sorted_call(p, p, 4, 10000, 10000, None, 1, 5000, None, None) == -1
+    assert "workspace" in _err(lib)
+    assert lib.kascade_topk_sorted_call(p, p, 4, 100, 100, None, 1, 101, p, None) == -1
+    assert "k <= uniform_len" in _err(lib)
+
+
 def test_null_pointers_are_rejected(lib):
     from kascade_amd._lib import Strides
     s = Strides(8, 8, 8)
