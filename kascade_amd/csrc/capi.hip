@@ -541,7 +541,7 @@ int kascade_topk_rows_call(const kascade_half* scores, int32_t* out_idx, int row
     if (period <= 0) period = 1;
     hipStream_t s = static_cast<hipStream_t>(stream);
     // rows of up to 131072 entries that start 16-byte aligned fit one workgroup's registers: one
-    // launch; longer (or unaligned long) rows go to several workgroups per row, six launches
+    // launch; longer (or unaligned long) rows go to several workgroups per row, four launches
     const bool one_workgroup = uniform_len <= topk_max_register_row() &&
                                (reinterpret_cast<uintptr_t>(scores) & 15) == 0 && row_stride % 8 == 0;
     if (!one_workgroup && workspace && topk_split_workspace_bytes(rows, uniform_len) > 0)

@@ -594,25 +594,44 @@ void topk_select_reg_kernel(
 
 // --------------------------------------------------------------------------
 // Long rows: the same radix select spread over several workgroups per row.
-// Every workgroup owns one chunk of kSplitChunk entries of one row; per-row state
-// lives in a caller-provided workspace:
-//   hist1 [rows][2048]            coarse histogram (atomically merged)
-//   sel   [rows][8]               {mode, b1, cum_above, T, r, n, len}
-//   cinfo [rows][chunks][34]      per chunk: fine histogram of bin b1 (32) and the
+// Every workgroup owns one chunk of kSplitChunk entries of one row and holds it in registers
+// (kSplitU 16-byte loads per thread, all in flight at once); per-row state lives in a
+// caller-provided workspace:
+//   hist1  [rows][2048]           coarse histogram (atomically merged)
+//   arrive [rows][2]              workgroups of the row that have finished pass 1 / pass 2
+//   sel    [rows][8]              {mode, b1, cum_above, T, r, n, len}
+//   cinfo  [rows][chunks][34]     per chunk: fine histogram of bin b1 (32) and the
 //                                 number of entries in bins above b1
-//   coff  [rows][chunks][2]       per chunk: selected-greater / equal counts before it
-// Launch sequence: zero -> hist1 -> scan1 -> hist2 -> scan2 -> write.
+//   coff   [rows][chunks][2]      per chunk: selected-greater / equal counts before it
+// Launch sequence: zero -> hist1 -> [scan1] -> hist2 -> [scan2] -> write.  With few workgroups
+// (a handful of very long rows: decode) the scan over a row's merged histogram is done by the
+// row's last workgroup to finish its pass (FUSED: an arrival counter per row), which saves the
+// two small launches; what one workgroup leaves for another of the same launch goes through
+// device-coherent atomics, stores and loads.  With thousands of rows (prefill) the counter's
+// round trip at the end of every workgroup costs more than the launches, so the scans stay
+// kernels of their own.
 // --------------------------------------------------------------------------
-constexpr int kSplitChunk = 16384;
+constexpr int kSplitU = 4;
+constexpr int kSplitChunk = kSplitU * kChunk;   // 32768 entries per workgroup
 constexpr int kSelWords = 8;
 constexpr int kInfoWords = 34;
+constexpr int kHistCopies = 4;
+constexpr long long kSplitFusedMax = 2048;   // workgroups up to which the scans are fused into the passes
 
 struct SplitWs {
     uint32_t* hist1;
+    uint32_t* arrive;
     uint32_t* sel;
     uint32_t* cinfo;
     uint32_t* coff;
 };
+
+__device__ __forceinline__ uint32_t load_device_u32(const uint32_t* p) {
+    return __hip_atomic_load(const_cast<uint32_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_device_u32(uint32_t* p, uint32_t v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 __device__ __forceinline__ void row_params(const int* valid_len, const int* n_sel, int period,
                                            int uniform_len, int k, long long row, int& len, int& n) {
@@ -622,161 +641,269 @@ __device__ __forceinline__ void row_params(const int* valid_len, const int* n_se
     n = max(0, min(n, k));
 }
 
+// The chunk [c0, c1) of a row as order keys: thread t holds entries c0 + u*8192 + 8t .. +8 for
+// u = 0..kSplitU-1 (every load instruction covers consecutive 16-byte pieces).
+__device__ __forceinline__ void load_chunk(const uint16_t* __restrict__ src, bool aligned, int c0, int c1,
+                                           uint32_t (&keys)[kSplitU][8], int (&nv)[kSplitU]) {
+#pragma unroll
+    for (int u = 0; u < kSplitU; ++u) {
+        const int base = c0 + u * kChunk + (int)threadIdx.x * 8;
+        nv[u] = 0;
+        if (base < c1) nv[u] = load_keys(src, aligned, base, c1, keys[u]);
+    }
+}
+
+// True in every thread of the row's last workgroup to get here (all of the row's `expected`
+// workgroups call it once per pass).  The caller's device-coherent stores and atomics are
+// waited for before the workgroup counts itself in.
+__device__ __forceinline__ bool last_of_row(uint32_t* counter, int expected, int* s_flag) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const uint32_t arrived = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *s_flag = (arrived == (uint32_t)(expected - 1));
+    }
+    __syncthreads();
+    return *s_flag != 0;
+}
+
 __global__ __launch_bounds__(256) void topk_zero_kernel(uint32_t* p, long long n) {
     long long i = (long long)blockIdx.x * 256 + threadIdx.x;
     if (i < n) p[i] = 0;
 }
 
-__global__ __launch_bounds__(kThreads) void topk_split_hist1_kernel(
+// The bin that holds the n-th largest entry of a row whose coarse histogram is complete (all
+// 1024 threads of a workgroup).
+__device__ __forceinline__ void split_scan1(const uint32_t* gh, uint32_t* sel, int n, int len, uint32_t* s_wave) {
+    const int tid = threadIdx.x;
+    const int rb0 = kBins1 - 1 - 2 * tid;   // this thread's bins, in descending order
+    const uint32_t h0 = load_device_u32(gh + rb0), h1 = load_device_u32(gh + rb0 - 1);
+    uint32_t total;
+    const uint32_t above0 = block_excl_scan(h0 + h1, s_wave, &total);
+    const uint32_t above1 = above0 + h0;
+    const uint32_t un = (uint32_t)n;
+    if (above0 < un && un <= above0 + h0) {
+        sel[1] = rb0; sel[2] = above0;
+    } else if (above1 < un && un <= above1 + h1) {
+        sel[1] = rb0 - 1; sel[2] = above1;
+    }
+    if (tid == 0) { sel[0] = 1; sel[5] = (uint32_t)n; sel[6] = (uint32_t)len; }
+}
+
+template <bool FUSED>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8))) void topk_split_hist1_kernel(
     const uint16_t* __restrict__ scores, long long row_stride, int uniform_len,
     const int* __restrict__ valid_len, const int* __restrict__ n_sel, int period, int k, SplitWs ws) {
-    __shared__ uint32_t s_hist[kBins1];
+    __shared__ uint32_t s_hist[kHistCopies][kBins1];
+    __shared__ uint32_t s_wave[kWaves];
+    __shared__ int s_flag;
     const int tid = threadIdx.x;
     const long long row = blockIdx.y;
     int len, n;
     row_params(valid_len, n_sel, period, uniform_len, k, row, len, n);
+    uint32_t* sel = ws.sel + row * kSelWords;
+    if (len <= n || n == 0) {   // nothing to select: the write pass lists the row's head
+        if (FUSED && blockIdx.x == 0 && tid == 0) { sel[0] = 0; sel[5] = (uint32_t)n; sel[6] = (uint32_t)len; }
+        return;
+    }
     const int c0 = blockIdx.x * kSplitChunk;
-    if (len <= n || n == 0 || c0 >= len) return;
+    if (c0 >= len) return;
     const int c1 = min(len, c0 + kSplitChunk);
     const uint16_t* src = scores + row * row_stride;
     const bool aligned = ((reinterpret_cast<uintptr_t>(src) & 15) == 0);
-    for (int i = tid; i < kBins1; i += kThreads) s_hist[i] = 0;
+    uint32_t keys[kSplitU][8];
+    int nv[kSplitU];
+    load_chunk(src, aligned, c0, c1, keys, nv);
+    for (int i = tid; i < kHistCopies * kBins1; i += kThreads) (&s_hist[0][0])[i] = 0;
     __syncthreads();
-    // zeros (pooled probabilities underflow to +0 by the thousand) are counted with a ballot
-    // per wavefront instead of that many atomics on one address; the loop bounds are uniform
-    // over a wavefront's lanes up to the ragged end, where absent lanes contribute nothing
-    uint32_t zeros = 0;
-    for (int base0 = c0; base0 < c1; base0 += kChunk) {
-        const int base = base0 + tid * 8;
-        uint32_t keys[8];
-        const int nv = (base < c1) ? load_keys(src, aligned, base, c1, keys) : 0;
+    // +0 (pooled probabilities underflow to it by the thousand) is not counted: its number is
+    // the chunk's length minus the sum of the others.  The other entries go to one of four
+    // copies of the histogram, chosen by the lane, which spreads the crowded bins.
+    uint32_t* mine = s_hist[tid & (kHistCopies - 1)];
+    uint32_t counted = 0;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const bool in = e < nv;
-            const bool zero = in && keys[e] == 0x8000u;
-            zeros += (uint32_t)__popcll(__ballot(zero));
-            if (in && !zero) atomicAdd(&s_hist[keys[e] >> 5], 1u);
-        }
-    }
-    if ((tid & 63) == 0 && zeros) atomicAdd(&s_hist[0x8000u >> 5], zeros);
+    for (int u = 0; u < kSplitU; ++u)
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            if (e < nv[u] && keys[u][e] != 0x8000u) {
+                atomicAdd(&mine[keys[u][e] >> 5], 1u);
+                ++counted;
+            }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) counted += __shfl_xor(counted, o);
+    if ((tid & 63) == 0) s_wave[tid >> 6] = counted;
     __syncthreads();
     uint32_t* gh = ws.hist1 + row * kBins1;
     for (int i = tid; i < kBins1; i += kThreads) {
-        uint32_t c = s_hist[i];
+        uint32_t c = 0;
+#pragma unroll
+        for (int j = 0; j < kHistCopies; ++j) c += s_hist[j][i];
+        if (i == (int)(0x8000u >> 5)) {
+            uint32_t all = 0;
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) all += s_wave[w];
+            c += (uint32_t)(c1 - c0) - all;
+        }
         if (c) atomicAdd(&gh[i], c);
     }
+    if (!FUSED) return;
+    const int nchunks = (len + kSplitChunk - 1) / kSplitChunk;
+    if (!last_of_row(ws.arrive + 2 * row, nchunks, &s_flag)) return;
+    split_scan1(gh, sel, n, len, s_wave);
 }
 
 __global__ __launch_bounds__(kThreads) void topk_split_scan1_kernel(
     int uniform_len, const int* __restrict__ valid_len, const int* __restrict__ n_sel, int period,
     int k, SplitWs ws) {
     __shared__ uint32_t s_wave[kWaves];
-    const int tid = threadIdx.x;
     const long long row = blockIdx.x;
     int len, n;
     row_params(valid_len, n_sel, period, uniform_len, k, row, len, n);
     uint32_t* sel = ws.sel + row * kSelWords;
     if (len <= n || n == 0) {
-        if (tid == 0) { sel[0] = 0; sel[5] = (uint32_t)n; sel[6] = (uint32_t)len; }
+        if (threadIdx.x == 0) { sel[0] = 0; sel[5] = (uint32_t)n; sel[6] = (uint32_t)len; }
         return;
     }
-    const uint32_t* gh = ws.hist1 + row * kBins1;
-    const int rb0 = kBins1 - 1 - 2 * tid;
-    const uint32_t c0 = gh[rb0], c1 = gh[rb0 - 1];
-    uint32_t total;
-    const uint32_t above0 = block_excl_scan(c0 + c1, s_wave, &total);
-    const uint32_t above1 = above0 + c0;
-    const uint32_t un = (uint32_t)n;
-    if (above0 < un && un <= above0 + c0) {
-        sel[1] = rb0; sel[2] = above0;
-    } else if (above1 < un && un <= above1 + c1) {
-        sel[1] = rb0 - 1; sel[2] = above1;
-    }
-    if (tid == 0) { sel[0] = 1; sel[5] = (uint32_t)n; sel[6] = (uint32_t)len; }
+    split_scan1(ws.hist1 + row * kBins1, sel, n, len, s_wave);
 }
 
-__global__ __launch_bounds__(kThreads) void topk_split_hist2_kernel(
-    const uint16_t* __restrict__ scores, long long row_stride, int max_chunks, SplitWs ws) {
+// From the chunks' fine histograms of a row: the threshold key T, the number r of entries equal
+// to T that still fit, and every chunk's offsets into the output.  One wavefront, lane c for
+// chunk c (64 chunks per round).
+__device__ __forceinline__ void split_scan2(uint32_t* sel, const uint32_t* rinfo, uint32_t* off, int nchunks) {
+    const int lane = threadIdx.x & 63;
+    const uint32_t n = sel[5], b1 = sel[1];
+    uint32_t h[32];
+#pragma unroll
+    for (int j = 0; j < 32; ++j) h[j] = 0;
+    for (int cb = 0; cb < nchunks; cb += 64) {
+        const int c = cb + lane;
+        if (c < nchunks) {
+#pragma unroll
+            for (int j = 0; j < 32; ++j) h[j] += load_device_u32(rinfo + c * kInfoWords + j);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 32; ++j)
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) h[j] += __shfl_xor(h[j], o);
+    // the fine bin of the n-th largest entry, from the top (bin 0 takes whatever is left)
+    uint32_t above = sel[2];
+    int b2 = 0;
+    bool found = false;
+#pragma unroll
+    for (int j = 31; j >= 1; --j) {
+        if (!found) {
+            if (above + h[j] >= n) { found = true; b2 = j; }
+            else above += h[j];
+        }
+    }
+    const uint32_t r = n - above;
+    if (lane == 0) { sel[3] = (b1 << 5) | (uint32_t)b2; sel[4] = r; }
+    // per-chunk counts of entries above T and equal to T, and their exclusive prefixes
+    uint32_t gt_run = 0, eq_run = 0;
+    for (int cb = 0; cb < nchunks; cb += 64) {
+        const int c = cb + lane;
+        uint32_t gt = 0, eq = 0;
+        if (c < nchunks) {
+            gt = load_device_u32(rinfo + c * kInfoWords + 32);
+#pragma unroll
+            for (int j = 0; j < 32; ++j) {
+                const uint32_t v = load_device_u32(rinfo + c * kInfoWords + j);
+                gt += (j > b2) ? v : 0u;
+                eq += (j == b2) ? v : 0u;
+            }
+        }
+        const uint32_t gi = wave_incl_scan(gt), ei = wave_incl_scan(eq);
+        if (c < nchunks) { off[2 * c] = gt_run + gi - gt; off[2 * c + 1] = eq_run + ei - eq; }
+        gt_run += __shfl(gi, 63);
+        eq_run += __shfl(ei, 63);
+    }
+}
+
+// Pass 2 of a chunk: the fine histogram of the threshold bin and the count of entries above it.
+// The chunk's loads are issued for the row's full width before the row's state (its length,
+// the threshold bin) has arrived, and cut down to the length afterwards.
+template <bool FUSED>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8))) void topk_split_hist2_kernel(
+    const uint16_t* __restrict__ scores, long long row_stride, int uniform_len, int max_chunks, SplitWs ws) {
     __shared__ uint32_t s_hist2[32];
     __shared__ uint32_t s_gt1;
-    const int tid = threadIdx.x;
+    __shared__ int s_flag;
+    const int tid = threadIdx.x, lane = tid & 63;
     const long long row = blockIdx.y;
-    const uint32_t* sel = ws.sel + row * kSelWords;
-    const int len = (int)sel[6];
+    uint32_t* sel = ws.sel + row * kSelWords;
     const int c0 = blockIdx.x * kSplitChunk;
-    if (sel[0] == 0 || c0 >= len) return;
-    const int c1 = min(len, c0 + kSplitChunk);
-    const uint32_t b1 = sel[1];
+    if (c0 >= uniform_len) return;
     const uint16_t* src = scores + row * row_stride;
     const bool aligned = ((reinterpret_cast<uintptr_t>(src) & 15) == 0);
+    uint32_t keys[kSplitU][8];
+    int nv[kSplitU];
+    load_chunk(src, aligned, c0, min(uniform_len, c0 + kSplitChunk), keys, nv);
+    const int len = (int)sel[6];
+    if (sel[0] == 0 || c0 >= len) return;
+    const uint32_t b1 = sel[1];
+#pragma unroll
+    for (int u = 0; u < kSplitU; ++u) nv[u] = max(0, min(nv[u], len - (c0 + u * kChunk + tid * 8)));
     if (tid < 32) s_hist2[tid] = 0;
     if (tid == 32) s_gt1 = 0;
     __syncthreads();
-    uint32_t gt1 = 0;
-    for (int base = c0 + tid * 8; base < c1; base += kChunk) {
-        uint32_t keys[8];
-        int nv = load_keys(src, aligned, base, c1, keys);
+    uint32_t gt1 = 0, zeros = 0;
+    const bool zero_bin = b1 == (0x8000u >> 5);   // uniform: the threshold lies among +0 and the smallest subnormals
+#pragma unroll
+    for (int u = 0; u < kSplitU; ++u)
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            if (e < nv) {
-                const uint32_t hb = keys[e] >> 5;
-                if (hb == b1) atomicAdd(&s_hist2[keys[e] & 31u], 1u);
-                gt1 += (hb > b1);
+            const bool in = e < nv[u];
+            const uint32_t hb = keys[u][e] >> 5;
+            if (zero_bin) {   // that many atomics on one address would serialise: a ballot per wavefront
+                const bool zero = in && keys[u][e] == 0x8000u;
+                zeros += (uint32_t)__popcll(__ballot(zero));
+                if (in && !zero && hb == b1) atomicAdd(&s_hist2[keys[u][e] & 31u], 1u);
+            } else if (in && hb == b1) {
+                atomicAdd(&s_hist2[keys[u][e] & 31u], 1u);
             }
+            gt1 += (in && hb > b1);
         }
-    }
-    if (gt1) atomicAdd(&s_gt1, gt1);
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) gt1 += __shfl_xor(gt1, o);
+    if (lane == 0 && gt1) atomicAdd(&s_gt1, gt1);
+    if (lane == 0 && zeros) atomicAdd(&s_hist2[0], zeros);   // +0 is entry 0 of its bin
     __syncthreads();
     uint32_t* info = ws.cinfo + (row * max_chunks + blockIdx.x) * kInfoWords;
-    if (tid < 32) info[tid] = s_hist2[tid];
-    if (tid == 32) info[32] = s_gt1;
+    if (tid < 32) store_device_u32(info + tid, s_hist2[tid]);
+    if (tid == 32) store_device_u32(info + 32, s_gt1);
+    if (!FUSED) return;
+    const int nchunks = (len + kSplitChunk - 1) / kSplitChunk;
+    if (!last_of_row(ws.arrive + 2 * row + 1, nchunks, &s_flag)) return;
+    if (tid >= 64) return;
+    split_scan2(sel, ws.cinfo + row * max_chunks * kInfoWords, ws.coff + row * max_chunks * 2, nchunks);
 }
 
 __global__ __launch_bounds__(64) void topk_split_scan2_kernel(int max_chunks, SplitWs ws) {
     const long long row = blockIdx.x;
     uint32_t* sel = ws.sel + row * kSelWords;
     if (sel[0] == 0) return;
-    const int lane = threadIdx.x;
-    const int len = (int)sel[6];
-    const uint32_t n = sel[5];
-    const int nchunks = (len + kSplitChunk - 1) / kSplitChunk;
-    const uint32_t* info = ws.cinfo + row * max_chunks * kInfoWords;
-    // lanes 0..31: total fine histogram
-    uint32_t h = 0;
-    if (lane < 32)
-        for (int c = 0; c < nchunks; ++c) h += info[c * kInfoWords + lane];
-    // suffix scan over the 32 bins (descending), done by every lane redundantly through shuffles
-    uint32_t above = sel[2];
-    int b2 = 31;
-    for (; b2 > 0; --b2) {
-        const uint32_t c = __shfl(h, b2);
-        if (above + c >= n) break;
-        above += c;
-    }
-    const uint32_t r = n - above;
-    if (lane == 0) { sel[3] = (sel[1] << 5) | (uint32_t)b2; sel[4] = r; }
-    // per-chunk counts and their exclusive prefix (chunks are few: serial over c, parallel over bins)
-    uint32_t gt_run = 0, eq_run = 0;
-    uint32_t* off = ws.coff + row * max_chunks * 2;
-    for (int c = 0; c < nchunks; ++c) {
-        uint32_t v = (lane < 32 && lane > b2) ? info[c * kInfoWords + lane] : 0u;
-#pragma unroll
-        for (int o = 16; o > 0; o >>= 1) v += __shfl_xor(v, o);
-        const uint32_t gt = info[c * kInfoWords + 32] + v;
-        const uint32_t eq = info[c * kInfoWords + b2];
-        if (lane == 0) { off[2 * c] = gt_run; off[2 * c + 1] = eq_run; }
-        gt_run += gt;
-        eq_run += eq;
-    }
+    const int nchunks = ((int)sel[6] + kSplitChunk - 1) / kSplitChunk;
+    split_scan2(sel, ws.cinfo + row * max_chunks * kInfoWords, ws.coff + row * max_chunks * 2, nchunks);
 }
 
-__global__ __launch_bounds__(kThreads) void topk_split_write_kernel(
-    const uint16_t* __restrict__ scores, int* __restrict__ out, long long row_stride, int k,
-    int fill, int max_chunks, SplitWs ws, RowsOut ro) {
-    __shared__ uint32_t s_wave[kWaves];
-    const int tid = threadIdx.x;
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8))) void topk_split_write_kernel(
+    const uint16_t* __restrict__ scores, int* __restrict__ out, long long row_stride, int uniform_len,
+    int k, int fill, int max_chunks, SplitWs ws, RowsOut ro) {
+    static_assert(kSplitU * kWaves == 64, "one wavefront scans the (load, wavefront) totals");
+    __shared__ uint32_t s_tot[kSplitU * kWaves];
+    __shared__ uint32_t s_pre[kSplitU * kWaves];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const long long row = blockIdx.y;
     const uint32_t* sel = ws.sel + row * kSelWords;
+    const int c0 = blockIdx.x * kSplitChunk;
+    const uint16_t* src = scores + row * row_stride;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(src) & 15) == 0);
+    // the chunk's loads go out before the row's state has arrived (cut down to its length below)
+    uint32_t keys[kSplitU][8];
+    int nv[kSplitU];
+    load_chunk(src, aligned, c0, min(uniform_len, c0 + kSplitChunk), keys, nv);
     const int len = (int)sel[6];
     const int n = (int)sel[5];
     int* dst = out + row * (long long)k;
@@ -785,7 +912,6 @@ __global__ __launch_bounds__(kThreads) void topk_split_write_kernel(
         dst[slot] = pos;
         if (rdst) rdst[slot] = to_cache_row(ro, row, pos);
     };
-    const int c0 = blockIdx.x * kSplitChunk;
     if (blockIdx.x == 0) {
         if (sel[0] == 0) {
             for (int i = tid; i < k; i += kThreads) put(i, (i < n) ? i : fill);
@@ -794,52 +920,64 @@ __global__ __launch_bounds__(kThreads) void topk_split_write_kernel(
         for (int i = n + tid; i < k; i += kThreads) put(i, fill);
     }
     if (sel[0] == 0 || c0 >= len) return;
-    const int c1 = min(len, c0 + kSplitChunk);
     const uint32_t T = sel[3];
     const uint32_t r = sel[4];
     const uint32_t* off = ws.coff + (row * max_chunks + blockIdx.x) * 2;
-    uint32_t gt_base = off[0], eq_base = off[1];
-    const uint16_t* src = scores + row * row_stride;
-    const bool aligned = ((reinterpret_cast<uintptr_t>(src) & 15) == 0);
-    for (int cbase = c0; cbase < c1; cbase += kChunk) {
-        const int base = cbase + tid * 8;
-        uint32_t keys[8];
-        int nv = (base < c1) ? load_keys(src, aligned, base, c1, keys) : 0;
+    const uint32_t gt_base = off[0], eq_base = off[1];
+#pragma unroll
+    for (int u = 0; u < kSplitU; ++u) nv[u] = max(0, min(nv[u], len - (c0 + u * kChunk + tid * 8)));
+    // counts above / equal to T per (load, thread), packed; position order is (load, thread, entry)
+    uint32_t cnt[kSplitU], inc[kSplitU];
+#pragma unroll
+    for (int u = 0; u < kSplitU; ++u) {
         uint32_t gt = 0, eq = 0;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            if (e < nv) {
-                gt += (keys[e] > T);
-                eq += (keys[e] == T);
+            if (e < nv[u]) {
+                gt += (keys[u][e] > T);
+                eq += (keys[u][e] == T);
             }
         }
-        uint32_t total;
-        const uint32_t ex = block_excl_scan(gt | (eq << 16), s_wave, &total);
+        cnt[u] = gt | (eq << 16);
+        inc[u] = wave_incl_scan(cnt[u]);
+        if (lane == 63) s_tot[u * kWaves + wave] = inc[u];
+    }
+    __syncthreads();
+    if (wave == 0) {
+        const uint32_t t = s_tot[lane];
+        s_pre[lane] = wave_incl_scan(t) - t;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < kSplitU; ++u) {
+        const uint32_t ex = s_pre[u * kWaves + wave] + inc[u] - cnt[u];
         uint32_t my_gt = gt_base + (ex & 0xFFFFu);
         uint32_t my_eq = eq_base + (ex >> 16);
+        const int base = c0 + u * kChunk + tid * 8;
+        // stores straight from the threads: staging the chunk's list in LDS for full-width stores
+        // was measured slower (its two extra barriers cost more than the narrow stores)
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            if (e < nv) {
-                if (keys[e] > T) {
+            if (e < nv[u]) {
+                if (keys[u][e] > T) {
                     put(my_gt + min(my_eq, r), base + e);
                     ++my_gt;
-                } else if (keys[e] == T) {
+                } else if (keys[u][e] == T) {
                     if (my_eq < r) put(my_gt + my_eq, base + e);
                     ++my_eq;
                 }
             }
         }
-        gt_base += total & 0xFFFFu;
-        eq_base += total >> 16;
     }
 }
 
 SplitWs carve_ws(void* workspace, int rows, int max_chunks) {
     SplitWs ws;
     uint32_t* p = reinterpret_cast<uint32_t*>(workspace);
-    ws.hist1 = p; p += (size_t)rows * kBins1;
-    ws.sel = p;   p += (size_t)rows * kSelWords;
-    ws.cinfo = p; p += (size_t)rows * max_chunks * kInfoWords;
+    ws.hist1 = p;  p += (size_t)rows * kBins1;
+    ws.arrive = p; p += (size_t)rows * 2;       // right behind hist1: one launch zeroes both
+    ws.sel = p;    p += (size_t)rows * kSelWords;
+    ws.cinfo = p;  p += (size_t)rows * max_chunks * kInfoWords;
     ws.coff = p;
     return ws;
 }
@@ -983,7 +1121,7 @@ int topk_max_register_row() { return 16 * kChunk; }
 long long topk_split_workspace_bytes(int rows, long long row_len) {
     if (row_len < kSplitMinLen || rows > kSplitMaxRows) return 0;
     const long long chunks = (row_len + kSplitChunk - 1) / kSplitChunk;
-    return 4ll * rows * (kBins1 + kSelWords + chunks * (kInfoWords + 2));
+    return 4ll * rows * (kBins1 + 2 + kSelWords + chunks * (kInfoWords + 2));
 }
 
 namespace {
@@ -1009,19 +1147,28 @@ hipError_t launch_topk_split(const half_t* scores, int* out_idx, int rows, long 
     const int max_chunks = (max_len + kSplitChunk - 1) / kSplitChunk;
     SplitWs ws = carve_ws(workspace, rows, max_chunks);
     const uint16_t* src = reinterpret_cast<const uint16_t*>(scores);
-    const long long nz = (long long)rows * kBins1;
+    const long long nz = (long long)rows * (kBins1 + 2);   // histograms and arrival counters
     hipLaunchKernelGGL(topk_zero_kernel, dim3((unsigned)((nz + 255) / 256)), dim3(256), 0, stream,
                        ws.hist1, nz);
     dim3 grid(max_chunks, rows);
-    hipLaunchKernelGGL(topk_split_hist1_kernel, grid, dim3(kThreads), 0, stream, src, row_stride,
-                       uniform_len, valid_len, n_sel, period, k, ws);
-    hipLaunchKernelGGL(topk_split_scan1_kernel, dim3(rows), dim3(kThreads), 0, stream, uniform_len,
-                       valid_len, n_sel, period, k, ws);
-    hipLaunchKernelGGL(topk_split_hist2_kernel, grid, dim3(kThreads), 0, stream, src, row_stride,
-                       max_chunks, ws);
-    hipLaunchKernelGGL(topk_split_scan2_kernel, dim3(rows), dim3(64), 0, stream, max_chunks, ws);
+    // few workgroups: the scans ride on the histogram passes; many: launches of their own
+    const bool fused = (long long)rows * max_chunks <= kSplitFusedMax;
+    if (fused) {
+        hipLaunchKernelGGL(topk_split_hist1_kernel<true>, grid, dim3(kThreads), 0, stream, src, row_stride,
+                           uniform_len, valid_len, n_sel, period, k, ws);
+        hipLaunchKernelGGL(topk_split_hist2_kernel<true>, grid, dim3(kThreads), 0, stream, src, row_stride,
+                           uniform_len, max_chunks, ws);
+    } else {
+        hipLaunchKernelGGL(topk_split_hist1_kernel<false>, grid, dim3(kThreads), 0, stream, src, row_stride,
+                           uniform_len, valid_len, n_sel, period, k, ws);
+        hipLaunchKernelGGL(topk_split_scan1_kernel, dim3(rows), dim3(kThreads), 0, stream, uniform_len,
+                           valid_len, n_sel, period, k, ws);
+        hipLaunchKernelGGL(topk_split_hist2_kernel<false>, grid, dim3(kThreads), 0, stream, src, row_stride,
+                           uniform_len, max_chunks, ws);
+        hipLaunchKernelGGL(topk_split_scan2_kernel, dim3(rows), dim3(64), 0, stream, max_chunks, ws);
+    }
     hipLaunchKernelGGL(topk_split_write_kernel, grid, dim3(kThreads), 0, stream, src, out_idx,
-                       row_stride, k, fill, max_chunks, ws, ro);
+                       row_stride, uniform_len, k, fill, max_chunks, ws, ro);
     if (tr && tr->out_rows)
         return launch_translate_indices(out_idx, tr->out_rows, tr->block_table, rows / tr->rows_per_seq,
                                         (long long)tr->rows_per_seq * k, tr->max_pages, tr->page_shift,

@@ -47,7 +47,7 @@ def test_topk_workspace_sizing(lib):
     assert lib.kascade_topk_workspace_bytes(128, 1000) == 0          # short rows: one workgroup per row
     assert lib.kascade_topk_workspace_bytes(8192, 32768) == 0        # too many rows for the workspace
     n = lib.kascade_topk_workspace_bytes(32, 524288)
-    assert n == 4 * 32 * (2048 + 8 + 32 * 36)
+    assert n == 4 * 32 * (2048 + 2 + 8 + 16 * 36)   # 16 chunks of 32768 entries
 
 
 def _err(lib):
