@@ -542,8 +542,8 @@ int kascade_topk_rows_call(const kascade_half* scores, int32_t* out_idx, int row
     hipStream_t s = static_cast<hipStream_t>(stream);
     // rows of up to 131072 entries that start 16-byte aligned fit one workgroup's registers: one
     // launch; longer (or unaligned long) rows go to several workgroups per row, four launches
-    const bool one_workgroup = uniform_len <= topk_max_register_row() &&
-                               (reinterpret_cast<uintptr_t>(scores) & 15) == 0 && row_stride % 8 == 0;
+    const bool one_workgroup = uniform_len + (row_stride % 8 != 0 ? 7 : 0) <= topk_max_register_row() &&
+                               (reinterpret_cast<uintptr_t>(scores) & 15) == 0;
     if (!one_workgroup && workspace && topk_split_workspace_bytes(rows, uniform_len) > 0)
         return check_hip(launch_topk_split(H(scores), out_idx, rows, row_stride, uniform_len,
                                            uniform_len, valid_len, n_sel, period, k, fill_value,

@@ -20,7 +20,8 @@ hipError_t launch_topk(const half_t* scores, int* out_idx, int rows, long long r
 // Multi-workgroup variant for long rows.  Returns 0 bytes when the single-workgroup kernel
 // is the right choice (short rows, or too many rows for the 8 KB/row workspace).
 long long topk_split_workspace_bytes(int rows, long long row_len);
-// longest row (entries) the one-workgroup selection keeps in registers (rows must be 16-byte aligned)
+// longest row (entries) the one-workgroup selection keeps in registers (the tensor must start 16-byte
+// aligned; rows that start off a boundary count 7 slots more)
 int topk_max_register_row();
 hipError_t launch_topk_split(const half_t* scores, int* out_idx, int rows, long long row_stride,
                              int max_len, int uniform_len, const int* valid_len, const int* n_sel,

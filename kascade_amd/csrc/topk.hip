@@ -267,7 +267,8 @@ __global__ __launch_bounds__(kThreads) void topk_select_kernel(
 //  * The compaction computes every (chunk, thread) offset with two barriers in all (per-chunk
 //    wavefront scans, then one scan over the chunk x wavefront totals), and stages the selected
 //    indices in LDS in their final order, so that the row's list leaves as full-width stores.
-// Rows must be 16-byte aligned and at most MAXC*8192 entries long (MAXC = 16: 131072 entries, 64
+// The tensor must start 16-byte aligned (its rows need not) and a row, with the up to 7 slots
+// between the boundary before it and its start, must fit MAXC*8192 slots (MAXC = 16: 131072, 64
 // registers of row data per thread, still one workgroup of 1024 threads per CU).
 template <int MAXC>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(MAXC <= 4 ? 8 : 4)))
@@ -300,7 +301,14 @@ void topk_select_reg_kernel(
     const int len = valid_len ? min(valid_len[pr], uniform_len) : uniform_len;
     int n = n_sel ? n_sel[pr] : k;
     n = max(0, min(n, k));
-    const uint16_t* src = scores + row * row_stride;
+    // A row that does not start on a 16-byte boundary (a row stride that is no multiple of 8) is
+    // read from the boundary before it: `lead` slots in front of the row count as absent, like
+    // the slots past its end, and every position below is taken in these shifted coordinates
+    // (the tensor itself starts on a boundary, so the slots in front belong to the row before).
+    const uint16_t* row_src = scores + row * row_stride;
+    const int lead = (int)((reinterpret_cast<uintptr_t>(row_src) & 15) >> 1);
+    const uint16_t* src = row_src - lead;
+    const int row_len = len;            // entries of the row itself
     int* dst = out + row * (long long)k;
     int* rdst = ro.rows ? ro.rows + row * (long long)k : nullptr;
     auto put = [&](int slot, int pos) {
@@ -308,33 +316,36 @@ void topk_select_reg_kernel(
         if (rdst) rdst[slot] = to_cache_row(ro, row, pos);
     };
 
-    if (len <= n || n == 0) {
+    if (row_len <= n || n == 0) {
         for (int i = tid; i < k; i += kThreads) put(i, (i < n) ? i : fill);
         return;
     }
-    const int nchunks = (len + kChunk - 1) / kChunk;   // <= MAXC (host)
+    const int slots = row_len + lead;   // the row in shifted coordinates: [lead, slots)
+    const int nchunks = (slots + kChunk - 1) / kChunk;   // <= MAXC (host)
 
-    // ---- the row: chunk c, entries [c*8192 + 8*tid, +8) as packed order keys ----
+    // ---- the row: chunk c, slots [c*8192 + 8*tid, +8) as packed order keys ----
     uint4_t data[MAXC];
-    // entries of chunk c that lie inside the row (recomputed where needed: an array of them
-    // would cost MAXC registers)
-    auto nv_of = [&](int c) { return max(0, min(8, len - (c * kChunk + tid * 8))); };
+    // slots of chunk c that lie before the row's end (recomputed where needed: an array of them
+    // would cost MAXC registers), and the absent slots in front (only the first thread has any)
+    auto nv_of = [&](int c) { return max(0, min(8, slots - (c * kChunk + tid * 8))); };
+    auto lead_of = [&](int c) { return (c == 0 && tid == 0) ? lead : 0; };
     // Every thread loads 16 bytes per chunk without a branch around the load, so that the loads
     // are in flight together: where the chunk's share lies past the end of the row the address
     // is pulled back inside it and the data replaced below.
-    const int last_full = max(len - 8, 0) & ~7;
+    const int last_full = max(slots - 8, 0) & ~7;
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
         data[c] = uint4_t{0, 0, 0, 0};
-        if (len >= 8)   // uniform
+        if (slots >= 8)   // uniform
             data[c] = *reinterpret_cast<const uint4_t*>(src + min(c * kChunk + tid * 8, last_full));
     }
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
         const int base = c * kChunk + tid * 8;
         const int nvc = nv_of(c);
+        const int ldc = lead_of(c);
         uint4_t raw = data[c];
-        if (nvc == 8) {
+        if (nvc == 8 && ldc == 0) {
             // order_key on both halves at once: negative values flip every bit, others the sign
             // bit; then at least 1
 #pragma unroll
@@ -344,8 +355,8 @@ void topk_select_reg_kernel(
             uint32_t w[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const uint32_t lo = (2 * e < nvc) ? max(order_key(src[base + 2 * e]), 1u) : 0u;
-                const uint32_t hi = (2 * e + 1 < nvc) ? max(order_key(src[base + 2 * e + 1]), 1u) : 0u;
+                const uint32_t lo = (2 * e < nvc && 2 * e >= ldc) ? max(order_key(src[base + 2 * e]), 1u) : 0u;
+                const uint32_t hi = (2 * e + 1 < nvc && 2 * e + 1 >= ldc) ? max(order_key(src[base + 2 * e + 1]), 1u) : 0u;
                 w[e] = lo | (hi << 16);
             }
             raw = uint4_t{w[0], w[1], w[2], w[3]};
@@ -371,7 +382,8 @@ void topk_select_reg_kernel(
     for (int c = 0; c < MAXC; ++c) {
         if (c < nchunks) {
             const int nvc = nv_of(c);
-            if (nvc == 8) {
+            const int ldc = lead_of(c);
+            if (nvc == 8 && ldc == 0) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     count1(data[c][j] & 0xFFFFu);
@@ -380,7 +392,7 @@ void topk_select_reg_kernel(
             } else if (nvc > 0) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e)
-                    if (e < nvc) count1((e & 1) ? (data[c][e >> 1] >> 16) : (data[c][e >> 1] & 0xFFFFu));
+                    if (e < nvc && e >= ldc) count1((e & 1) ? (data[c][e >> 1] >> 16) : (data[c][e >> 1] & 0xFFFFu));
             }
         }
     }
@@ -397,7 +409,7 @@ void topk_select_reg_kernel(
         uint32_t c1 = h1[0] + h1[1] + h1[2] + h1[3];
         uint32_t total;
         uint32_t above0 = block_excl_scan(c0 + c1, s_wave, &total);
-        const uint32_t skipped = (uint32_t)len - total;
+        const uint32_t skipped = (uint32_t)row_len - total;
         if (tid == kSkipOwner) c1 += skipped;
         if (tid > kSkipOwner) above0 += skipped;
         const uint32_t above1 = above0 + c0;
@@ -537,7 +549,7 @@ void topk_select_reg_kernel(
                 // where the next selected entry goes: after the earlier ones above T and the
                 // earlier ties taken
                 uint32_t pos = s_pgt[c * kWaves + wave] + (ex & 0xFFFFu) + min(my_eq, r);
-                const int base = c * kChunk + tid * 8;
+                const int base = c * kChunk + tid * 8 - lead;   // back to positions of the row
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const uint32_t code = pk_min_u16(pk_sub_sat_u16(data[c][j], tm1_r), kTwo);
@@ -1182,16 +1194,18 @@ hipError_t launch_topk(const half_t* scores, int* out_idx, int rows, long long r
     if (rows == 0) return hipSuccess;
     const RowsOut ro = rows_out(tr);
     const uint16_t* src = reinterpret_cast<const uint16_t*>(scores);
-    // rows that start 16-byte aligned and fit the register file of a workgroup are selected
-    // from registers; anything else streams the row three times
-    const bool aligned_rows = (reinterpret_cast<uintptr_t>(scores) & 15) == 0 && row_stride % 8 == 0;
-    if (aligned_rows && uniform_len <= 4 * kChunk)
+    // rows of a tensor that starts 16-byte aligned and that fit the register file of a workgroup
+    // are selected from registers (rows that start off a boundary bring up to 7 slots in front);
+    // anything else streams the row three times
+    const bool aligned_rows = (reinterpret_cast<uintptr_t>(scores) & 15) == 0;
+    const int slots = uniform_len + (row_stride % 8 != 0 ? 7 : 0);
+    if (aligned_rows && slots <= 4 * kChunk)
         hipLaunchKernelGGL(topk_select_reg_kernel<4>, dim3(rows), dim3(kThreads), 0, stream, src, out_idx,
                            row_stride, uniform_len, valid_len, n_sel, period, k, fill, ro);
-    else if (aligned_rows && uniform_len <= 8 * kChunk)
+    else if (aligned_rows && slots <= 8 * kChunk)
         hipLaunchKernelGGL(topk_select_reg_kernel<8>, dim3(rows), dim3(kThreads), 0, stream, src, out_idx,
                            row_stride, uniform_len, valid_len, n_sel, period, k, fill, ro);
-    else if (aligned_rows && uniform_len <= 16 * kChunk)
+    else if (aligned_rows && slots <= 16 * kChunk)
         hipLaunchKernelGGL(topk_select_reg_kernel<16>, dim3(rows), dim3(kThreads), 0, stream, src, out_idx,
                            row_stride, uniform_len, valid_len, n_sel, period, k, fill, ro);
     else

@@ -73,6 +73,37 @@ def test_topk_strided_unaligned_rows(cuda):
     _check(base.cpu()[:, :L], idx.cpu(), lambda r: K, lambda r: L, K, 0)
 
 
+@pytest.mark.parametrize("L,K", [(32763, 3328), (32765, 3328), (8191, 896), (65537, 6656), (131065, 13184), (1001, 128)])
+def test_topk_rows_of_odd_length_equal_aligned_rows(cuda, L, K):
+    """A prompt whose length is no multiple of 8 gives score rows that start off a 16-byte
+    boundary (all but every eighth).  They are read from the boundary before them, the slots in
+    front counted as absent; the result must be bit-equal to the same values in aligned rows, on
+    ragged lengths, ties, -inf runs and rows next to a neighbour full of large values."""
+    from kascade_amd import kernels
+    rows = 16
+    sc = _scores(rows, L, seed=L + 3)
+    sc[1, 500:900] = float("-inf")
+    sc[2] = 0.25
+    sc[3, : L // 2] = 0.0
+    sc[4, -7:] = 60000.0        # the slots in front of row 5 hold the largest values of the tensor
+    sc[6, :7] = 60000.0
+    valid = torch.tensor([L, L - 1, min(L, 8192), min(L, 8193), min(L, 5000), L, L - 3, min(L, 100)], dtype=torch.int32)
+    nsel = torch.tensor([K, K, 512, 512, 256, 0, K, 64], dtype=torch.int32).clamp(max=K)
+    Lp = (L + 7) // 8 * 8
+    padded = torch.zeros(rows, Lp, dtype=torch.float16)
+    padded[:, :L] = sc
+    dvalid, dnsel = valid.to(cuda), nsel.to(cuda)
+    tight = sc.to(cuda)                               # row stride L: rows 1.. start off a boundary
+    assert tight.data_ptr() % 16 == 0 and (L * 2) % 16 != 0
+    a = kernels.topk_indices(padded.to(cuda)[:, :L], K, valid_len=dvalid, n_sel=dnsel, fill_value=-1)
+    b = kernels.topk_indices(tight, K, valid_len=dvalid, n_sel=dnsel, fill_value=-1)
+    torch.cuda.synchronize()
+    assert torch.equal(a.cpu(), b.cpu())
+    _check(sc, b.cpu(), lambda r: nsel[r % 8], lambda r: valid[r % 8], K, -1)
+    u = kernels.topk_indices(tight, K, fill_value=-1)          # uniform rows: the full length
+    _check(sc, u.cpu(), lambda r: K, lambda r: L, K, -1)
+
+
 def test_topk_matches_torch_topk_sets_when_no_ties(cuda):
     from kascade_amd import kernels
     g = torch.Generator().manual_seed(4)
